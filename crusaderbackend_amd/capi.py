@@ -1,0 +1,141 @@
+"""ctypes binding of the C ABI declared in include/crusader_hip.h.
+
+This module is plumbing for tests and the benchmark: it loads the in-tree
+``lib/libcrusader_hip.so`` and passes raw device pointers (``tensor.data_ptr()``) and sizes
+straight through. There is no CPU fallback: if the shared library is missing, loading raises.
+"""
+import ctypes
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "lib", "libcrusader_hip.so")
+
+CRB_OK = 0
+CRB_EINVAL_SHAPE = -1
+CRB_ENULL = -2
+CRB_EHIP = -3
+CRB_EWORKSPACE = -4
+CRB_FLAG_RELU = 1
+
+_u32 = ctypes.c_uint32
+_ptr = ctypes.c_void_p
+
+
+class ConvGeom(ctypes.Structure):
+    """Mirror of ``crb_conv_geom``."""
+
+    _fields_ = [(n, _u32) for n in ("N", "IC", "IH", "IW", "OC", "FH", "FW", "OH", "OW", "sH", "sW", "pH", "pW")]
+
+    @classmethod
+    def make(cls, N, IC, IH, IW, OC, FH, FW, sH=1, sW=1, pH=0, pW=0, OH=None, OW=None):
+        if OH is None:
+            OH = (IH - FH + 2 * pH) // sH + 1
+        if OW is None:
+            OW = (IW - FW + 2 * pW) // sW + 1
+        return cls(N, IC, IH, IW, OC, FH, FW, OH, OW, sH, sW, pH, pW)
+
+
+# name -> (restype, argtypes); every symbol include/crusader_hip.h declares
+SIGNATURES = {
+    "crb_abi_version": (ctypes.c_int, []),
+    "crb_last_error_string": (ctypes.c_char_p, []),
+    "crb_release_workspace": (None, []),
+    "crb_sgemm_nn": (ctypes.c_int, [_ptr, _ptr, _ptr, _u32, _u32, _u32, _u32, _ptr]),
+    "crb_sgemm_tn": (ctypes.c_int, [_ptr, _ptr, _ptr, _u32, _u32, _u32, _u32, _ptr]),
+    "crb_sgemm_nt": (ctypes.c_int, [_ptr, _ptr, _ptr, _u32, _u32, _u32, _ptr]),
+    "crb_sgemm_nta": (ctypes.c_int, [_ptr, _ptr, _ptr, _u32, _u32, _u32, _u32, _ptr]),
+    "crb_linear_fwd": (ctypes.c_int, [_ptr, _ptr, _ptr, _ptr, _u32, _u32, _u32, _u32, _ptr]),
+    "crb_linear_dgrad": (ctypes.c_int, [_ptr, _ptr, _ptr, _u32, _u32, _u32, _ptr]),
+    "crb_linear_wgrad": (ctypes.c_int, [_ptr, _ptr, _ptr, _ptr, _u32, _u32, _u32, _ptr]),
+    "crb_conv_fwd": (ctypes.c_int, [_ptr, _ptr, _ptr, _ptr, ctypes.POINTER(ConvGeom), _u32, _ptr]),
+    "crb_conv_dgrad": (ctypes.c_int, [_ptr, _ptr, _ptr, ctypes.POINTER(ConvGeom), _ptr]),
+    "crb_conv_wgrad_workspace_bytes": (ctypes.c_size_t, [ctypes.POINTER(ConvGeom)]),
+    "crb_conv_wgrad": (ctypes.c_int, [_ptr, _ptr, _ptr, ctypes.POINTER(ConvGeom), _ptr, ctypes.c_size_t, _ptr]),
+    "crb_conv_bias": (ctypes.c_int, [_ptr, _ptr, _u32, _u32, _u32, _ptr]),
+}
+
+_lib = None
+
+
+def load():
+    """Load the HIP library (once) and attach signatures. Raises OSError if it has not been built."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise OSError(f"{LIB_PATH} not found: build it with `make -C crusaderbackend_amd/csrc`")
+        lib = ctypes.CDLL(LIB_PATH)
+        for name, (res, args) in SIGNATURES.items():
+            fn = getattr(lib, name)
+            fn.restype = res
+            fn.argtypes = args
+        _lib = lib
+    return _lib
+
+
+class CrbError(RuntimeError):
+    def __init__(self, status, message):
+        super().__init__(f"crb status {status}: {message}")
+        self.status = status
+
+
+def check(status):
+    if status != CRB_OK:
+        raise CrbError(status, load().crb_last_error_string().decode())
+
+
+def _p(t):
+    return None if t is None else t.data_ptr()
+
+
+def _stream(stream):
+    return None if stream is None else stream.cuda_stream
+
+
+# Thin helpers over torch CUDA tensors (device memory + streams only; no torch math).
+def sgemm_nn(A, B, C, M, N, K, batch=1, stream=None):
+    check(load().crb_sgemm_nn(_p(A), _p(B), _p(C), M, N, K, batch, _stream(stream)))
+
+
+def sgemm_tn(A, B, C, M, N, K, batch=1, stream=None):
+    check(load().crb_sgemm_tn(_p(A), _p(B), _p(C), M, N, K, batch, _stream(stream)))
+
+
+def sgemm_nt(A, B, C, M, N, K, stream=None):
+    check(load().crb_sgemm_nt(_p(A), _p(B), _p(C), M, N, K, _stream(stream)))
+
+
+def sgemm_nta(A, B, C, M, N, K, batch=1, stream=None):
+    check(load().crb_sgemm_nta(_p(A), _p(B), _p(C), M, N, K, batch, _stream(stream)))
+
+
+def linear_fwd(X, W, bias, Y, batch, IN, OUT, flags=0, stream=None):
+    check(load().crb_linear_fwd(_p(X), _p(W), _p(bias), _p(Y), batch, IN, OUT, flags, _stream(stream)))
+
+
+def linear_dgrad(dY, W, dX, batch, IN, OUT, stream=None):
+    check(load().crb_linear_dgrad(_p(dY), _p(W), _p(dX), batch, IN, OUT, _stream(stream)))
+
+
+def linear_wgrad(dY, X, dW, dB, batch, IN, OUT, stream=None):
+    check(load().crb_linear_wgrad(_p(dY), _p(X), _p(dW), _p(dB), batch, IN, OUT, _stream(stream)))
+
+
+def conv_fwd(W, X, Y, bias, geom, flags=0, stream=None):
+    check(load().crb_conv_fwd(_p(W), _p(X), _p(Y), _p(bias), ctypes.byref(geom), flags, _stream(stream)))
+
+
+def conv_dgrad(W, dY, dX, geom, stream=None):
+    check(load().crb_conv_dgrad(_p(W), _p(dY), _p(dX), ctypes.byref(geom), _stream(stream)))
+
+
+def conv_wgrad_workspace_bytes(geom):
+    return load().crb_conv_wgrad_workspace_bytes(ctypes.byref(geom))
+
+
+def conv_wgrad(dY, X, dW, geom, workspace=None, stream=None):
+    nbytes = 0 if workspace is None else workspace.numel() * workspace.element_size()
+    check(load().crb_conv_wgrad(_p(dY), _p(X), _p(dW), ctypes.byref(geom), _p(workspace), nbytes, _stream(stream)))
+
+
+def conv_bias(Y, bias, N, C, HW, stream=None):
+    check(load().crb_conv_bias(_p(Y), _p(bias), N, C, HW, _stream(stream)))

@@ -1,0 +1,170 @@
+// C-ABI entry points of the convolution family: forward, data gradient, weight gradient and the
+// standalone bias add, all as implicit GEMMs on the MFMA engine (no im2col buffer is materialised).
+#include "operands.h"
+
+namespace crb {
+
+// Macro-tiles chosen by the channel extent on the GEMM-M side; the pixel (or tap) side is 128 wide.
+typedef TileCfg<32, 128, 16, 1, 4, 2> CfgM32;
+typedef TileCfg<64, 128, 16, 2, 2, 2> CfgM64;
+typedef TileCfg<128, 128, 16, 2, 2, 2> CfgM128;
+
+static inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+static int check_geom(const char *what, const crb_conv_geom *g) {
+    if (!g) return fail(CRB_ENULL, "%s: null geometry", what);
+    if (!g->N || !g->IC || !g->IH || !g->IW || !g->OC || !g->FH || !g->FW || !g->OH || !g->OW || !g->sH || !g->sW)
+        return fail(CRB_EINVAL_SHAPE, "%s: zero dimension or stride", what);
+    // the relations the reference's assertConv enforces (cuConv.cu:731-755)
+    if (g->IH + 2 * g->pH < g->FH || g->OH != (g->IH + 2 * g->pH - g->FH) / g->sH + 1)
+        return fail(CRB_EINVAL_SHAPE, "%s: assertConv: rows (h) relationship did not satisfy", what);
+    if (g->IW + 2 * g->pW < g->FW || g->OW != (g->IW + 2 * g->pW - g->FW) / g->sW + 1)
+        return fail(CRB_EINVAL_SHAPE, "%s: assertConv: cols (w) relationship did not satisfy", what);
+    const uint64_t lim = 0x7fffffffull;
+    if (uint64_t(g->N) * g->IC * g->IH * g->IW > lim || uint64_t(g->N) * g->OC * g->OH * g->OW > lim ||
+        uint64_t(g->OC) * g->IC * g->FH * g->FW > lim)
+        return fail(CRB_EINVAL_SHAPE, "%s: tensor exceeds 2^31 elements", what);
+    return CRB_OK;
+}
+
+static Im2col make_im2col(const float *X, const crb_conv_geom *g) {
+    Im2col m;
+    m.X = X;
+    m.npix = g->N * g->OH * g->OW;
+    m.ntap = g->IC * g->FH * g->FW;
+    m.IH = g->IH, m.IW = g->IW;
+    m.img_stride = g->IC * g->IH * g->IW;
+    m.chan_stride = g->IH * g->IW;
+    m.sH = g->sH, m.sW = g->sW, m.pH = g->pH, m.pW = g->pW;
+    m.ohw.init(g->OH * g->OW), m.ow.init(g->OW), m.fhw.init(g->FH * g->FW), m.fw.init(g->FW);
+    return m;
+}
+
+template <class AOp, class BOp, class Epi>
+static int run_by_m(const AOp &a, const BOp &b, const Epi &e, u32 M, u32 N, u32 K, u32 zdim, u32 split_k, u32 k_per_z,
+                    hipStream_t s, const char *what) {
+    if (M <= 32) return launch_igemm<CfgM32>(a, b, e, M, N, K, zdim, split_k, k_per_z, s, what);
+    if (M <= 64) return launch_igemm<CfgM64>(a, b, e, M, N, K, zdim, split_k, k_per_z, s, what);
+    return launch_igemm<CfgM128>(a, b, e, M, N, K, zdim, split_k, k_per_z, s, what);
+}
+
+static u32 tile_m_for(u32 M) { return M <= 32 ? 32 : (M <= 64 ? 64 : 128); }
+
+// Split plan of the weight gradient: the contraction runs over n*OH*OW (up to 131072) while the result
+// is only OC x IC*FH*FW, so the K range is cut into `splits` slices handled by separate workgroups.
+struct WgradPlan {
+    u32 M, Ncols, K, splits, k_per_z;
+};
+static WgradPlan wgrad_plan(const crb_conv_geom *g) {
+    WgradPlan p;
+    p.M = g->OC;
+    p.Ncols = g->IC * g->FH * g->FW;
+    p.K = g->N * g->OH * g->OW;
+    const u32 tiles = ceil_div(p.M, tile_m_for(p.M)) * ceil_div(p.Ncols, 128);
+    const u32 target_wgs = 1024;  // ~4 workgroups per CU
+    u32 splits = tiles >= target_wgs ? 1 : target_wgs / tiles;
+    const u32 min_k = 256;  // do not cut slices thinner than 16 slabs
+    if (splits > ceil_div(p.K, min_k)) splits = ceil_div(p.K, min_k);
+    if (splits < 1) splits = 1;
+    u32 kz = ceil_div(ceil_div(p.K, splits), 16) * 16;
+    p.k_per_z = kz;
+    p.splits = ceil_div(p.K, kz);
+    return p;
+}
+
+__global__ void __launch_bounds__(256) conv_bias_kernel(float *__restrict__ Y, const float *__restrict__ bias,
+                                                        u32 total, u32 C, FastDiv hw) {
+    const u32 i = blockIdx.x * 256 + threadIdx.x;
+    if (i >= total) return;
+    const u32 plane = hw.div(i);
+    Y[i] += bias[plane % C];
+}
+
+}  // namespace crb
+
+using namespace crb;
+
+extern "C" {
+
+int crb_conv_fwd(const float *W, const float *X, float *Y, const float *bias_or_null, const crb_conv_geom *g,
+                 uint32_t flags, void *stream) {
+    if (!W || !X || !Y) return fail(CRB_ENULL, "crb_conv_fwd: null operand");
+    if (int st = check_geom("crb_conv_fwd", g)) return st;
+    const u32 M = g->OC, N = g->N * g->OH * g->OW, K = g->IC * g->FH * g->FW;
+    Im2colPixRows b{make_im2col(X, g)};
+    NchwEpi e{Y, bias_or_null, g->OC, g->OH * g->OW, (flags & CRB_FLAG_RELU) ? u32(EPI_RELU) : 0u,
+              FastDiv(g->OH * g->OW)};
+    hipStream_t s = hipStream_t(stream);
+    if (K % 4 == 0 && aligned16(W)) {
+        MatK<true> a{W, M, K, 0};
+        return run_by_m(a, b, e, M, N, K, 1, 0, K, s, "crb_conv_fwd");
+    }
+    MatK<false> a{W, M, K, 0};
+    return run_by_m(a, b, e, M, N, K, 1, 0, K, s, "crb_conv_fwd");
+}
+
+int crb_conv_dgrad(const float *W, const float *dY, float *dX, const crb_conv_geom *g, void *stream) {
+    if (!W || !dY || !dX) return fail(CRB_ENULL, "crb_conv_dgrad: null operand");
+    if (int st = check_geom("crb_conv_dgrad", g)) return st;
+    const u32 FHW = g->FH * g->FW;
+    const u32 M = g->IC, N = g->N * g->IH * g->IW, K = g->OC * FHW;
+    SepK a{W, g->IC, FHW, g->IC * FHW, 1, FastDiv(FHW)};
+    DgradGather b;
+    b.dY = dY;
+    b.npix = N;
+    b.OH = g->OH, b.OW = g->OW;
+    b.img_stride = g->OC * g->OH * g->OW;
+    b.chan_stride = g->OH * g->OW;
+    b.pH = g->pH, b.pW = g->pW;
+    b.ihw.init(g->IH * g->IW), b.iw.init(g->IW), b.fhw.init(FHW), b.fw.init(g->FW);
+    b.sH.init(g->sH), b.sW.init(g->sW);
+    NchwEpi e{dX, nullptr, g->IC, g->IH * g->IW, 0u, FastDiv(g->IH * g->IW)};
+    return run_by_m(a, b, e, M, N, K, 1, 0, K, hipStream_t(stream), "crb_conv_dgrad");
+}
+
+size_t crb_conv_wgrad_workspace_bytes(const crb_conv_geom *g) {
+    if (check_geom("crb_conv_wgrad_workspace_bytes", g)) return 0;
+    const WgradPlan p = wgrad_plan(g);
+    return p.splits > 1 ? size_t(p.splits) * p.M * p.Ncols * sizeof(float) : 0;
+}
+
+int crb_conv_wgrad(const float *dY, const float *X, float *dW, const crb_conv_geom *g, void *workspace,
+                   size_t workspace_bytes, void *stream) {
+    if (!dY || !X || !dW) return fail(CRB_ENULL, "crb_conv_wgrad: null operand");
+    if (int st = check_geom("crb_conv_wgrad", g)) return st;
+    const WgradPlan p = wgrad_plan(g);
+    hipStream_t s = hipStream_t(stream);
+    const u32 OHW = g->OH * g->OW;
+    SepK a{dY, g->OC, OHW, g->OC * OHW, 1, FastDiv(OHW)};
+    Im2colTapRows b{make_im2col(X, g)};
+    if (p.splits == 1) {
+        RowMajorEpi e{dW, nullptr, p.Ncols, 0, EPI_ACCUM};
+        return run_by_m(a, b, e, p.M, p.Ncols, p.K, 1, 0, p.K, s, "crb_conv_wgrad");
+    }
+    const size_t need = size_t(p.splits) * p.M * p.Ncols * sizeof(float);
+    float *ws = static_cast<float *>(workspace);
+    if (ws) {
+        if (workspace_bytes < need)
+            return fail(CRB_EWORKSPACE, "crb_conv_wgrad: workspace %zu bytes < required %zu", workspace_bytes, need);
+    } else {
+        ws = static_cast<float *>(arena_get(need));
+        if (!ws) return fail(CRB_EHIP, "crb_conv_wgrad: cannot allocate %zu bytes of scratch", need);
+    }
+    RowMajorEpi e{ws, nullptr, p.Ncols, p.M * p.Ncols, 0u};
+    if (int st = run_by_m(a, b, e, p.M, p.Ncols, p.K, p.splits, 1, p.k_per_z, s, "crb_conv_wgrad")) return st;
+    const u32 count = p.M * p.Ncols;
+    hipLaunchKernelGGL(splitk_reduce_kernel, dim3(ceil_div(count, 256)), dim3(256), 0, s, ws, dW, count, p.splits, 1u);
+    return check_launch("crb_conv_wgrad(reduce)");
+}
+
+int crb_conv_bias(float *Y, const float *bias, uint32_t N, uint32_t C, uint32_t HW, void *stream) {
+    if (!Y || !bias) return fail(CRB_ENULL, "crb_conv_bias: null operand");
+    if (!N || !C || !HW) return fail(CRB_EINVAL_SHAPE, "crb_conv_bias: zero dimension");
+    if (uint64_t(N) * C * HW > 0x7fffffffull) return fail(CRB_EINVAL_SHAPE, "crb_conv_bias: tensor exceeds 2^31 elements");
+    const u32 total = N * C * HW;
+    hipLaunchKernelGGL(conv_bias_kernel, dim3(ceil_div(total, 256)), dim3(256), 0, hipStream_t(stream), Y, bias, total, C,
+                       FastDiv(HW));
+    return check_launch("crb_conv_bias");
+}
+
+}  // extern "C"

@@ -1,0 +1,154 @@
+// C-ABI entry points of the GEMM and dense-layer families (fp32, row-major) on the MFMA engine.
+#include "operands.h"
+
+namespace crb {
+
+// Macro-tiles. Large: 128x128, each wave a 64x64 block of four 32x32 MFMA tiles. Small: 64x64 for
+// problems that would not fill 256 CUs with large tiles.
+typedef TileCfg<128, 128, 16, 2, 2, 2> CfgLarge;
+typedef TileCfg<64, 64, 16, 2, 2, 2> CfgSmall;
+
+static inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+template <class AOp, class BOp, class Epi>
+static int run_tiles(const AOp &a, const BOp &b, const Epi &e, u32 M, u32 N, u32 K, u32 zdim, hipStream_t s,
+                     const char *what) {
+    const uint64_t large_tiles = uint64_t(ceil_div(M, 128)) * ceil_div(N, 128) * zdim;
+    if (large_tiles >= 256 && M > 64 && N > 64)
+        return launch_igemm<CfgLarge>(a, b, e, M, N, K, zdim, 0, K, s, what);
+    return launch_igemm<CfgSmall>(a, b, e, M, N, K, zdim, 0, K, s, what);
+}
+
+static int check_dims(const char *what, u32 M, u32 N, u32 K, u32 batch) {
+    if (M == 0 || N == 0 || K == 0 || batch == 0) return fail(CRB_EINVAL_SHAPE, "%s: zero dimension", what);
+    const uint64_t lim = 0x7fffffffull;
+    if (uint64_t(M) * K * batch > lim || uint64_t(K) * N * batch > lim || uint64_t(M) * N * batch > lim)
+        return fail(CRB_EINVAL_SHAPE, "%s: operand exceeds 2^31 elements", what);
+    return CRB_OK;
+}
+
+// column sums of a (rows x cols) row-major matrix: out[c] += sum_r in[r*cols + c], ascending r.
+__global__ void __launch_bounds__(256) colsum_accum_kernel(const float *__restrict__ in, float *__restrict__ out,
+                                                           u32 rows, u32 cols) {
+    const u32 c = blockIdx.x * 256 + threadIdx.x;
+    if (c >= cols) return;
+    float s = 0.0f;
+    for (u32 r = 0; r < rows; ++r) s += in[size_t(r) * cols + c];
+    out[c] += s;
+}
+
+static int gemm_nn(const float *A, const float *B, float *C, u32 M, u32 N, u32 K, u32 batch, const float *col_bias,
+                   u32 flags, hipStream_t s, const char *what) {
+    RowMajorEpi e{C, col_bias, N, M * N, flags};
+    if (K % 4 == 0 && N % 4 == 0 && aligned16(A) && aligned16(B)) {
+        MatK<true> a{A, M, K, 0};
+        MatR<true> b{B, N, N, K * N};
+        return run_tiles(a, b, e, M, N, K, batch, s, what);
+    }
+    MatK<false> a{A, M, K, 0};
+    MatR<false> b{B, N, N, K * N};
+    return run_tiles(a, b, e, M, N, K, batch, s, what);
+}
+
+static int gemm_tn(const float *A, const float *B, float *C, u32 M, u32 N, u32 K, u32 batch, u32 flags,
+                   hipStream_t s, const char *what) {
+    RowMajorEpi e{C, nullptr, N, M * N, flags};
+    if (M % 4 == 0 && N % 4 == 0 && aligned16(A) && aligned16(B)) {
+        MatR<true> a{A, M, M, 0};
+        MatR<true> b{B, N, N, K * N};
+        return run_tiles(a, b, e, M, N, K, batch, s, what);
+    }
+    MatR<false> a{A, M, M, 0};
+    MatR<false> b{B, N, N, K * N};
+    return run_tiles(a, b, e, M, N, K, batch, s, what);
+}
+
+static int gemm_nt(const float *A, const float *B, float *C, u32 M, u32 N, u32 K, const float *col_bias, u32 flags,
+                   hipStream_t s, const char *what) {
+    RowMajorEpi e{C, col_bias, N, 0, flags};
+    if (K % 4 == 0 && aligned16(A) && aligned16(B)) {
+        MatK<true> a{A, M, K, 0};
+        MatK<true> b{B, N, K, 0};
+        return run_tiles(a, b, e, M, N, K, 1, s, what);
+    }
+    MatK<false> a{A, M, K, 0};
+    MatK<false> b{B, N, K, 0};
+    return run_tiles(a, b, e, M, N, K, 1, s, what);
+}
+
+}  // namespace crb
+
+using namespace crb;
+
+extern "C" {
+
+int crb_sgemm_nn(const float *A, const float *B, float *C, uint32_t M, uint32_t N, uint32_t K, uint32_t batch,
+                 void *stream) {
+    if (!A || !B || !C) return fail(CRB_ENULL, "crb_sgemm_nn: null operand");
+    if (int st = check_dims("crb_sgemm_nn", M, N, K, batch)) return st;
+    return gemm_nn(A, B, C, M, N, K, batch, nullptr, 0, hipStream_t(stream), "crb_sgemm_nn");
+}
+
+int crb_sgemm_tn(const float *A, const float *B, float *C, uint32_t M, uint32_t N, uint32_t K, uint32_t batch,
+                 void *stream) {
+    if (!A || !B || !C) return fail(CRB_ENULL, "crb_sgemm_tn: null operand");
+    if (int st = check_dims("crb_sgemm_tn", M, N, K, batch)) return st;
+    return gemm_tn(A, B, C, M, N, K, batch, 0, hipStream_t(stream), "crb_sgemm_tn");
+}
+
+int crb_sgemm_nt(const float *A, const float *B, float *C, uint32_t M, uint32_t N, uint32_t K, void *stream) {
+    if (!A || !B || !C) return fail(CRB_ENULL, "crb_sgemm_nt: null operand");
+    if (int st = check_dims("crb_sgemm_nt", M, N, K, 1)) return st;
+    return gemm_nt(A, B, C, M, N, K, nullptr, 0, hipStream_t(stream), "crb_sgemm_nt");
+}
+
+int crb_sgemm_nta(const float *A, const float *B, float *C, uint32_t M, uint32_t N, uint32_t K, uint32_t batch,
+                  void *stream) {
+    if (!A || !B || !C) return fail(CRB_ENULL, "crb_sgemm_nta: null operand");
+    if (int st = check_dims("crb_sgemm_nta", M, N, K, batch)) return st;
+    if (uint64_t(K) * batch > 0x7fffffffull) return fail(CRB_EINVAL_SHAPE, "crb_sgemm_nta: K*batch too large");
+    const u32 KK = K * batch;
+    RowMajorEpi e{C, nullptr, N, 0, EPI_ACCUM};
+    hipStream_t s = hipStream_t(stream);
+    if (K % 4 == 0 && aligned16(A) && aligned16(B)) {
+        MatKCat<true> a{A, M, K, M * K, FastDiv(K)};
+        MatKCat<true> b{B, N, K, N * K, FastDiv(K)};
+        return run_tiles(a, b, e, M, N, KK, 1, s, "crb_sgemm_nta");
+    }
+    MatKCat<false> a{A, M, K, M * K, FastDiv(K)};
+    MatKCat<false> b{B, N, K, N * K, FastDiv(K)};
+    return run_tiles(a, b, e, M, N, KK, 1, s, "crb_sgemm_nta");
+}
+
+int crb_linear_fwd(const float *X, const float *W, const float *bias, float *Y, uint32_t batch, uint32_t IN,
+                   uint32_t OUT, uint32_t flags, void *stream) {
+    if (!X || !W || !bias || !Y) return fail(CRB_ENULL, "crb_linear_fwd: null operand");
+    if (int st = check_dims("crb_linear_fwd", batch, OUT, IN, 1)) return st;
+    // Y (batch x OUT) = X (batch x IN) * W^T, bias broadcast along rows
+    return gemm_nt(X, W, Y, batch, OUT, IN, bias, (flags & CRB_FLAG_RELU) ? EPI_RELU : 0u, hipStream_t(stream),
+                   "crb_linear_fwd");
+}
+
+int crb_linear_dgrad(const float *dY, const float *W, float *dX, uint32_t batch, uint32_t IN, uint32_t OUT,
+                     void *stream) {
+    if (!dY || !W || !dX) return fail(CRB_ENULL, "crb_linear_dgrad: null operand");
+    if (int st = check_dims("crb_linear_dgrad", batch, IN, OUT, 1)) return st;
+    // dX (batch x IN) = dY (batch x OUT) * W (OUT x IN)
+    return gemm_nn(dY, W, dX, batch, IN, OUT, 1, nullptr, 0, hipStream_t(stream), "crb_linear_dgrad");
+}
+
+int crb_linear_wgrad(const float *dY, const float *X, float *dW, float *dB, uint32_t batch, uint32_t IN,
+                     uint32_t OUT, void *stream) {
+    if (!dY || !X || !dW) return fail(CRB_ENULL, "crb_linear_wgrad: null operand");
+    if (int st = check_dims("crb_linear_wgrad", OUT, IN, batch, 1)) return st;
+    hipStream_t s = hipStream_t(stream);
+    // dW (OUT x IN) += dY^T (dY stored batch x OUT) * X (batch x IN)
+    if (int st = gemm_tn(dY, X, dW, OUT, IN, batch, 1, EPI_ACCUM, s, "crb_linear_wgrad")) return st;
+    if (dB) {
+        hipLaunchKernelGGL(colsum_accum_kernel, dim3(ceil_div(OUT, 256)), dim3(256), 0, s, dY, dB, batch, OUT);
+        return check_launch("crb_linear_wgrad(dB)");
+    }
+    return CRB_OK;
+}
+
+}  // extern "C"

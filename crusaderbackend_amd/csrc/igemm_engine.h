@@ -1,0 +1,317 @@
+// Generic fp32 MFMA contraction engine for gfx950:  D(M x N) = sum_k A(m,k) * B(k,n).
+//
+// One 256-thread workgroup (4 wave64) owns a BM x BN macro-tile. Operand panels are staged through
+// double-buffered LDS one BK-wide K slab at a time (global -> registers -> LDS prefetch of slab s+1
+// overlaps the MFMAs of slab s; one barrier per slab) and fed to v_mfma_f32_32x32x2_f32.
+//
+// Operands are functors, so the same mainloop serves plain matrices (any transposition), K-concatenated
+// batches and the implicit im2col gathers of the convolution passes. Each operand declares which of
+// its two indices is contiguous in memory:
+//   kKFast = true  : LDS panel is [row][k] (row stride BK+4 floats). A lane reads one 16-byte vector
+//                    = the k values of 4 consecutive MFMA steps.
+//   kKFast = false : LDS panel is [k][row] (row stride ROWS+4 floats). MFMA block `b` of a wave owns
+//                    rows {T*i + b}, so a lane reads its T blocks' values for one step as one vector.
+// Either way global->LDS copies are straight (no transposition) and LDS reads are vector reads.
+// Within a group of 8 k's, MFMA step s of lane-half h consumes k = 4*h + s for both operands.
+//
+// MFMA 32x32x2 f32 operand mapping (wave64, lane l): A value = A[i = l%32][k = l/32],
+// B value = B[k = l/32][j = l%32], accumulator register r = D[8*(r/4) + 4*(l/32) + r%4][l%32].
+#pragma once
+#include "crb_common.h"
+
+namespace crb {
+
+typedef float v2f __attribute__((ext_vector_type(2)));
+typedef float v4f __attribute__((ext_vector_type(4)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+
+constexpr int kThreads = 256;
+constexpr u32 kXcds = 8;
+
+struct IgemmDims {
+    u32 M, N, K;
+    u32 tiles_m, tiles_n;
+    u32 k_per_z;  // K range handled per blockIdx.z when split_k != 0 (multiple of BK)
+    u32 split_k;  // 0: blockIdx.z is a batch index; 1: blockIdx.z is a K-split index
+};
+
+template <int BM_, int BN_, int BK_, int WM_, int WN_, int OCC_>
+struct TileCfg {
+    static constexpr int BM = BM_, BN = BN_, BK = BK_, WM = WM_, WN = WN_, OCC = OCC_;
+    static constexpr int WTM = BM / WM, WTN = BN / WN;  // wave tile
+    static constexpr int TM = WTM / 32, TN = WTN / 32;  // 32x32 MFMA blocks per wave tile
+    static_assert(WM * WN == 4, "4 waves per workgroup");
+    static_assert(TM >= 1 && TN >= 1 && TM * 32 * WM == BM && TN * 32 * WN == BN, "tile shape");
+    static_assert(BK % 8 == 0, "K slab is a multiple of 8");
+};
+
+// ---- global -> register -> LDS staging of one operand panel (ROWS x BK) -----------------------------
+template <class Op, int ROWS, int BK>
+struct PanelLoader {
+    static constexpr bool KF = Op::kKFast;
+    static constexpr bool VEC = Op::kVec;
+    static constexpr int LD = KF ? BK + 4 : ROWS + 4;
+    static constexpr int SIZE = KF ? ROWS * LD : BK * LD;
+    // number of register-resident items per thread per slab
+    static constexpr int ITEMS = VEC ? ROWS * BK / 4 : ROWS * BK;
+    static constexpr int NP = (ITEMS + kThreads - 1) / kThreads;
+    static_assert(ITEMS % kThreads == 0 || ITEMS < kThreads, "panel must split evenly over 256 threads");
+    // panels with fewer items than threads are staged by the first ITEMS threads only
+    static __device__ __forceinline__ bool active() { return ITEMS >= kThreads || threadIdx.x < ITEMS; }
+    static_assert(VEC || KF || ROWS <= kThreads, "row-fast scalar staging needs ROWS <= 256");
+
+    // scalar, k-fast: thread owns k lane t%BK and rows t/BK + i*(256/BK): NP row states kept
+    // scalar, row-fast: thread owns row t%ROWS and k's t/ROWS + i*(256/ROWS): one row state kept
+    static constexpr int NROWSTATE = VEC ? 1 : (KF ? NP : 1);
+    typename Op::RowS rs[NROWSTATE];
+    float reg[VEC ? NP * 4 : NP];
+    u32 row0;
+
+    __device__ __forceinline__ void init(const Op &op, u32 row0_) {
+        row0 = row0_;
+        const u32 t = threadIdx.x;
+        if constexpr (!VEC) {
+            if constexpr (KF) {
+#pragma unroll
+                for (int i = 0; i < NP; ++i) rs[i] = op.prep_row(row0 + t / BK + i * (kThreads / BK));
+            } else {
+                rs[0] = op.prep_row(row0 + t % ROWS);
+            }
+        }
+    }
+
+    __device__ __forceinline__ void fetch(const Op &op, u32 k0, u32 klimit) {
+        const u32 t = threadIdx.x;
+        if (!active()) return;
+        if constexpr (VEC) {
+            if constexpr (KF) {
+                constexpr int QK = BK / 4, RP = kThreads / QK;
+#pragma unroll
+                for (int i = 0; i < NP; ++i) {
+                    v4f v = op.fetch4(row0 + t / QK + i * RP, k0 + 4 * (t % QK), klimit);
+                    reg[4 * i + 0] = v.x, reg[4 * i + 1] = v.y, reg[4 * i + 2] = v.z, reg[4 * i + 3] = v.w;
+                }
+            } else {
+                constexpr int QR = ROWS / 4, KP = kThreads / QR;
+#pragma unroll
+                for (int i = 0; i < NP; ++i) {
+                    v4f v = op.fetch4(row0 + 4 * (t % QR), k0 + t / QR + i * KP, klimit);
+                    reg[4 * i + 0] = v.x, reg[4 * i + 1] = v.y, reg[4 * i + 2] = v.z, reg[4 * i + 3] = v.w;
+                }
+            }
+        } else {
+            if constexpr (KF) {
+                typename Op::KS ks = op.prep_k(k0 + t % BK, klimit);
+#pragma unroll
+                for (int i = 0; i < NP; ++i) reg[i] = op.fetch(rs[i], ks);
+            } else {
+                constexpr int KP = kThreads / ROWS;
+#pragma unroll
+                for (int i = 0; i < NP; ++i) {
+                    typename Op::KS ks = op.prep_k(k0 + t / ROWS + i * KP, klimit);
+                    reg[i] = op.fetch(rs[0], ks);
+                }
+            }
+        }
+    }
+
+    __device__ __forceinline__ void commit(float *lds) const {
+        const u32 t = threadIdx.x;
+        if (!active()) return;
+        if constexpr (VEC) {
+            if constexpr (KF) {
+                constexpr int QK = BK / 4, RP = kThreads / QK;
+#pragma unroll
+                for (int i = 0; i < NP; ++i) {
+                    v4f v = {reg[4 * i], reg[4 * i + 1], reg[4 * i + 2], reg[4 * i + 3]};
+                    *reinterpret_cast<v4f *>(lds + (t / QK + i * RP) * LD + 4 * (t % QK)) = v;
+                }
+            } else {
+                constexpr int QR = ROWS / 4, KP = kThreads / QR;
+#pragma unroll
+                for (int i = 0; i < NP; ++i) {
+                    v4f v = {reg[4 * i], reg[4 * i + 1], reg[4 * i + 2], reg[4 * i + 3]};
+                    *reinterpret_cast<v4f *>(lds + (t / QR + i * KP) * LD + 4 * (t % QR)) = v;
+                }
+            }
+        } else {
+            if constexpr (KF) {
+#pragma unroll
+                for (int i = 0; i < NP; ++i) lds[(t / BK + i * (kThreads / BK)) * LD + t % BK] = reg[i];
+            } else {
+                constexpr int KP = kThreads / ROWS;
+#pragma unroll
+                for (int i = 0; i < NP; ++i) lds[(t / ROWS + i * KP) * LD + t % ROWS] = reg[i];
+            }
+        }
+    }
+};
+
+// ---- LDS -> MFMA fragments for one group of 8 k's (4 MFMA steps) ------------------------------------
+// frag[s][b]: value this lane feeds to MFMA step s for 32-row block b of the wave tile.
+template <bool KF, int T, int LD>
+__device__ __forceinline__ void read_frags(const float *lds, int wave_row0, int g, int lane, float (&frag)[4][T]) {
+    const int i = lane & 31, h = lane >> 5;
+    if constexpr (KF) {
+#pragma unroll
+        for (int b = 0; b < T; ++b) {
+            v4f v = *reinterpret_cast<const v4f *>(lds + (wave_row0 + b * 32 + i) * LD + 8 * g + 4 * h);
+            frag[0][b] = v.x, frag[1][b] = v.y, frag[2][b] = v.z, frag[3][b] = v.w;
+        }
+    } else {
+#pragma unroll
+        for (int s = 0; s < 4; ++s) {
+            const float *p = lds + (8 * g + 4 * h + s) * LD + wave_row0 + i * T;
+            if constexpr (T == 1) {
+                frag[s][0] = p[0];
+            } else if constexpr (T == 2) {
+                v2f v = *reinterpret_cast<const v2f *>(p);
+                frag[s][0] = v.x, frag[s][1] = v.y;
+            } else {
+                static_assert(T % 4 == 0 || T <= 2, "row-fast wave tiles use 1, 2 or 4k blocks");
+#pragma unroll
+                for (int q = 0; q < T / 4; ++q) {
+                    v4f v = *reinterpret_cast<const v4f *>(p + 4 * q);
+                    frag[s][4 * q + 0] = v.x, frag[s][4 * q + 1] = v.y, frag[s][4 * q + 2] = v.z,
+                                    frag[s][4 * q + 3] = v.w;
+                }
+            }
+        }
+    }
+}
+
+// Workgroups are dealt round-robin to the 8 XCDs (each with its own L2). Give every XCD a contiguous
+// run of the tile sequence, and order that sequence in bands of 8 tile-rows walked column by column,
+// so the workgroups resident on one XCD share A and B panels through that XCD's L2.
+__device__ __forceinline__ void swizzled_tile(u32 bid, u32 tiles_m, u32 tiles_n, u32 &tm, u32 &tn) {
+    const u32 nt = tiles_m * tiles_n;
+    const u32 q = nt / kXcds, r = nt % kXcds;
+    const u32 xcd = bid % kXcds, loc = bid / kXcds;
+    const u32 tile = xcd * q + (xcd < r ? xcd : r) + loc;
+    constexpr u32 BAND = 8;
+    const u32 per_band = BAND * tiles_n;
+    const u32 band = tile / per_band, in_band = tile % per_band;
+    const u32 first_m = band * BAND;
+    const u32 rows = tiles_m - first_m < BAND ? tiles_m - first_m : BAND;
+    tm = first_m + in_band % rows;
+    tn = in_band / rows;
+}
+
+template <class Cfg, class AOp, class BOp, class Epi>
+__global__ void __launch_bounds__(kThreads, Cfg::OCC) igemm_kernel(AOp a, BOp b, Epi epi, IgemmDims d) {
+    constexpr int BM = Cfg::BM, BN = Cfg::BN, BK = Cfg::BK, TM = Cfg::TM, TN = Cfg::TN;
+    using LA = PanelLoader<AOp, BM, BK>;
+    using LB = PanelLoader<BOp, BN, BK>;
+    __shared__ __attribute__((aligned(16))) float sA[2][LA::SIZE];
+    __shared__ __attribute__((aligned(16))) float sB[2][LB::SIZE];
+
+    u32 tm, tn;
+    swizzled_tile(blockIdx.x, d.tiles_m, d.tiles_n, tm, tn);
+    const u32 z = blockIdx.z;
+    u32 kbeg = 0, kend = d.K;
+    if (d.split_k) {
+        kbeg = z * d.k_per_z;
+        kend = kbeg + d.k_per_z < d.K ? kbeg + d.k_per_z : d.K;
+        a.bind(0), b.bind(0);
+    } else {
+        a.bind(z), b.bind(z);
+    }
+    epi.bind(z);
+
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int wave_m = wave / Cfg::WN, wave_n = wave % Cfg::WN;
+    const u32 row0 = tm * BM, col0 = tn * BN;
+
+    LA la;
+    LB lb;
+    la.init(a, row0);
+    lb.init(b, col0);
+
+    v16f acc[TM][TN];
+#pragma unroll
+    for (int mi = 0; mi < TM; ++mi)
+#pragma unroll
+        for (int ni = 0; ni < TN; ++ni)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[mi][ni][r] = 0.0f;
+
+    if (kbeg < kend) {
+        la.fetch(a, kbeg, kend);
+        lb.fetch(b, kbeg, kend);
+        la.commit(sA[0]);
+        lb.commit(sB[0]);
+    }
+    __syncthreads();
+
+    int buf = 0;
+    for (u32 k0 = kbeg; k0 < kend; k0 += BK, buf ^= 1) {
+        const bool more = k0 + BK < kend;
+        if (more) {
+            la.fetch(a, k0 + BK, kend);
+            lb.fetch(b, k0 + BK, kend);
+        }
+        const float *pa = sA[buf], *pb = sB[buf];
+#pragma unroll
+        for (int g = 0; g < BK / 8; ++g) {
+            float fa[4][TM], fb[4][TN];
+            read_frags<AOp::kKFast, TM, LA::LD>(pa, wave_m * Cfg::WTM, g, lane, fa);
+            read_frags<BOp::kKFast, TN, LB::LD>(pb, wave_n * Cfg::WTN, g, lane, fb);
+#pragma unroll
+            for (int s = 0; s < 4; ++s)
+#pragma unroll
+                for (int mi = 0; mi < TM; ++mi)
+#pragma unroll
+                    for (int ni = 0; ni < TN; ++ni)
+                        acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[s][mi], fb[s][ni], acc[mi][ni], 0, 0, 0);
+        }
+        if (more) {
+            la.commit(sA[buf ^ 1]);
+            lb.commit(sB[buf ^ 1]);
+        }
+        __syncthreads();
+    }
+
+    // epilogue: accumulator register r of lane l is D[8*(r/4) + 4*(l/32) + r%4][l%32] of its block
+    const int j = lane & 31, h = lane >> 5;
+#pragma unroll
+    for (int ni = 0; ni < TN; ++ni) {
+        const u32 col = col0 + wave_n * Cfg::WTN + (BOp::kKFast ? ni * 32 + j : j * TN + ni);
+        const typename Epi::ColS cs = epi.prep_col(col, d.N);
+#pragma unroll
+        for (int mi = 0; mi < TM; ++mi)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int id = 8 * (r / 4) + 4 * h + (r % 4);
+                const u32 row = row0 + wave_m * Cfg::WTM + (AOp::kKFast ? mi * 32 + id : id * TM + mi);
+                if (row < d.M) epi.store(row, cs, acc[mi][ni][r]);
+            }
+    }
+}
+
+// ---- split-K second pass: C[i] (+)= sum_z partial[z][i], fixed ascending-z order ---------------------
+static __global__ void __launch_bounds__(256) splitk_reduce_kernel(const float *__restrict__ partial, float *__restrict__ C,
+                                                            u32 count, u32 splits, u32 accumulate) {
+    const u32 i = blockIdx.x * 256 + threadIdx.x;
+    if (i >= count) return;
+    float s = 0.0f;
+    for (u32 zz = 0; zz < splits; ++zz) s += partial[size_t(zz) * count + i];
+    C[i] = accumulate ? C[i] + s : s;
+}
+
+template <class Cfg, class AOp, class BOp, class Epi>
+inline int launch_igemm(const AOp &a, const BOp &b, const Epi &epi, u32 M, u32 N, u32 K, u32 zdim, u32 split_k,
+                        u32 k_per_z, hipStream_t stream, const char *what) {
+    IgemmDims d;
+    d.M = M, d.N = N, d.K = K;
+    d.tiles_m = ceil_div(M, Cfg::BM);
+    d.tiles_n = ceil_div(N, Cfg::BN);
+    d.split_k = split_k;
+    d.k_per_z = k_per_z;
+    const uint64_t tiles = uint64_t(d.tiles_m) * d.tiles_n;
+    if (tiles > 0x7fffffffull || zdim > 65535u) return fail(CRB_EINVAL_SHAPE, "%s: launch grid too large", what);
+    dim3 grid(u32(tiles), 1, zdim);
+    hipLaunchKernelGGL((igemm_kernel<Cfg, AOp, BOp, Epi>), grid, dim3(kThreads), 0, stream, a, b, epi, d);
+    return check_launch(what);
+}
+
+}  // namespace crb

@@ -1,0 +1,281 @@
+// Operand and epilogue functors for the contraction engine. An operand maps (row, k) of its panel to
+// a global-memory value (or 0 outside its extent); an epilogue maps (row, col, value) of the result to
+// a store. All offsets are uint32 element offsets (each tensor holds fewer than 2^31 elements).
+#pragma once
+#include "igemm_engine.h"
+
+namespace crb {
+
+// ---- plain matrices -----------------------------------------------------------------------------------
+// element(row, k) = base[row*ld + k]  (k contiguous): A of NN/NT, B of NT.
+template <bool VEC>
+struct MatK {
+    static constexpr bool kKFast = true, kVec = VEC;
+    const float *base;
+    u32 rows, ld, zstride;
+    struct RowS {
+        u32 off;
+        bool ok;
+    };
+    struct KS {
+        u32 k;
+        bool ok;
+    };
+    __device__ __forceinline__ void bind(u32 z) { base += size_t(z) * zstride; }
+    __device__ __forceinline__ RowS prep_row(u32 row) const { return {row * ld, row < rows}; }
+    __device__ __forceinline__ KS prep_k(u32 k, u32 klimit) const { return {k, k < klimit}; }
+    __device__ __forceinline__ float fetch(const RowS &r, const KS &k) const {
+        return (r.ok && k.ok) ? base[r.off + k.k] : 0.0f;
+    }
+    __device__ __forceinline__ v4f fetch4(u32 row, u32 k, u32 klimit) const {
+        if (row < rows && k < klimit) return *reinterpret_cast<const v4f *>(base + size_t(row) * ld + k);
+        return v4f{0.f, 0.f, 0.f, 0.f};
+    }
+};
+
+// element(row, k) = base[k*ld + row]  (row contiguous): B of NN/TN, A of TN.
+template <bool VEC>
+struct MatR {
+    static constexpr bool kKFast = false, kVec = VEC;
+    const float *base;
+    u32 rows, ld, zstride;
+    struct RowS {
+        u32 row;
+        bool ok;
+    };
+    struct KS {
+        u32 off;
+        bool ok;
+    };
+    __device__ __forceinline__ void bind(u32 z) { base += size_t(z) * zstride; }
+    __device__ __forceinline__ RowS prep_row(u32 row) const { return {row, row < rows}; }
+    __device__ __forceinline__ KS prep_k(u32 k, u32 klimit) const { return {k * ld, k < klimit}; }
+    __device__ __forceinline__ float fetch(const RowS &r, const KS &k) const {
+        return (r.ok && k.ok) ? base[k.off + r.row] : 0.0f;
+    }
+    __device__ __forceinline__ v4f fetch4(u32 row, u32 k, u32 klimit) const {
+        if (row < rows && k < klimit) return *reinterpret_cast<const v4f *>(base + size_t(k) * ld + row);
+        return v4f{0.f, 0.f, 0.f, 0.f};
+    }
+};
+
+// K-concatenated batch of k-contiguous matrices: kk -> (nd = kk / Kb, k = kk % Kb),
+// element(row, kk) = base[nd*bstride + row*ld + k]. Operands of the accumulate-NT form.
+template <bool VEC>
+struct MatKCat {
+    static constexpr bool kKFast = true, kVec = VEC;
+    const float *base;
+    u32 rows, ld, bstride;
+    FastDiv kb;
+    struct RowS {
+        u32 off;
+        bool ok;
+    };
+    struct KS {
+        u32 off;
+        bool ok;
+    };
+    __device__ __forceinline__ void bind(u32) {}
+    __device__ __forceinline__ u32 koff(u32 kk) const {
+        u32 nd, k;
+        kb.divmod(kk, nd, k);
+        return nd * bstride + k;
+    }
+    __device__ __forceinline__ RowS prep_row(u32 row) const { return {row * ld, row < rows}; }
+    __device__ __forceinline__ KS prep_k(u32 k, u32 klimit) const { return {koff(k), k < klimit}; }
+    __device__ __forceinline__ float fetch(const RowS &r, const KS &k) const {
+        return (r.ok && k.ok) ? base[r.off + k.off] : 0.0f;
+    }
+    __device__ __forceinline__ v4f fetch4(u32 row, u32 k, u32 klimit) const {
+        if (row < rows && k < klimit) return *reinterpret_cast<const v4f *>(base + size_t(row) * ld + koff(k));
+        return v4f{0.f, 0.f, 0.f, 0.f};
+    }
+};
+
+// element(row, k) = base[roff(row) + koff(k)] with roff = row*rstride and
+// koff(k) = (k / kdiv)*kouter + (k % kdiv)*kinner. Scalar only. Used for
+//   dgrad filters  A(ic, (oc,fh,fw)) = W[oc*IC*FHW + ic*FHW + r]      (kdiv = FHW, kouter = IC*FHW, kinner = 1)
+//   wgrad dY       A(oc, (n,oh,ow))  = dY[n*OC*OHW + oc*OHW + p]      (kdiv = OHW, kouter = OC*OHW, kinner = 1)
+struct SepK {
+    static constexpr bool kKFast = true, kVec = false;
+    const float *base;
+    u32 rows, rstride, kouter, kinner;
+    FastDiv kdiv;
+    struct RowS {
+        u32 off;
+        bool ok;
+    };
+    struct KS {
+        u32 off;
+        bool ok;
+    };
+    __device__ __forceinline__ void bind(u32) {}
+    __device__ __forceinline__ RowS prep_row(u32 row) const { return {row * rstride, row < rows}; }
+    __device__ __forceinline__ KS prep_k(u32 k, u32 klimit) const {
+        u32 q, r;
+        kdiv.divmod(k, q, r);
+        return {q * kouter + r * kinner, k < klimit};
+    }
+    __device__ __forceinline__ float fetch(const RowS &r, const KS &k) const {
+        return (r.ok && k.ok) ? base[r.off + k.off] : 0.0f;
+    }
+};
+
+// ---- implicit im2col gather ---------------------------------------------------------------------------
+// value(pixel j = (n, oh, ow), tap t = (ic, fh, fw)) = X[n, ic, oh*sH - pH + fh, ow*sW - pW + fw], 0 outside.
+struct Im2col {
+    const float *X;
+    u32 npix, ntap;  // N*OH*OW, IC*FH*FW
+    u32 IH, IW, img_stride /* IC*IH*IW */, chan_stride /* IH*IW */;
+    u32 sH, sW, pH, pW;
+    FastDiv ohw, ow, fhw, fw;
+    struct Pix {
+        u32 off;
+        int ih0, iw0;
+        bool ok;
+    };
+    struct Tap {
+        u32 off;
+        int fh, fw;
+        bool ok;
+    };
+    __device__ __forceinline__ Pix pixel(u32 j, u32 limit) const {
+        u32 n, p, oh, owi;
+        ohw.divmod(j, n, p);
+        ow.divmod(p, oh, owi);
+        return {n * img_stride, int(oh * sH) - int(pH), int(owi * sW) - int(pW), j < limit};
+    }
+    __device__ __forceinline__ Tap tap(u32 t, u32 limit) const {
+        u32 ic, r, fhi, fwi;
+        fhw.divmod(t, ic, r);
+        fw.divmod(r, fhi, fwi);
+        return {ic * chan_stride, int(fhi), int(fwi), t < limit};
+    }
+    __device__ __forceinline__ float fetch(const Pix &p, const Tap &t) const {
+        const int ih = p.ih0 + t.fh, iw = p.iw0 + t.fw;
+        const bool in = p.ok && t.ok && u32(ih) < IH && u32(iw) < IW;
+        return in ? X[p.off + t.off + u32(ih) * IW + u32(iw)] : 0.0f;
+    }
+};
+
+// conv forward B operand: rows are output pixels (contiguous in memory for a fixed tap), k are taps.
+struct Im2colPixRows {
+    static constexpr bool kKFast = false, kVec = false;
+    Im2col g;
+    typedef Im2col::Pix RowS;
+    typedef Im2col::Tap KS;
+    __device__ __forceinline__ void bind(u32) {}
+    __device__ __forceinline__ RowS prep_row(u32 row) const { return g.pixel(row, g.npix); }
+    __device__ __forceinline__ KS prep_k(u32 k, u32 klimit) const { return g.tap(k, klimit); }
+    __device__ __forceinline__ float fetch(const RowS &r, const KS &k) const { return g.fetch(r, k); }
+};
+
+// conv wgrad B operand: rows are taps (ic,fh,fw), k are output pixels (contiguous for a fixed tap).
+struct Im2colTapRows {
+    static constexpr bool kKFast = true, kVec = false;
+    Im2col g;
+    typedef Im2col::Tap RowS;
+    typedef Im2col::Pix KS;
+    __device__ __forceinline__ void bind(u32) {}
+    __device__ __forceinline__ RowS prep_row(u32 row) const { return g.tap(row, g.ntap); }
+    __device__ __forceinline__ KS prep_k(u32 k, u32 klimit) const { return g.pixel(k, klimit); }
+    __device__ __forceinline__ float fetch(const RowS &r, const KS &k) const { return g.fetch(k, r); }
+};
+
+// conv dgrad B operand: rows are input pixels j = (n, y, x); k = (oc, fh, fw);
+// value = dY[n, oc, (y+pH-fh)/sH, (x+pW-fw)/sW] where both divisions are exact and in range, else 0.
+struct DgradGather {
+    static constexpr bool kKFast = false, kVec = false;
+    const float *dY;
+    u32 npix;  // N*IH*IW
+    u32 OH, OW, img_stride /* OC*OH*OW */, chan_stride /* OH*OW */;
+    u32 pH, pW;
+    FastDiv ihw, iw, fhw, fw, sH, sW;
+    struct RowS {
+        u32 off;
+        int yp, xp;
+        bool ok;
+    };
+    struct KS {
+        u32 off;
+        int fh, fw;
+        bool ok;
+    };
+    __device__ __forceinline__ void bind(u32) {}
+    __device__ __forceinline__ RowS prep_row(u32 j) const {
+        u32 n, p, y, x;
+        ihw.divmod(j, n, p);
+        iw.divmod(p, y, x);
+        return {n * img_stride, int(y + pH), int(x + pW), j < npix};
+    }
+    __device__ __forceinline__ KS prep_k(u32 k, u32 klimit) const {
+        u32 oc, r, fhi, fwi;
+        fhw.divmod(k, oc, r);
+        fw.divmod(r, fhi, fwi);
+        return {oc * chan_stride, int(fhi), int(fwi), k < klimit};
+    }
+    __device__ __forceinline__ float fetch(const RowS &r, const KS &k) const {
+        const int th = r.yp - k.fh, tw = r.xp - k.fw;
+        if (!(r.ok && k.ok) || th < 0 || tw < 0) return 0.0f;
+        u32 oh, rh, ow, rw;
+        sH.divmod(u32(th), oh, rh);
+        sW.divmod(u32(tw), ow, rw);
+        if (rh != 0 || rw != 0 || oh >= OH || ow >= OW) return 0.0f;
+        return dY[r.off + k.off + oh * OW + ow];
+    }
+};
+
+// ---- epilogues ----------------------------------------------------------------------------------------
+enum : u32 { EPI_ACCUM = 1u, EPI_RELU = 2u };
+
+// Row-major result C[z*zstride + row*ld + col], optional per-column bias (dense layer), optional
+// accumulate (C += v) and ReLU.
+struct RowMajorEpi {
+    float *C;
+    const float *col_bias;
+    u32 ld, zstride, flags;
+    struct ColS {
+        u32 col;
+        float bias;
+        bool ok;
+    };
+    __device__ __forceinline__ void bind(u32 z) { C += size_t(z) * zstride; }
+    __device__ __forceinline__ ColS prep_col(u32 col, u32 ncols) const {
+        const bool ok = col < ncols;
+        return {col, (ok && col_bias) ? col_bias[col] : 0.0f, ok};
+    }
+    __device__ __forceinline__ void store(u32 row, const ColS &c, float v) const {
+        if (!c.ok) return;
+        float *p = C + size_t(row) * ld + c.col;
+        v += c.bias;
+        if (flags & EPI_ACCUM) v += *p;
+        if (flags & EPI_RELU) v = v > 0.0f ? v : 0.0f;
+        *p = v;
+    }
+};
+
+// NCHW scatter: row = channel, col = n*HW + p  ->  T[(n*C + row)*HW + p], optional per-row bias, ReLU.
+struct NchwEpi {
+    float *T;
+    const float *row_bias;
+    u32 C, HW, flags;
+    FastDiv hw;
+    struct ColS {
+        u32 off;
+        bool ok;
+    };
+    __device__ __forceinline__ void bind(u32) {}
+    __device__ __forceinline__ ColS prep_col(u32 col, u32 ncols) const {
+        u32 n, p;
+        hw.divmod(col, n, p);
+        return {n * C * HW + p, col < ncols};
+    }
+    __device__ __forceinline__ void store(u32 row, const ColS &c, float v) const {
+        if (!c.ok) return;
+        if (row_bias) v += row_bias[row];
+        if (flags & EPI_RELU) v = v > 0.0f ? v : 0.0f;
+        T[c.off + row * HW] = v;
+    }
+};
+
+}  // namespace crb

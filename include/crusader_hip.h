@@ -1,0 +1,139 @@
+/*
+ * crusader_hip.h — C ABI of the MI355X (gfx950) implementation of the seblas fp32 GEMM /
+ * linear / convolution hot path.
+ *
+ * Conventions
+ *   - Every pointer is a DEVICE pointer to row-major fp32 (tensors are NCHW), owned by the caller.
+ *     The library never frees caller memory and never retains a pointer after the call returns.
+ *   - Dimensions are passed by value as uint32_t. Any dimension >= 1 is accepted; element counts of
+ *     a single operand must stay below 2^31.
+ *   - `stream` is a hipStream_t passed as void* (NULL = the default stream). Calls only enqueue work;
+ *     they do not synchronise. The reference's blocking behaviour (cudaDeviceSynchronize after every
+ *     op, e.g. seblas/operations/cuGEMM.cu:1661) is restored by the C++ seblas wrappers, which
+ *     synchronise the stream after the call.
+ *   - Return value: CRB_OK (0) or a negative crb_status. The reference signals the same conditions
+ *     with assert()/std::invalid_argument (shape) and std::runtime_error (device error,
+ *     seblas/assist/CudaAssert.cu:8-15); the C++ wrappers translate. crb_last_error_string() gives
+ *     the message of the calling thread's most recent failure.
+ *   - "overwrite" entry points write every element of their output; "accumulate" entry points
+ *     read-modify-write it (C += ...), exactly once per element, deterministically.
+ */
+#ifndef CRUSADER_HIP_H
+#define CRUSADER_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum crb_status {
+    CRB_OK = 0,
+    CRB_EINVAL_SHAPE = -1, /* a shape relation the reference asserts does not hold, or a zero dim */
+    CRB_ENULL = -2,        /* a required pointer is NULL */
+    CRB_EHIP = -3,         /* a HIP runtime call or kernel launch failed */
+    CRB_EWORKSPACE = -4    /* caller-provided workspace is too small */
+} crb_status;
+
+/* Flags for crb_conv_fwd / crb_linear_fwd. Default 0 reproduces the reference (bias only). */
+#define CRB_FLAG_NONE 0u
+#define CRB_FLAG_RELU 1u /* extra, not in the reference: clamp the output at 0 in the epilogue */
+
+/* Library / device ------------------------------------------------------------------------- */
+
+/* Version of this ABI (major*1000 + minor). */
+int crb_abi_version(void);
+
+/* Message for the most recent non-OK status returned to the calling thread ("" if none). */
+const char *crb_last_error_string(void);
+
+/* Releases the library's lazily grown split-K scratch arena (safe to call at any time when no
+ * library kernel is in flight). */
+void crb_release_workspace(void);
+
+/* GEMM family ------------------------------------------------------------------------------ */
+
+/* Replaces seblas::sgemm (seblas/operations/cuGEMM.cu:1649-1664; kernels :34-210, :791-999).
+ * For nd in [0,batch): C[nd] (MxN) = A (MxK) * B[nd] (KxN). A is shared across the batch
+ * (batch = B.n in the reference). Overwrite. */
+int crb_sgemm_nn(const float *A, const float *B, float *C, uint32_t M, uint32_t N, uint32_t K, uint32_t batch,
+                 void *stream);
+
+/* Replaces seblas::sgemmTN (cuGEMM.cu:1667-1682; kernels :229-409, :1016-1217).
+ * For nd in [0,batch): C[nd] (MxN) = A^T * B[nd], A stored K x M. Overwrite. */
+int crb_sgemm_tn(const float *A, const float *B, float *C, uint32_t M, uint32_t N, uint32_t K, uint32_t batch,
+                 void *stream);
+
+/* Replaces seblas::sgemmNT (cuGEMM.cu:1685-1699; kernels :427-595, :1222-1429).
+ * C (MxN) = A (MxK) * B^T, B stored N x K. No batch. Overwrite. */
+int crb_sgemm_nt(const float *A, const float *B, float *C, uint32_t M, uint32_t N, uint32_t K, void *stream);
+
+/* Replaces seblas::sgemmNTA (cuGEMM.cu:1701-1714; kernels :600-773, :1434-1647).
+ * C (MxN) += sum_{nd<batch} A[nd] (MxK) * B[nd]^T (B[nd] stored N x K). Accumulate. */
+int crb_sgemm_nta(const float *A, const float *B, float *C, uint32_t M, uint32_t N, uint32_t K, uint32_t batch,
+                  void *stream);
+
+/* Dense-layer family ------------------------------------------------------------------------ */
+
+/* Replaces seblas::linear (seblas/operations/cuLinear.cu:1052-1072; kernels :33-206, :224-439).
+ * Y (batch x OUT) = X (batch x IN) * W^T (W stored OUT x IN) + bias (OUT). bias must not be NULL
+ * (the reference dereferences it unconditionally). Overwrite. flags: CRB_FLAG_*. */
+int crb_linear_fwd(const float *X, const float *W, const float *bias, float *Y, uint32_t batch, uint32_t IN,
+                   uint32_t OUT, uint32_t flags, void *stream);
+
+/* Replaces seblas::linearXGrad (cuLinear.cu:1075-1095; kernels :457-631, :649-854).
+ * dX (batch x IN) = dY (batch x OUT) * W (OUT x IN). Overwrite. */
+int crb_linear_dgrad(const float *dY, const float *W, float *dX, uint32_t batch, uint32_t IN, uint32_t OUT,
+                     void *stream);
+
+/* Replaces seblas::linearParamGrad (cuLinear.cu:1098-1113; kernel :872-1049).
+ * dW (OUT x IN) += dY^T * X; dB (OUT) += column sums of dY (each element updated exactly once;
+ * dB may be NULL to skip it). Accumulate. */
+int crb_linear_wgrad(const float *dY, const float *X, float *dW, float *dB, uint32_t batch, uint32_t IN,
+                     uint32_t OUT, void *stream);
+
+/* Convolution family ------------------------------------------------------------------------ */
+
+/* Geometry shared by the three convolution passes. OH/OW are the output-feature extents the caller's
+ * tensors have; they must satisfy the relation the reference's assertConv checks
+ * (cuConv.cu:731-755): OH == (IH - FH + 2*pH)/sH + 1 and likewise for OW (integer division). */
+typedef struct crb_conv_geom {
+    uint32_t N;          /* batch */
+    uint32_t IC, IH, IW; /* input features  N x IC x IH x IW */
+    uint32_t OC, FH, FW; /* filters         OC x IC x FH x FW */
+    uint32_t OH, OW;     /* output features N x OC x OH x OW */
+    uint32_t sH, sW;     /* strides (>= 1) */
+    uint32_t pH, pW;     /* zero padding */
+} crb_conv_geom;
+
+/* Replaces seblas::conv (seblas/operations/cuConv.cu:757-770; kernel :32-243).
+ * Y[n,oc,oh,ow] = sum_{ic,fh,fw} W[oc,ic,fh,fw] * X[n,ic,oh*sH-pH+fh,ow*sW-pW+fw] (+ bias[oc]);
+ * taps outside the image contribute 0; bias may be NULL. Overwrite. flags: CRB_FLAG_*. */
+int crb_conv_fwd(const float *W, const float *X, float *Y, const float *bias_or_null, const crb_conv_geom *g,
+                 uint32_t flags, void *stream);
+
+/* Replaces seblas::convDerive (cuConv.cu:774-790; kernel :262-483).
+ * dX[n,ic,y,x] = sum over (oc,fh,fw) with y+pH-fh = oh*sH, x+pW-fw = ow*sW, 0<=oh<OH, 0<=ow<OW of
+ * W[oc,ic,fh,fw] * dY[n,oc,oh,ow]. Overwrite. */
+int crb_conv_dgrad(const float *W, const float *dY, float *dX, const crb_conv_geom *g, void *stream);
+
+/* Bytes of scratch crb_conv_wgrad needs for this geometry (0 if none). */
+size_t crb_conv_wgrad_workspace_bytes(const crb_conv_geom *g);
+
+/* Replaces seblas::convError (cuConv.cu:793-806; kernel :488-707).
+ * dW[oc,ic,fh,fw] += sum_{n,oh,ow} dY[n,oc,oh,ow] * X[n,ic,oh*sH-pH+fh,ow*sW-pW+fw]. Accumulate.
+ * The reduction over n*OH*OW is split across workgroups and combined in a fixed order (no atomics),
+ * so results are bit-reproducible. `workspace` may be NULL: the library then uses its own lazily
+ * grown arena (which may call hipMalloc on first use / growth); otherwise it must hold at least
+ * crb_conv_wgrad_workspace_bytes(g) bytes. */
+int crb_conv_wgrad(const float *dY, const float *X, float *dW, const crb_conv_geom *g, void *workspace,
+                   size_t workspace_bytes, void *stream);
+
+/* Replaces seblas::convBias (cuConv.cu:808-818; kernel :709-729). Y[n,c,:,:] += bias[c], in place. */
+int crb_conv_bias(float *Y, const float *bias, uint32_t N, uint32_t C, uint32_t HW, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* CRUSADER_HIP_H */

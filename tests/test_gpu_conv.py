@@ -1,0 +1,189 @@
+"""GPU parity of the convolution entry points (through the C ABI) against the CPU oracle.
+
+The reference only ever tested dgrad with stride 1 / pad 0 (validation/UnitTestTools.cu:172-300);
+this grid keeps that family and adds strides, padding, forward, wgrad, bias and the BASELINE layer shapes.
+"""
+import numpy as np
+import pytest
+
+from tests.util import assert_close, he_normal, normal, to_dev, to_np
+
+pytestmark = pytest.mark.gpu
+
+
+def _capi():
+    from crusaderbackend_amd import capi
+    return capi
+
+
+def _oracle():
+    from oracle import seblas_oracle
+    return seblas_oracle
+
+
+def _nan(dev, *shape):
+    import torch
+    return torch.full(shape, float("nan"), dtype=torch.float32, device=dev)
+
+
+def run_layer(dev, N, IC, IH, IW, OC, FH, FW, sH, sW, pH, pW, bias=False, seed=0, ws=False):
+    import torch
+    capi, orc = _capi(), _oracle()
+    g = capi.ConvGeom.make(N, IC, IH, IW, OC, FH, FW, sH, sW, pH, pW)
+    X = normal(seed + 10, N, IC, IH, IW)
+    W = he_normal(seed + 20, OC, IC, FH, FW)
+    dY = normal(seed + 30, N, OC, g.OH, g.OW)
+    b = normal(seed + 40, OC) if bias else None
+    tag = f"N{N} {IC}->{OC} {IH}x{IW} f{FH}x{FW} s{sH}{sW} p{pH}{pW}"
+    dX_, dW_, dYd = to_dev(X, dev), to_dev(W, dev), to_dev(dY, dev)
+
+    Y = _nan(dev, N, OC, g.OH, g.OW)
+    capi.conv_fwd(dW_, dX_, Y, None if b is None else to_dev(b, dev), g)
+    assert_close(to_np(Y), orc.conv(W, X, b, sH, sW, pH, pW, threads=8), IC * FH * FW, "conv fwd " + tag)
+
+    dX = _nan(dev, N, IC, IH, IW)
+    capi.conv_dgrad(dW_, dYd, dX, g)
+    assert_close(to_np(dX), orc.convDerive(W, dY, (IH, IW), sH, sW, pH, pW, threads=8), OC * FH * FW,
+                 "conv dgrad " + tag)
+
+    dW0 = normal(seed + 50, OC, IC, FH, FW)
+    dWt = to_dev(dW0, dev)
+    wsbuf = None
+    if ws:
+        nbytes = capi.conv_wgrad_workspace_bytes(g)
+        wsbuf = torch.empty(max(nbytes // 4, 1), dtype=torch.float32, device=dev)
+    capi.conv_wgrad(dYd, dX_, dWt, g, workspace=wsbuf)
+    assert_close(to_np(dWt), orc.convError(dY, X, dW0, sH, sW, pH, pW, threads=8), N * g.OH * g.OW,
+                 "conv wgrad " + tag)
+
+
+# (N, IC, IH, IW, OC, FH, FW, sH, sW, pH, pW)
+SMALL = [
+    (1, 1, 4, 4, 1, 1, 1, 1, 1, 0, 0),
+    (2, 3, 8, 8, 4, 3, 3, 1, 1, 1, 1),
+    (2, 3, 9, 7, 5, 3, 3, 2, 2, 1, 1),
+    (3, 5, 11, 13, 7, 2, 4, 1, 2, 0, 1),
+    (2, 4, 16, 16, 6, 5, 5, 2, 1, 2, 2),
+    (1, 8, 10, 10, 130, 3, 3, 1, 1, 1, 1),
+    (2, 130, 6, 6, 9, 1, 1, 1, 1, 0, 0),
+    (4, 6, 12, 12, 12, 1, 1, 2, 2, 0, 0),
+    (2, 2, 7, 7, 3, 7, 7, 1, 1, 0, 0),
+    (2, 2, 5, 6, 3, 3, 3, 3, 3, 2, 2),
+]
+
+
+@pytest.mark.parametrize("shape", SMALL)
+def test_conv_small_grid(dev, shape):
+    run_layer(dev, *shape, bias=False, seed=1)
+    run_layer(dev, *shape, bias=True, seed=2, ws=True)
+
+
+@pytest.mark.parametrize("feature,filt,C1,C2,N", [(8, 2, 4, 8, 2), (16, 4, 16, 3, 4), (32, 8, 2, 5, 1), (4, 1, 64, 32, 8)])
+def test_conv_reference_unit_grid(dev, feature, filt, C1, C2, N):
+    """Shape family of the reference's convUnitTest: square features/filters, stride 1, pad 0."""
+    run_layer(dev, N, C1, feature, feature, C2, filt, filt, 1, 1, 0, 0, seed=3)
+
+
+RESNET = [
+    (16, 32, 16, 1),  # 16->16 @32x32
+    (32, 16, 32, 1),  # 32->32 @16x16
+    (64, 8, 64, 1),   # 64->64 @8x8
+    (16, 32, 32, 2),  # 16->32 stride 2
+    (32, 16, 64, 2),  # 32->64 stride 2
+]
+
+
+@pytest.mark.parametrize("IC,H,OC,s", RESNET)
+def test_conv_resnet56_layers(dev, IC, H, OC, s):
+    """BASELINE config 2 layer shapes (3x3, pad 1) at batch 16; the full batch-128 shapes are covered by the
+    adjoint property test below."""
+    run_layer(dev, 16, IC, H, H, OC, 3, 3, s, s, 1, 1, seed=4)
+
+
+@pytest.mark.parametrize("IC,H", [(24, 32), (108, 16), (330, 8)])
+def test_conv_densenet_layers(dev, IC, H):
+    """BASELINE config 4: 1x1 IC->48 bottleneck then 3x3 48->12, with bias, batch 8."""
+    run_layer(dev, 8, IC, H, H, 48, 1, 1, 1, 1, 0, 0, bias=True, seed=5)
+    run_layer(dev, 8, 48, H, H, 12, 3, 3, 1, 1, 1, 1, bias=True, seed=6)
+
+
+def test_conv_vgg_stem_and_wide(dev):
+    run_layer(dev, 4, 3, 32, 32, 64, 3, 3, 1, 1, 1, 1, bias=True, seed=7)
+    run_layer(dev, 2, 256, 4, 4, 512, 3, 3, 1, 1, 1, 1, bias=True, seed=8)
+
+
+@pytest.mark.parametrize("IC,H,OC,s", RESNET)
+def test_conv_full_batch_adjoint(dev, IC, H, OC, s):
+    """Size-independent property at the full BASELINE batch (128): <conv(W,X), dY> = <X, dgrad(W,dY)> =
+    <W, wgrad(dY,X)>, inner products accumulated in float64 on the device results."""
+    import torch
+    capi = _capi()
+    N = 128
+    g = capi.ConvGeom.make(N, IC, H, H, OC, 3, 3, s, s, 1, 1)
+    X, W, dY = normal(10, N, IC, H, H), he_normal(20, OC, IC, 3, 3), normal(30, N, OC, g.OH, g.OW)
+    Xd, Wd, dYd = to_dev(X, dev), to_dev(W, dev), to_dev(dY, dev)
+    Y = _nan(dev, N, OC, g.OH, g.OW)
+    dX = _nan(dev, N, IC, H, H)
+    dW = torch.zeros(OC, IC, 3, 3, device=dev)
+    capi.conv_fwd(Wd, Xd, Y, None, g)
+    capi.conv_dgrad(Wd, dYd, dX, g)
+    capi.conv_wgrad(dYd, Xd, dW, g)
+    a = float(np.vdot(to_np(Y).astype(np.float64), dY.astype(np.float64)))
+    b = float(np.vdot(to_np(dX).astype(np.float64), X.astype(np.float64)))
+    c = float(np.vdot(to_np(dW).astype(np.float64), W.astype(np.float64)))
+    scale = float(np.linalg.norm(to_np(Y).astype(np.float64)) * np.linalg.norm(dY.astype(np.float64)))
+    assert abs(a - b) <= 1e-5 * scale and abs(a - c) <= 1e-5 * scale, (a, b, c, scale)
+
+
+def test_conv_wgrad_accumulates_and_is_deterministic(dev):
+    import torch
+    capi = _capi()
+    g = capi.ConvGeom.make(32, 16, 32, 32, 16, 3, 3, 1, 1, 1, 1)
+    X, dY = normal(1, 32, 16, 32, 32), normal(2, 32, 16, 32, 32)
+    Xd, dYd = to_dev(X, dev), to_dev(dY, dev)
+    dW = torch.zeros(16, 16, 3, 3, device=dev)
+    capi.conv_wgrad(dYd, Xd, dW, g)
+    once = to_np(dW).copy()
+    capi.conv_wgrad(dYd, Xd, dW, g)
+    np.testing.assert_allclose(to_np(dW), 2 * once, rtol=1e-6, atol=0)
+    dW2 = torch.zeros(16, 16, 3, 3, device=dev)
+    capi.conv_wgrad(dYd, Xd, dW2, g)
+    assert np.array_equal(to_np(dW2), once), "split-K reduction must be bit-reproducible"
+
+
+def test_conv_bias_entry(dev):
+    capi, orc = _capi(), _oracle()
+    Y0, b = normal(1, 5, 7, 6, 3), normal(2, 7)
+    Y = to_dev(Y0, dev)
+    capi.conv_bias(Y, to_dev(b, dev), 5, 7, 18)
+    assert np.array_equal(to_np(Y), orc.convBias(Y0, b))
+
+
+def test_conv_bias_null_equals_zero_bias(dev):
+    import torch
+    capi = _capi()
+    g = capi.ConvGeom.make(2, 3, 8, 8, 4, 3, 3, 1, 1, 1, 1)
+    X, W = to_dev(normal(1, 2, 3, 8, 8), dev), to_dev(he_normal(2, 4, 3, 3, 3), dev)
+    Y1, Y2 = _nan(dev, 2, 4, 8, 8), _nan(dev, 2, 4, 8, 8)
+    capi.conv_fwd(W, X, Y1, None, g)
+    capi.conv_fwd(W, X, Y2, torch.zeros(4, device=dev), g)
+    assert np.array_equal(to_np(Y1), to_np(Y2))
+
+
+def test_conv_shape_errors(dev):
+    import ctypes
+    import torch
+    capi = _capi()
+    lib = capi.load()
+    t = torch.zeros(4096, device=dev)
+    g = capi.ConvGeom.make(1, 2, 8, 8, 2, 3, 3, 1, 1, 1, 1, OH=7, OW=8)
+    st = lib.crb_conv_fwd(t.data_ptr(), t.data_ptr(), t.data_ptr(), None, ctypes.byref(g), 0, None)
+    assert st == capi.CRB_EINVAL_SHAPE and b"rows (h) relationship" in lib.crb_last_error_string()
+    g = capi.ConvGeom.make(1, 2, 8, 8, 2, 3, 3, 1, 1, 1, 1, OH=8, OW=9)
+    st = lib.crb_conv_dgrad(t.data_ptr(), t.data_ptr(), t.data_ptr(), ctypes.byref(g), None)
+    assert st == capi.CRB_EINVAL_SHAPE and b"cols (w) relationship" in lib.crb_last_error_string()
+    g = capi.ConvGeom.make(64, 16, 32, 32, 16, 3, 3, 1, 1, 1, 1)
+    need = capi.conv_wgrad_workspace_bytes(g)
+    assert need > 0
+    st = lib.crb_conv_wgrad(t.data_ptr(), t.data_ptr(), t.data_ptr(), ctypes.byref(g), t.data_ptr(), 16, None)
+    assert st == capi.CRB_EWORKSPACE

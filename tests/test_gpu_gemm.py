@@ -1,0 +1,165 @@
+"""GPU parity of the GEMM and dense-layer entry points (through the C ABI) against the CPU oracle.
+
+Case grids follow the reference's own differential tests (validation/UnitTestTools.cu:130-170 for the
+linear/NTA identity) plus the sizes its `%4` kernel-selection rules and 128-wide tiles make interesting
+(seblas/operations/cuGEMM.cu:1653-1660).
+"""
+import numpy as np
+import pytest
+
+from tests.util import assert_close, to_dev, to_np, uniform, normal
+
+pytestmark = pytest.mark.gpu
+
+ODD = [1, 2, 3, 5, 7, 127, 129, 130]
+
+
+def _capi():
+    from crusaderbackend_amd import capi
+    return capi
+
+
+def _oracle():
+    from oracle import seblas_oracle
+    return seblas_oracle
+
+
+def _empty(dev, *shape):
+    import torch
+    return torch.full(shape, float("nan"), dtype=torch.float32, device=dev)
+
+
+def run_nn(dev, M, N, K, batch, seed):
+    A = uniform(seed, M, K)
+    B = uniform(seed + 1, batch, K, N)
+    C = _empty(dev, batch, M, N)
+    _capi().sgemm_nn(to_dev(A, dev), to_dev(B, dev), C, M, N, K, batch)
+    assert_close(to_np(C), _oracle().sgemm(A, B, threads=8), K, f"sgemm_nn {M}x{N}x{K} b{batch}")
+
+
+def run_tn(dev, M, N, K, batch, seed):
+    A = uniform(seed, K, M)
+    B = uniform(seed + 1, batch, K, N)
+    C = _empty(dev, batch, M, N)
+    _capi().sgemm_tn(to_dev(A, dev), to_dev(B, dev), C, M, N, K, batch)
+    assert_close(to_np(C), _oracle().sgemmTN(A, B, threads=8), K, f"sgemm_tn {M}x{N}x{K} b{batch}")
+
+
+def run_nt(dev, M, N, K, seed):
+    A = uniform(seed, M, K)
+    B = uniform(seed + 1, N, K)
+    C = _empty(dev, M, N)
+    _capi().sgemm_nt(to_dev(A, dev), to_dev(B, dev), C, M, N, K)
+    assert_close(to_np(C), _oracle().sgemmNT(A, B, threads=8), K, f"sgemm_nt {M}x{N}x{K}")
+
+
+def run_nta(dev, M, N, K, batch, seed):
+    A = uniform(seed, batch, M, K)
+    B = uniform(seed + 1, batch, N, K)
+    C0 = uniform(seed + 2, M, N)
+    C = to_dev(C0, dev)
+    _capi().sgemm_nta(to_dev(A, dev), to_dev(B, dev), C, M, N, K, batch)
+    assert_close(to_np(C), _oracle().sgemmNTA(A, B, C0, threads=8), K * batch, f"sgemm_nta {M}x{N}x{K} b{batch}")
+
+
+def test_sgemm_config1_1024(dev):
+    """BASELINE config 1: M=N=K=1024, uniform[-1,1], fixed seeds."""
+    run_nn(dev, 1024, 1024, 1024, 1, seed=1)
+
+
+@pytest.mark.parametrize("M,N,K", [(m, n, k) for m in ODD for n in (1, 5, 129) for k in (1, 7, 130)])
+def test_sgemm_nn_odd(dev, M, N, K):
+    run_nn(dev, M, N, K, 1, seed=100 + M + N + K)
+
+
+@pytest.mark.parametrize("M,N,K,batch", [(64, 64, 64, 3), (130, 36, 20, 2), (256, 384, 128, 2), (8, 260, 24, 5)])
+def test_sgemm_nn_batched(dev, M, N, K, batch):
+    run_nn(dev, M, N, K, batch, seed=7)
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 1, 1), (3, 5, 7), (127, 129, 130), (128, 128, 16), (132, 260, 33),
+                                   (512, 256, 100), (64, 512, 12)])
+def test_sgemm_tn(dev, M, N, K):
+    run_tn(dev, M, N, K, 1, seed=11)
+    run_tn(dev, M, N, K, 2, seed=12)
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 1, 1), (3, 5, 7), (127, 129, 130), (129, 257, 64), (256, 130, 36),
+                                   (260, 260, 260), (512, 512, 128)])
+def test_sgemm_nt(dev, M, N, K):
+    run_nt(dev, M, N, K, seed=21)
+
+
+@pytest.mark.parametrize("M,N,K,batch", [(4, 6, 1, 128), (130, 66, 1, 16), (64, 64, 8, 4), (200, 100, 12, 3),
+                                         (129, 3, 5, 7), (256, 256, 64, 2)])
+def test_sgemm_nta(dev, M, N, K, batch):
+    run_nta(dev, M, N, K, batch, seed=31)
+
+
+def test_sgemm_nta_accumulates_twice(dev):
+    """Calling the accumulate form twice on a zero C doubles the single-call result."""
+    M, N, K, batch = 96, 80, 20, 3
+    A, B = uniform(1, batch, M, K), uniform(2, batch, N, K)
+    import torch
+    C = torch.zeros(M, N, device=dev)
+    dA, dB = to_dev(A, dev), to_dev(B, dev)
+    _capi().sgemm_nta(dA, dB, C, M, N, K, batch)
+    once = to_np(C).copy()
+    _capi().sgemm_nta(dA, dB, C, M, N, K, batch)
+    np.testing.assert_allclose(to_np(C), 2 * once, rtol=1e-6, atol=0)
+
+
+@pytest.mark.parametrize("batch,IN,OUT", [(1, 1, 1), (3, 7, 5), (128, 512, 512), (128, 512, 10), (64, 130, 66),
+                                          (33, 1024, 10), (256, 260, 132)])
+def test_linear_family(dev, batch, IN, OUT):
+    capi, orc = _capi(), _oracle()
+    X, W, b = normal(1, batch, IN), normal(2, OUT, IN, std=(2.0 / IN) ** 0.5), normal(3, OUT)
+    dY = normal(4, batch, OUT)
+    Y = _empty(dev, batch, OUT)
+    capi.linear_fwd(to_dev(X, dev), to_dev(W, dev), to_dev(b, dev), Y, batch, IN, OUT)
+    assert_close(to_np(Y), orc.linear(X, W, b, threads=8), IN, "linear")
+    dX = _empty(dev, batch, IN)
+    capi.linear_dgrad(to_dev(dY, dev), to_dev(W, dev), dX, batch, IN, OUT)
+    assert_close(to_np(dX), orc.linearXGrad(dY, W, threads=8), OUT, "linearXGrad")
+    dW0, dB0 = normal(5, OUT, IN), normal(6, OUT)
+    dW, dB = to_dev(dW0, dev), to_dev(dB0, dev)
+    capi.linear_wgrad(to_dev(dY, dev), to_dev(X, dev), dW, dB, batch, IN, OUT)
+    rW, rB = orc.linearParamGrad(dY, X, dW0, dB0, threads=8)
+    assert_close(to_np(dW), rW, batch, "linearParamGrad dW")
+    assert_close(to_np(dB), rB, batch, "linearParamGrad dB")
+
+
+def test_linear_param_grad_equals_nta_outer_products(dev):
+    """The reference's linearUnitTest identity (validation/UnitTestTools.cu:143-144): dW from
+    linearParamGrad equals sgemmNTA over the batch of K=1 outer products dY[n] x X[n]^T."""
+    import torch
+    capi = _capi()
+    batch, IN, OUT = 32, 48, 40
+    dY, X = normal(1, batch, OUT), normal(2, batch, IN)
+    dW1 = torch.zeros(OUT, IN, device=dev)
+    dB = torch.zeros(OUT, device=dev)
+    capi.linear_wgrad(to_dev(dY, dev), to_dev(X, dev), dW1, dB, batch, IN, OUT)
+    dW2 = torch.zeros(OUT, IN, device=dev)
+    # A = dY viewed as (batch, OUT, 1), B = X viewed as (batch, IN, 1)
+    capi.sgemm_nta(to_dev(dY, dev), to_dev(X, dev), dW2, OUT, IN, 1, batch)
+    np.testing.assert_allclose(to_np(dW1), to_np(dW2), atol=1e-3, rtol=0)  # abs 1e-3 as in the reference test
+
+
+def test_linear_relu_flag(dev):
+    capi, orc = _capi(), _oracle()
+    batch, IN, OUT = 16, 64, 48
+    X, W, b = normal(1, batch, IN), normal(2, OUT, IN), normal(3, OUT)
+    Y = _empty(dev, batch, OUT)
+    capi.linear_fwd(to_dev(X, dev), to_dev(W, dev), to_dev(b, dev), Y, batch, IN, OUT, flags=capi.CRB_FLAG_RELU)
+    assert_close(to_np(Y), np.maximum(orc.linear(X, W, b), 0), IN, "linear+relu")
+
+
+def test_error_paths(dev):
+    import torch
+    capi = _capi()
+    t = torch.zeros(16, device=dev)
+    lib = capi.load()
+    assert lib.crb_sgemm_nn(None, t.data_ptr(), t.data_ptr(), 4, 4, 1, 1, None) == capi.CRB_ENULL
+    assert lib.crb_sgemm_nn(t.data_ptr(), t.data_ptr(), t.data_ptr(), 0, 4, 1, 1, None) == capi.CRB_EINVAL_SHAPE
+    assert b"zero dimension" in lib.crb_last_error_string()
+    assert lib.crb_linear_fwd(t.data_ptr(), t.data_ptr(), None, t.data_ptr(), 1, 4, 4, 0, None) == capi.CRB_ENULL
