@@ -1,0 +1,234 @@
+#!/usr/bin/env python3
+"""Benchmark of the seblas conv/GEMM hot path on one MI355X.
+
+Default workload (BASELINE config 2): the convolution layers of ResNet-56 on CIFAR-shaped tensors, fp32 NCHW,
+batch 128. One *step* = forward + data-gradient + weight-gradient of every 3x3 conv layer of the network's three
+stages and two stride-2 transitions, with the layer multiplicities of the reference's archived model
+(archive/Resnet56: 19x 16->16@32, 17x 32->32@16, 18x 64->64@8, 1x 16->32 s2, 1x 32->64 s2), on synthetic
+N(0,1) activations/gradients and He-normal filters already resident in HBM. Flops are nominal
+(2*N*OC*OH*OW*IC*FH*FW per pass; zeros from stride/padding are not discounted).
+
+Prints ONE JSON line. `value` is TFLOP/s over the timed steps; `extra` carries images/s and the 4096^3 sgemm rate.
+`roofline` describes the kernel that takes the most time in the step, timed per launch with HIP events on the
+launch stream in a separate instrumented pass. `cpu_baseline` is the CPU oracle on a bounded sample.
+
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--report FILE]   (--report adds every BASELINE config)
+"""
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_FP32_MFMA_TFLOPS = 157.3  # 256 CU x 2.4 GHz x 256 flop/clk/CU
+PEAK_HBM_GBS = 8000.0
+
+# (name, IC, H, OC, stride, multiplicity) — 3x3, pad 1
+RESNET56 = [
+    ("L1_16-16@32", 16, 32, 16, 1, 19),
+    ("L2_32-32@16", 32, 16, 32, 1, 17),
+    ("L3_64-64@8", 64, 8, 64, 1, 18),
+    ("T1_16-32s2", 16, 32, 32, 2, 1),
+    ("T2_32-64s2", 32, 16, 64, 2, 1),
+]
+BATCH = 128
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--report", type=str, default=None, help="also time every BASELINE config and write a JSON report")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
+    return ap.parse_args()
+
+
+class Layer:
+    def __init__(self, torch, capi, dev, name, IC, H, OC, s, mult, seed, batch=BATCH, F=3, pad=1, bias=False):
+        self.name, self.mult = name, mult
+        self.g = capi.ConvGeom.make(batch, IC, H, H, OC, F, F, s, s, pad, pad)
+        g = self.g
+        gen = torch.Generator(device="cpu").manual_seed(seed)
+        self.X = torch.randn(batch, IC, H, H, generator=gen).to(dev)
+        self.W = (torch.randn(OC, IC, F, F, generator=gen) * math.sqrt(2.0 / (IC * F * F))).to(dev)
+        self.dY = torch.randn(batch, OC, g.OH, g.OW, generator=gen).to(dev)
+        self.b = torch.randn(OC, generator=gen).to(dev) if bias else None
+        self.Y = torch.empty(batch, OC, g.OH, g.OW, device=dev)
+        self.dX = torch.empty(batch, IC, H, H, device=dev)
+        self.dW = torch.zeros(OC, IC, F, F, device=dev)
+        nbytes = capi.conv_wgrad_workspace_bytes(g)
+        self.ws = torch.empty(max(nbytes // 4, 1), dtype=torch.float32, device=dev) if nbytes else None
+        self.flops = 2.0 * batch * OC * g.OH * g.OW * IC * F * F
+        nb = 0 if self.b is None else OC
+        self.bytes = {
+            "fwd": 4.0 * (self.X.numel() + self.W.numel() + self.Y.numel() + nb),
+            "dgrad": 4.0 * (self.dY.numel() + self.W.numel() + self.dX.numel()),
+            "wgrad": 4.0 * (self.dY.numel() + self.X.numel() + 2 * self.dW.numel()),
+        }
+        self.capi = capi
+
+    def fwd(self):
+        self.capi.conv_fwd(self.W, self.X, self.Y, self.b, self.g)
+
+    def dgrad(self):
+        self.capi.conv_dgrad(self.W, self.dY, self.dX, self.g)
+
+    def wgrad(self):
+        self.capi.conv_wgrad(self.dY, self.X, self.dW, self.g, workspace=self.ws)
+
+    def passes(self):
+        return (("fwd", self.fwd), ("dgrad", self.dgrad), ("wgrad", self.wgrad))
+
+
+def event_time_ms(torch, fn, reps, warm=3):
+    """Average duration of `fn` (ms) over `reps` back-to-back launches between two events on the launch stream."""
+    for _ in range(warm):
+        fn()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(reps):
+        fn()
+    e1.record()
+    e1.synchronize()
+    return e0.elapsed_time(e1) / reps
+
+
+def cpu_baseline(layers_spec):
+    """CPU oracle on a bounded sample: the same step at batch 64 (half of the images), all host cores capped at 16."""
+    import numpy as np
+
+    from oracle import seblas_oracle as orc
+
+    threads = min(os.cpu_count() or 1, 16)
+    nb = 64
+    rng = np.random.default_rng(0)
+    work = []
+    flops = 0.0
+    for (_, IC, H, OC, s, mult) in layers_spec:
+        OH = (H + 2 - 3) // s + 1
+        X = rng.standard_normal((nb, IC, H, H)).astype(np.float32)
+        W = (rng.standard_normal((OC, IC, 3, 3)) * math.sqrt(2.0 / (IC * 9))).astype(np.float32)
+        dY = rng.standard_normal((nb, OC, OH, OH)).astype(np.float32)
+        work.append((X, W, dY, H, s, mult))
+        flops += 3 * mult * 2.0 * nb * OC * OH * OH * IC * 9
+    t0 = time.perf_counter()
+    for (X, W, dY, H, s, mult) in work:
+        for _ in range(mult):
+            orc.conv(W, X, None, s, s, 1, 1, threads=threads)
+            orc.convDerive(W, dY, (H, H), s, s, 1, 1, threads=threads)
+            orc.convError(dY, X, np.zeros_like(W), s, s, 1, 1, threads=threads)
+    dt = time.perf_counter() - t0
+    return {
+        "value": flops / dt / 1e12, "unit": "TFLOP/s", "cores": threads, "kind": "port",
+        "images_per_s": nb / dt, "seconds": dt,
+        "sample": f"one full ResNet-56 conv step (fwd+dgrad+wgrad, all 56 layers) at batch {nb} instead of {BATCH}, "
+                  f"fp32 loop oracle, {threads} threads",
+    }
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print("bench.py: this build targets one GPU per process and has no multi-GPU path; run with --gpus 1",
+              file=sys.stderr)
+        sys.exit(2)
+    import torch
+
+    from crusaderbackend_amd import capi
+
+    capi.load()
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    dev = torch.device("cuda:0")
+    props = torch.cuda.get_device_properties(0)
+
+    layers = [Layer(torch, capi, dev, n, IC, H, OC, s, m, seed=10 + i) for i, (n, IC, H, OC, s, m) in enumerate(RESNET56)]
+    step_flops = sum(3 * L.mult * L.flops for L in layers)
+
+    def step():
+        for L in layers:
+            for _ in range(L.mult):
+                L.fwd()
+        for L in reversed(layers):
+            for _ in range(L.mult):
+                L.dgrad()
+                L.wgrad()
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    ms_per_step = dt / args.steps * 1e3
+    tflops = step_flops * args.steps / dt / 1e12
+    images_per_s = BATCH * args.steps / dt
+
+    # instrumented pass: per-(layer, pass) launch duration with events on the launch stream
+    per = {}
+    for L in layers:
+        for pname, fn in L.passes():
+            ms = event_time_ms(torch, fn, reps=50)
+            per[f"{L.name}.{pname}"] = {
+                "ms": ms, "tflops": L.flops / ms / 1e9, "gbs": L.bytes[pname] / ms / 1e6, "mult": L.mult,
+                "flops": L.flops, "bytes": L.bytes[pname],
+            }
+    dom = max(per, key=lambda k: per[k]["ms"] * per[k]["mult"])
+    d = per[dom]
+    roofline = {
+        "bound": "mfma", "kernel": dom, "achieved": d["tflops"], "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s",
+        "frac": d["tflops"] / PEAK_FP32_MFMA_TFLOPS, "traffic": None,
+        "flops_per_launch": d["flops"], "avg_launch_ms": d["ms"],
+        "share_of_step": d["ms"] * d["mult"] / sum(v["ms"] * v["mult"] for v in per.values()),
+    }
+    kern_sum_ms = sum(v["ms"] * v["mult"] for v in per.values())
+
+    # headline GEMM target: 4096^3 sgemm
+    n = 4096
+    A = torch.rand(n, n, device=dev) * 2 - 1
+    B = torch.rand(n, n, device=dev) * 2 - 1
+    C = torch.empty(n, n, device=dev)
+    gemm_ms = event_time_ms(torch, lambda: capi.sgemm_nn(A, B, C, n, n, n), reps=10)
+    gemm_tflops = 2.0 * n ** 3 / gemm_ms / 1e9
+    del A, B, C
+
+    out = {
+        "metric": "fp32 conv TFLOP/s, ResNet-56 conv layers fwd+dgrad+wgrad (also % FP32 MFMA peak, images/s in extra)",
+        "value": tflops, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "ResNet-56 CIFAR conv shapes, fp32 NCHW, batch 128, 3x3 pad 1: 19x16->16@32, 17x32->32@16, "
+                               "18x64->64@8, 16->32 s2, 32->64 s2; forward + dgrad + wgrad per layer",
+                   "batch": BATCH, "flops_per_step": step_flops},
+        "roofline": roofline,
+        "extra": {
+            "frac_fp32_mfma_peak": tflops / PEAK_FP32_MFMA_TFLOPS,
+            "resnet56_conv_images_per_s": images_per_s,
+            "resnet56_conv_images_per_s_kernel_only": BATCH / (kern_sum_ms / 1e3),
+            "kernel_only_tflops": step_flops / kern_sum_ms / 1e9,
+            "sgemm_4096_tflops": gemm_tflops, "sgemm_4096_ms": gemm_ms,
+            "sgemm_4096_frac_peak": gemm_tflops / PEAK_FP32_MFMA_TFLOPS,
+            "per_kernel": {k: {"ms": round(v["ms"], 5), "tflops": round(v["tflops"], 2), "gbs": round(v["gbs"], 1)}
+                           for k, v in per.items()},
+            "device": props.name, "cus": props.multi_processor_count,
+        },
+    }
+    if not args.no_cpu:
+        out["cpu_baseline"] = cpu_baseline(RESNET56)
+    if args.report:
+        from crusaderbackend_amd import bench_report
+
+        rep = bench_report.run(torch, capi, dev, event_time_ms, Layer)
+        with open(args.report, "w") as f:
+            json.dump(rep, f, indent=1)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()
