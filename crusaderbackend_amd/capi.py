@@ -52,6 +52,9 @@ SIGNATURES = {
     "crb_conv_wgrad_workspace_bytes": (ctypes.c_size_t, [ctypes.POINTER(ConvGeom)]),
     "crb_conv_wgrad": (ctypes.c_int, [_ptr, _ptr, _ptr, ctypes.POINTER(ConvGeom), _ptr, ctypes.c_size_t, _ptr]),
     "crb_conv_bias": (ctypes.c_int, [_ptr, _ptr, _u32, _u32, _u32, _ptr]),
+    "crb_conv_bias_grad": (ctypes.c_int, [_ptr, _ptr, _u32, _u32, _u32, _ptr]),
+    "crb_tensor_add_inplace": (ctypes.c_int, [_ptr, _ptr, _u32, _ptr]),
+    "crb_tensor_fill": (ctypes.c_int, [_ptr, ctypes.c_float, _u32, _ptr]),
 }
 
 _lib = None
@@ -139,3 +142,15 @@ def conv_wgrad(dY, X, dW, geom, workspace=None, stream=None):
 
 def conv_bias(Y, bias, N, C, HW, stream=None):
     check(load().crb_conv_bias(_p(Y), _p(bias), N, C, HW, _stream(stream)))
+
+
+def conv_bias_grad(dY, dB, N, C, HW, stream=None):
+    check(load().crb_conv_bias_grad(_p(dY), _p(dB), N, C, HW, _stream(stream)))
+
+
+def tensor_add_inplace(a, b, count, stream=None):
+    check(load().crb_tensor_add_inplace(_p(a), _p(b), count, _stream(stream)))
+
+
+def tensor_fill(a, value, count, stream=None):
+    check(load().crb_tensor_fill(_p(a), value, count, _stream(stream)))

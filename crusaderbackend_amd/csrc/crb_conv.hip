@@ -80,6 +80,25 @@ __global__ void __launch_bounds__(256) conv_bias_kernel(float *__restrict__ Y, c
     Y[i] += bias[plane % C];
 }
 
+// One workgroup per channel: dB[c] += sum over (n, hw) of dY[n,c,hw]; fixed-order tree reduction in LDS.
+__global__ void __launch_bounds__(256) conv_bias_grad_kernel(const float *__restrict__ dY, float *__restrict__ dB, u32 N,
+                                                             u32 C, u32 HW) {
+    __shared__ float red[256];
+    const u32 c = blockIdx.x;
+    float s = 0.0f;
+    for (u32 n = 0; n < N; ++n) {
+        const float *p = dY + (size_t(n) * C + c) * HW;
+        for (u32 i = threadIdx.x; i < HW; i += 256) s += p[i];
+    }
+    red[threadIdx.x] = s;
+    __syncthreads();
+    for (u32 w = 128; w > 0; w >>= 1) {
+        if (threadIdx.x < w) red[threadIdx.x] += red[threadIdx.x + w];
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) dB[c] += red[0];
+}
+
 }  // namespace crb
 
 using namespace crb;
@@ -155,6 +174,15 @@ int crb_conv_wgrad(const float *dY, const float *X, float *dW, const crb_conv_ge
     const u32 count = p.M * p.Ncols;
     hipLaunchKernelGGL(splitk_reduce_kernel, dim3(ceil_div(count, 256)), dim3(256), 0, s, ws, dW, count, p.splits, 1u);
     return check_launch("crb_conv_wgrad(reduce)");
+}
+
+int crb_conv_bias_grad(const float *dY, float *dB, uint32_t N, uint32_t C, uint32_t HW, void *stream) {
+    if (!dY || !dB) return fail(CRB_ENULL, "crb_conv_bias_grad: null operand");
+    if (!N || !C || !HW) return fail(CRB_EINVAL_SHAPE, "crb_conv_bias_grad: zero dimension");
+    if (uint64_t(N) * C * HW > 0x7fffffffull)
+        return fail(CRB_EINVAL_SHAPE, "crb_conv_bias_grad: tensor exceeds 2^31 elements");
+    hipLaunchKernelGGL(conv_bias_grad_kernel, dim3(C), dim3(256), 0, hipStream_t(stream), dY, dB, N, C, HW);
+    return check_launch("crb_conv_bias_grad");
 }
 
 int crb_conv_bias(float *Y, const float *bias, uint32_t N, uint32_t C, uint32_t HW, void *stream) {

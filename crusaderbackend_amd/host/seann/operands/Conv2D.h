@@ -1,0 +1,34 @@
+// seann::Conv2D — the convolution operand calling the seblas path, with the reference's members, constructor
+// and method set (seann/operands/seblas/Conv2D.cuh:14-100, Conv2D.cu:8-57).
+#pragma once
+#include "OperandBase.h"
+
+#define OPR_SEBLAS_CONV2D 0x0002
+
+namespace seann {
+
+class Conv2D : public OperandBase {
+public:
+    shape4 filterShape;
+    NetParam *filter{};
+    NetParam *bias = nullptr;
+    uint32 strideH, strideW, padH, padW;
+    bool WITH_BIAS = false;
+
+    Conv2D(shape4 filterShape, uint32 strideH, uint32 strideW, uint32 padH, uint32 padW, bool WITH_BIAS)
+        : filterShape(filterShape), strideH(strideH), strideW(strideW), padH(padH), padW(padW), WITH_BIAS(WITH_BIAS) {}
+
+    std::string info() override {
+        return "Conv2D        { filter: " + filter->data()->dims.toString() + ", input feature: " + X->A->dims.toString() + " }";
+    }
+
+    // output shape (N, OC, (H + 2p - FH)/s + 1, (W + 2p - FW)/s + 1)  — Conv2D.cuh:40-44
+    void initNetParams(OptimizerInfo *info, shape4 inShape) override;
+    void forward() override;
+    void xGrads() override;
+    void paramGrads() override;
+    void randFillNetParams() override;
+    void zeroGrads() override;
+    uint32 OPERAND_ID() override { return OPR_SEBLAS_CONV2D; }
+};
+}  // namespace seann

@@ -1,0 +1,31 @@
+// seann::Linear — the dense operand calling the seblas path (seann/operands/seblas/Linear.cuh:14-73,
+// Linear.cu:8-60). The input is flattened to (N, 1, IN, 1); weights are stored OUT x IN.
+#pragma once
+#include "OperandBase.h"
+
+#define OPR_SEBLAS_LINEAR 0x0001
+
+namespace seann {
+
+class Linear : public OperandBase {
+public:
+    NetParam *weights{};
+    NetParam *biases{};
+    uint32 INPUT_SIZE{};
+    uint32 OUTPUT_SIZE;
+
+    explicit Linear(uint32 OUTPUT_SIZE) : OUTPUT_SIZE(OUTPUT_SIZE) {}
+
+    std::string info() override {
+        return "Linear        { " + std::to_string(INPUT_SIZE) + ", " + std::to_string(OUTPUT_SIZE) + " }";
+    }
+
+    void initNetParams(OptimizerInfo *info, shape4 inShape) override;
+    void forward() override;
+    void paramGrads() override;
+    void xGrads() override;
+    void randFillNetParams() override;
+    void zeroGrads() override;
+    uint32 OPERAND_ID() override { return OPR_SEBLAS_LINEAR; }
+};
+}  // namespace seann

@@ -1,0 +1,136 @@
+// seblas operator API over the C ABI: shape checks as in the reference, launch on the default stream,
+// block until done, translate status codes to exceptions. See operations.h.
+#include "operations.h"
+
+#include <hip/hip_runtime_api.h>
+
+#include <stdexcept>
+
+#include "../../../../include/crusader_hip.h"
+#include "../assist/HipAssert.h"
+
+namespace seblas {
+
+static void require(bool ok, const char *what) {
+    if (!ok) throw std::invalid_argument(what);
+}
+
+// every reference op ends with cudaDeviceSynchronize(); assertCuda(...)
+static void finish(int status, const char *file, int line) {
+    throwOnStatus(status, file, line);
+    if (hipStreamSynchronize(nullptr) != hipSuccess) assertHip(file, line);
+    assertHip(file, line);
+}
+
+Tensor *sgemm(Tensor *A, Tensor *B, Tensor *C) {
+    require(A->dims.w == B->dims.h, "sgemm: A.w != B.h");       // cuGEMM.cu:1650
+    require(A->dims.h == C->dims.h, "sgemm: A.h != C.h");       // :1651
+    require(B->dims.w == C->dims.w, "sgemm: B.w != C.w");       // :1652
+    finish(crb_sgemm_nn(A->elements, B->elements, C->elements, A->dims.h, B->dims.w, A->dims.w, B->dims.n, nullptr),
+           __FILE__, __LINE__);
+    return C;
+}
+
+Tensor *sgemmTN(Tensor *A, Tensor *B, Tensor *C) {
+    require(A->dims.h == B->dims.h, "sgemmTN: A.h != B.h");                                // :1668
+    require(A->dims.w == C->dims.h && B->dims.w == C->dims.w, "sgemmTN: C shape mismatch");  // :1669
+    finish(crb_sgemm_tn(A->elements, B->elements, C->elements, A->dims.w, B->dims.w, A->dims.h, B->dims.n, nullptr),
+           __FILE__, __LINE__);
+    return C;
+}
+
+Tensor *sgemmNT(Tensor *A, Tensor *B, Tensor *C) {
+    require(A->dims.w == B->dims.w, "sgemmNT: A.w != B.w");                                // :1686
+    require(A->dims.h == C->dims.h && B->dims.h == C->dims.w, "sgemmNT: C shape mismatch");  // :1687
+    finish(crb_sgemm_nt(A->elements, B->elements, C->elements, A->dims.h, B->dims.h, A->dims.w, nullptr), __FILE__,
+           __LINE__);
+    return C;
+}
+
+Tensor *sgemmNTA(Tensor *A, Tensor *B, Tensor *C) {
+    require(A->dims.w == B->dims.w, "sgemmNTA: A.w != B.w");                                // :1702
+    require(A->dims.h == C->dims.h && B->dims.h == C->dims.w, "sgemmNTA: C shape mismatch");  // :1703
+    finish(crb_sgemm_nta(A->elements, B->elements, C->elements, A->dims.h, B->dims.h, A->dims.w, A->dims.n, nullptr),
+           __FILE__, __LINE__);
+    return C;
+}
+
+Tensor *linear(Tensor *X, Tensor *W, Tensor *B, Tensor *Y) {
+    const uint32 M = Y->dims.h;                                  // cuLinear.cu:1053
+    const uint32 N = Y->dims.n * Y->dims.w;                      // :1054
+    require(W->dims.w == X->dims.h, "linear: W.w != X.h");       // :1056
+    require(B->dims.h == M, "linear: B.h != Y.h");               // :1057
+    require(Y->dims.w == 1 && B->dims.w == 1 && X->dims.w == 1, "linear: X, B, Y must have w == 1");  // :1058
+    require(X->dims.n == Y->dims.n, "linear: batch mismatch");   // :1059
+    require(W->dims.h == M, "linear: W.h != Y.h");
+    finish(crb_linear_fwd(X->elements, W->elements, B->elements, Y->elements, N, W->dims.w, M, 0, nullptr), __FILE__,
+           __LINE__);
+    return Y;
+}
+
+Tensor *linearXGrad(Tensor *dY, Tensor *W, Tensor *dX) {
+    const uint32 N = dX->dims.n * dX->dims.w;                                // :1077
+    require(W->dims.h == dY->dims.h, "linearXGrad: W.h != dY.h");            // :1079
+    require(dX->dims.n == dY->dims.n, "linearXGrad: batch mismatch");        // :1080
+    require(dX->dims.w == 1 && dY->dims.w == 1, "linearXGrad: w must be 1");  // :1081
+    require(W->dims.w == dX->dims.h, "linearXGrad: W.w != dX.h");            // :1082
+    finish(crb_linear_dgrad(dY->elements, W->elements, dX->elements, N, W->dims.w, W->dims.h, nullptr), __FILE__,
+           __LINE__);
+    return dX;
+}
+
+Tensor *linearParamGrad(Tensor *dY, Tensor *X, Tensor *dW, Tensor *dB) {
+    const uint32 M = dW->dims.h, N = dW->dims.w;                          // :1099-1100
+    require(X->dims.h == N, "linearParamGrad: X.h != dW.w");             // :1102
+    require(dY->dims.h == M, "linearParamGrad: dY.h != dW.h");           // :1103
+    require(X->dims.n == dY->dims.n, "linearParamGrad: batch mismatch");  // :1104
+    require(dB->dims.size == M, "linearParamGrad: dB size != dW.h");
+    finish(crb_linear_wgrad(dY->elements, X->elements, dW->elements, dB->elements, X->dims.n, N, M, nullptr), __FILE__,
+           __LINE__);
+    return dW;
+}
+
+// Geometry + the four relations of assertConv (cuConv.cu:731-755); h/w relations are checked by the C ABI with
+// the reference's messages, channel/batch relations here.
+static crb_conv_geom geom(Tensor *filters, Tensor *features, Tensor *featureOut, int sH, int sW, int pH, int pW) {
+    require(sH > 0 && sW > 0 && pH >= 0 && pW >= 0, "assertConv: stride must be positive and padding non-negative");
+    if (featureOut->dims.c != filters->dims.n || features->dims.c != filters->dims.c)
+        throw std::invalid_argument("assertConv: channels relationship did not satisfy");
+    if (featureOut->dims.n != features->dims.n) throw std::invalid_argument("assertConv: batch relationship did not satisfy");
+    crb_conv_geom g;
+    g.N = features->dims.n;
+    g.IC = features->dims.c, g.IH = features->dims.h, g.IW = features->dims.w;
+    g.OC = filters->dims.n, g.FH = filters->dims.h, g.FW = filters->dims.w;
+    g.OH = featureOut->dims.h, g.OW = featureOut->dims.w;
+    g.sH = uint32(sH), g.sW = uint32(sW), g.pH = uint32(pH), g.pW = uint32(pW);
+    return g;
+}
+
+Tensor *conv(Tensor *A, Tensor *B, Tensor *C, int strideH, int strideW, int padH, int padW, Tensor *biases) {
+    crb_conv_geom g = geom(A, B, C, strideH, strideW, padH, padW);
+    if (biases) require(biases->dims.size == g.OC, "conv: biases must hold OC elements");
+    finish(crb_conv_fwd(A->elements, B->elements, C->elements, biases ? biases->elements : nullptr, &g, 0, nullptr),
+           __FILE__, __LINE__);
+    return C;
+}
+
+Tensor *convDerive(Tensor *A, Tensor *B, Tensor *C, int strideH, int strideW, int padH, int padW) {
+    crb_conv_geom g = geom(A, C, B, strideH, strideW, padH, padW);  // assertConv(A, C, B, ...) cuConv.cu:775
+    finish(crb_conv_dgrad(A->elements, B->elements, C->elements, &g, nullptr), __FILE__, __LINE__);
+    return C;
+}
+
+Tensor *convError(Tensor *A, Tensor *B, Tensor *C, int strideH, int strideW, int padH, int padW) {
+    crb_conv_geom g = geom(C, B, A, strideH, strideW, padH, padW);  // assertConv(C, B, A, ...) cuConv.cu:794
+    finish(crb_conv_wgrad(A->elements, B->elements, C->elements, &g, nullptr, 0, nullptr), __FILE__, __LINE__);
+    return A;  // the reference returns its first argument (cuConv.cu:805)
+}
+
+Tensor *convBias(Tensor *Y, Tensor *biases) {
+    require(biases->dims.size == Y->dims.c, "convBias: bias size != channels");  // cuConv.cu:809
+    finish(crb_conv_bias(Y->elements, biases->elements, Y->dims.n, Y->dims.c, Y->dims.h * Y->dims.w, nullptr), __FILE__,
+           __LINE__);
+    return Y;
+}
+
+}  // namespace seblas

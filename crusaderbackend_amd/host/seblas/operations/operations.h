@@ -1,0 +1,33 @@
+// The seblas free-function operator API of the GEMM / linear / convolution path, with the reference's
+// signatures, argument meaning, return-pointer quirks, blocking behaviour and error behaviour
+// (seblas/operations/cuGEMM.cuh:12-21, cuConv.cuh:20-42, cuLinear.cuh:14-18). Each function validates shapes
+// the way the reference does, calls the C ABI in include/crusader_hip.h on the default stream, synchronises
+// (the reference ends every op with cudaDeviceSynchronize) and throws on failure.
+//
+// Shape violations: the reference uses assert() for GEMM/linear (abort in debug builds, unchecked in release)
+// and std::invalid_argument for conv; here both throw std::invalid_argument. Device errors throw
+// std::runtime_error.
+#pragma once
+#include "../tensor/Parameter.h"
+#include "../tensor/Tensor.h"
+
+namespace seblas {
+// cuGEMM.cu:1649-1714
+Tensor *sgemm(Tensor *A, Tensor *B, Tensor *C);     // C[n] = A * B[n]
+Tensor *sgemmTN(Tensor *A, Tensor *B, Tensor *C);   // C[n] = A^T * B[n]
+Tensor *sgemmNT(Tensor *A, Tensor *B, Tensor *C);   // C = A * B^T
+Tensor *sgemmNTA(Tensor *A, Tensor *B, Tensor *C);  // C += sum_n A[n] * B[n]^T
+
+// cuLinear.cu:1052-1113
+Tensor *linear(Tensor *X, Tensor *W, Tensor *B, Tensor *Y);
+Tensor *linearXGrad(Tensor *dY, Tensor *W, Tensor *dX);
+Tensor *linearParamGrad(Tensor *dY, Tensor *X, Tensor *dW, Tensor *dB);  // returns dW
+
+// cuConv.cu:757-818. A: filters OC x IC x FH x FW.
+Tensor *conv(Tensor *A, Tensor *B, Tensor *C, int strideH, int strideW, int padH, int padW, Tensor *biases);
+Tensor *convDerive(Tensor *A, Tensor *B, Tensor *C, int strideH, int strideW, int padH, int padW);
+// A: errors N x OC x OH x OW, B: inputs N x IC x IH x IW, C: filter grads (accumulated). Returns A, as the
+// reference does (cuConv.cu:805).
+Tensor *convError(Tensor *A, Tensor *B, Tensor *C, int strideH, int strideW, int padH, int padW);
+Tensor *convBias(Tensor *Y, Tensor *biases);
+}  // namespace seblas

@@ -133,6 +133,22 @@ int crb_conv_wgrad(const float *dY, const float *X, float *dW, const crb_conv_ge
 /* Replaces seblas::convBias (cuConv.cu:808-818; kernel :709-729). Y[n,c,:,:] += bias[c], in place. */
 int crb_conv_bias(float *Y, const float *bias, uint32_t N, uint32_t C, uint32_t HW, void *stream);
 
+/* Bias gradient of a conv operand: dB[c] += sum_{n,h,w} dY[n,c,h,w], each element updated exactly once.
+ * Stands in for the channelReduce call of Conv2D::paramGrads (seann/operands/seblas/Conv2D.cu:26-28), whose
+ * size assertion (seblas/operations/cuReduce.cu:237) cannot hold for a C-element bias; this computes the
+ * per-channel sum that call is meant to produce. Accumulate. */
+int crb_conv_bias_grad(const float *dY, float *dB, uint32_t N, uint32_t C, uint32_t HW, void *stream);
+
+/* Tensor helpers the conv / linear operands use around the hot path ---------------------------- */
+
+/* Replaces the device branch of seblas::Tensor::operator+(Tensor*) (seblas/tensor/Tensor.cu:118-132,
+ * 462-483): a[i] += b[i] for i < count, in place. Used by Conv2D::xGrads / Linear::xGrads to fold the
+ * reserve gradient into dA (seann/operands/seblas/Conv2D.cu:19). */
+int crb_tensor_add_inplace(float *a, const float *b, uint32_t count, void *stream);
+
+/* Replaces the device branch of seblas::Tensor::constFill (Tensor.cu:294-304, 638-657): a[i] = value. */
+int crb_tensor_fill(float *a, float value, uint32_t count, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

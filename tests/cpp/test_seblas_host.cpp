@@ -1,0 +1,253 @@
+// Host-side tests of the C++ seblas / seann layer. Mode "host" needs no GPU (shape rules, exact division helper,
+// shape-error translation, which all happen before any device work). Mode "gpu" drives the reference-shaped API
+// end to end on the device — Tensor::create / copy / seblas::conv ... / seann::Conv2D, Linear — and checks results
+// against the CPU oracle (linked here as the checker only).
+#include <cmath>
+#include <cstdio>
+#include <cstring>
+#include <random>
+#include <stdexcept>
+#include <vector>
+
+#include "../../crusaderbackend_amd/csrc/crb_common.h"
+#include "../../crusaderbackend_amd/host/seann/operands/Conv2D.h"
+#include "../../crusaderbackend_amd/host/seann/operands/Linear.h"
+
+extern "C" {
+void oracle_sgemm(const float *, const float *, float *, uint32_t, uint32_t, uint32_t, uint32_t, int);
+void oracle_sgemmNT(const float *, const float *, float *, uint32_t, uint32_t, uint32_t, int);
+void oracle_linear(const float *, const float *, const float *, float *, uint32_t, uint32_t, uint32_t, int);
+void oracle_linearXGrad(const float *, const float *, float *, uint32_t, uint32_t, uint32_t, int);
+void oracle_linearParamGrad(const float *, const float *, float *, float *, uint32_t, uint32_t, uint32_t, int);
+void oracle_conv(const float *, const float *, float *, const float *, uint32_t, uint32_t, uint32_t, uint32_t, uint32_t,
+                 uint32_t, uint32_t, uint32_t, uint32_t, uint32_t, uint32_t, uint32_t, uint32_t, int);
+void oracle_convDerive(const float *, const float *, float *, uint32_t, uint32_t, uint32_t, uint32_t, uint32_t, uint32_t,
+                       uint32_t, uint32_t, uint32_t, uint32_t, uint32_t, uint32_t, uint32_t, int);
+void oracle_convError(const float *, const float *, float *, uint32_t, uint32_t, uint32_t, uint32_t, uint32_t, uint32_t,
+                      uint32_t, uint32_t, uint32_t, uint32_t, uint32_t, uint32_t, uint32_t, int);
+}
+
+using namespace seblas;
+static int g_fail = 0;
+#define CHECK(cond)                                                          \
+    do {                                                                     \
+        if (!(cond)) {                                                       \
+            std::printf("FAIL %s:%d: %s\n", __FILE__, __LINE__, #cond);      \
+            ++g_fail;                                                        \
+        }                                                                    \
+    } while (0)
+
+template <class F>
+static bool throws_invalid(F f) {
+    try {
+        f();
+    } catch (const std::invalid_argument &) {
+        return true;
+    } catch (...) {
+        return false;
+    }
+    return false;
+}
+
+static void host_tests() {
+    // shape constructor rules (Tensor.cuh:67-76)
+    shape4 a(3, 5), b(2, 3, 5), c(7, 2, 3, 5);
+    CHECK(a.n == 1 && a.c == 1 && a.h == 3 && a.w == 5 && a.size == 15);
+    CHECK(b.n == 1 && b.c == 2 && b.h == 3 && b.w == 5 && b.size == 30);
+    CHECK(c.n == 7 && c.size == 210);
+    CHECK(c.toString() == "(7,2,3,5)");
+    CHECK((index4(1, 2, 3, 4) + index4(1, 1, 1, 1)) == index4(2, 3, 4, 5));
+
+    // exact division helper against the hardware divide
+    std::mt19937 gen(7);
+    const uint32_t divisors[] = {1, 2, 3, 5, 7, 9, 16, 17, 64, 144, 255, 256, 1000, 1024, 65535, 65536, 1u << 20, 0x7fffffffu, 0xffffffffu};
+    for (uint32_t d : divisors) {
+        crb::FastDiv fd(d);
+        const uint32_t edge[] = {0, 1, d - 1, d, d + 1, 2 * d - 1, 2 * d, 0x7fffffffu, 0xfffffffeu, 0xffffffffu};
+        for (uint32_t n : edge) CHECK(fd.div(n) == n / d);
+        for (int i = 0; i < 20000; ++i) {
+            uint32_t n = gen();
+            uint32_t q, r;
+            fd.divmod(n, q, r);
+            CHECK(q == n / d && r == n % d);
+        }
+    }
+
+    // descriptors can be declared, reshaped and attached without a device
+    Tensor *t = Tensor::declare(2, 3, 4, 5);
+    CHECK(t->dims.size == 120 && t->elements == nullptr);
+    t->reshape(6, 20);
+    CHECK(t->dims.h == 6 && t->dims.w == 20 && t->dims.n == 1);
+    CHECK(throws_invalid([&] { t->reshape(7, 20); }));
+    float backing[120];
+    t->attach(backing, -1);
+    CHECK(t->elements == backing && t->deviceId == -1);
+    t->constFill(2.0f);
+    Tensor *u = Tensor::declare(6, 20)->attach(backing, -1);
+    *t + u;  // host branch of operator+: in-place add (aliasing itself doubles)
+    CHECK(backing[0] == 4.0f && backing[119] == 4.0f);
+
+    // shape violations are reported as std::invalid_argument before any device work
+    Tensor *A = Tensor::declare(4, 6), *B = Tensor::declare(5, 8), *C = Tensor::declare(4, 8);
+    CHECK(throws_invalid([&] { sgemm(A, B, C); }));       // A.w != B.h
+    CHECK(throws_invalid([&] { sgemmNT(A, B, C); }));     // A.w != B.w
+    CHECK(throws_invalid([&] { sgemmTN(A, B, C); }));
+    Tensor *W = Tensor::declare(8, 3, 3, 3), *X = Tensor::declare(2, 3, 8, 8), *Y = Tensor::declare(2, 8, 7, 8);
+    CHECK(throws_invalid([&] { conv(W, X, Y, 1, 1, 1, 1, nullptr); }));                      // rows relation
+    Tensor *Y2 = Tensor::declare(2, 9, 8, 8);
+    CHECK(throws_invalid([&] { conv(W, X, Y2, 1, 1, 1, 1, nullptr); }));                     // channels relation
+    Tensor *Y3 = Tensor::declare(3, 8, 8, 8);
+    CHECK(throws_invalid([&] { conv(W, X, Y3, 1, 1, 1, 1, nullptr); }));                     // batch relation
+    Tensor *lx = Tensor::declare(4, 1, 10, 1), *lw = Tensor::declare(6, 11), *lb = Tensor::declare(6, 1), *ly = Tensor::declare(4, 1, 6, 1);
+    CHECK(throws_invalid([&] { linear(lx, lw, lb, ly); }));                                  // W.w != X.h
+
+    // operand shape inference (Conv2D.cuh:40-44, Linear.cu:9-13) is pure host arithmetic on declared shapes
+    shape4 in(128, 16, 32, 32);
+    uint32_t oh = (in.h + 2 * 1 - 3) / 2 + 1;
+    CHECK(oh == 16);
+}
+
+static double tol(double ref, double rms, uint32_t K) { return 1e-5 * std::sqrt(double(K)) * std::fmax(std::fabs(ref), rms); }
+
+static void compare(const char *what, const std::vector<float> &got, const std::vector<float> &ref, uint32_t K) {
+    double ss = 0;
+    for (float v : ref) ss += double(v) * v;
+    double rms = std::sqrt(ss / double(ref.size()));
+    size_t bad = 0;
+    for (size_t i = 0; i < ref.size(); ++i)
+        if (!(std::fabs(double(got[i]) - ref[i]) <= tol(ref[i], rms, K))) ++bad;
+    if (bad) {
+        std::printf("FAIL %s: %zu/%zu outside tolerance\n", what, bad, ref.size());
+        ++g_fail;
+    }
+}
+
+static std::vector<float> pull(Tensor *t) {
+    std::vector<float> v(t->dims.size);
+    Tensor *h = t->ripOffDevice();
+    std::memcpy(v.data(), h->elements, sizeof(float) * v.size());
+    h->eliminateHost();
+    return v;
+}
+
+static Tensor *push(shape4 s, const std::vector<float> &v) {
+    Tensor *h = Tensor::createHost(s);
+    std::memcpy(h->elements, v.data(), sizeof(float) * v.size());
+    return h->toDevice();
+}
+
+static std::vector<float> randn(size_t n, uint32_t seed, float sd = 1.0f) {
+    std::mt19937 g(seed);
+    std::normal_distribution<float> d(0.f, sd);
+    std::vector<float> v(n);
+    for (auto &x : v) x = d(g);
+    return v;
+}
+
+static void gpu_tests() {
+    // raw operator API: sgemm with a batched B, and sgemmNT
+    {
+        const uint32_t M = 70, K = 36, N = 52, batch = 3;
+        auto a = randn(M * K, 1), b = randn(batch * K * N, 2);
+        Tensor *A = push(shape4(M, K), a), *B = push(shape4(batch, 1, K, N), b), *C = Tensor::create(batch, 1, M, N);
+        CHECK(sgemm(A, B, C) == C);
+        std::vector<float> ref(batch * M * N);
+        oracle_sgemm(a.data(), b.data(), ref.data(), M, N, K, batch, 4);
+        compare("seblas::sgemm", pull(C), ref, K);
+        A->eliminate(), B->eliminate(), C->eliminate();
+    }
+    // seann::Conv2D: forward, xGrads (with a non-zero reserve gradient folded in first), paramGrads
+    for (int stride = 1; stride <= 2; ++stride) {
+        const uint32_t N = 4, IC = 6, H = 12, OC = 10;
+        seann::Conv2D op(shape4(OC, IC, 3, 3), stride, stride, 1, 1, true);
+        op.initNetParams(nullptr, shape4(N, IC, H, H));
+        seann::Parameter *src = seann::Parameter::create(N, IC, H, H);
+        op.bindInput(src);
+        op.randFillNetParams();
+        const uint32_t OH = op.Y->A->dims.h;
+        CHECK(OH == (H + 2 - 3) / stride + 1 && op.Y->A->dims.c == OC && op.Y->A->dims.n == N);
+        auto x = randn(N * IC * H * H, 3), dy = randn(N * OC * OH * OH, 4), rs = randn(N * OC * OH * OH, 5);
+        Tensor *hx = Tensor::createHost(src->A->dims);
+        std::memcpy(hx->elements, x.data(), x.size() * 4);
+        hx->copyToH2D(src->A);
+        Tensor *hd = Tensor::createHost(op.Y->dA->dims);
+        std::memcpy(hd->elements, dy.data(), dy.size() * 4);
+        hd->copyToH2D(op.Y->dA);
+        std::memcpy(hd->elements, rs.data(), rs.size() * 4);
+        hd->copyToH2D(op.Y->dAReserve);
+        auto w = pull(op.filter->data()), bv = pull(op.bias->data());
+
+        op.forward();
+        std::vector<float> ref(N * OC * OH * OH);
+        oracle_conv(w.data(), x.data(), ref.data(), bv.data(), N, IC, H, H, OC, 3, 3, OH, OH, stride, stride, 1, 1, 4);
+        compare("Conv2D::forward", pull(op.Y->A), ref, IC * 9);
+
+        op.xGrads();  // dA += dAReserve; dX = dgrad(dA); reserve zeroed
+        std::vector<float> dsum(dy.size());
+        for (size_t i = 0; i < dy.size(); ++i) dsum[i] = dy[i] + rs[i];
+        std::vector<float> refdx(x.size());
+        oracle_convDerive(w.data(), dsum.data(), refdx.data(), N, IC, H, H, OC, 3, 3, OH, OH, stride, stride, 1, 1, 4);
+        compare("Conv2D::xGrads", pull(src->dA), refdx, OC * 9);
+        auto z = pull(op.Y->dAReserve);
+        bool allzero = true;
+        for (float v : z) allzero = allzero && v == 0.0f;
+        CHECK(allzero);
+
+        op.zeroGrads();
+        op.paramGrads();
+        std::vector<float> refdw(w.size(), 0.0f);
+        oracle_convError(dsum.data(), x.data(), refdw.data(), N, IC, H, H, OC, 3, 3, OH, OH, stride, stride, 1, 1, 4);
+        compare("Conv2D::paramGrads dW", pull(op.filter->grad()), refdw, N * OH * OH);
+        std::vector<float> refdb(OC, 0.0f);
+        for (uint32_t n = 0; n < N; ++n)
+            for (uint32_t c = 0; c < OC; ++c)
+                for (uint32_t i = 0; i < OH * OH; ++i) refdb[c] += dsum[(n * OC + c) * OH * OH + i];
+        compare("Conv2D::paramGrads dB", pull(op.bias->grad()), refdb, N * OH * OH);
+        // convError returns its first argument
+        CHECK(convError(op.Y->dA, op.X->A, op.filter->grad(), stride, stride, 1, 1) == op.Y->dA);
+    }
+    // seann::Linear on a 4-D input (flattened to IN = c*h*w)
+    {
+        const uint32_t N = 9, OUT = 20;
+        seann::Linear op(OUT);
+        op.initNetParams(nullptr, shape4(N, 4, 3, 5));
+        CHECK(op.INPUT_SIZE == 60 && op.X->A->dims.h == 60 && op.X->A->dims.w == 1);
+        seann::Parameter *src = seann::Parameter::create(N, 4, 3, 5);
+        op.bindInput(src);
+        op.randFillNetParams();
+        auto x = randn(N * 60, 6), dy = randn(N * OUT, 7);
+        Tensor *hx = Tensor::createHost(src->A->dims);
+        std::memcpy(hx->elements, x.data(), x.size() * 4);
+        hx->copyToH2D(src->A);
+        Tensor *hd = Tensor::createHost(op.Y->dA->dims);
+        std::memcpy(hd->elements, dy.data(), dy.size() * 4);
+        hd->copyToH2D(op.Y->dA);
+        auto w = pull(op.weights->data()), b = pull(op.biases->data());
+        op.forward();
+        std::vector<float> ref(N * OUT), refdx(N * 60), refdw(OUT * 60, 0.f), refdb(OUT, 0.f);
+        oracle_linear(x.data(), w.data(), b.data(), ref.data(), N, 60, OUT, 2);
+        compare("Linear::forward", pull(op.Y->A), ref, 60);
+        op.xGrads();
+        oracle_linearXGrad(dy.data(), w.data(), refdx.data(), N, 60, OUT, 2);
+        compare("Linear::xGrads", pull(src->dA), refdx, OUT);
+        op.paramGrads();
+        oracle_linearParamGrad(dy.data(), x.data(), refdw.data(), refdb.data(), N, 60, OUT, 2);
+        compare("Linear::paramGrads dW", pull(op.weights->grad()), refdw, N);
+        compare("Linear::paramGrads dB", pull(op.biases->grad()), refdb, N);
+    }
+}
+
+int main(int argc, char **argv) {
+    const bool gpu = argc > 1 && std::strcmp(argv[1], "gpu") == 0;
+    try {
+        if (gpu)
+            gpu_tests();
+        else
+            host_tests();
+    } catch (const std::exception &e) {
+        std::printf("FAIL: unexpected exception: %s\n", e.what());
+        return 2;
+    }
+    std::printf("%s: %s\n", gpu ? "gpu" : "host", g_fail ? "FAILED" : "OK");
+    return g_fail ? 1 : 0;
+}

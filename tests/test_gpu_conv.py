@@ -187,3 +187,23 @@ def test_conv_shape_errors(dev):
     assert need > 0
     st = lib.crb_conv_wgrad(t.data_ptr(), t.data_ptr(), t.data_ptr(), ctypes.byref(g), t.data_ptr(), 16, None)
     assert st == capi.CRB_EWORKSPACE
+
+
+def test_bias_grad_and_tensor_helpers(dev):
+    import torch
+    capi = _capi()
+    dY0, dB0 = normal(1, 6, 5, 7, 9), normal(2, 5)
+    dB = to_dev(dB0, dev)
+    capi.conv_bias_grad(to_dev(dY0, dev), dB, 6, 5, 63)
+    assert_close(to_np(dB), dB0 + dY0.astype(np.float64).sum(axis=(0, 2, 3)), 6 * 63, "conv bias grad")
+    for count in (1, 3, 4, 1027, 65536 + 5):
+        a0, b0 = normal(3, count), normal(4, count)
+        a = to_dev(a0, dev)
+        capi.tensor_add_inplace(a, to_dev(b0, dev), count)
+        assert np.array_equal(to_np(a), a0 + b0)
+        capi.tensor_fill(a, 1.5, count)
+        assert np.array_equal(to_np(a), np.full(count, 1.5, np.float32))
+    # unaligned views take the scalar path
+    base = torch.zeros(130, device=dev)
+    capi.tensor_fill(base[1:], 2.0, 129)
+    assert float(base[0]) == 0.0 and bool((base[1:] == 2.0).all())
