@@ -1,5 +1,6 @@
 // C-ABI entry points of the convolution family: forward, data gradient, weight gradient and the
 // standalone bias add, all as implicit GEMMs on the MFMA engine (no im2col buffer is materialised).
+#include "conv3x3_direct.h"
 #include "operands.h"
 
 namespace crb {
@@ -72,6 +73,45 @@ static WgradPlan wgrad_plan(const crb_conv_geom *g) {
     return p;
 }
 
+// ---- direct 3x3 / stride 1 / pad 1 path -------------------------------------------------------------------
+// Configurations <W, ROWS, CI, OCT, PBW, OBW, DGRAD, OCC, NBUF>, picked by image width and channel counts.
+// Tried in order; the first whose divisibility constraints hold is used, otherwise the implicit-GEMM engine runs.
+template <bool DG>
+static int try_direct(const float *Wt, const float *X, float *Y, const float *bias, u32 N, u32 C_IN, u32 C_OUT, u32 H,
+                      u32 Wd, u32 relu, hipStream_t s, const char *what, bool &done) {
+    done = true;
+#define CRB_TRY(...)                                                                                         \
+    if (direct_fits<DirectCfg<__VA_ARGS__>>(C_IN, C_OUT, H, Wd))                                              \
+        return launch_direct<DirectCfg<__VA_ARGS__>>(Wt, X, Y, bias, N, C_IN, C_OUT, H, relu, s, what);
+    if (Wd == 32) {
+        CRB_TRY(32, 8, 16, 16, 4, 1, DG, 2, 1)  // C_IN == 16: whole contraction in one LDS-resident chunk
+        if (C_OUT >= 64) { CRB_TRY(32, 8, 8, 64, 4, 4, DG, 2, 2) }
+        if (C_OUT >= 32) { CRB_TRY(32, 8, 8, 32, 4, 2, DG, 2, 2) }
+        CRB_TRY(32, 8, 8, 16, 4, 1, DG, 2, 2)
+        CRB_TRY(32, 4, 8, 16, 2, 1, DG, 2, 2)
+    } else if (Wd == 16) {
+        if (C_OUT >= 128) { CRB_TRY(16, 8, 8, 64, 2, 4, DG, 2, 2) }
+        CRB_TRY(16, 4, 16, 32, 1, 2, DG, 2, 2)
+        CRB_TRY(16, 4, 8, 32, 1, 2, DG, 2, 2)
+        CRB_TRY(16, 8, 8, 16, 2, 1, DG, 2, 2)
+        CRB_TRY(16, 4, 8, 16, 1, 1, DG, 2, 2)
+    } else if (Wd == 8) {
+        if (C_OUT >= 256) { CRB_TRY(8, 8, 16, 64, 1, 4, DG, 2, 2) }
+        if (C_OUT >= 128) { CRB_TRY(8, 8, 16, 32, 1, 2, DG, 2, 2) }
+        CRB_TRY(8, 8, 16, 16, 1, 1, DG, 2, 2)
+        CRB_TRY(8, 8, 8, 16, 1, 1, DG, 2, 2)
+        CRB_TRY(8, 4, 8, 32, 1, 1, DG, 2, 2)
+    }
+#undef CRB_TRY
+    done = false;
+    return CRB_OK;
+}
+
+static bool direct_shape(const crb_conv_geom *g) {
+    return g->FH == 3 && g->FW == 3 && g->sH == 1 && g->sW == 1 && g->pH == 1 && g->pW == 1 && g->IH == g->OH &&
+           g->IW == g->OW;
+}
+
 __global__ void __launch_bounds__(256) conv_bias_kernel(float *__restrict__ Y, const float *__restrict__ bias,
                                                         u32 total, u32 C, FastDiv hw) {
     const u32 i = blockIdx.x * 256 + threadIdx.x;
@@ -114,6 +154,12 @@ int crb_conv_fwd(const float *W, const float *X, float *Y, const float *bias_or_
     NchwEpi e{Y, bias_or_null, g->OC, g->OH * g->OW, (flags & CRB_FLAG_RELU) ? u32(EPI_RELU) : 0u,
               FastDiv(g->OH * g->OW)};
     hipStream_t s = hipStream_t(stream);
+    if (direct_shape(g) && aligned16(X) && aligned16(Y)) {
+        bool done;
+        int st = try_direct<false>(W, X, Y, bias_or_null, g->N, g->IC, g->OC, g->IH, g->IW, flags & CRB_FLAG_RELU, s,
+                                   "crb_conv_fwd", done);
+        if (done) return st;
+    }
     if (K % 4 == 0 && aligned16(W)) {
         MatK<true> a{W, M, K, 0};
         return run_by_m(a, b, e, M, N, K, 1, 0, K, s, "crb_conv_fwd");
@@ -125,6 +171,12 @@ int crb_conv_fwd(const float *W, const float *X, float *Y, const float *bias_or_
 int crb_conv_dgrad(const float *W, const float *dY, float *dX, const crb_conv_geom *g, void *stream) {
     if (!W || !dY || !dX) return fail(CRB_ENULL, "crb_conv_dgrad: null operand");
     if (int st = check_geom("crb_conv_dgrad", g)) return st;
+    if (direct_shape(g) && aligned16(dY) && aligned16(dX)) {
+        bool done;
+        int st = try_direct<true>(W, dY, dX, nullptr, g->N, g->OC, g->IC, g->IH, g->IW, 0, hipStream_t(stream),
+                                  "crb_conv_dgrad", done);
+        if (done) return st;
+    }
     const u32 FHW = g->FH * g->FW;
     const u32 M = g->IC, N = g->N * g->IH * g->IW, K = g->OC * FHW;
     SepK a{W, g->IC, FHW, g->IC * FHW, 1, FastDiv(FHW)};

@@ -207,3 +207,31 @@ def test_bias_grad_and_tensor_helpers(dev):
     base = torch.zeros(130, device=dev)
     capi.tensor_fill(base[1:], 2.0, 129)
     assert float(base[0]) == 0.0 and bool((base[1:] == 2.0).all())
+
+
+# 3x3 / stride 1 / pad 1 shapes chosen so that every configuration of the direct (LDS-staged) path is exercised,
+# plus neighbours that must fall back to the implicit-GEMM engine (odd height, channel counts not divisible by 8/16).
+# (N, IC, H, W, OC)
+DIRECT = [
+    (3, 16, 32, 32, 16), (2, 16, 32, 32, 64), (2, 64, 32, 32, 64), (2, 8, 32, 32, 32), (2, 24, 32, 32, 48),
+    (2, 8, 36, 32, 16), (2, 8, 12, 32, 16),
+    (3, 32, 16, 16, 32), (2, 64, 16, 16, 128), (2, 24, 16, 16, 32), (2, 8, 16, 16, 16), (2, 16, 8, 16, 48),
+    (2, 16, 12, 16, 16),
+    (3, 64, 8, 8, 64), (2, 128, 8, 8, 256), (2, 32, 8, 8, 128), (2, 8, 8, 8, 16), (2, 24, 8, 8, 32), (2, 8, 4, 8, 32),
+    (2, 16, 30, 32, 16), (2, 12, 16, 16, 16), (2, 16, 8, 8, 24), (2, 16, 6, 8, 16),
+]
+
+
+@pytest.mark.parametrize("N,IC,H,W,OC", DIRECT)
+def test_conv3x3_direct_configs(dev, N, IC, H, W, OC):
+    run_layer(dev, N, IC, H, W, OC, 3, 3, 1, 1, 1, 1, bias=True, seed=11)
+
+
+def test_conv_relu_flag(dev):
+    capi, orc = _capi(), _oracle()
+    for (N, IC, H, OC) in [(2, 16, 32, 16), (2, 5, 9, 7)]:  # direct path and implicit-GEMM path
+        g = capi.ConvGeom.make(N, IC, H, H, OC, 3, 3, 1, 1, 1, 1)
+        X, W, b = normal(1, N, IC, H, H), he_normal(2, OC, IC, 3, 3), normal(3, OC)
+        Y = _nan(dev, N, OC, H, H)
+        capi.conv_fwd(to_dev(W, dev), to_dev(X, dev), Y, to_dev(b, dev), g, flags=capi.CRB_FLAG_RELU)
+        assert_close(to_np(Y), np.maximum(orc.conv(W, X, b, 1, 1, 1, 1), 0), IC * 9, "conv+bias+relu")
