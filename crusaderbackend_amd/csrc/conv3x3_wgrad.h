@@ -1,0 +1,285 @@
+// Weight gradient of a 3x3 / stride 1 / pad 1 convolution for gfx950.
+//
+// dW[oc][ic][fh][fw] = sum over (n, y, x) of dY[n][oc][y][x] * X[n][ic][y+fh-1][x+fw-1]: for each of the 9 taps a
+// (OC x IC) matrix product whose contraction index is the pixel. A workgroup owns ONE 16x16 (oc-block, ic-block)
+// pair for all 9 taps and a slice of the pixel range (split z). It walks its slice tile by tile (TI images x TR
+// rows), staging the 16 dY planes and the 16 X planes (with their one-row halo, zero outside the image) in
+// double-buffered LDS. Inside a tile the pixels are a flat run k' = y*W + x, and tap (fh, fw) of X is the same
+// run shifted by the constant fh*W + fw - 1, so every fragment read is base + immediate. The wrap-around that
+// the shift causes at the left/right image border is removed by zeroing the dY value of the lanes that sit on
+// column 0 (taps fw = 0) or column W-1 (taps fw = 2) — a select on one step in W/4, decided at compile time.
+//
+// v_mfma_f32_16x16x4_f32 mapping (wave64, lane l): A = dY[oc = l%16][k' = 4s + l/16], B = X[k'][ic = l%16],
+// accumulator register r = dW[oc = 4*(l/16) + r][ic = l%16]; 9 accumulator tiles (one per tap) per wave.
+// The 4 waves take different rows (or images) of the tile; their accumulators are summed through LDS in fixed
+// wave order at the end and written either as this split's partial result or, without splitting, added to dW.
+#pragma once
+#include "igemm_engine.h"
+
+namespace crb {
+
+template <int W_, int TR_, int TI_, int OCC_>
+struct WgradCfg {
+    static constexpr int W = W_, TR = TR_, TI = TI_, OCC = OCC_;
+    static constexpr int WPI = 4 / TI;         // waves per image of the tile
+    static constexpr int RW = TR / WPI;        // rows per wave
+    static constexpr int KW = RW * W;          // pixels per wave per tile
+    static constexpr int NSTEP = KW / 4;       // MFMA steps per wave per tile
+    static constexpr int YIMG = TR * W;        // dY floats per image per plane
+    static constexpr int XIMG = (TR + 2) * W;  // X floats per image per plane (halo rows included)
+    // plane strides == 2 mod 4 (and even): 16 planes x 2 lane groups of a half-wave land on 32 distinct banks
+    static constexpr int YP = TI * YIMG + 2;
+    static constexpr int XP = TI * XIMG + 8 + 2;  // 4 leading + 4 trailing pad floats (kept zero)
+    static constexpr int Y_SIZE = 16 * YP, X_SIZE = 16 * XP;
+    static constexpr int BUF = Y_SIZE + X_SIZE;      // one staging buffer (floats)
+    static constexpr int RED_SIZE = 4 * 9 * 64 * 4;  // cross-wave reduction scratch (floats), reuses the staging space
+    static constexpr int SMEM = 2 * BUF > RED_SIZE ? 2 * BUF : RED_SIZE;
+    static_assert(TI == 1 || TI == 2 || TI == 4, "images per tile");
+    static_assert(TR % WPI == 0 && KW % 4 == 0, "rows must split evenly over the waves");
+};
+
+struct WgradArgs {
+    const float *dY;  // N x OC x H x W
+    const float *X;   // N x IC x H x W
+    float *out;       // splits > 1: partials [z][OC][IC][9]; splits == 1: dW (accumulated)
+    u32 OC, IC, H;
+    u32 ic_blocks;        // IC / 16
+    u32 tiles, tiles_per_z;  // tile count (N/TI * H/TR) and tiles per split
+    u32 tiles_per_img;    // H / TR
+    u32 accumulate;       // add to `out` instead of overwriting (splits == 1)
+};
+
+template <class Cfg>
+__global__ void __launch_bounds__(kThreads, Cfg::OCC) wgrad3x3s1_kernel(WgradArgs a) {
+    constexpr int W = Cfg::W, TR = Cfg::TR, TI = Cfg::TI, YP = Cfg::YP, XP = Cfg::XP, NSTEP = Cfg::NSTEP;
+    constexpr int YIMG = Cfg::YIMG, XIMG = Cfg::XIMG;
+    __shared__ __attribute__((aligned(16))) float smem[Cfg::SMEM];  // buffer b: dY planes at b*BUF, X planes after them
+
+    const u32 t = threadIdx.x;
+    const u32 pair = blockIdx.x, z = blockIdx.y;
+    const u32 ob = pair / a.ic_blocks, ib = pair % a.ic_blocks;
+    const u32 HW = a.H * W;
+    const u32 t_begin = z * a.tiles_per_z;
+    const u32 t_end = t_begin + a.tiles_per_z < a.tiles ? t_begin + a.tiles_per_z : a.tiles;
+
+    // ---- staging: 16-byte global loads, 8-byte LDS stores (plane strides are even, not multiples of 4) ------
+    constexpr int YQ = TI * 16 * (YIMG / 4), XQ = TI * 16 * (XIMG / 4);
+    constexpr int YNP = (YQ + kThreads - 1) / kThreads, XNP = (XQ + kThreads - 1) / kThreads;
+    v4f yreg[YNP], xreg[XNP];
+
+    auto fetch = [&](u32 tile) {
+        const u32 n0 = (tile / a.tiles_per_img) * TI;
+        const int r0 = int(tile % a.tiles_per_img) * TR;
+#pragma unroll
+        for (int i = 0; i < YNP; ++i) {
+            const u32 e = t + i * kThreads;
+            v4f v = {0.f, 0.f, 0.f, 0.f};
+            if (YQ % kThreads == 0 || e < YQ) {
+                const u32 q = e % (YIMG / 4), c = (e / (YIMG / 4)) % 16, img = e / ((YIMG / 4) * 16);
+                v = *reinterpret_cast<const v4f *>(a.dY + (size_t(n0 + img) * a.OC + ob * 16 + c) * HW + u32(r0) * W + 4 * q);
+            }
+            yreg[i] = v;
+        }
+#pragma unroll
+        for (int i = 0; i < XNP; ++i) {
+            const u32 e = t + i * kThreads;
+            v4f v = {0.f, 0.f, 0.f, 0.f};
+            if (XQ % kThreads == 0 || e < XQ) {
+                const u32 q = e % (XIMG / 4), c = (e / (XIMG / 4)) % 16, img = e / ((XIMG / 4) * 16);
+                const int row = r0 - 1 + int(q / (W / 4));
+                if (row >= 0 && row < int(a.H))
+                    v = *reinterpret_cast<const v4f *>(a.X + (size_t(n0 + img) * a.IC + ib * 16 + c) * HW + u32(row) * W +
+                                                       4 * (q % (W / 4)));
+            }
+            xreg[i] = v;
+        }
+    };
+
+    auto commit = [&](float *dYs, float *dXs) {
+#pragma unroll
+        for (int i = 0; i < YNP; ++i) {
+            const u32 e = t + i * kThreads;
+            if (YQ % kThreads == 0 || e < YQ) {
+                const u32 q = e % (YIMG / 4), c = (e / (YIMG / 4)) % 16, img = e / ((YIMG / 4) * 16);
+                float *p = dYs + c * YP + img * YIMG + 4 * q;
+                *reinterpret_cast<v2f *>(p) = v2f{yreg[i].x, yreg[i].y};
+                *reinterpret_cast<v2f *>(p + 2) = v2f{yreg[i].z, yreg[i].w};
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < XNP; ++i) {
+            const u32 e = t + i * kThreads;
+            if (XQ % kThreads == 0 || e < XQ) {
+                const u32 q = e % (XIMG / 4), c = (e / (XIMG / 4)) % 16, img = e / ((XIMG / 4) * 16);
+                float *p = dXs + c * XP + 4 + img * XIMG + 4 * q;
+                *reinterpret_cast<v2f *>(p) = v2f{xreg[i].x, xreg[i].y};
+                *reinterpret_cast<v2f *>(p + 2) = v2f{xreg[i].z, xreg[i].w};
+            }
+        }
+    };
+
+    // leading / trailing pad floats of every X plane stay zero (they are read, multiplied by a zeroed dY value)
+    for (u32 e = t; e < 2u * 16 * 8; e += kThreads) {
+        float *plane = smem + (e / 128) * Cfg::BUF + Cfg::Y_SIZE + ((e % 128) / 8) * XP;
+        const u32 k = e % 8;
+        plane[k < 4 ? k : 4 + TI * XIMG + (k - 4)] = 0.f;
+    }
+
+    // ---- per-lane fragment addressing ---------------------------------------------------------------------
+    const int lane = t & 63, wave = t >> 6;
+    const int li = lane & 15, kq = lane >> 4;
+    const int img_w = wave / Cfg::WPI, row_w = (wave % Cfg::WPI) * Cfg::RW;
+    const int ybase = li * YP + kq + img_w * YIMG + row_w * W;
+    const int xbase = li * XP + kq + 3 + img_w * XIMG + row_w * W;  // +4 pad, -1 for the fw shift
+
+    v4f acc[9];
+#pragma unroll
+    for (int k = 0; k < 9; ++k) acc[k] = v4f{0.f, 0.f, 0.f, 0.f};
+
+    auto compute = [&](const float *cy, const float *cx) {
+        const float *py = cy + ybase, *px = cx + xbase;
+        float av[2], bv[2][9];
+        auto read_step = [&](int s, int slot) {
+            av[slot] = py[4 * s];
+#pragma unroll
+            for (int k = 0; k < 9; ++k) bv[slot][k] = px[4 * s + (k / 3) * W + (k % 3)];
+        };
+        read_step(0, 0);
+#pragma unroll
+        for (int s = 0; s < NSTEP; ++s) {
+            if (s + 1 < NSTEP) read_step(s + 1, (s + 1) & 1);
+            __builtin_amdgcn_sched_barrier(0);
+            const float am = av[s & 1];
+            // lanes on image column 0 contribute nothing to the fw = 0 taps, lanes on column W-1 nothing to fw = 2
+            const float a0 = ((4 * s) % W == 0) ? (kq == 0 ? 0.f : am) : am;
+            const float a2 = ((4 * s + 4) % W == 0) ? (kq == 3 ? 0.f : am) : am;
+#pragma unroll
+            for (int k = 0; k < 9; ++k)
+                acc[k] = __builtin_amdgcn_mfma_f32_16x16x4f32(k % 3 == 0 ? a0 : (k % 3 == 2 ? a2 : am), bv[s & 1][k], acc[k], 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+
+    // ---- main loop over this split's tiles (double-buffered) ------------------------------------------------
+    if (t_begin < t_end) {
+        fetch(t_begin);
+        commit(smem, smem + Cfg::Y_SIZE);
+    }
+    __syncthreads();
+    for (u32 tile = t_begin; tile < t_end; ++tile) {
+        const u32 b = (tile - t_begin) & 1;
+        const bool more = tile + 1 < t_end;
+        if (more) fetch(tile + 1);
+        compute(smem + b * Cfg::BUF, smem + b * Cfg::BUF + Cfg::Y_SIZE);
+        if (more) commit(smem + (b ^ 1) * Cfg::BUF, smem + (b ^ 1) * Cfg::BUF + Cfg::Y_SIZE);
+        __syncthreads();
+    }
+
+    // ---- sum the 4 waves' accumulators in wave order, write this (pair, split) block --------------------------
+    float *red = smem;  // [wave][tap][lane][4]
+#pragma unroll
+    for (int k = 0; k < 9; ++k) *reinterpret_cast<v4f *>(red + ((wave * 9 + k) * 64 + lane) * 4) = acc[k];
+    __syncthreads();
+    const size_t count = size_t(a.OC) * a.IC * 9;
+    float *out = a.out + size_t(z) * count * (a.accumulate ? 0 : 1);
+    for (u32 e = t; e < 16 * 16 * 9; e += kThreads) {
+        const u32 oc = e / 144, ic = (e % 144) / 9, tap = e % 9;
+        const u32 src = (tap * 64 + (oc / 4) * 16 + ic) * 4 + (oc % 4);
+        float s = red[src];
+#pragma unroll
+        for (int w = 1; w < 4; ++w) s += red[w * 9 * 64 * 4 + src];
+        float *dst = out + (size_t(ob * 16 + oc) * a.IC + ib * 16 + ic) * 9 + tap;
+        *dst = a.accumulate ? *dst + s : s;
+    }
+}
+
+// C[i] (+)= sum_z partial[z][i]. A workgroup covers OUTS consecutive outputs with 256/OUTS z-lanes per output; every
+// z-lane keeps 4 independent running sums over its strided subset of z (loads in flight instead of one dependent
+// chain), then the lanes are combined through LDS in lane order. The association is fixed by (splits, OUTS) alone,
+// so repeated runs are bit-identical.
+template <int OUTS>
+static __global__ void __launch_bounds__(256) splitk_reduce_wide_kernel(const float *__restrict__ partial, float *__restrict__ C,
+                                                                        u32 count, u32 splits, u32 accumulate) {
+    constexpr u32 ZL = 256 / OUTS;
+    __shared__ float red[ZL][OUTS];
+    const u32 o = threadIdx.x % OUTS, g = threadIdx.x / OUTS;
+    const u32 i = blockIdx.x * OUTS + o;
+    float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
+    if (i < count) {
+        const float *p = partial + i;
+        u32 zz = g;
+        for (; zz + 3 * ZL < splits; zz += 4 * ZL) {
+            s0 += p[size_t(zz) * count];
+            s1 += p[size_t(zz + ZL) * count];
+            s2 += p[size_t(zz + 2 * ZL) * count];
+            s3 += p[size_t(zz + 3 * ZL) * count];
+        }
+        for (; zz < splits; zz += ZL) s0 += p[size_t(zz) * count];
+    }
+    red[g][o] = (s0 + s1) + (s2 + s3);
+    __syncthreads();
+    if (g == 0 && i < count) {
+        float r = red[0][o];
+#pragma unroll
+        for (u32 k = 1; k < ZL; ++k) r += red[k][o];
+        C[i] = accumulate ? C[i] + r : r;
+    }
+}
+
+inline int launch_splitk_reduce_wide(const float *partial, float *C, u32 count, u32 splits, u32 accumulate, hipStream_t s,
+                                     const char *what) {
+    // enough workgroups to cover the chip even when the result is small
+    if (count >= 32u * 512u)
+        hipLaunchKernelGGL(splitk_reduce_wide_kernel<32>, dim3(ceil_div(count, 32)), dim3(256), 0, s, partial, C, count, splits, accumulate);
+    else if (count >= 16u * 256u)
+        hipLaunchKernelGGL(splitk_reduce_wide_kernel<16>, dim3(ceil_div(count, 16)), dim3(256), 0, s, partial, C, count, splits, accumulate);
+    else
+        hipLaunchKernelGGL(splitk_reduce_wide_kernel<8>, dim3(ceil_div(count, 8)), dim3(256), 0, s, partial, C, count, splits, accumulate);
+    return check_launch(what);
+}
+
+struct WgradDirectPlan {
+    u32 pairs, tiles, splits, tiles_per_z;
+    size_t workspace_bytes;
+};
+
+template <class Cfg>
+inline bool wgrad_direct_fits(u32 N, u32 IC, u32 OC, u32 H, u32 Wd) {
+    return Wd == u32(Cfg::W) && H % Cfg::TR == 0 && N % Cfg::TI == 0 && IC % 16 == 0 && OC % 16 == 0;
+}
+
+template <class Cfg>
+inline WgradDirectPlan wgrad_direct_plan(u32 N, u32 IC, u32 OC, u32 H, u32 target_wgs) {
+    WgradDirectPlan p;
+    p.pairs = (OC / 16) * (IC / 16);
+    p.tiles = (N / Cfg::TI) * (H / Cfg::TR);
+    u32 splits = p.pairs >= target_wgs ? 1 : target_wgs / p.pairs;
+    if (splits > p.tiles) splits = p.tiles;
+    p.tiles_per_z = ceil_div(p.tiles, splits);
+    p.splits = ceil_div(p.tiles, p.tiles_per_z);
+    p.workspace_bytes = p.splits > 1 ? size_t(p.splits) * OC * IC * 9 * sizeof(float) : 0;
+    return p;
+}
+
+template <class Cfg>
+inline int launch_wgrad_direct(const float *dY, const float *X, float *dW, float *ws, const WgradDirectPlan &p, u32 N, u32 IC,
+                               u32 OC, u32 H, hipStream_t s, const char *what) {
+    (void)N;
+    WgradArgs a;
+    a.dY = dY, a.X = X;
+    a.out = p.splits > 1 ? ws : dW;
+    a.OC = OC, a.IC = IC, a.H = H;
+    a.ic_blocks = IC / 16;
+    a.tiles = p.tiles, a.tiles_per_z = p.tiles_per_z;
+    a.tiles_per_img = H / Cfg::TR;
+    a.accumulate = p.splits > 1 ? 0u : 1u;
+    if (p.splits > 65535u) return fail(CRB_EINVAL_SHAPE, "%s: too many splits", what);
+    hipLaunchKernelGGL((wgrad3x3s1_kernel<Cfg>), dim3(p.pairs, p.splits), dim3(kThreads), 0, s, a);
+    if (int st = check_launch(what)) return st;
+    if (p.splits > 1) {
+        return launch_splitk_reduce_wide(ws, dW, OC * IC * 9, p.splits, 1u, s, what);
+    }
+    return CRB_OK;
+}
+
+}  // namespace crb

@@ -1,6 +1,7 @@
 // C-ABI entry points of the convolution family: forward, data gradient, weight gradient and the
 // standalone bias add, all as implicit GEMMs on the MFMA engine (no im2col buffer is materialised).
 #include "conv3x3_direct.h"
+#include "conv3x3_wgrad.h"
 #include "operands.h"
 
 namespace crb {
@@ -112,6 +113,32 @@ static bool direct_shape(const crb_conv_geom *g) {
            g->IW == g->OW;
 }
 
+// ---- direct 3x3 / stride 1 / pad 1 weight gradient ---------------------------------------------------------
+// One entry per configuration <W, TR, TI, OCC>; `run` = false only computes the plan (workspace size).
+constexpr u32 kWgradTargetWgs = 256;  // one workgroup per CU: pairs x splits
+
+template <class Cfg>
+static bool wgrad_cfg(const crb_conv_geom *g, bool run, const float *dY, const float *X, float *dW, float *ws, hipStream_t s,
+                      WgradDirectPlan &plan, int &status) {
+    if (!wgrad_direct_fits<Cfg>(g->N, g->IC, g->OC, g->IH, g->IW)) return false;
+    plan = wgrad_direct_plan<Cfg>(g->N, g->IC, g->OC, g->IH, kWgradTargetWgs);
+    if (run) status = launch_wgrad_direct<Cfg>(dY, X, dW, ws, plan, g->N, g->IC, g->OC, g->IH, s, "crb_conv_wgrad");
+    return true;
+}
+
+static bool wgrad_direct(const crb_conv_geom *g, bool run, const float *dY, const float *X, float *dW, float *ws,
+                         hipStream_t s, WgradDirectPlan &plan, int &status) {
+    if (!direct_shape(g)) return false;
+    if (g->IW == 32) return wgrad_cfg<WgradCfg<32, 8, 1, 2>>(g, run, dY, X, dW, ws, s, plan, status);
+    if (g->IW == 16)
+        return wgrad_cfg<WgradCfg<16, 16, 1, 2>>(g, run, dY, X, dW, ws, s, plan, status) ||
+               wgrad_cfg<WgradCfg<16, 8, 1, 2>>(g, run, dY, X, dW, ws, s, plan, status);
+    if (g->IW == 8)
+        return wgrad_cfg<WgradCfg<8, 8, 4, 2>>(g, run, dY, X, dW, ws, s, plan, status) ||
+               wgrad_cfg<WgradCfg<8, 8, 2, 2>>(g, run, dY, X, dW, ws, s, plan, status);
+    return false;
+}
+
 __global__ void __launch_bounds__(256) conv_bias_kernel(float *__restrict__ Y, const float *__restrict__ bias,
                                                         u32 total, u32 C, FastDiv hw) {
     const u32 i = blockIdx.x * 256 + threadIdx.x;
@@ -195,6 +222,11 @@ int crb_conv_dgrad(const float *W, const float *dY, float *dX, const crb_conv_ge
 
 size_t crb_conv_wgrad_workspace_bytes(const crb_conv_geom *g) {
     if (check_geom("crb_conv_wgrad_workspace_bytes", g)) return 0;
+    {
+        WgradDirectPlan dp;
+        int st = 0;
+        if (wgrad_direct(g, false, nullptr, nullptr, nullptr, nullptr, nullptr, dp, st)) return dp.workspace_bytes;
+    }
     const WgradPlan p = wgrad_plan(g);
     return p.splits > 1 ? size_t(p.splits) * p.M * p.Ncols * sizeof(float) : 0;
 }
@@ -203,8 +235,27 @@ int crb_conv_wgrad(const float *dY, const float *X, float *dW, const crb_conv_ge
                    size_t workspace_bytes, void *stream) {
     if (!dY || !X || !dW) return fail(CRB_ENULL, "crb_conv_wgrad: null operand");
     if (int st = check_geom("crb_conv_wgrad", g)) return st;
-    const WgradPlan p = wgrad_plan(g);
     hipStream_t s = hipStream_t(stream);
+    if (aligned16(dY) && aligned16(X)) {
+        WgradDirectPlan dp;
+        int st = CRB_OK;
+        if (wgrad_direct(g, false, nullptr, nullptr, nullptr, nullptr, nullptr, dp, st)) {
+            float *dws = static_cast<float *>(workspace);
+            if (dp.workspace_bytes) {
+                if (dws) {
+                    if (workspace_bytes < dp.workspace_bytes)
+                        return fail(CRB_EWORKSPACE, "crb_conv_wgrad: workspace %zu bytes < required %zu", workspace_bytes,
+                                    dp.workspace_bytes);
+                } else {
+                    dws = static_cast<float *>(arena_get(dp.workspace_bytes));
+                    if (!dws) return fail(CRB_EHIP, "crb_conv_wgrad: cannot allocate %zu bytes of scratch", dp.workspace_bytes);
+                }
+            }
+            wgrad_direct(g, true, dY, X, dW, dws, s, dp, st);
+            return st;
+        }
+    }
+    const WgradPlan p = wgrad_plan(g);
     const u32 OHW = g->OH * g->OW;
     SepK a{dY, g->OC, OHW, g->OC * OHW, 1, FastDiv(OHW)};
     Im2colTapRows b{make_im2col(X, g)};
@@ -223,9 +274,7 @@ int crb_conv_wgrad(const float *dY, const float *X, float *dW, const crb_conv_ge
     }
     RowMajorEpi e{ws, nullptr, p.Ncols, p.M * p.Ncols, 0u};
     if (int st = run_by_m(a, b, e, p.M, p.Ncols, p.K, p.splits, 1, p.k_per_z, s, "crb_conv_wgrad")) return st;
-    const u32 count = p.M * p.Ncols;
-    hipLaunchKernelGGL(splitk_reduce_kernel, dim3(ceil_div(count, 256)), dim3(256), 0, s, ws, dW, count, p.splits, 1u);
-    return check_launch("crb_conv_wgrad(reduce)");
+    return launch_splitk_reduce_wide(ws, dW, p.M * p.Ncols, p.splits, 1u, s, "crb_conv_wgrad(reduce)");
 }
 
 int crb_conv_bias_grad(const float *dY, float *dB, uint32_t N, uint32_t C, uint32_t HW, void *stream) {

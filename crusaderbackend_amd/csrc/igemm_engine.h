@@ -288,16 +288,6 @@ __global__ void __launch_bounds__(kThreads, Cfg::OCC) igemm_kernel(AOp a, BOp b,
     }
 }
 
-// ---- split-K second pass: C[i] (+)= sum_z partial[z][i], fixed ascending-z order ---------------------
-static __global__ void __launch_bounds__(256) splitk_reduce_kernel(const float *__restrict__ partial, float *__restrict__ C,
-                                                            u32 count, u32 splits, u32 accumulate) {
-    const u32 i = blockIdx.x * 256 + threadIdx.x;
-    if (i >= count) return;
-    float s = 0.0f;
-    for (u32 zz = 0; zz < splits; ++zz) s += partial[size_t(zz) * count + i];
-    C[i] = accumulate ? C[i] + s : s;
-}
-
 template <class Cfg, class AOp, class BOp, class Epi>
 inline int launch_igemm(const AOp &a, const BOp &b, const Epi &epi, u32 M, u32 N, u32 K, u32 zdim, u32 split_k,
                         u32 k_per_z, hipStream_t stream, const char *what) {
