@@ -45,6 +45,9 @@ def parse():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--report", type=str, default=None, help="also time every BASELINE config and write a JSON report")
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
+    ap.add_argument("--calibrate", action="store_true",
+                    help="only run a plain streaming kernel of known size (a += b on 64 Mi floats: reads 512 MiB, writes "
+                         "256 MiB per launch) so hardware byte counters can be scaled against it, then exit")
     return ap.parse_args()
 
 
@@ -145,6 +148,15 @@ def main():
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     dev = torch.device("cuda:0")
     props = torch.cuda.get_device_properties(0)
+
+    if args.calibrate:
+        n = 64 << 20
+        x, y = torch.ones(n, device=dev), torch.ones(n, device=dev)
+        for _ in range(3):
+            capi.tensor_add_inplace(x, y, n)
+        torch.cuda.synchronize()
+        print(json.dumps({"calibrate": "add_inplace_kernel", "floats": n, "read_bytes": 8 * n, "write_bytes": 4 * n}))
+        return
 
     layers = [Layer(torch, capi, dev, n, IC, H, OC, s, m, seed=10 + i) for i, (n, IC, H, OC, s, m) in enumerate(RESNET56)]
     step_flops = sum(3 * L.mult * L.flops for L in layers)
