@@ -1,0 +1,107 @@
+"""Extended timing report over every BASELINE configuration (used by ``bench.py --report FILE``).
+
+Each entry: launch duration from HIP events on the launch stream (average of back-to-back launches), nominal
+flops, algorithmic bytes (each operand read once, output written once), TFLOP/s, GB/s and the fraction of the
+roofline that bounds the shape (FP32 matrix peak above ~19.7 flop/B, HBM bandwidth below).
+"""
+import math
+
+PEAK_TF = 157.3
+PEAK_GBS = 8000.0
+RIDGE = PEAK_TF * 1e3 / PEAK_GBS  # flop per byte
+
+
+def _entry(name, ms, flops, nbytes):
+    ai = flops / nbytes
+    tf, gbs = flops / ms / 1e9, nbytes / ms / 1e6
+    bound = "mfma" if ai >= RIDGE else "hbm"
+    frac = tf / PEAK_TF if bound == "mfma" else gbs / PEAK_GBS
+    return {"name": name, "us": round(ms * 1e3, 2), "gflop": round(flops / 1e9, 3), "mbytes": round(nbytes / 1e6, 2),
+            "ai": round(ai, 1), "tflops": round(tf, 2), "gbs": round(gbs, 1), "bound": bound, "frac": round(frac, 4)}
+
+
+def run(torch, capi, dev, event_time_ms, Layer):
+    out = {"gemm": [], "resnet56": [], "vgg16": [], "densenet": [], "dense": []}
+
+    def rnd(*shape):
+        return torch.rand(*shape, device=dev) * 2 - 1
+
+    # config 1 + target GEMM
+    for n in (1024, 4096):
+        A, B, C = rnd(n, n), rnd(n, n), torch.empty(n, n, device=dev)
+        ms = event_time_ms(torch, lambda: capi.sgemm_nn(A, B, C, n, n, n), reps=20 if n == 1024 else 10)
+        out["gemm"].append(_entry(f"sgemm {n}^3", ms, 2.0 * n ** 3, 12.0 * n * n))
+
+    def conv_entries(key, specs, batch, bias):
+        for i, (name, IC, H, OC, F, s, p) in enumerate(specs):
+            L = Layer(torch, capi, dev, name, IC, H, OC, s, 1, seed=100 + i, batch=batch, F=F, pad=p, bias=bias)
+            for pname, fn in L.passes():
+                reps = 30 if L.flops < 2e9 else 10
+                out[key].append(_entry(f"{name}.{pname}", event_time_ms(torch, fn, reps=reps), L.flops, L.bytes[pname]))
+            del L
+            torch.cuda.empty_cache()
+
+    # config 2: the five 3x3 shapes + stem + the two 1x1 stride-2 shortcuts
+    conv_entries("resnet56", [("16-16@32", 16, 32, 16, 3, 1, 1), ("32-32@16", 32, 16, 32, 3, 1, 1),
+                              ("64-64@8", 64, 8, 64, 3, 1, 1), ("16-32s2", 16, 32, 32, 3, 2, 1),
+                              ("32-64s2", 32, 16, 64, 3, 2, 1), ("stem3-16@32", 3, 32, 16, 3, 1, 1),
+                              ("sc16-32_1x1s2", 16, 32, 32, 1, 2, 0), ("sc32-64_1x1s2", 32, 16, 64, 1, 2, 0)], 128, False)
+
+    # config 3: VGG-16 (CIFAR) conv layers, bias fused, batch 128
+    vgg = [(3, 32, 64), (64, 32, 64), (64, 16, 128), (128, 16, 128), (128, 8, 256), (256, 8, 256), (256, 8, 256),
+           (256, 4, 512), (512, 4, 512), (512, 4, 512), (512, 2, 512), (512, 2, 512), (512, 2, 512)]
+    conv_entries("vgg16", [(f"c{i + 1}_{ic}-{oc}@{h}", ic, h, oc, 3, 1, 1) for i, (ic, h, oc) in enumerate(vgg)], 128, True)
+    for (IN, OUT) in ((512, 512), (512, 10)):
+        b = 128
+        X, W, bias = rnd(b, IN), rnd(OUT, IN), rnd(OUT)
+        Y, dY, dX, dW, dB = (torch.empty(b, OUT, device=dev), rnd(b, OUT), torch.empty(b, IN, device=dev),
+                             torch.zeros(OUT, IN, device=dev), torch.zeros(OUT, device=dev))
+        fl, by = 2.0 * b * IN * OUT, 4.0 * (b * IN + IN * OUT + b * OUT)
+        out["vgg16"].append(_entry(f"fc{IN}-{OUT}.fwd", event_time_ms(torch, lambda: capi.linear_fwd(X, W, bias, Y, b, IN, OUT), 30), fl, by))
+        out["vgg16"].append(_entry(f"fc{IN}-{OUT}.dgrad", event_time_ms(torch, lambda: capi.linear_dgrad(dY, W, dX, b, IN, OUT), 30), fl, by))
+        out["vgg16"].append(_entry(f"fc{IN}-{OUT}.wgrad", event_time_ms(torch, lambda: capi.linear_wgrad(dY, X, dW, dB, b, IN, OUT), 30), fl, by))
+
+    # config 4: DenseNet-BC-100 (k = 12), batch 64: first / middle / last bottleneck of each stage + the 3x3
+    dn = []
+    for (H, base) in ((32, 24), (16, 108), (8, 150)):
+        for i in (0, 8, 15):
+            dn.append((f"1x1_{base + 12 * i}-48@{H}", base + 12 * i, H, 48, 1, 1, 0))
+        dn.append((f"3x3_48-12@{H}", 48, H, 12, 3, 1, 1))
+    conv_entries("densenet", dn, 64, True)
+
+    # config 5: dense sweep (batch 256, 4096 <-> 4096) through linear* and the raw GEMM forms, plus tall-skinny
+    b, n = 256, 4096
+    X, W, bias = rnd(b, n), rnd(n, n), rnd(n)
+    Y, dX, dW, dB = torch.empty(b, n, device=dev), torch.empty(b, n, device=dev), torch.zeros(n, n, device=dev), torch.zeros(n, device=dev)
+    fl, by = 2.0 * b * n * n, 4.0 * (2 * b * n + n * n)
+    for nm, fn in (("linear (Y=X*W^T+b)", lambda: capi.linear_fwd(X, W, bias, Y, b, n, n)),
+                   ("linearXGrad (dX=dY*W)", lambda: capi.linear_dgrad(X, W, dX, b, n, n)),
+                   ("linearParamGrad (dW+=dY^T*X)", lambda: capi.linear_wgrad(X, X, dW, dB, b, n, n)),
+                   ("sgemmNT 256x4096x4096", lambda: capi.sgemm_nt(X, W, Y, b, n, n)),
+                   ("sgemm 256x4096x4096", lambda: capi.sgemm_nn(X, W, Y, b, n, n)),
+                   ("sgemmTN 4096x4096x256", lambda: capi.sgemm_tn(X, X, dW, n, n, b))):
+        out["dense"].append(_entry(nm, event_time_ms(torch, fn, 20), fl, by))
+    M, K, N = 32768, 576, 64
+    A, B, C = rnd(M, K), rnd(K, N), torch.empty(M, N, device=dev)
+    out["dense"].append(_entry("sgemm tall-skinny 32768x64x576", event_time_ms(torch, lambda: capi.sgemm_nn(A, B, C, M, N, K), 20),
+                               2.0 * M * N * K, 4.0 * (M * K + K * N + M * N)))
+
+    # summary lines
+    def total(key, suffix=None):
+        es = [e for e in out[key] if suffix is None or e["name"].endswith(suffix)]
+        return {"us": round(sum(e["us"] for e in es), 1), "gflop": round(sum(e["gflop"] for e in es), 2),
+                "tflops": round(sum(e["gflop"] for e in es) / max(sum(e["us"] for e in es), 1e-9) * 1e3, 2)}
+
+    out["summary"] = {"vgg16_conv_fc_train_step": total("vgg16"), "vgg16_fwd": total("vgg16", ".fwd"),
+                      "peak_fp32_mfma_tflops": PEAK_TF, "peak_hbm_gbs": PEAK_GBS, "ridge_flop_per_byte": round(RIDGE, 2)}
+    return out
+
+
+def to_markdown(rep):
+    lines = []
+    for key in ("gemm", "resnet56", "vgg16", "densenet", "dense"):
+        lines += [f"### {key}", "", "| shape.pass | us | GFLOP | MB | AI | TFLOP/s | GB/s | bound | fraction of roofline |", "|---|---|---|---|---|---|---|---|---|"]
+        for e in rep[key]:
+            lines.append(f"| {e['name']} | {e['us']} | {e['gflop']} | {e['mbytes']} | {e['ai']} | {e['tflops']} | {e['gbs']} | {e['bound']} | {e['frac'] * 100:.1f} % |")
+        lines.append("")
+    return "\n".join(lines)

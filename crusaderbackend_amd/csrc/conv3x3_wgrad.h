@@ -193,51 +193,6 @@ __global__ void __launch_bounds__(kThreads, Cfg::OCC) wgrad3x3s1_kernel(WgradArg
     }
 }
 
-// C[i] (+)= sum_z partial[z][i]. A workgroup covers OUTS consecutive outputs with 256/OUTS z-lanes per output; every
-// z-lane keeps 4 independent running sums over its strided subset of z (loads in flight instead of one dependent
-// chain), then the lanes are combined through LDS in lane order. The association is fixed by (splits, OUTS) alone,
-// so repeated runs are bit-identical.
-template <int OUTS>
-static __global__ void __launch_bounds__(256) splitk_reduce_wide_kernel(const float *__restrict__ partial, float *__restrict__ C,
-                                                                        u32 count, u32 splits, u32 accumulate) {
-    constexpr u32 ZL = 256 / OUTS;
-    __shared__ float red[ZL][OUTS];
-    const u32 o = threadIdx.x % OUTS, g = threadIdx.x / OUTS;
-    const u32 i = blockIdx.x * OUTS + o;
-    float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
-    if (i < count) {
-        const float *p = partial + i;
-        u32 zz = g;
-        for (; zz + 3 * ZL < splits; zz += 4 * ZL) {
-            s0 += p[size_t(zz) * count];
-            s1 += p[size_t(zz + ZL) * count];
-            s2 += p[size_t(zz + 2 * ZL) * count];
-            s3 += p[size_t(zz + 3 * ZL) * count];
-        }
-        for (; zz < splits; zz += ZL) s0 += p[size_t(zz) * count];
-    }
-    red[g][o] = (s0 + s1) + (s2 + s3);
-    __syncthreads();
-    if (g == 0 && i < count) {
-        float r = red[0][o];
-#pragma unroll
-        for (u32 k = 1; k < ZL; ++k) r += red[k][o];
-        C[i] = accumulate ? C[i] + r : r;
-    }
-}
-
-inline int launch_splitk_reduce_wide(const float *partial, float *C, u32 count, u32 splits, u32 accumulate, hipStream_t s,
-                                     const char *what) {
-    // enough workgroups to cover the chip even when the result is small
-    if (count >= 32u * 512u)
-        hipLaunchKernelGGL(splitk_reduce_wide_kernel<32>, dim3(ceil_div(count, 32)), dim3(256), 0, s, partial, C, count, splits, accumulate);
-    else if (count >= 16u * 256u)
-        hipLaunchKernelGGL(splitk_reduce_wide_kernel<16>, dim3(ceil_div(count, 16)), dim3(256), 0, s, partial, C, count, splits, accumulate);
-    else
-        hipLaunchKernelGGL(splitk_reduce_wide_kernel<8>, dim3(ceil_div(count, 8)), dim3(256), 0, s, partial, C, count, splits, accumulate);
-    return check_launch(what);
-}
-
 struct WgradDirectPlan {
     u32 pairs, tiles, splits, tiles_per_z;
     size_t workspace_bytes;
@@ -277,7 +232,7 @@ inline int launch_wgrad_direct(const float *dY, const float *X, float *dW, float
     hipLaunchKernelGGL((wgrad3x3s1_kernel<Cfg>), dim3(p.pairs, p.splits), dim3(kThreads), 0, s, a);
     if (int st = check_launch(what)) return st;
     if (p.splits > 1) {
-        return launch_splitk_reduce_wide(ws, dW, OC * IC * 9, p.splits, 1u, s, what);
+        return launch_splitk_reduce(ws, dW, OC * IC * 9, p.splits, ReduceEpi{nullptr, 1, 1, EPI_ACCUM}, s, what);
     }
     return CRB_OK;
 }

@@ -42,12 +42,36 @@ static Im2col make_im2col(const float *X, const crb_conv_geom *g) {
     return m;
 }
 
+template <class Cfg, class AOp, class BOp, class Epi>
+static int launch_cfg(const AOp &a, const BOp &b, const Epi &e, u32 M, u32 N, u32 K, u32 zdim, u32 split_k, u32 k_per_z,
+                      hipStream_t s, const char *what) {
+    return launch_igemm<Cfg>(a, b, e, M, N, K, zdim, split_k, k_per_z, s, what);
+}
+
 template <class AOp, class BOp, class Epi>
 static int run_by_m(const AOp &a, const BOp &b, const Epi &e, u32 M, u32 N, u32 K, u32 zdim, u32 split_k, u32 k_per_z,
                     hipStream_t s, const char *what) {
-    if (M <= 32) return launch_igemm<CfgM32>(a, b, e, M, N, K, zdim, split_k, k_per_z, s, what);
-    if (M <= 64) return launch_igemm<CfgM64>(a, b, e, M, N, K, zdim, split_k, k_per_z, s, what);
-    return launch_igemm<CfgM128>(a, b, e, M, N, K, zdim, split_k, k_per_z, s, what);
+    if (M <= 32) return launch_cfg<CfgM32>(a, b, e, M, N, K, zdim, split_k, k_per_z, s, what);
+    if (M <= 64) return launch_cfg<CfgM64>(a, b, e, M, N, K, zdim, split_k, k_per_z, s, what);
+    return launch_cfg<CfgM128>(a, b, e, M, N, K, zdim, split_k, k_per_z, s, what);
+}
+
+// Forward / data gradient through the engine with an NCHW result. When the tile grid is too small to occupy the chip
+// the contraction is cut into slices: partial NCHW results go to scratch, a second kernel sums them in fixed order and
+// applies bias / ReLU.
+template <class AOp, class BOp>
+static int run_nchw(const AOp &a, const BOp &b, NchwEpi e, u32 M, u32 N, u32 K, hipStream_t s, const char *what) {
+    const u32 bm = M <= 32 ? 32 : (M <= 64 ? 64 : 128);
+    const SplitPlan sp = plan_split(M, N, K, bm, 128, 16, 1);
+    if (sp.splits == 1) return run_by_m(a, b, e, M, N, K, 1, 0, K, s, what);
+    const u32 count = M * N;  // N = batch * H * W, so M*N is the whole NCHW tensor
+    const size_t need = size_t(sp.splits) * count * sizeof(float);
+    float *ws = static_cast<float *>(arena_get(need));
+    if (!ws) return fail(CRB_EHIP, "%s: cannot allocate %zu bytes of split-K scratch", what, need);
+    NchwEpi pe = e;
+    pe.T = ws, pe.row_bias = nullptr, pe.flags = 0u, pe.zstride = count;
+    if (int st = run_by_m(a, b, pe, M, N, K, sp.splits, 1, sp.k_per_z, s, what)) return st;
+    return launch_splitk_reduce(ws, e.T, count, sp.splits, ReduceEpi{e.row_bias, e.HW, e.C, e.flags}, s, what);
 }
 
 static u32 tile_m_for(u32 M) { return M <= 32 ? 32 : (M <= 64 ? 64 : 128); }
@@ -179,7 +203,7 @@ int crb_conv_fwd(const float *W, const float *X, float *Y, const float *bias_or_
     const u32 M = g->OC, N = g->N * g->OH * g->OW, K = g->IC * g->FH * g->FW;
     Im2colPixRows b{make_im2col(X, g)};
     NchwEpi e{Y, bias_or_null, g->OC, g->OH * g->OW, (flags & CRB_FLAG_RELU) ? u32(EPI_RELU) : 0u,
-              FastDiv(g->OH * g->OW)};
+              FastDiv(g->OH * g->OW), 0u};
     hipStream_t s = hipStream_t(stream);
     if (direct_shape(g) && aligned16(X) && aligned16(Y)) {
         bool done;
@@ -189,10 +213,10 @@ int crb_conv_fwd(const float *W, const float *X, float *Y, const float *bias_or_
     }
     if (K % 4 == 0 && aligned16(W)) {
         MatK<true> a{W, M, K, 0};
-        return run_by_m(a, b, e, M, N, K, 1, 0, K, s, "crb_conv_fwd");
+        return run_nchw(a, b, e, M, N, K, s, "crb_conv_fwd");
     }
     MatK<false> a{W, M, K, 0};
-    return run_by_m(a, b, e, M, N, K, 1, 0, K, s, "crb_conv_fwd");
+    return run_nchw(a, b, e, M, N, K, s, "crb_conv_fwd");
 }
 
 int crb_conv_dgrad(const float *W, const float *dY, float *dX, const crb_conv_geom *g, void *stream) {
@@ -216,8 +240,8 @@ int crb_conv_dgrad(const float *W, const float *dY, float *dX, const crb_conv_ge
     b.pH = g->pH, b.pW = g->pW;
     b.ihw.init(g->IH * g->IW), b.iw.init(g->IW), b.fhw.init(FHW), b.fw.init(g->FW);
     b.sH.init(g->sH), b.sW.init(g->sW);
-    NchwEpi e{dX, nullptr, g->IC, g->IH * g->IW, 0u, FastDiv(g->IH * g->IW)};
-    return run_by_m(a, b, e, M, N, K, 1, 0, K, hipStream_t(stream), "crb_conv_dgrad");
+    NchwEpi e{dX, nullptr, g->IC, g->IH * g->IW, 0u, FastDiv(g->IH * g->IW), 0u};
+    return run_nchw(a, b, e, M, N, K, hipStream_t(stream), "crb_conv_dgrad");
 }
 
 size_t crb_conv_wgrad_workspace_bytes(const crb_conv_geom *g) {
@@ -274,7 +298,7 @@ int crb_conv_wgrad(const float *dY, const float *X, float *dW, const crb_conv_ge
     }
     RowMajorEpi e{ws, nullptr, p.Ncols, p.M * p.Ncols, 0u};
     if (int st = run_by_m(a, b, e, p.M, p.Ncols, p.K, p.splits, 1, p.k_per_z, s, "crb_conv_wgrad")) return st;
-    return launch_splitk_reduce_wide(ws, dW, p.M * p.Ncols, p.splits, 1u, s, "crb_conv_wgrad(reduce)");
+    return launch_splitk_reduce(ws, dW, p.M * p.Ncols, p.splits, ReduceEpi{nullptr, 1, 1, EPI_ACCUM}, s, "crb_conv_wgrad(reduce)");
 }
 
 int crb_conv_bias_grad(const float *dY, float *dB, uint32_t N, uint32_t C, uint32_t HW, void *stream) {

@@ -10,13 +10,37 @@ typedef TileCfg<64, 64, 16, 2, 2, 2> CfgSmall;
 
 static inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
-template <class AOp, class BOp, class Epi>
-static int run_tiles(const AOp &a, const BOp &b, const Epi &e, u32 M, u32 N, u32 K, u32 zdim, hipStream_t s,
+// Runs C = A*B through the engine. `e` describes the final result; when the M x N tile grid is too small to occupy the
+// chip (and there is no batch), K is cut into slices whose partial results go to scratch and a second kernel combines
+// them in fixed order and applies the epilogue (bias / accumulate / ReLU).
+template <class Cfg, class AOp, class BOp>
+static int run_cfg(const AOp &a, const BOp &b, const RowMajorEpi &e, u32 M, u32 N, u32 K, u32 zdim, hipStream_t s,
+                   const char *what) {
+    const SplitPlan sp = plan_split(M, N, K, Cfg::BM, Cfg::BN, Cfg::BK, zdim);
+    if (sp.splits == 1) return launch_igemm<Cfg>(a, b, e, M, N, K, zdim, 0, K, s, what);
+    if (e.ld != N) return launch_igemm<Cfg>(a, b, e, M, N, K, zdim, 0, K, s, what);  // partials assume a dense result
+    const size_t need = size_t(sp.splits) * M * N * sizeof(float);
+    float *ws = static_cast<float *>(arena_get(need));
+    if (!ws) return fail(CRB_EHIP, "%s: cannot allocate %zu bytes of split-K scratch", what, need);
+    RowMajorEpi pe{ws, nullptr, N, M * N, 0u};
+    if (int st = launch_igemm<Cfg>(a, b, pe, M, N, K, sp.splits, 1, sp.k_per_z, s, what)) return st;
+    return launch_splitk_reduce(ws, e.C, M * N, sp.splits, ReduceEpi{e.col_bias, 1, N, e.flags}, s, what);
+}
+
+template <class AOp, class BOp>
+static int run_tiles(const AOp &a, const BOp &b, const RowMajorEpi &e, u32 M, u32 N, u32 K, u32 zdim, hipStream_t s,
                      const char *what) {
-    const uint64_t large_tiles = uint64_t(ceil_div(M, 128)) * ceil_div(N, 128) * zdim;
-    if (large_tiles >= 256 && M > 64 && N > 64)
-        return launch_igemm<CfgLarge>(a, b, e, M, N, K, zdim, 0, K, s, what);
-    return launch_igemm<CfgSmall>(a, b, e, M, N, K, zdim, 0, K, s, what);
+    // Large tiles when their grid alone occupies the chip; otherwise small tiles if those do; otherwise split K —
+    // with large tiles only when each slice keeps a long contraction (the split costs a second pass over the result).
+    const uint64_t tiles_l = uint64_t(ceil_div(M, 128)) * ceil_div(N, 128) * zdim;
+    const uint64_t tiles_s = uint64_t(ceil_div(M, 64)) * ceil_div(N, 64) * zdim;
+    if (M > 64 && N > 64) {
+        if (tiles_l >= 160) return run_cfg<CfgLarge>(a, b, e, M, N, K, zdim, s, what);
+        if (tiles_s >= 160 && K < 2048) return run_cfg<CfgSmall>(a, b, e, M, N, K, zdim, s, what);
+        const SplitPlan sp = plan_split(M, N, K, 128, 128, 16, zdim);
+        if (sp.splits > 1 && sp.k_per_z >= 512) return run_cfg<CfgLarge>(a, b, e, M, N, K, zdim, s, what);
+    }
+    return run_cfg<CfgSmall>(a, b, e, M, N, K, zdim, s, what);
 }
 
 static int check_dims(const char *what, u32 M, u32 N, u32 K, u32 batch) {

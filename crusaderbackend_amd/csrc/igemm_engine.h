@@ -28,6 +28,8 @@ typedef float v16f __attribute__((ext_vector_type(16)));
 constexpr int kThreads = 256;
 constexpr u32 kXcds = 8;
 
+enum : u32 { EPI_ACCUM = 1u, EPI_RELU = 2u };
+
 struct IgemmDims {
     u32 M, N, K;
     u32 tiles_m, tiles_n;
@@ -286,6 +288,82 @@ __global__ void __launch_bounds__(kThreads, Cfg::OCC) igemm_kernel(AOp a, BOp b,
                 if (row < d.M) epi.store(row, cs, acc[mi][ni][r]);
             }
     }
+}
+
+// ---- split-K second pass --------------------------------------------------------------------------------
+// C[i] (+)= sum_z partial[z][i] (+ bias) (ReLU). A workgroup covers OUTS consecutive outputs with 256/OUTS z-lanes per
+// output; every z-lane keeps 4 independent running sums over its strided subset of z (loads in flight instead of one
+// dependent chain), then the lanes are combined through LDS in lane order. The association is fixed by (splits, OUTS)
+// alone, so repeated runs are bit-identical. Bias index of output i: (i / bias_div) % bias_mod
+// (row-major result with per-column bias: div 1, mod N; NCHW with per-channel bias: div H*W, mod C).
+struct ReduceEpi {
+    const float *bias;
+    u32 bias_div, bias_mod;
+    u32 flags;  // EPI_ACCUM | EPI_RELU
+};
+
+template <int OUTS>
+static __global__ void __launch_bounds__(256) splitk_reduce_kernel(const float *__restrict__ partial, float *__restrict__ C, u32 count,
+                                                                   u32 splits, ReduceEpi e, FastDiv bdiv) {
+    constexpr u32 ZL = 256 / OUTS;
+    __shared__ float red[ZL][OUTS];
+    const u32 o = threadIdx.x % OUTS, g = threadIdx.x / OUTS;
+    const u32 i = blockIdx.x * OUTS + o;
+    float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
+    if (i < count) {
+        const float *p = partial + i;
+        u32 zz = g;
+        for (; zz + 3 * ZL < splits; zz += 4 * ZL) {
+            s0 += p[size_t(zz) * count];
+            s1 += p[size_t(zz + ZL) * count];
+            s2 += p[size_t(zz + 2 * ZL) * count];
+            s3 += p[size_t(zz + 3 * ZL) * count];
+        }
+        for (; zz < splits; zz += ZL) s0 += p[size_t(zz) * count];
+    }
+    red[g][o] = (s0 + s1) + (s2 + s3);
+    __syncthreads();
+    if (g == 0 && i < count) {
+        float r = red[0][o];
+#pragma unroll
+        for (u32 k = 1; k < ZL; ++k) r += red[k][o];
+        if (e.bias) r += e.bias[bdiv.div(i) % e.bias_mod];
+        if (e.flags & EPI_ACCUM) r += C[i];
+        if (e.flags & EPI_RELU) r = r > 0.f ? r : 0.f;
+        C[i] = r;
+    }
+}
+
+inline int launch_splitk_reduce(const float *partial, float *C, u32 count, u32 splits, ReduceEpi e, hipStream_t s,
+                                const char *what) {
+    FastDiv bdiv(e.bias_div ? e.bias_div : 1);
+    if (!e.bias_mod) e.bias_mod = 1;
+    // enough workgroups to cover the chip even when the result is small
+    if (count >= 32u * 512u)
+        hipLaunchKernelGGL(splitk_reduce_kernel<32>, dim3(ceil_div(count, 32)), dim3(256), 0, s, partial, C, count, splits, e, bdiv);
+    else if (count >= 16u * 256u)
+        hipLaunchKernelGGL(splitk_reduce_kernel<16>, dim3(ceil_div(count, 16)), dim3(256), 0, s, partial, C, count, splits, e, bdiv);
+    else
+        hipLaunchKernelGGL(splitk_reduce_kernel<8>, dim3(ceil_div(count, 8)), dim3(256), 0, s, partial, C, count, splits, e, bdiv);
+    return check_launch(what);
+}
+
+// How to cut K when an M x N result gives too few macro-tiles to occupy 256 CUs.
+struct SplitPlan {
+    u32 splits, k_per_z;
+};
+inline SplitPlan plan_split(u32 M, u32 N, u32 K, u32 BM, u32 BN, u32 BK, u32 zdim) {
+    SplitPlan p{1, K};
+    const uint64_t tiles = uint64_t(ceil_div(M, BM)) * ceil_div(N, BN) * zdim;
+    if (zdim != 1 || tiles >= 160) return p;
+    u32 want = u32(ceil_div(256u, u32(tiles)));
+    const u32 max_by_k = K / (8 * BK) ? K / (8 * BK) : 1;  // keep at least 8 slabs per slice
+    if (want > max_by_k) want = max_by_k;
+    if (want <= 1) return p;
+    p.k_per_z = ceil_div(ceil_div(K, want), BK) * BK;
+    p.splits = ceil_div(K, p.k_per_z);
+    if (p.splits <= 1) p = SplitPlan{1, K};
+    return p;
 }
 
 template <class Cfg, class AOp, class BOp, class Epi>

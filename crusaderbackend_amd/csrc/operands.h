@@ -226,8 +226,6 @@ struct DgradGather {
 };
 
 // ---- epilogues ----------------------------------------------------------------------------------------
-enum : u32 { EPI_ACCUM = 1u, EPI_RELU = 2u };
-
 // Row-major result C[z*zstride + row*ld + col], optional per-column bias (dense layer), optional
 // accumulate (C += v) and ReLU.
 struct RowMajorEpi {
@@ -260,11 +258,12 @@ struct NchwEpi {
     const float *row_bias;
     u32 C, HW, flags;
     FastDiv hw;
+    u32 zstride;  // elements between split-K partial results (0 when not splitting)
     struct ColS {
         u32 off;
         bool ok;
     };
-    __device__ __forceinline__ void bind(u32) {}
+    __device__ __forceinline__ void bind(u32 z) { T += size_t(z) * zstride; }
     __device__ __forceinline__ ColS prep_col(u32 col, u32 ncols) const {
         u32 n, p;
         hw.divmod(col, n, p);

@@ -163,3 +163,25 @@ def test_error_paths(dev):
     assert lib.crb_sgemm_nn(t.data_ptr(), t.data_ptr(), t.data_ptr(), 0, 4, 1, 1, None) == capi.CRB_EINVAL_SHAPE
     assert b"zero dimension" in lib.crb_last_error_string()
     assert lib.crb_linear_fwd(t.data_ptr(), t.data_ptr(), None, t.data_ptr(), 1, 4, 4, 0, None) == capi.CRB_ENULL
+
+
+@pytest.mark.parametrize("M,N,K", [(256, 256, 4096), (100, 200, 3000), (64, 48, 8192), (130, 1000, 2049), (1, 1, 5000)])
+def test_split_k_paths(dev, M, N, K):
+    """Few output tiles and a long contraction: the K range is split over workgroups and recombined in fixed order."""
+    run_nn(dev, M, N, K, 1, seed=41)
+    run_tn(dev, M, N, K, 1, seed=42)
+    run_nt(dev, M, N, K, seed=43)
+
+
+def test_split_k_nta_small_output_and_bias_epilogue(dev):
+    run_nta(dev, 48, 24, 1024, 64, seed=44)
+    capi, orc = _capi(), _oracle()
+    batch, IN, OUT = 32, 2048, 300
+    X, W, b = normal(1, batch, IN), normal(2, OUT, IN, std=0.02), normal(3, OUT)
+    Y = _empty(dev, batch, OUT)
+    capi.linear_fwd(to_dev(X, dev), to_dev(W, dev), to_dev(b, dev), Y, batch, IN, OUT, flags=capi.CRB_FLAG_RELU)
+    assert_close(to_np(Y), np.maximum(orc.linear(X, W, b, threads=8), 0), IN, "split-K linear + bias + relu")
+    # bit-reproducible
+    Y2 = _empty(dev, batch, OUT)
+    capi.linear_fwd(to_dev(X, dev), to_dev(W, dev), to_dev(b, dev), Y2, batch, IN, OUT, flags=capi.CRB_FLAG_RELU)
+    assert np.array_equal(to_np(Y), to_np(Y2))
