@@ -22,8 +22,8 @@
 
 namespace crb {
 
-// NBUF_ = 2: double-buffered chunk pipeline (any C_IN that is a multiple of CI). NBUF_ = 1: the whole contraction is one
-// chunk (C_IN == CI), half the LDS, so more workgroups fit on a CU and overlap each other's staging.
+// NBUF_ = 2: double-buffered chunk pipeline (any C_IN). NBUF_ = 1: the whole contraction is one
+// chunk (C_IN <= CI), half the LDS, so more workgroups fit on a CU and overlap each other's staging.
 template <int W_, int ROWS_, int CI_, int OCT_, int PBW_, int OBW_, bool DGRAD_, int OCC_, int NBUF_ = 2>
 struct DirectCfg {
     static constexpr int W = W_, ROWS = ROWS_, CI = CI_, OCT = OCT_, PBW = PBW_, OBW = OBW_, OCC = OCC_, NBUF = NBUF_;
@@ -100,7 +100,7 @@ __global__ void __launch_bounds__(kThreads, Cfg::OCC) conv3x3s1_kernel(DirectArg
             if (XQ % kThreads == 0 || e < XQ) {
                 const u32 q = e % (W / 4), lr = (e / (W / 4)) % XR, c = e / ((W / 4) * XR);
                 const int row = r0 - 1 + int(lr);
-                if (row >= 0 && row < int(a.H))
+                if (row >= 0 && row < int(a.H) && c0 + c < a.C_IN)
                     v = *reinterpret_cast<const v4f *>(a.X + (size_t(n) * a.C_IN + c0 + c) * HW + u32(row) * W + 4 * q);
             }
             xreg[i] = v;
@@ -113,9 +113,15 @@ __global__ void __launch_bounds__(kThreads, Cfg::OCC) conv3x3s1_kernel(DirectArg
             const u32 j = Cfg::DGRAD ? e % OCT : e / CI, c = Cfg::DGRAD ? e / OCT : e % CI;
             const float *src = Cfg::DGRAD ? a.Wt + ((size_t(c0) + c) * a.C_OUT + oc0 + j) * 9
                                           : a.Wt + ((size_t(oc0) + j) * a.C_IN + c0 + c) * 9;
-            const bool ok = WQ % kThreads == 0 || e < WQ;
+            // channels past the tensor's extent (ragged last chunk / last channel tile) are staged as zeros
+            const bool ok = (WQ % kThreads == 0 || e < WQ) && c0 + c < a.C_IN && oc0 + j < a.C_OUT;
+            if (ok) {  // one branch around the 9 contiguous loads keeps them mergeable into wide loads
 #pragma unroll
-            for (int tap = 0; tap < 9; ++tap) wreg[i * 9 + tap] = ok ? src[tap] : 0.f;
+                for (int tap = 0; tap < 9; ++tap) wreg[i * 9 + tap] = src[tap];
+            } else {
+#pragma unroll
+                for (int tap = 0; tap < 9; ++tap) wreg[i * 9 + tap] = 0.f;
+            }
         }
     };
 
@@ -196,7 +202,7 @@ __global__ void __launch_bounds__(kThreads, Cfg::OCC) conv3x3s1_kernel(DirectArg
     if constexpr (NBUF == 1) {
         compute(sX[0], sW[0]);
     } else {
-        const u32 nchunk = a.C_IN / CI;
+        const u32 nchunk = (a.C_IN + CI - 1) / CI;
         for (u32 ch = 0; ch < nchunk; ++ch) {
             const bool more = ch + 1 < nchunk;
             if (more) fetch((ch + 1) * CI);
@@ -215,6 +221,7 @@ __global__ void __launch_bounds__(kThreads, Cfg::OCC) conv3x3s1_kernel(DirectArg
 #pragma unroll
     for (int o = 0; o < OBW; ++o) {
         const u32 oc = oc0 + (wo * OBW + o) * 16 + li;
+        if (oc >= a.C_OUT) continue;
         const float b = a.bias ? a.bias[oc] : 0.f;
 #pragma unroll
         for (int p = 0; p < PBW; ++p) {
@@ -237,7 +244,7 @@ inline int launch_direct(const float *Wt, const float *X, float *Y, const float 
     a.Wt = Wt, a.X = X, a.Y = Y, a.bias = bias;
     a.C_IN = C_IN, a.C_OUT = C_OUT, a.H = H;
     a.tiles_per_img = H / Cfg::ROWS;
-    a.oc_tiles = C_OUT / Cfg::OCT;
+    a.oc_tiles = ceil_div(C_OUT, u32(Cfg::OCT));
     a.relu = relu;
     const uint64_t wgs = uint64_t(N) * a.tiles_per_img * a.oc_tiles;
     if (wgs > 0x7fffffffull) return fail(CRB_EINVAL_SHAPE, "%s: launch grid too large", what);
@@ -245,11 +252,11 @@ inline int launch_direct(const float *Wt, const float *X, float *Y, const float 
     return check_launch(what);
 }
 
-// shape gate shared by all configurations of one image width
+// Shape gate of one configuration. Channel counts need not divide CI / OCT: ragged chunks and tiles are zero-filled.
 template <class Cfg>
 inline bool direct_fits(u32 C_IN, u32 C_OUT, u32 H, u32 Wd) {
-    return Wd == u32(Cfg::W) && H % Cfg::ROWS == 0 && C_OUT % Cfg::OCT == 0 &&
-           (Cfg::NBUF == 1 ? C_IN == u32(Cfg::CI) : C_IN % Cfg::CI == 0);
+    (void)C_OUT;
+    return Wd == u32(Cfg::W) && H % Cfg::ROWS == 0 && (Cfg::NBUF == 1 ? C_IN <= u32(Cfg::CI) : true);
 }
 
 }  // namespace crb

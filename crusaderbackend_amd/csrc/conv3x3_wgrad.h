@@ -43,7 +43,7 @@ struct WgradArgs {
     const float *X;   // N x IC x H x W
     float *out;       // splits > 1: partials [z][OC][IC][9]; splits == 1: dW (accumulated)
     u32 OC, IC, H;
-    u32 ic_blocks;        // IC / 16
+    u32 ic_blocks;        // ceil(IC / 16)
     u32 tiles, tiles_per_z;  // tile count (N/TI * H/TR) and tiles per split
     u32 tiles_per_img;    // H / TR
     u32 accumulate;       // add to `out` instead of overwriting (splits == 1)
@@ -76,7 +76,8 @@ __global__ void __launch_bounds__(kThreads, Cfg::OCC) wgrad3x3s1_kernel(WgradArg
             v4f v = {0.f, 0.f, 0.f, 0.f};
             if (YQ % kThreads == 0 || e < YQ) {
                 const u32 q = e % (YIMG / 4), c = (e / (YIMG / 4)) % 16, img = e / ((YIMG / 4) * 16);
-                v = *reinterpret_cast<const v4f *>(a.dY + (size_t(n0 + img) * a.OC + ob * 16 + c) * HW + u32(r0) * W + 4 * q);
+                if (ob * 16 + c < a.OC)  // channels past the tensor's extent are staged as zeros
+                    v = *reinterpret_cast<const v4f *>(a.dY + (size_t(n0 + img) * a.OC + ob * 16 + c) * HW + u32(r0) * W + 4 * q);
             }
             yreg[i] = v;
         }
@@ -87,7 +88,7 @@ __global__ void __launch_bounds__(kThreads, Cfg::OCC) wgrad3x3s1_kernel(WgradArg
             if (XQ % kThreads == 0 || e < XQ) {
                 const u32 q = e % (XIMG / 4), c = (e / (XIMG / 4)) % 16, img = e / ((XIMG / 4) * 16);
                 const int row = r0 - 1 + int(q / (W / 4));
-                if (row >= 0 && row < int(a.H))
+                if (row >= 0 && row < int(a.H) && ib * 16 + c < a.IC)
                     v = *reinterpret_cast<const v4f *>(a.X + (size_t(n0 + img) * a.IC + ib * 16 + c) * HW + u32(row) * W +
                                                        4 * (q % (W / 4)));
             }
@@ -184,6 +185,7 @@ __global__ void __launch_bounds__(kThreads, Cfg::OCC) wgrad3x3s1_kernel(WgradArg
     float *out = a.out + size_t(z) * count * (a.accumulate ? 0 : 1);
     for (u32 e = t; e < 16 * 16 * 9; e += kThreads) {
         const u32 oc = e / 144, ic = (e % 144) / 9, tap = e % 9;
+        if (ob * 16 + oc >= a.OC || ib * 16 + ic >= a.IC) continue;
         const u32 src = (tap * 64 + (oc / 4) * 16 + ic) * 4 + (oc % 4);
         float s = red[src];
 #pragma unroll
@@ -200,13 +202,14 @@ struct WgradDirectPlan {
 
 template <class Cfg>
 inline bool wgrad_direct_fits(u32 N, u32 IC, u32 OC, u32 H, u32 Wd) {
-    return Wd == u32(Cfg::W) && H % Cfg::TR == 0 && N % Cfg::TI == 0 && IC % 16 == 0 && OC % 16 == 0;
+    (void)IC, (void)OC;  // ragged channel blocks are zero-filled
+    return Wd == u32(Cfg::W) && H % Cfg::TR == 0 && N % Cfg::TI == 0;
 }
 
 template <class Cfg>
 inline WgradDirectPlan wgrad_direct_plan(u32 N, u32 IC, u32 OC, u32 H, u32 target_wgs) {
     WgradDirectPlan p;
-    p.pairs = (OC / 16) * (IC / 16);
+    p.pairs = ceil_div(OC, 16u) * ceil_div(IC, 16u);
     p.tiles = (N / Cfg::TI) * (H / Cfg::TR);
     u32 splits = p.pairs >= target_wgs ? 1 : target_wgs / p.pairs;
     if (splits > p.tiles) splits = p.tiles;
@@ -224,7 +227,7 @@ inline int launch_wgrad_direct(const float *dY, const float *X, float *dW, float
     a.dY = dY, a.X = X;
     a.out = p.splits > 1 ? ws : dW;
     a.OC = OC, a.IC = IC, a.H = H;
-    a.ic_blocks = IC / 16;
+    a.ic_blocks = ceil_div(IC, 16u);
     a.tiles = p.tiles, a.tiles_per_z = p.tiles_per_z;
     a.tiles_per_img = H / Cfg::TR;
     a.accumulate = p.splits > 1 ? 0u : 1u;

@@ -2,6 +2,7 @@
 // standalone bias add, all as implicit GEMMs on the MFMA engine (no im2col buffer is materialised).
 #include "conv3x3_direct.h"
 #include "conv3x3_wgrad.h"
+#include "gemm_internal.h"
 #include "operands.h"
 
 namespace crb {
@@ -108,28 +109,36 @@ static int try_direct(const float *Wt, const float *X, float *Y, const float *bi
 #define CRB_TRY(...)                                                                                         \
     if (direct_fits<DirectCfg<__VA_ARGS__>>(C_IN, C_OUT, H, Wd))                                              \
         return launch_direct<DirectCfg<__VA_ARGS__>>(Wt, X, Y, bias, N, C_IN, C_OUT, H, relu, s, what);
+    // output-channel tile: the smallest of 16 / 32 / 64 that covers C_OUT, 64 beyond; chunk of 16 input channels
+    // unless C_IN <= 8
     if (Wd == 32) {
-        CRB_TRY(32, 8, 16, 16, 4, 1, DG, 2, 1)  // C_IN == 16: whole contraction in one LDS-resident chunk
-        if (C_OUT >= 64) { CRB_TRY(32, 8, 8, 64, 4, 4, DG, 2, 2) }
-        if (C_OUT >= 32) { CRB_TRY(32, 8, 8, 32, 4, 2, DG, 2, 2) }
+        if (C_IN <= 16 && C_IN > 8 && C_OUT <= 16) { CRB_TRY(32, 8, 16, 16, 4, 1, DG, 2, 1) }  // one LDS-resident chunk
+        if (C_OUT > 32) { CRB_TRY(32, 8, 8, 64, 4, 4, DG, 2, 2) }
+        if (C_OUT > 16) { CRB_TRY(32, 8, 8, 32, 4, 2, DG, 2, 2) }
         CRB_TRY(32, 8, 8, 16, 4, 1, DG, 2, 2)
         CRB_TRY(32, 4, 8, 16, 2, 1, DG, 2, 2)
     } else if (Wd == 16) {
-        if (C_OUT >= 128) { CRB_TRY(16, 8, 8, 64, 2, 4, DG, 2, 2) }
-        CRB_TRY(16, 4, 16, 32, 1, 2, DG, 2, 2)
-        CRB_TRY(16, 4, 8, 32, 1, 2, DG, 2, 2)
+        if (C_OUT > 64) { CRB_TRY(16, 8, 8, 64, 2, 4, DG, 2, 2) }
+        if (C_OUT > 16 && C_IN > 8) { CRB_TRY(16, 4, 16, 32, 1, 2, DG, 2, 2) }
+        if (C_OUT > 16) { CRB_TRY(16, 4, 8, 32, 1, 2, DG, 2, 2) }
         CRB_TRY(16, 8, 8, 16, 2, 1, DG, 2, 2)
         CRB_TRY(16, 4, 8, 16, 1, 1, DG, 2, 2)
     } else if (Wd == 8) {
-        if (C_OUT >= 256) { CRB_TRY(8, 8, 16, 64, 1, 4, DG, 2, 2) }
-        if (C_OUT >= 128) { CRB_TRY(8, 8, 16, 32, 1, 2, DG, 2, 2) }
-        CRB_TRY(8, 8, 16, 16, 1, 1, DG, 2, 2)
+        if (C_OUT > 128 && C_IN > 8) { CRB_TRY(8, 8, 16, 64, 1, 4, DG, 2, 2) }
+        if (C_OUT > 64 && C_IN > 8) { CRB_TRY(8, 8, 16, 32, 1, 2, DG, 2, 2) }
+        if (C_IN > 8) { CRB_TRY(8, 8, 16, 16, 1, 1, DG, 2, 2) }
         CRB_TRY(8, 8, 8, 16, 1, 1, DG, 2, 2)
         CRB_TRY(8, 4, 8, 32, 1, 1, DG, 2, 2)
     }
 #undef CRB_TRY
     done = false;
     return CRB_OK;
+}
+
+// 1x1 / stride 1 / no padding: per image Y[n] (OC x HW) = W (OC x IC) * X[n] (IC x HW) on the native layout, i.e. the
+// batched forms of the GEMM family (forward NN with a per-row bias, data gradient TN, weight gradient accumulate-NT).
+static bool pointwise_shape(const crb_conv_geom *g) {
+    return g->FH == 1 && g->FW == 1 && g->sH == 1 && g->sW == 1 && g->pH == 0 && g->pW == 0;
 }
 
 static bool direct_shape(const crb_conv_geom *g) {
@@ -205,6 +214,9 @@ int crb_conv_fwd(const float *W, const float *X, float *Y, const float *bias_or_
     NchwEpi e{Y, bias_or_null, g->OC, g->OH * g->OW, (flags & CRB_FLAG_RELU) ? u32(EPI_RELU) : 0u,
               FastDiv(g->OH * g->OW), 0u};
     hipStream_t s = hipStream_t(stream);
+    if (pointwise_shape(g))
+        return gemm_nn_rowbias(W, X, Y, g->OC, g->IH * g->IW, g->IC, g->N, bias_or_null,
+                               (flags & CRB_FLAG_RELU) ? u32(EPI_RELU) : 0u, s, "crb_conv_fwd");
     if (direct_shape(g) && aligned16(X) && aligned16(Y)) {
         bool done;
         int st = try_direct<false>(W, X, Y, bias_or_null, g->N, g->IC, g->OC, g->IH, g->IW, flags & CRB_FLAG_RELU, s,
@@ -222,6 +234,8 @@ int crb_conv_fwd(const float *W, const float *X, float *Y, const float *bias_or_
 int crb_conv_dgrad(const float *W, const float *dY, float *dX, const crb_conv_geom *g, void *stream) {
     if (!W || !dY || !dX) return fail(CRB_ENULL, "crb_conv_dgrad: null operand");
     if (int st = check_geom("crb_conv_dgrad", g)) return st;
+    if (pointwise_shape(g))
+        return gemm_tn_batched(W, dY, dX, g->IC, g->IH * g->IW, g->OC, g->N, hipStream_t(stream), "crb_conv_dgrad");
     if (direct_shape(g) && aligned16(dY) && aligned16(dX)) {
         bool done;
         int st = try_direct<true>(W, dY, dX, nullptr, g->N, g->OC, g->IC, g->IH, g->IW, 0, hipStream_t(stream),
@@ -246,6 +260,7 @@ int crb_conv_dgrad(const float *W, const float *dY, float *dX, const crb_conv_ge
 
 size_t crb_conv_wgrad_workspace_bytes(const crb_conv_geom *g) {
     if (check_geom("crb_conv_wgrad_workspace_bytes", g)) return 0;
+    if (pointwise_shape(g)) return 0;  // accumulate-NT GEMM form; its split scratch comes from the library arena
     {
         WgradDirectPlan dp;
         int st = 0;
@@ -260,6 +275,7 @@ int crb_conv_wgrad(const float *dY, const float *X, float *dW, const crb_conv_ge
     if (!dY || !X || !dW) return fail(CRB_ENULL, "crb_conv_wgrad: null operand");
     if (int st = check_geom("crb_conv_wgrad", g)) return st;
     hipStream_t s = hipStream_t(stream);
+    if (pointwise_shape(g)) return crb_sgemm_nta(dY, X, dW, g->OC, g->IC, g->IH * g->IW, g->N, stream);
     if (aligned16(dY) && aligned16(X)) {
         WgradDirectPlan dp;
         int st = CRB_OK;

@@ -1,4 +1,5 @@
 // C-ABI entry points of the GEMM and dense-layer families (fp32, row-major) on the MFMA engine.
+#include "gemm_internal.h"
 #include "operands.h"
 
 namespace crb {
@@ -24,6 +25,7 @@ static int run_cfg(const AOp &a, const BOp &b, const RowMajorEpi &e, u32 M, u32 
     if (!ws) return fail(CRB_EHIP, "%s: cannot allocate %zu bytes of split-K scratch", what, need);
     RowMajorEpi pe{ws, nullptr, N, M * N, 0u};
     if (int st = launch_igemm<Cfg>(a, b, pe, M, N, K, sp.splits, 1, sp.k_per_z, s, what)) return st;
+    if (e.row_bias) return launch_splitk_reduce(ws, e.C, M * N, sp.splits, ReduceEpi{e.row_bias, N, M, e.flags}, s, what);
     return launch_splitk_reduce(ws, e.C, M * N, sp.splits, ReduceEpi{e.col_bias, 1, N, e.flags}, s, what);
 }
 
@@ -62,8 +64,9 @@ __global__ void __launch_bounds__(256) colsum_accum_kernel(const float *__restri
 }
 
 static int gemm_nn(const float *A, const float *B, float *C, u32 M, u32 N, u32 K, u32 batch, const float *col_bias,
-                   u32 flags, hipStream_t s, const char *what) {
+                   u32 flags, hipStream_t s, const char *what, const float *row_bias = nullptr) {
     RowMajorEpi e{C, col_bias, N, M * N, flags};
+    e.row_bias = row_bias;
     if (K % 4 == 0 && N % 4 == 0 && aligned16(A) && aligned16(B)) {
         MatK<true> a{A, M, K, 0};
         MatR<true> b{B, N, N, K * N};
@@ -98,6 +101,15 @@ static int gemm_nt(const float *A, const float *B, float *C, u32 M, u32 N, u32 K
     MatK<false> a{A, M, K, 0};
     MatK<false> b{B, N, K, 0};
     return run_tiles(a, b, e, M, N, K, 1, s, what);
+}
+
+int gemm_nn_rowbias(const float *A, const float *B, float *C, u32 M, u32 N, u32 K, u32 batch, const float *row_bias, u32 flags,
+                    hipStream_t s, const char *what) {
+    return gemm_nn(A, B, C, M, N, K, batch, nullptr, flags, s, what, row_bias);
+}
+
+int gemm_tn_batched(const float *A, const float *B, float *C, u32 M, u32 N, u32 K, u32 batch, hipStream_t s, const char *what) {
+    return gemm_tn(A, B, C, M, N, K, batch, 0, s, what);
 }
 
 }  // namespace crb

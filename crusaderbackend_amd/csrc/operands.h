@@ -226,12 +226,13 @@ struct DgradGather {
 };
 
 // ---- epilogues ----------------------------------------------------------------------------------------
-// Row-major result C[z*zstride + row*ld + col], optional per-column bias (dense layer), optional
-// accumulate (C += v) and ReLU.
+// Row-major result C[z*zstride + row*ld + col], optional per-column bias (dense layer) or per-row bias (1x1
+// convolution as a batched GEMM), optional accumulate (C += v) and ReLU.
 struct RowMajorEpi {
     float *C;
     const float *col_bias;
     u32 ld, zstride, flags;
+    const float *row_bias = nullptr;
     struct ColS {
         u32 col;
         float bias;
@@ -246,6 +247,7 @@ struct RowMajorEpi {
         if (!c.ok) return;
         float *p = C + size_t(row) * ld + c.col;
         v += c.bias;
+        if (row_bias) v += row_bias[row];
         if (flags & EPI_ACCUM) v += *p;
         if (flags & EPI_RELU) v = v > 0.0f ? v : 0.0f;
         *p = v;

@@ -220,6 +220,9 @@ DIRECT = [
     (3, 64, 8, 8, 64), (2, 128, 8, 8, 256), (2, 32, 8, 8, 128), (2, 8, 8, 8, 16), (2, 24, 8, 8, 32), (2, 8, 4, 8, 32),
     (2, 16, 30, 32, 16), (2, 12, 16, 16, 16), (2, 16, 8, 8, 24), (2, 16, 6, 8, 16),
     (4, 64, 8, 8, 64), (8, 32, 8, 8, 16), (5, 16, 16, 16, 32), (1, 16, 32, 32, 16), (6, 48, 8, 8, 32),
+    # channel counts that divide neither the channel chunk nor the channel tile (zero-filled tails)
+    (2, 3, 32, 32, 16), (2, 48, 32, 32, 12), (2, 5, 16, 16, 7), (4, 13, 8, 8, 19), (2, 3, 32, 32, 64), (2, 17, 16, 16, 33),
+    (4, 1, 8, 8, 1), (2, 9, 32, 32, 70),
 ]
 
 
