@@ -61,7 +61,7 @@ struct DirectArgs {
     float *Y;           // output of this pass (forward: Y, dgrad: dX), N x C_OUT x H x W
     const float *bias;  // per output channel or nullptr
     u32 C_IN, C_OUT, H;
-    u32 tiles_per_img, oc_tiles;
+    u32 tiles_per_img, oc_tiles, tiles_total;  // tiles_total = N * tiles_per_img
     u32 relu;
 };
 
@@ -74,8 +74,12 @@ __global__ void __launch_bounds__(kThreads, Cfg::OCC) conv3x3s1_kernel(DirectArg
     __shared__ __attribute__((aligned(16))) float sW[NBUF][Cfg::W_SIZE];
 
     const u32 t = threadIdx.x;
-    const u32 oct = blockIdx.x % a.oc_tiles;
-    const u32 rest = blockIdx.x / a.oc_tiles;
+    // Workgroups are dealt round-robin to the 8 XCDs. Decode the id so that the oc_tiles workgroups that read the same
+    // input rows get ids 8 apart: they land on the same XCD, back to back, and share those rows through its L2.
+    const u32 xcd = blockIdx.x % kXcds, slot = blockIdx.x / kXcds;
+    const u32 oct = slot % a.oc_tiles;
+    const u32 rest = (slot / a.oc_tiles) * kXcds + xcd;
+    if (rest >= a.tiles_total) return;
     const u32 tile = rest % a.tiles_per_img;
     const u32 n = rest / a.tiles_per_img;
     const int r0 = int(tile) * ROWS;  // first output row of this tile
@@ -246,7 +250,8 @@ inline int launch_direct(const float *Wt, const float *X, float *Y, const float 
     a.tiles_per_img = H / Cfg::ROWS;
     a.oc_tiles = ceil_div(C_OUT, u32(Cfg::OCT));
     a.relu = relu;
-    const uint64_t wgs = uint64_t(N) * a.tiles_per_img * a.oc_tiles;
+    a.tiles_total = N * a.tiles_per_img;
+    const uint64_t wgs = uint64_t(ceil_div(a.tiles_total, kXcds)) * kXcds * a.oc_tiles;  // padded to whole XCD rounds
     if (wgs > 0x7fffffffull) return fail(CRB_EINVAL_SHAPE, "%s: launch grid too large", what);
     hipLaunchKernelGGL((conv3x3s1_kernel<Cfg>), dim3(u32(wgs)), dim3(kThreads), 0, s, a);
     return check_launch(what);

@@ -46,6 +46,7 @@ struct WgradArgs {
     u32 ic_blocks;        // ceil(IC / 16)
     u32 tiles, tiles_per_z;  // tile count (N/TI * H/TR) and tiles per split
     u32 tiles_per_img;    // H / TR
+    u32 pairs, splits;
     u32 accumulate;       // add to `out` instead of overwriting (splits == 1)
 };
 
@@ -56,7 +57,17 @@ __global__ void __launch_bounds__(kThreads, Cfg::OCC) wgrad3x3s1_kernel(WgradArg
     __shared__ __attribute__((aligned(16))) float smem[Cfg::SMEM];  // buffer b: dY planes at b*BUF, X planes after them
 
     const u32 t = threadIdx.x;
-    const u32 pair = blockIdx.x, z = blockIdx.y;
+    // The workgroups of one split z read the same tiles (different channel blocks). With ids 8 apart they run on the
+    // same XCD and share the tiles through its L2 (workgroups are dealt round-robin to the 8 XCDs).
+    // Only done when there are at least 8 splits; with fewer, ids map plainly so every XCD still gets work.
+    u32 pair, z;
+    if (a.splits >= kXcds) {
+        const u32 xcd = blockIdx.x % kXcds, slot = blockIdx.x / kXcds;
+        pair = slot % a.pairs, z = (slot / a.pairs) * kXcds + xcd;
+        if (z >= a.splits) return;
+    } else {
+        pair = blockIdx.x % a.pairs, z = blockIdx.x / a.pairs;
+    }
     const u32 ob = pair / a.ic_blocks, ib = pair % a.ic_blocks;
     const u32 HW = a.H * W;
     const u32 t_begin = z * a.tiles_per_z;
@@ -231,8 +242,11 @@ inline int launch_wgrad_direct(const float *dY, const float *X, float *dW, float
     a.tiles = p.tiles, a.tiles_per_z = p.tiles_per_z;
     a.tiles_per_img = H / Cfg::TR;
     a.accumulate = p.splits > 1 ? 0u : 1u;
-    if (p.splits > 65535u) return fail(CRB_EINVAL_SHAPE, "%s: too many splits", what);
-    hipLaunchKernelGGL((wgrad3x3s1_kernel<Cfg>), dim3(p.pairs, p.splits), dim3(kThreads), 0, s, a);
+    a.pairs = p.pairs, a.splits = p.splits;
+    const uint64_t wgs = p.splits >= kXcds ? uint64_t(ceil_div(p.splits, kXcds)) * kXcds * p.pairs  // whole XCD rounds
+                                           : uint64_t(p.splits) * p.pairs;
+    if (wgs > 0x7fffffffull) return fail(CRB_EINVAL_SHAPE, "%s: launch grid too large", what);
+    hipLaunchKernelGGL((wgrad3x3s1_kernel<Cfg>), dim3(u32(wgs)), dim3(kThreads), 0, s, a);
     if (int st = check_launch(what)) return st;
     if (p.splits > 1) {
         return launch_splitk_reduce(ws, dW, OC * IC * 9, p.splits, ReduceEpi{nullptr, 1, 1, EPI_ACCUM}, s, what);
