@@ -1,75 +1,105 @@
-// Direct 3x3 / stride 1 / pad 1 convolution for gfx950: forward and data gradient in one template.
+// Direct 3x3 / pad 1 convolution for gfx950, stride 1 or 2: forward and data gradient in one template.
 //
-// A workgroup (4 wave64) owns ROWS full image rows of one image and OCT output channels. The contraction
-// runs over input channels in chunks of CI: for each chunk the raw input rows (with their one-pixel halo,
-// zero outside the image) and the matching OCT x CI x 9 filter slice are staged in LDS, and every wave
-// feeds v_mfma_f32_16x16x4_f32 directly from them. Inside a chunk the contraction index is ordered tap-major
-// (k = tap*CI + channel), so MFMA step s covers one tap and four consecutive channels: the im2col gather is
-// a per-lane base address (pixel + (lane/16) channel planes) plus a compile-time immediate per step, and the
-// inner loop contains nothing but ds_read and MFMA. Fragments are read PF steps ahead of the MFMAs that
-// consume them (explicit software pipeline; the scheduler is fenced so it cannot undo it).
+// A workgroup (4 wave64) owns ROWS rows of a "pixel grid" of one image and OCT output channels. The grid is the
+// output image for the forward pass and for the stride-1 data gradient; for the stride-2 data gradient it is the
+// dY image, each of whose pixels yields a 2x2 block of dX. The contraction runs over input channels in chunks of CI:
+// for each chunk the raw input rows the tile needs (with their halo, zero outside the image) and the matching
+// OCT x CI x 9 filter slice are staged in LDS, and every wave feeds v_mfma_f32_16x16x4_f32 directly from them.
+// Inside a chunk the contraction index is ordered tap-major (k = tap*(CI+1) + channel), so an MFMA step covers one
+// tap and four consecutive channels: the im2col gather is a per-lane base address (pixel + (lane/16) channel planes)
+// plus a compile-time immediate per step, and the inner loop contains nothing but ds_read and MFMA. Fragments are
+// read PF steps ahead of the MFMAs that consume them (explicit software pipeline; the scheduler is fenced so it
+// cannot undo it).
 //
 // MFMA 16x16x4 f32 mapping (wave64, lane l): A value = A[i = l%16][k = l/16], B value = B[k = l/16][j = l%16],
-// accumulator register r = D[i = 4*(l/16) + r][j = l%16]. Here i = pixel within a 16-pixel block,
-// j = output channel within a 16-channel block, so a lane ends up with 4 consecutive pixels of one output
-// channel: one 16-byte store per MFMA tile, and bias / ReLU are per-lane scalars.
+// accumulator register r = D[i = 4*(l/16) + r][j = l%16]. Here i = pixel within a 16-pixel block of the grid,
+// j = output channel within a 16-channel block, so a lane ends up with 4 consecutive grid pixels of one output
+// channel: 16-byte stores, and bias / ReLU are per-lane scalars.
 //
-// The data gradient of a stride-1 pad-1 3x3 convolution is the same computation on dY with the filter's
-// channel roles swapped and its taps mirrored: DGRAD only changes how the filter slice is gathered into LDS
-// and the sign of the tap offsets.
+// Variants:
+//   forward, stride S: grid pixel (y, x) reads input (S*y + fh - 1, S*x + fw - 1).
+//   data gradient, stride 1: the same computation on dY with the filter's channel roles swapped and its taps
+//     mirrored: grid pixel (y, x) reads dY (y + 1 - fh, x + 1 - fw).
+//   data gradient, stride 2: dX (2y'+py, 2x'+px) only receives the taps with fh = 1 - py (mod 2), fw = 1 - px (mod 2):
+//     four interleaved sub-convolutions of dY with 1, 2, 2 and 4 taps. Each tap accumulates into the accumulator of
+//     its parity class, reading dY (y' + (fh == 0), x' + (fw == 0)); the structural zeros a zero-upsampled
+//     formulation would multiply are never touched. The two column parities held by a lane interleave into 8
+//     consecutive dX floats per row parity.
 #pragma once
 #include "igemm_engine.h"
 
 namespace crb {
 
-// NBUF_ = 2: double-buffered chunk pipeline (any C_IN). NBUF_ = 1: the whole contraction is one
-// chunk (C_IN <= CI), half the LDS, so more workgroups fit on a CU and overlap each other's staging.
-template <int W_, int ROWS_, int CI_, int OCT_, int PBW_, int OBW_, bool DGRAD_, int OCC_, int NBUF_ = 2>
+// NBUF_ = 2: double-buffered chunk pipeline (any C_IN). NBUF_ = 1: the whole contraction is one chunk (C_IN <= CI),
+// half the LDS, so more workgroups fit on a CU and overlap each other's staging.
+template <int W_, int ROWS_, int CI_, int OCT_, int PBW_, int OBW_, bool DGRAD_, int OCC_, int NBUF_ = 2, int S_ = 1>
 struct DirectCfg {
-    static constexpr int W = W_, ROWS = ROWS_, CI = CI_, OCT = OCT_, PBW = PBW_, OBW = OBW_, OCC = OCC_, NBUF = NBUF_;
+    static constexpr int W = W_, ROWS = ROWS_, CI = CI_, OCT = OCT_, PBW = PBW_, OBW = OBW_, OCC = OCC_, NBUF = NBUF_, S = S_;
     static constexpr bool DGRAD = DGRAD_;
-    static constexpr int TP = ROWS * W;          // pixels per workgroup tile
-    static constexpr int NPB = TP / 16;          // 16-pixel blocks
-    static constexpr int NOB = OCT / 16;         // 16-channel blocks
-    static constexpr int NPBW = NPB / PBW;       // wave groups along pixels
-    static constexpr int NOBW = NOB / OBW;       // wave groups along channels
-    static constexpr int XS = W + 8;             // LDS row stride: 3 pad, left halo, W interior (16-byte aligned), right halo, 3 pad
-    static constexpr int XR = ROWS + 2;          // rows incl. halo
+    static constexpr bool DG2 = DGRAD && S == 2;  // stride-2 data gradient (4 parity classes)
+    static constexpr bool FW2 = !DGRAD && S == 2; // stride-2 forward
+    static constexpr int NPH = DG2 ? 4 : 1;       // accumulator sets per MFMA tile
+    static constexpr int TP = ROWS * W;           // grid pixels per workgroup tile
+    static constexpr int NPB = TP / 16;           // 16-pixel blocks
+    static constexpr int NOB = OCT / 16;          // 16-channel blocks
+    static constexpr int NPBW = NPB / PBW;        // wave groups along pixels
+    static constexpr int NOBW = NOB / OBW;        // wave groups along channels
+    // staged input: row width, row count, the input row LDS row 0 holds (ROW0_MUL*r0 + ROW0_ADD for first grid row r0)
+    static constexpr int SW = FW2 ? 2 * W : W;
+    static constexpr int XR = DG2 ? ROWS + 1 : S * (ROWS - 1) + 3;
+    static constexpr int ROW0_MUL = FW2 ? 2 : 1;
+    static constexpr int ROW0_ADD = DG2 ? 0 : -1;
+    static constexpr int PSTEP = FW2 ? 2 : 1;     // LDS distance of neighbouring grid pixels
+    static constexpr int XS = SW + 8;  // LDS row stride: 3 pad, left halo, SW interior (16-byte aligned), right halo, 3 pad
     // channel plane stride (floats): the four lane groups (lane/16) of a fragment read sit one plane apart;
     // 16 mod 32 (8 mod 32 for the 2-row blocks of W = 8) puts them on disjoint LDS banks. Multiple of 4.
     static constexpr int XP_MIN = XR * XS;
     static constexpr int XP_RES = W == 8 ? 8 : 16;
     static constexpr int XP = XP_MIN + ((XP_RES - XP_MIN % 32) + 32) % 32;
-    static constexpr int KC = CI * 9;            // contraction length per chunk
-    static constexpr int NSTEP = KC / 4;         // MFMA steps per chunk
-    static constexpr int CQ = CI / 4;            // steps per tap
-    static constexpr int PF = (8 / (PBW * OBW)) < 1 ? 1 : ((8 / (PBW * OBW)) > 4 ? 4 : (8 / (PBW * OBW)));  // read-ahead
-    static constexpr int CIP = CI + 1;           // k index of (tap, channel) in a filter row is tap*CIP + channel: odd tap stride
-    static constexpr int WSTR_MIN = 9 * CIP;     // filter row stride == 2 mod 4: the 32 lanes of a half-wave (16 rows x 2 k) hit distinct banks
+    static constexpr int NSTEP = CI * 9 / 4;      // MFMA steps per chunk
+    static constexpr int CQ = CI / 4;             // steps per tap
+    static constexpr int MPS = PBW * OBW;         // MFMAs per step
+    static constexpr int PF = (8 / MPS) < 1 ? 1 : ((8 / MPS) > 4 ? 4 : (8 / MPS));  // read-ahead (steps)
+    static constexpr int CIP = CI + 1;            // k index of (tap, channel) in a filter row is tap*CIP + channel: odd tap stride
+    static constexpr int WSTR_MIN = 9 * CIP;      // filter row stride == 2 mod 4: the 32 lanes of a half-wave (16 rows x 2 k) hit distinct banks
     static constexpr int WSTR = WSTR_MIN + ((2 - WSTR_MIN % 4) + 4) % 4;
     static constexpr int X_SIZE = CI * XP;
     static constexpr int W_SIZE = OCT * WSTR;
-    static_assert(W == 8 || W == 16 || W == 32, "image width");
+    static_assert(W == 8 || W == 16 || W == 32, "grid width");
+    static_assert(S == 1 || S == 2, "stride");
     static_assert(TP % 16 == 0 && NPB % PBW == 0 && NOB % OBW == 0 && NPBW * NOBW == 4, "wave tiling must use 4 waves");
     static_assert((PBW * 16) % W == 0 || PBW == 1, "a wave's pixel blocks must start on a row boundary");
     static_assert(CI % 4 == 0, "chunk channel count");
+
+    // LDS offset of tap (fh, fw) relative to the lane's pixel base (which points one float left of the pixel)
+    static constexpr int tap_off(int tap) {
+        const int fh = tap / 3, fw = tap % 3;
+        if (DG2) return (fh == 0 ? 1 : 0) * XS + (fw == 0 ? 1 : 0) + 1;
+        if (DGRAD) return (2 - fh) * XS + (2 - fw);
+        return fh * XS + fw;
+    }
+    // parity class 2*py + px of dX that tap (fh, fw) contributes to (stride-2 data gradient), else 0
+    static constexpr int tap_phase(int tap) { return DG2 ? (tap / 3 == 1 ? 0 : 2) + (tap % 3 == 1 ? 0 : 1) : 0; }
+    static constexpr int pix_off(int q) { return (q / W) * PSTEP * XS + (q % W) * PSTEP; }
 };
 
 struct DirectArgs {
     const float *Wt;    // filters, OC x IC x 3 x 3 of the forward convolution
-    const float *X;     // input of this pass  (forward: X, dgrad: dY), N x C_IN x H x W
-    float *Y;           // output of this pass (forward: Y, dgrad: dX), N x C_OUT x H x W
+    const float *X;     // input of this pass  (forward: X, dgrad: dY), N x C_IN x in_H x SW
+    float *Y;           // output of this pass (forward: Y, dgrad: dX), N x C_OUT x (grid_H x W, or twice that for stride-2 dgrad)
     const float *bias;  // per output channel or nullptr
-    u32 C_IN, C_OUT, H;
+    u32 C_IN, C_OUT;
+    u32 in_H;           // rows of the staged tensor
+    u32 grid_H;         // rows of the pixel grid
     u32 tiles_per_img, oc_tiles, tiles_total;  // tiles_total = N * tiles_per_img
     u32 relu;
 };
 
 template <class Cfg>
-__global__ void __launch_bounds__(kThreads, Cfg::OCC) conv3x3s1_kernel(DirectArgs a) {
+__global__ void __launch_bounds__(kThreads, Cfg::OCC) conv3x3_kernel(DirectArgs a) {
     constexpr int W = Cfg::W, ROWS = Cfg::ROWS, CI = Cfg::CI, OCT = Cfg::OCT, PBW = Cfg::PBW, OBW = Cfg::OBW;
-    constexpr int XS = Cfg::XS, XR = Cfg::XR, XP = Cfg::XP, NSTEP = Cfg::NSTEP, WSTR = Cfg::WSTR;
-    constexpr int NBUF = Cfg::NBUF;
+    constexpr int XS = Cfg::XS, XR = Cfg::XR, XP = Cfg::XP, NSTEP = Cfg::NSTEP, WSTR = Cfg::WSTR, SW = Cfg::SW;
+    constexpr int NBUF = Cfg::NBUF, NPH = Cfg::NPH;
     __shared__ __attribute__((aligned(16))) float sX[NBUF][Cfg::X_SIZE];
     __shared__ __attribute__((aligned(16))) float sW[NBUF][Cfg::W_SIZE];
 
@@ -82,13 +112,14 @@ __global__ void __launch_bounds__(kThreads, Cfg::OCC) conv3x3s1_kernel(DirectArg
     if (rest >= a.tiles_total) return;
     const u32 tile = rest % a.tiles_per_img;
     const u32 n = rest / a.tiles_per_img;
-    const int r0 = int(tile) * ROWS;  // first output row of this tile
+    const int r0 = int(tile) * ROWS;  // first grid row of this tile
+    const int srow0 = Cfg::ROW0_MUL * r0 + Cfg::ROW0_ADD;  // input row held by LDS row 0
     const u32 oc0 = oct * OCT;
-    const u32 HW = a.H * W;
+    const u32 in_HW = a.in_H * SW;
 
     // ---- staging helpers ----------------------------------------------------------------------------
-    // input rows: CI planes x XR rows x W/4 quads
-    constexpr int XQ = CI * XR * (W / 4);
+    // input rows: CI planes x XR rows x SW/4 quads
+    constexpr int XQ = CI * XR * (SW / 4);
     constexpr int XNP = (XQ + kThreads - 1) / kThreads;
     // filter slice: one (filter row j, chunk channel c) pair per item, 9 contiguous taps each
     constexpr int WQ = OCT * CI;
@@ -102,10 +133,10 @@ __global__ void __launch_bounds__(kThreads, Cfg::OCC) conv3x3s1_kernel(DirectArg
             const u32 e = t + i * kThreads;
             v4f v = {0.f, 0.f, 0.f, 0.f};
             if (XQ % kThreads == 0 || e < XQ) {
-                const u32 q = e % (W / 4), lr = (e / (W / 4)) % XR, c = e / ((W / 4) * XR);
-                const int row = r0 - 1 + int(lr);
-                if (row >= 0 && row < int(a.H) && c0 + c < a.C_IN)
-                    v = *reinterpret_cast<const v4f *>(a.X + (size_t(n) * a.C_IN + c0 + c) * HW + u32(row) * W + 4 * q);
+                const u32 q = e % (SW / 4), lr = (e / (SW / 4)) % XR, c = e / ((SW / 4) * XR);
+                const int row = srow0 + int(lr);
+                if (row >= 0 && row < int(a.in_H) && c0 + c < a.C_IN)
+                    v = *reinterpret_cast<const v4f *>(a.X + (size_t(n) * a.C_IN + c0 + c) * in_HW + u32(row) * SW + 4 * q);
             }
             xreg[i] = v;
         }
@@ -134,7 +165,7 @@ __global__ void __launch_bounds__(kThreads, Cfg::OCC) conv3x3s1_kernel(DirectArg
         for (int i = 0; i < XNP; ++i) {
             const u32 e = t + i * kThreads;
             if (XQ % kThreads == 0 || e < XQ) {
-                const u32 q = e % (W / 4), lr = (e / (W / 4)) % XR, c = e / ((W / 4) * XR);
+                const u32 q = e % (SW / 4), lr = (e / (SW / 4)) % XR, c = e / ((SW / 4) * XR);
                 *reinterpret_cast<v4f *>(dX + c * XP + lr * XS + 4 + 4 * q) = xreg[i];
             }
         }
@@ -153,23 +184,25 @@ __global__ void __launch_bounds__(kThreads, Cfg::OCC) conv3x3s1_kernel(DirectArg
     for (u32 e = t; e < u32(NBUF) * CI * XR; e += kThreads) {
         float *row = &sX[0][0] + (e / (CI * XR)) * Cfg::X_SIZE + ((e % (CI * XR)) / XR) * XP + (e % XR) * XS;
         row[3] = 0.f;
-        row[W + 4] = 0.f;
+        row[SW + 4] = 0.f;
     }
 
     // ---- per-lane fragment addressing ---------------------------------------------------------------------
     const int lane = t & 63, wave = t >> 6;
     const int wp = wave % Cfg::NPBW, wo = wave / Cfg::NPBW;
     const int li = lane & 15, kq = lane >> 4;
-    // pixel of this lane in the wave's first block; lane group kq reads channel plane kq of each 4-channel step
+    // grid pixel of this lane in the wave's first block; lane group kq reads channel plane kq of each 4-channel step
     const int q0 = (wp * PBW) * 16 + li;
-    const int xbase = kq * XP + (q0 / W) * XS + (q0 % W) + 3;
+    const int xbase = kq * XP + Cfg::pix_off(q0) + 3;
     const int wbase = (wo * OBW * 16 + li) * WSTR + kq;
 
-    v4f acc[PBW][OBW];
+    v4f acc[NPH][PBW][OBW];
 #pragma unroll
-    for (int p = 0; p < PBW; ++p)
+    for (int ph = 0; ph < NPH; ++ph)
 #pragma unroll
-        for (int o = 0; o < OBW; ++o) acc[p][o] = v4f{0.f, 0.f, 0.f, 0.f};
+        for (int p = 0; p < PBW; ++p)
+#pragma unroll
+            for (int o = 0; o < OBW; ++o) acc[ph][p][o] = v4f{0.f, 0.f, 0.f, 0.f};
 
     constexpr int PF = Cfg::PF, CQ = Cfg::CQ;
     auto compute = [&](const float *cx, const float *cw) {
@@ -177,10 +210,9 @@ __global__ void __launch_bounds__(kThreads, Cfg::OCC) conv3x3s1_kernel(DirectArg
         float av[PF + 1][PBW], bv[PF + 1][OBW];
         auto read_step = [&](int s, int slot) {
             const int tap = s / CQ, cq = s % CQ;
-            const int fh = Cfg::DGRAD ? 2 - tap / 3 : tap / 3, fw = Cfg::DGRAD ? 2 - tap % 3 : tap % 3;
-            const int xo = cq * 4 * XP + fh * XS + fw;
+            const int xo = cq * 4 * XP + Cfg::tap_off(tap);
 #pragma unroll
-            for (int p = 0; p < PBW; ++p) av[slot][p] = px[xo + ((p * 16) / W) * XS + (p * 16) % W];
+            for (int p = 0; p < PBW; ++p) av[slot][p] = px[xo + Cfg::pix_off(p * 16)];
 #pragma unroll
             for (int o = 0; o < OBW; ++o) bv[slot][o] = pw[o * 16 * WSTR + tap * Cfg::CIP + 4 * cq];
         };
@@ -190,11 +222,12 @@ __global__ void __launch_bounds__(kThreads, Cfg::OCC) conv3x3s1_kernel(DirectArg
         for (int s = 0; s < NSTEP; ++s) {
             if (s + PF < NSTEP) read_step(s + PF, (s + PF) % (PF + 1));
             __builtin_amdgcn_sched_barrier(0);
+            const int ph = Cfg::tap_phase(s / CQ);
 #pragma unroll
             for (int p = 0; p < PBW; ++p)
 #pragma unroll
                 for (int o = 0; o < OBW; ++o)
-                    acc[p][o] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[s % (PF + 1)][p], bv[s % (PF + 1)][o], acc[p][o], 0, 0, 0);
+                    acc[ph][p][o] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[s % (PF + 1)][p], bv[s % (PF + 1)][o], acc[ph][p][o], 0, 0, 0);
             __builtin_amdgcn_sched_barrier(0);
         }
     };
@@ -221,7 +254,7 @@ __global__ void __launch_bounds__(kThreads, Cfg::OCC) conv3x3s1_kernel(DirectArg
         }
     }
 
-    // ---- epilogue: lane holds 4 consecutive pixels of one output channel per tile ---------------------------
+    // ---- epilogue: a lane holds 4 consecutive grid pixels of one output channel per tile ----------------------
 #pragma unroll
     for (int o = 0; o < OBW; ++o) {
         const u32 oc = oc0 + (wo * OBW + o) * 16 + li;
@@ -230,38 +263,50 @@ __global__ void __launch_bounds__(kThreads, Cfg::OCC) conv3x3s1_kernel(DirectArg
 #pragma unroll
         for (int p = 0; p < PBW; ++p) {
             const int q = (wp * PBW + p) * 16 + 4 * kq;
-            v4f v = acc[p][o];
-            v.x += b, v.y += b, v.z += b, v.w += b;
-            if (a.relu) {
-                v.x = v.x > 0.f ? v.x : 0.f, v.y = v.y > 0.f ? v.y : 0.f;
-                v.z = v.z > 0.f ? v.z : 0.f, v.w = v.w > 0.f ? v.w : 0.f;
+            const u32 gy = u32(r0 + q / W), gx = u32(q % W);
+            if constexpr (Cfg::DG2) {
+                // grid pixel (gy, gx..gx+3) -> dX rows 2gy, 2gy+1, columns 2gx .. 2gx+7 (column parities interleaved)
+                float *base = a.Y + ((size_t(n) * a.C_OUT + oc) * (2 * a.grid_H) + 2 * gy) * (2 * W) + 2 * gx;
+#pragma unroll
+                for (int py = 0; py < 2; ++py) {
+                    const v4f e = acc[2 * py][p][o], d = acc[2 * py + 1][p][o];  // px = 0, px = 1
+                    *reinterpret_cast<v4f *>(base + py * 2 * W) = v4f{e.x, d.x, e.y, d.y};
+                    *reinterpret_cast<v4f *>(base + py * 2 * W + 4) = v4f{e.z, d.z, e.w, d.w};
+                }
+            } else {
+                v4f v = acc[0][p][o];
+                v.x += b, v.y += b, v.z += b, v.w += b;
+                if (a.relu) {
+                    v.x = v.x > 0.f ? v.x : 0.f, v.y = v.y > 0.f ? v.y : 0.f;
+                    v.z = v.z > 0.f ? v.z : 0.f, v.w = v.w > 0.f ? v.w : 0.f;
+                }
+                *reinterpret_cast<v4f *>(a.Y + ((size_t(n) * a.C_OUT + oc) * a.grid_H + gy) * W + gx) = v;
             }
-            *reinterpret_cast<v4f *>(a.Y + (size_t(n) * a.C_OUT + oc) * HW + u32(r0 + q / W) * W + (q % W)) = v;
         }
     }
 }
 
+// Shape gate of one configuration. Channel counts need not divide CI / OCT: ragged chunks and tiles are zero-filled.
+// (grid_H, grid_W) = extent of the pixel grid: the output image, or dY for the stride-2 data gradient.
 template <class Cfg>
-inline int launch_direct(const float *Wt, const float *X, float *Y, const float *bias, u32 N, u32 C_IN, u32 C_OUT, u32 H,
-                         u32 relu, hipStream_t s, const char *what) {
-    DirectArgs a;
-    a.Wt = Wt, a.X = X, a.Y = Y, a.bias = bias;
-    a.C_IN = C_IN, a.C_OUT = C_OUT, a.H = H;
-    a.tiles_per_img = H / Cfg::ROWS;
-    a.oc_tiles = ceil_div(C_OUT, u32(Cfg::OCT));
-    a.relu = relu;
-    a.tiles_total = N * a.tiles_per_img;
-    const uint64_t wgs = uint64_t(ceil_div(a.tiles_total, kXcds)) * kXcds * a.oc_tiles;  // padded to whole XCD rounds
-    if (wgs > 0x7fffffffull) return fail(CRB_EINVAL_SHAPE, "%s: launch grid too large", what);
-    hipLaunchKernelGGL((conv3x3s1_kernel<Cfg>), dim3(u32(wgs)), dim3(kThreads), 0, s, a);
-    return check_launch(what);
+inline bool direct_fits(u32 C_IN, u32 grid_H, u32 grid_W) {
+    return grid_W == u32(Cfg::W) && grid_H % Cfg::ROWS == 0 && (Cfg::NBUF == 1 ? C_IN <= u32(Cfg::CI) : true);
 }
 
-// Shape gate of one configuration. Channel counts need not divide CI / OCT: ragged chunks and tiles are zero-filled.
 template <class Cfg>
-inline bool direct_fits(u32 C_IN, u32 C_OUT, u32 H, u32 Wd) {
-    (void)C_OUT;
-    return Wd == u32(Cfg::W) && H % Cfg::ROWS == 0 && (Cfg::NBUF == 1 ? C_IN <= u32(Cfg::CI) : true);
+inline int launch_direct(const float *Wt, const float *X, float *Y, const float *bias, u32 N, u32 C_IN, u32 C_OUT, u32 grid_H,
+                         u32 in_H, u32 relu, hipStream_t s, const char *what) {
+    DirectArgs a;
+    a.Wt = Wt, a.X = X, a.Y = Y, a.bias = bias;
+    a.C_IN = C_IN, a.C_OUT = C_OUT, a.grid_H = grid_H, a.in_H = in_H;
+    a.tiles_per_img = grid_H / Cfg::ROWS;
+    a.oc_tiles = ceil_div(C_OUT, u32(Cfg::OCT));
+    a.tiles_total = N * a.tiles_per_img;
+    a.relu = relu;
+    const uint64_t wgs = uint64_t(ceil_div(a.tiles_total, kXcds)) * kXcds * a.oc_tiles;  // padded to whole XCD rounds
+    if (wgs > 0x7fffffffull) return fail(CRB_EINVAL_SHAPE, "%s: launch grid too large", what);
+    hipLaunchKernelGGL((conv3x3_kernel<Cfg>), dim3(u32(wgs)), dim3(kThreads), 0, s, a);
+    return check_launch(what);
 }
 
 }  // namespace crb

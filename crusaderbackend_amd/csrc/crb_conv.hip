@@ -99,36 +99,53 @@ static WgradPlan wgrad_plan(const crb_conv_geom *g) {
     return p;
 }
 
-// ---- direct 3x3 / stride 1 / pad 1 path -------------------------------------------------------------------
-// Configurations <W, ROWS, CI, OCT, PBW, OBW, DGRAD, OCC, NBUF>, picked by image width and channel counts.
-// Tried in order; the first whose divisibility constraints hold is used, otherwise the implicit-GEMM engine runs.
-template <bool DG>
-static int try_direct(const float *Wt, const float *X, float *Y, const float *bias, u32 N, u32 C_IN, u32 C_OUT, u32 H,
-                      u32 Wd, u32 relu, hipStream_t s, const char *what, bool &done) {
+// ---- direct 3x3 / pad 1 path (stride 1 and 2) ----------------------------------------------------------------
+// Configurations <W, ROWS, CI, OCT, PBW, OBW, DGRAD, OCC, NBUF, S>, picked by grid width and channel counts.
+// Tried in order; the first whose constraints hold is used, otherwise the implicit-GEMM engine runs.
+// (gH, gW) is the pixel grid: the output image, or dY for the stride-2 data gradient; in_H the rows of the staged tensor.
+template <bool DG, int S>
+static int try_direct(const float *Wt, const float *X, float *Y, const float *bias, u32 N, u32 C_IN, u32 C_OUT, u32 gH,
+                      u32 gW, u32 in_H, u32 relu, hipStream_t s, const char *what, bool &done) {
     done = true;
-#define CRB_TRY(...)                                                                                         \
-    if (direct_fits<DirectCfg<__VA_ARGS__>>(C_IN, C_OUT, H, Wd))                                              \
-        return launch_direct<DirectCfg<__VA_ARGS__>>(Wt, X, Y, bias, N, C_IN, C_OUT, H, relu, s, what);
-    // output-channel tile: the smallest of 16 / 32 / 64 that covers C_OUT, 64 beyond; chunk of 16 input channels
-    // unless C_IN <= 8
-    if (Wd == 32) {
-        if (C_IN <= 16 && C_IN > 8 && C_OUT <= 16) { CRB_TRY(32, 8, 16, 16, 4, 1, DG, 2, 1) }  // one LDS-resident chunk
-        if (C_OUT > 32) { CRB_TRY(32, 8, 8, 64, 4, 4, DG, 2, 2) }
-        if (C_OUT > 16) { CRB_TRY(32, 8, 8, 32, 4, 2, DG, 2, 2) }
-        CRB_TRY(32, 8, 8, 16, 4, 1, DG, 2, 2)
-        CRB_TRY(32, 4, 8, 16, 2, 1, DG, 2, 2)
-    } else if (Wd == 16) {
-        if (C_OUT > 64) { CRB_TRY(16, 8, 8, 64, 2, 4, DG, 2, 2) }
-        if (C_OUT > 16 && C_IN > 8) { CRB_TRY(16, 4, 16, 32, 1, 2, DG, 2, 2) }
-        if (C_OUT > 16) { CRB_TRY(16, 4, 8, 32, 1, 2, DG, 2, 2) }
-        CRB_TRY(16, 8, 8, 16, 2, 1, DG, 2, 2)
-        CRB_TRY(16, 4, 8, 16, 1, 1, DG, 2, 2)
-    } else if (Wd == 8) {
-        if (C_OUT > 128 && C_IN > 8) { CRB_TRY(8, 8, 16, 64, 1, 4, DG, 2, 2) }
-        if (C_OUT > 64 && C_IN > 8) { CRB_TRY(8, 8, 16, 32, 1, 2, DG, 2, 2) }
-        if (C_IN > 8) { CRB_TRY(8, 8, 16, 16, 1, 1, DG, 2, 2) }
-        CRB_TRY(8, 8, 8, 16, 1, 1, DG, 2, 2)
-        CRB_TRY(8, 4, 8, 32, 1, 1, DG, 2, 2)
+#define CRB_TRY(...)                                                                                          \
+    if (direct_fits<DirectCfg<__VA_ARGS__>>(C_IN, gH, gW))                                                     \
+        return launch_direct<DirectCfg<__VA_ARGS__>>(Wt, X, Y, bias, N, C_IN, C_OUT, gH, in_H, relu, s, what);
+    // output-channel tile: the smallest of 16 / 32 / 64 that covers C_OUT, 64 beyond; chunks of 16 input channels at
+    // stride 1 when C_IN > 8, chunks of 8 otherwise (stride 2 stages wider / more rows per chunk)
+    if constexpr (S == 1) {
+        if (gW == 32) {
+            if (C_IN <= 16 && C_IN > 8 && C_OUT <= 16) { CRB_TRY(32, 8, 16, 16, 4, 1, DG, 2, 1, 1) }  // one LDS-resident chunk
+            if (C_OUT > 32) { CRB_TRY(32, 8, 8, 64, 4, 4, DG, 2, 2, 1) }
+            if (C_OUT > 16) { CRB_TRY(32, 8, 8, 32, 4, 2, DG, 2, 2, 1) }
+            CRB_TRY(32, 8, 8, 16, 4, 1, DG, 2, 2, 1)
+            CRB_TRY(32, 4, 8, 16, 2, 1, DG, 2, 2, 1)
+        } else if (gW == 16) {
+            if (C_OUT > 64) { CRB_TRY(16, 8, 8, 64, 2, 4, DG, 2, 2, 1) }
+            if (C_OUT > 16 && C_IN > 8) { CRB_TRY(16, 4, 16, 32, 1, 2, DG, 2, 2, 1) }
+            if (C_OUT > 16) { CRB_TRY(16, 4, 8, 32, 1, 2, DG, 2, 2, 1) }
+            CRB_TRY(16, 8, 8, 16, 2, 1, DG, 2, 2, 1)
+            CRB_TRY(16, 4, 8, 16, 1, 1, DG, 2, 2, 1)
+        } else if (gW == 8) {
+            if (C_OUT > 128 && C_IN > 8) { CRB_TRY(8, 8, 16, 64, 1, 4, DG, 2, 2, 1) }
+            if (C_OUT > 64 && C_IN > 8) { CRB_TRY(8, 8, 16, 32, 1, 2, DG, 2, 2, 1) }
+            if (C_IN > 8) { CRB_TRY(8, 8, 16, 16, 1, 1, DG, 2, 2, 1) }
+            CRB_TRY(8, 8, 8, 16, 1, 1, DG, 2, 2, 1)
+            CRB_TRY(8, 4, 8, 32, 1, 1, DG, 2, 2, 1)
+        }
+    } else {
+        if (gW == 32) {
+            if (C_OUT > 16) { CRB_TRY(32, 8, 8, 32, 4, 2, DG, 2, 2, 2) }
+            CRB_TRY(32, 8, 8, 16, 4, 1, DG, 2, 2, 2)
+            CRB_TRY(32, 4, 8, 16, 2, 1, DG, 2, 2, 2)
+        } else if (gW == 16) {
+            if (C_OUT > 16) { CRB_TRY(16, 8, 8, 32, 2, 2, DG, 2, 2, 2) }
+            CRB_TRY(16, 8, 8, 16, 2, 1, DG, 2, 2, 2)
+            CRB_TRY(16, 4, 8, 16, 1, 1, DG, 2, 2, 2)
+        } else if (gW == 8) {
+            if (C_OUT > 16) { CRB_TRY(8, 8, 8, 32, 1, 2, DG, 2, 2, 2) }
+            CRB_TRY(8, 8, 8, 16, 1, 1, DG, 2, 2, 2)
+            CRB_TRY(8, 4, 8, 32, 1, 1, DG, 2, 2, 2)
+        }
     }
 #undef CRB_TRY
     done = false;
@@ -141,9 +158,10 @@ static bool pointwise_shape(const crb_conv_geom *g) {
     return g->FH == 1 && g->FW == 1 && g->sH == 1 && g->sW == 1 && g->pH == 0 && g->pW == 0;
 }
 
-static bool direct_shape(const crb_conv_geom *g) {
-    return g->FH == 3 && g->FW == 3 && g->sH == 1 && g->sW == 1 && g->pH == 1 && g->pW == 1 && g->IH == g->OH &&
-           g->IW == g->OW;
+// 3x3, pad 1, stride 1 (output = input extent) or stride 2 with even input extents (output = half)
+static bool direct_shape(const crb_conv_geom *g, u32 stride) {
+    return g->FH == 3 && g->FW == 3 && g->sH == stride && g->sW == stride && g->pH == 1 && g->pW == 1 &&
+           g->IH == stride * g->OH && g->IW == stride * g->OW;
 }
 
 // ---- direct 3x3 / stride 1 / pad 1 weight gradient ---------------------------------------------------------
@@ -161,7 +179,7 @@ static bool wgrad_cfg(const crb_conv_geom *g, bool run, const float *dY, const f
 
 static bool wgrad_direct(const crb_conv_geom *g, bool run, const float *dY, const float *X, float *dW, float *ws,
                          hipStream_t s, WgradDirectPlan &plan, int &status) {
-    if (!direct_shape(g)) return false;
+    if (!direct_shape(g, 1)) return false;
     if (g->IW == 32) return wgrad_cfg<WgradCfg<32, 8, 1, 2>>(g, run, dY, X, dW, ws, s, plan, status);
     if (g->IW == 16)
         return wgrad_cfg<WgradCfg<16, 16, 1, 2>>(g, run, dY, X, dW, ws, s, plan, status) ||
@@ -217,10 +235,12 @@ int crb_conv_fwd(const float *W, const float *X, float *Y, const float *bias_or_
     if (pointwise_shape(g))
         return gemm_nn_rowbias(W, X, Y, g->OC, g->IH * g->IW, g->IC, g->N, bias_or_null,
                                (flags & CRB_FLAG_RELU) ? u32(EPI_RELU) : 0u, s, "crb_conv_fwd");
-    if (direct_shape(g) && aligned16(X) && aligned16(Y)) {
+    if (aligned16(X) && aligned16(Y) && (direct_shape(g, 1) || direct_shape(g, 2))) {
         bool done;
-        int st = try_direct<false>(W, X, Y, bias_or_null, g->N, g->IC, g->OC, g->IH, g->IW, flags & CRB_FLAG_RELU, s,
-                                   "crb_conv_fwd", done);
+        int st = g->sH == 1 ? try_direct<false, 1>(W, X, Y, bias_or_null, g->N, g->IC, g->OC, g->OH, g->OW, g->IH,
+                                                   flags & CRB_FLAG_RELU, s, "crb_conv_fwd", done)
+                            : try_direct<false, 2>(W, X, Y, bias_or_null, g->N, g->IC, g->OC, g->OH, g->OW, g->IH,
+                                                   flags & CRB_FLAG_RELU, s, "crb_conv_fwd", done);
         if (done) return st;
     }
     if (K % 4 == 0 && aligned16(W)) {
@@ -236,10 +256,13 @@ int crb_conv_dgrad(const float *W, const float *dY, float *dX, const crb_conv_ge
     if (int st = check_geom("crb_conv_dgrad", g)) return st;
     if (pointwise_shape(g))
         return gemm_tn_batched(W, dY, dX, g->IC, g->IH * g->IW, g->OC, g->N, hipStream_t(stream), "crb_conv_dgrad");
-    if (direct_shape(g) && aligned16(dY) && aligned16(dX)) {
+    if (aligned16(dY) && aligned16(dX) && (direct_shape(g, 1) || direct_shape(g, 2))) {
         bool done;
-        int st = try_direct<true>(W, dY, dX, nullptr, g->N, g->OC, g->IC, g->IH, g->IW, 0, hipStream_t(stream),
-                                  "crb_conv_dgrad", done);
+        // the pixel grid and the staged tensor are dY in both cases (at stride 1 dY and dX have the same extent)
+        int st = g->sH == 1 ? try_direct<true, 1>(W, dY, dX, nullptr, g->N, g->OC, g->IC, g->OH, g->OW, g->OH, 0,
+                                                  hipStream_t(stream), "crb_conv_dgrad", done)
+                            : try_direct<true, 2>(W, dY, dX, nullptr, g->N, g->OC, g->IC, g->OH, g->OW, g->OH, 0,
+                                                  hipStream_t(stream), "crb_conv_dgrad", done);
         if (done) return st;
     }
     const u32 FHW = g->FH * g->FW;

@@ -239,3 +239,16 @@ def test_conv_relu_flag(dev):
         Y = _nan(dev, N, OC, H, H)
         capi.conv_fwd(to_dev(W, dev), to_dev(X, dev), Y, to_dev(b, dev), g, flags=capi.CRB_FLAG_RELU)
         assert_close(to_np(Y), np.maximum(orc.conv(W, X, b, 1, 1, 1, 1), 0), IC * 9, "conv+bias+relu")
+
+
+# 3x3 / stride 2 / pad 1 with even input extents: direct forward (input stride 2) and direct data gradient (parity classes).
+# (N, IC, IH, IW, OC); output is IH/2 x IW/2. Widths 64/32/16 hit the grid widths 32/16/8; the others fall back.
+STRIDE2 = [
+    (3, 16, 32, 32, 32), (2, 32, 16, 16, 64), (2, 8, 64, 64, 16), (2, 24, 32, 32, 48), (2, 5, 16, 16, 7), (2, 16, 16, 32, 20),
+    (2, 3, 32, 32, 16), (4, 40, 16, 16, 33), (2, 16, 8, 16, 16), (2, 6, 24, 16, 9), (2, 4, 12, 12, 5), (2, 4, 16, 8, 5),
+]
+
+
+@pytest.mark.parametrize("N,IC,IH,IW,OC", STRIDE2)
+def test_conv3x3_stride2_direct(dev, N, IC, IH, IW, OC):
+    run_layer(dev, N, IC, IH, IW, OC, 3, 3, 2, 2, 1, 1, bias=True, seed=21)
