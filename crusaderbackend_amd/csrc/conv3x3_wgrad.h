@@ -1,4 +1,4 @@
-// Weight gradient of a 3x3 / stride 1 / pad 1 convolution for gfx950.
+// Weight gradient of a 3x3 / pad 1 convolution (stride 1 or 2) for gfx950.
 //
 // dW[oc][ic][fh][fw] = sum over (n, y, x) of dY[n][oc][y][x] * X[n][ic][y+fh-1][x+fw-1]: for each of the 9 taps a
 // (OC x IC) matrix product whose contraction index is the pixel. A workgroup owns ONE 16x16 (oc-block, ic-block)
@@ -9,6 +9,11 @@
 // the shift causes at the left/right image border is removed by zeroing the dY value of the lanes that sit on
 // column 0 (taps fw = 0) or column W-1 (taps fw = 2) — a select on one step in W/4, decided at compile time.
 //
+// Stride 2 (even input extents): X is staged de-interleaved into its four (row parity, column parity) planes, each the
+// size of dY plus one halo row above. Input (2oh + fh - 1, 2ow + fw - 1) then lives in plane (fh != 1, fw != 1) at
+// (oh - (fh == 0), ow - (fw == 0)): again a constant shift of the flat dY run, so the inner loop is unchanged. Only
+// the fw = 0 taps can wrap (at ow = 0) and need the select.
+//
 // v_mfma_f32_16x16x4_f32 mapping (wave64, lane l): A = dY[oc = l%16][k' = 4s + l/16], B = X[k'][ic = l%16],
 // accumulator register r = dW[oc = 4*(l/16) + r][ic = l%16]; 9 accumulator tiles (one per tap) per wave.
 // The 4 waves take different rows (or images) of the tile; their accumulators are summed through LDS in fixed
@@ -18,15 +23,19 @@
 
 namespace crb {
 
-template <int W_, int TR_, int TI_, int OCC_>
+// W_: dY width; TR_: dY rows per image per tile; TI_: images per tile; S_: stride.
+template <int W_, int TR_, int TI_, int OCC_, int S_ = 1>
 struct WgradCfg {
-    static constexpr int W = W_, TR = TR_, TI = TI_, OCC = OCC_;
+    static constexpr int W = W_, TR = TR_, TI = TI_, OCC = OCC_, S = S_;
     static constexpr int WPI = 4 / TI;         // waves per image of the tile
     static constexpr int RW = TR / WPI;        // rows per wave
     static constexpr int KW = RW * W;          // pixels per wave per tile
     static constexpr int NSTEP = KW / 4;       // MFMA steps per wave per tile
     static constexpr int YIMG = TR * W;        // dY floats per image per plane
-    static constexpr int XIMG = (TR + 2) * W;  // X floats per image per plane (halo rows included)
+    static constexpr int PL = (TR + 1) * W;    // stride 2: one parity plane (halo row above + TR rows)
+    static constexpr int XIMG = S == 1 ? (TR + 2) * W : 4 * PL;  // X floats per image per channel (halo rows included)
+    static constexpr int XROWS = S == 1 ? TR + 2 : 2 * (TR + 1);  // input rows staged per image
+    static constexpr int XRW = S * W;                             // input row width
     // plane strides == 2 mod 4 (and even): 16 planes x 2 lane groups of a half-wave land on 32 distinct banks
     static constexpr int YP = TI * YIMG + 2;
     static constexpr int XP = TI * XIMG + 8 + 2;  // 4 leading + 4 trailing pad floats (kept zero)
@@ -36,11 +45,18 @@ struct WgradCfg {
     static constexpr int SMEM = 2 * BUF > RED_SIZE ? 2 * BUF : RED_SIZE;
     static_assert(TI == 1 || TI == 2 || TI == 4, "images per tile");
     static_assert(TR % WPI == 0 && KW % 4 == 0, "rows must split evenly over the waves");
+    static_assert(S == 1 || S == 2, "stride");
+    // LDS offset of tap (fh, fw) relative to the lane's X base (which already carries the 4 leading pad floats)
+    static constexpr int tap_off(int tap) {
+        const int fh = tap / 3, fw = tap % 3;
+        if (S == 1) return fh * W + fw - 1;
+        return ((fh != 1 ? 2 : 0) + (fw != 1 ? 1 : 0)) * PL + (fh == 0 ? 0 : 1) * W + (fw == 0 ? -1 : 0);
+    }
 };
 
 struct WgradArgs {
     const float *dY;  // N x OC x H x W
-    const float *X;   // N x IC x H x W
+    const float *X;   // N x IC x (S*H) x (S*W)
     float *out;       // splits > 1: partials [z][OC][IC][9]; splits == 1: dW (accumulated)
     u32 OC, IC, H;
     u32 ic_blocks;        // ceil(IC / 16)
@@ -51,7 +67,7 @@ struct WgradArgs {
 };
 
 template <class Cfg>
-__global__ void __launch_bounds__(kThreads, Cfg::OCC) wgrad3x3s1_kernel(WgradArgs a) {
+__global__ void __launch_bounds__(kThreads, Cfg::OCC) wgrad3x3_kernel(WgradArgs a) {
     constexpr int W = Cfg::W, TR = Cfg::TR, TI = Cfg::TI, YP = Cfg::YP, XP = Cfg::XP, NSTEP = Cfg::NSTEP;
     constexpr int YIMG = Cfg::YIMG, XIMG = Cfg::XIMG;
     __shared__ __attribute__((aligned(16))) float smem[Cfg::SMEM];  // buffer b: dY planes at b*BUF, X planes after them
@@ -69,12 +85,15 @@ __global__ void __launch_bounds__(kThreads, Cfg::OCC) wgrad3x3s1_kernel(WgradArg
         pair = blockIdx.x % a.pairs, z = blockIdx.x / a.pairs;
     }
     const u32 ob = pair / a.ic_blocks, ib = pair % a.ic_blocks;
-    const u32 HW = a.H * W;
+    const u32 HW = a.H * W;                            // dY plane
+    const u32 in_H = a.H * Cfg::S, in_HW = in_H * Cfg::XRW;  // X plane
     const u32 t_begin = z * a.tiles_per_z;
     const u32 t_end = t_begin + a.tiles_per_z < a.tiles ? t_begin + a.tiles_per_z : a.tiles;
 
     // ---- staging: 16-byte global loads, 8-byte LDS stores (plane strides are even, not multiples of 4) ------
-    constexpr int YQ = TI * 16 * (YIMG / 4), XQ = TI * 16 * (XIMG / 4);
+    constexpr int XRQ = Cfg::XRW / 4;                  // quads per input row
+    constexpr int XIQ = Cfg::XROWS * XRQ;              // quads per image per channel
+    constexpr int YQ = TI * 16 * (YIMG / 4), XQ = TI * 16 * XIQ;
     constexpr int YNP = (YQ + kThreads - 1) / kThreads, XNP = (XQ + kThreads - 1) / kThreads;
     v4f yreg[YNP], xreg[XNP];
 
@@ -97,11 +116,12 @@ __global__ void __launch_bounds__(kThreads, Cfg::OCC) wgrad3x3s1_kernel(WgradArg
             const u32 e = t + i * kThreads;
             v4f v = {0.f, 0.f, 0.f, 0.f};
             if (XQ % kThreads == 0 || e < XQ) {
-                const u32 q = e % (XIMG / 4), c = (e / (XIMG / 4)) % 16, img = e / ((XIMG / 4) * 16);
-                const int row = r0 - 1 + int(q / (W / 4));
-                if (row >= 0 && row < int(a.H) && ib * 16 + c < a.IC)
-                    v = *reinterpret_cast<const v4f *>(a.X + (size_t(n0 + img) * a.IC + ib * 16 + c) * HW + u32(row) * W +
-                                                       4 * (q % (W / 4)));
+                const u32 q = e % XIQ, c = (e / XIQ) % 16, img = e / (XIQ * 16);
+                // first staged input row: r0 - 1 (stride 1), 2*(r0 - 1) (stride 2: both parities of the halo row pair)
+                const int row = (Cfg::S == 1 ? r0 - 1 : 2 * (r0 - 1)) + int(q / XRQ);
+                if (row >= 0 && row < int(in_H) && ib * 16 + c < a.IC)
+                    v = *reinterpret_cast<const v4f *>(a.X + (size_t(n0 + img) * a.IC + ib * 16 + c) * in_HW +
+                                                       u32(row) * Cfg::XRW + 4 * (q % XRQ));
             }
             xreg[i] = v;
         }
@@ -122,10 +142,20 @@ __global__ void __launch_bounds__(kThreads, Cfg::OCC) wgrad3x3s1_kernel(WgradArg
         for (int i = 0; i < XNP; ++i) {
             const u32 e = t + i * kThreads;
             if (XQ % kThreads == 0 || e < XQ) {
-                const u32 q = e % (XIMG / 4), c = (e / (XIMG / 4)) % 16, img = e / ((XIMG / 4) * 16);
-                float *p = dXs + c * XP + 4 + img * XIMG + 4 * q;
-                *reinterpret_cast<v2f *>(p) = v2f{xreg[i].x, xreg[i].y};
-                *reinterpret_cast<v2f *>(p + 2) = v2f{xreg[i].z, xreg[i].w};
+                const u32 q = e % XIQ, c = (e / XIQ) % 16, img = e / (XIQ * 16);
+                float *p = dXs + c * XP + 4 + img * XIMG;
+                if constexpr (Cfg::S == 1) {
+                    p += 4 * q;
+                    *reinterpret_cast<v2f *>(p) = v2f{xreg[i].x, xreg[i].y};
+                    *reinterpret_cast<v2f *>(p + 2) = v2f{xreg[i].z, xreg[i].w};
+                } else {
+                    // de-interleave: staged row j = q / XRQ has row parity j % 2 and plane row j / 2; the quad's
+                    // even columns go to the column-parity-0 plane, its odd columns to the column-parity-1 plane
+                    const u32 j = q / XRQ, qq = q % XRQ;
+                    p += (j & 1) * 2 * Cfg::PL + (j >> 1) * W + 2 * qq;
+                    *reinterpret_cast<v2f *>(p) = v2f{xreg[i].x, xreg[i].z};
+                    *reinterpret_cast<v2f *>(p + Cfg::PL) = v2f{xreg[i].y, xreg[i].w};
+                }
             }
         }
     };
@@ -142,7 +172,7 @@ __global__ void __launch_bounds__(kThreads, Cfg::OCC) wgrad3x3s1_kernel(WgradArg
     const int li = lane & 15, kq = lane >> 4;
     const int img_w = wave / Cfg::WPI, row_w = (wave % Cfg::WPI) * Cfg::RW;
     const int ybase = li * YP + kq + img_w * YIMG + row_w * W;
-    const int xbase = li * XP + kq + 3 + img_w * XIMG + row_w * W;  // +4 pad, -1 for the fw shift
+    const int xbase = li * XP + kq + 4 + img_w * XIMG + row_w * W;  // +4: leading pad floats
 
     v4f acc[9];
 #pragma unroll
@@ -154,7 +184,7 @@ __global__ void __launch_bounds__(kThreads, Cfg::OCC) wgrad3x3s1_kernel(WgradArg
         auto read_step = [&](int s, int slot) {
             av[slot] = py[4 * s];
 #pragma unroll
-            for (int k = 0; k < 9; ++k) bv[slot][k] = px[4 * s + (k / 3) * W + (k % 3)];
+            for (int k = 0; k < 9; ++k) bv[slot][k] = px[4 * s + Cfg::tap_off(k)];
         };
         read_step(0, 0);
 #pragma unroll
@@ -162,9 +192,9 @@ __global__ void __launch_bounds__(kThreads, Cfg::OCC) wgrad3x3s1_kernel(WgradArg
             if (s + 1 < NSTEP) read_step(s + 1, (s + 1) & 1);
             __builtin_amdgcn_sched_barrier(0);
             const float am = av[s & 1];
-            // lanes on image column 0 contribute nothing to the fw = 0 taps, lanes on column W-1 nothing to fw = 2
+            // lanes on dY column 0 contribute nothing to the fw = 0 taps; at stride 1 lanes on column W-1 nothing to fw = 2
             const float a0 = ((4 * s) % W == 0) ? (kq == 0 ? 0.f : am) : am;
-            const float a2 = ((4 * s + 4) % W == 0) ? (kq == 3 ? 0.f : am) : am;
+            const float a2 = (Cfg::S == 1 && (4 * s + 4) % W == 0) ? (kq == 3 ? 0.f : am) : am;
 #pragma unroll
             for (int k = 0; k < 9; ++k)
                 acc[k] = __builtin_amdgcn_mfma_f32_16x16x4f32(k % 3 == 0 ? a0 : (k % 3 == 2 ? a2 : am), bv[s & 1][k], acc[k], 0, 0, 0);
@@ -246,7 +276,7 @@ inline int launch_wgrad_direct(const float *dY, const float *X, float *dW, float
     const uint64_t wgs = p.splits >= kXcds ? uint64_t(ceil_div(p.splits, kXcds)) * kXcds * p.pairs  // whole XCD rounds
                                            : uint64_t(p.splits) * p.pairs;
     if (wgs > 0x7fffffffull) return fail(CRB_EINVAL_SHAPE, "%s: launch grid too large", what);
-    hipLaunchKernelGGL((wgrad3x3s1_kernel<Cfg>), dim3(u32(wgs)), dim3(kThreads), 0, s, a);
+    hipLaunchKernelGGL((wgrad3x3_kernel<Cfg>), dim3(u32(wgs)), dim3(kThreads), 0, s, a);
     if (int st = check_launch(what)) return st;
     if (p.splits > 1) {
         return launch_splitk_reduce(ws, dW, OC * IC * 9, p.splits, ReduceEpi{nullptr, 1, 1, EPI_ACCUM}, s, what);

@@ -164,29 +164,37 @@ static bool direct_shape(const crb_conv_geom *g, u32 stride) {
            g->IH == stride * g->OH && g->IW == stride * g->OW;
 }
 
-// ---- direct 3x3 / stride 1 / pad 1 weight gradient ---------------------------------------------------------
+// ---- direct 3x3 / pad 1 weight gradient (stride 1 and 2) ---------------------------------------------------------
 // One entry per configuration <W, TR, TI, OCC>; `run` = false only computes the plan (workspace size).
 constexpr u32 kWgradTargetWgs = 256;  // one workgroup per CU: pairs x splits
 
 template <class Cfg>
 static bool wgrad_cfg(const crb_conv_geom *g, bool run, const float *dY, const float *X, float *dW, float *ws, hipStream_t s,
                       WgradDirectPlan &plan, int &status) {
-    if (!wgrad_direct_fits<Cfg>(g->N, g->IC, g->OC, g->IH, g->IW)) return false;
-    plan = wgrad_direct_plan<Cfg>(g->N, g->IC, g->OC, g->IH, kWgradTargetWgs);
-    if (run) status = launch_wgrad_direct<Cfg>(dY, X, dW, ws, plan, g->N, g->IC, g->OC, g->IH, s, "crb_conv_wgrad");
+    if (!wgrad_direct_fits<Cfg>(g->N, g->IC, g->OC, g->OH, g->OW)) return false;
+    plan = wgrad_direct_plan<Cfg>(g->N, g->IC, g->OC, g->OH, kWgradTargetWgs);
+    if (run) status = launch_wgrad_direct<Cfg>(dY, X, dW, ws, plan, g->N, g->IC, g->OC, g->OH, s, "crb_conv_wgrad");
     return true;
 }
 
+// Configurations <W (dY width), TR, TI, OCC, S>.
 static bool wgrad_direct(const crb_conv_geom *g, bool run, const float *dY, const float *X, float *dW, float *ws,
                          hipStream_t s, WgradDirectPlan &plan, int &status) {
-    if (!direct_shape(g, 1)) return false;
-    if (g->IW == 32) return wgrad_cfg<WgradCfg<32, 8, 1, 2>>(g, run, dY, X, dW, ws, s, plan, status);
-    if (g->IW == 16)
-        return wgrad_cfg<WgradCfg<16, 16, 1, 2>>(g, run, dY, X, dW, ws, s, plan, status) ||
-               wgrad_cfg<WgradCfg<16, 8, 1, 2>>(g, run, dY, X, dW, ws, s, plan, status);
-    if (g->IW == 8)
-        return wgrad_cfg<WgradCfg<8, 8, 4, 2>>(g, run, dY, X, dW, ws, s, plan, status) ||
-               wgrad_cfg<WgradCfg<8, 8, 2, 2>>(g, run, dY, X, dW, ws, s, plan, status);
+    if (direct_shape(g, 1)) {
+        if (g->OW == 32) return wgrad_cfg<WgradCfg<32, 8, 1, 2, 1>>(g, run, dY, X, dW, ws, s, plan, status);
+        if (g->OW == 16)
+            return wgrad_cfg<WgradCfg<16, 16, 1, 2, 1>>(g, run, dY, X, dW, ws, s, plan, status) ||
+                   wgrad_cfg<WgradCfg<16, 8, 1, 2, 1>>(g, run, dY, X, dW, ws, s, plan, status);
+        if (g->OW == 8)
+            return wgrad_cfg<WgradCfg<8, 8, 4, 2, 1>>(g, run, dY, X, dW, ws, s, plan, status) ||
+                   wgrad_cfg<WgradCfg<8, 8, 2, 2, 1>>(g, run, dY, X, dW, ws, s, plan, status);
+    } else if (direct_shape(g, 2)) {
+        if (g->OW == 32) return wgrad_cfg<WgradCfg<32, 4, 1, 1, 2>>(g, run, dY, X, dW, ws, s, plan, status);
+        if (g->OW == 16) return wgrad_cfg<WgradCfg<16, 8, 1, 1, 2>>(g, run, dY, X, dW, ws, s, plan, status);
+        if (g->OW == 8)
+            return wgrad_cfg<WgradCfg<8, 8, 2, 1, 2>>(g, run, dY, X, dW, ws, s, plan, status) ||
+                   wgrad_cfg<WgradCfg<8, 4, 2, 1, 2>>(g, run, dY, X, dW, ws, s, plan, status);
+    }
     return false;
 }
 
