@@ -41,7 +41,7 @@ struct WgradCfg {
     static constexpr int XP = TI * XIMG + 8 + 2;  // 4 leading + 4 trailing pad floats (kept zero)
     static constexpr int Y_SIZE = 16 * YP, X_SIZE = 16 * XP;
     static constexpr int BUF = Y_SIZE + X_SIZE;      // one staging buffer (floats)
-    static constexpr int RED_SIZE = 4 * 9 * 64 * 4;  // cross-wave reduction scratch (floats), reuses the staging space
+    static constexpr int RED_SIZE = 4 * 9 * 256 + 2304;  // cross-wave reduction scratch (floats), reuses the staging space
     static constexpr int SMEM = 2 * BUF > RED_SIZE ? 2 * BUF : RED_SIZE;
     static_assert(TI == 1 || TI == 2 || TI == 4, "images per tile");
     static_assert(TR % WPI == 0 && KW % 4 == 0, "rows must split evenly over the waves");
@@ -91,74 +91,77 @@ __global__ void __launch_bounds__(kThreads, Cfg::OCC) wgrad3x3_kernel(WgradArgs 
     const u32 t_end = t_begin + a.tiles_per_z < a.tiles ? t_begin + a.tiles_per_z : a.tiles;
 
     // ---- staging: 16-byte global loads, 8-byte LDS stores (plane strides are even, not multiples of 4) ------
-    constexpr int XRQ = Cfg::XRW / 4;                  // quads per input row
-    constexpr int XIQ = Cfg::XROWS * XRQ;              // quads per image per channel
-    constexpr int YQ = TI * 16 * (YIMG / 4), XQ = TI * 16 * XIQ;
-    constexpr int YNP = (YQ + kThreads - 1) / kThreads, XNP = (XQ + kThreads - 1) / kThreads;
+    // A thread owns one (image, channel, quad-of-a-row) column of the tile for the whole kernel and walks down its rows,
+    // so per tile and item the address arithmetic is one add of a compile-time multiple of the row pitch.
+    constexpr int YRQ = W / 4, XRQ = Cfg::XRW / 4;      // quads per dY row / per input row
+    constexpr int YC = TI * 16 * YRQ, XC = TI * 16 * XRQ;  // columns
+    static_assert(kThreads % YC == 0 && kThreads % XC == 0, "columns must divide the workgroup");
+    constexpr int YRPP = kThreads / YC, XRPP = kThreads / XC;  // rows covered per pass
+    constexpr int YNP = (TR + YRPP - 1) / YRPP, XNP = (Cfg::XROWS + XRPP - 1) / XRPP;
     v4f yreg[YNP], xreg[XNP];
+
+    const u32 ycol = t % YC, yrp = t / YC;
+    const u32 yq = ycol % YRQ, yc = (ycol / YRQ) % 16, yimg = ycol / (YRQ * 16);
+    const bool ychan_ok = ob * 16 + yc < a.OC;  // channels past the tensor's extent are staged as zeros
+    const float *ysrc = a.dY + (size_t(yimg) * a.OC + ob * 16 + yc) * HW + yrp * W + 4 * yq;
+    const u32 ylds = yc * YP + yimg * YIMG + yrp * W + 4 * yq;
+
+    const u32 xcol = t % XC, xrp = t / XC;
+    const u32 xq = xcol % XRQ, xc = (xcol / XRQ) % 16, ximg = xcol / (XRQ * 16);
+    const bool xchan_ok = ib * 16 + xc < a.IC;
+    const float *xsrc = a.X + (size_t(ximg) * a.IC + ib * 16 + xc) * in_HW + 4 * xq;
+    const u32 xlds = xc * XP + 4 + ximg * XIMG + (Cfg::S == 1 ? 4 * xq : 2 * xq);
 
     auto fetch = [&](u32 tile) {
         const u32 n0 = (tile / a.tiles_per_img) * TI;
         const int r0 = int(tile % a.tiles_per_img) * TR;
+        const float *yp = ysrc + size_t(n0) * a.OC * HW + u32(r0) * W;
 #pragma unroll
         for (int i = 0; i < YNP; ++i) {
-            const u32 e = t + i * kThreads;
             v4f v = {0.f, 0.f, 0.f, 0.f};
-            if (YQ % kThreads == 0 || e < YQ) {
-                const u32 q = e % (YIMG / 4), c = (e / (YIMG / 4)) % 16, img = e / ((YIMG / 4) * 16);
-                if (ob * 16 + c < a.OC)  // channels past the tensor's extent are staged as zeros
-                    v = *reinterpret_cast<const v4f *>(a.dY + (size_t(n0 + img) * a.OC + ob * 16 + c) * HW + u32(r0) * W + 4 * q);
-            }
+            if (ychan_ok && (TR % YRPP == 0 || i * YRPP + int(yrp) < TR)) v = *reinterpret_cast<const v4f *>(yp + i * YRPP * W);
             yreg[i] = v;
         }
+        // first staged input row: r0 - 1 (stride 1), 2*(r0 - 1) (stride 2: both parities of the halo row pair)
+        const int row0 = (Cfg::S == 1 ? r0 - 1 : 2 * (r0 - 1)) + int(xrp);
+        const float *xp = xsrc + size_t(n0) * a.IC * in_HW;
 #pragma unroll
         for (int i = 0; i < XNP; ++i) {
-            const u32 e = t + i * kThreads;
             v4f v = {0.f, 0.f, 0.f, 0.f};
-            if (XQ % kThreads == 0 || e < XQ) {
-                const u32 q = e % XIQ, c = (e / XIQ) % 16, img = e / (XIQ * 16);
-                // first staged input row: r0 - 1 (stride 1), 2*(r0 - 1) (stride 2: both parities of the halo row pair)
-                const int row = (Cfg::S == 1 ? r0 - 1 : 2 * (r0 - 1)) + int(q / XRQ);
-                if (row >= 0 && row < int(in_H) && ib * 16 + c < a.IC)
-                    v = *reinterpret_cast<const v4f *>(a.X + (size_t(n0 + img) * a.IC + ib * 16 + c) * in_HW +
-                                                       u32(row) * Cfg::XRW + 4 * (q % XRQ));
-            }
+            const int row = row0 + i * XRPP;
+            if (xchan_ok && (Cfg::XROWS % XRPP == 0 || i * XRPP + int(xrp) < Cfg::XROWS) && row >= 0 && row < int(in_H))
+                v = *reinterpret_cast<const v4f *>(xp + row * Cfg::XRW);
             xreg[i] = v;
         }
     };
 
-    auto commit = [&](float *dYs, float *dXs) {
-#pragma unroll
-        for (int i = 0; i < YNP; ++i) {
-            const u32 e = t + i * kThreads;
-            if (YQ % kThreads == 0 || e < YQ) {
-                const u32 q = e % (YIMG / 4), c = (e / (YIMG / 4)) % 16, img = e / ((YIMG / 4) * 16);
-                float *p = dYs + c * YP + img * YIMG + 4 * q;
+    // LDS store of staged item i (dY items first, then X items)
+    auto commit_item = [&](int i, float *dYs, float *dXs) {
+        if (i < YNP) {
+            if (TR % YRPP == 0 || i * YRPP + int(yrp) < TR) {
+                float *p = dYs + ylds + i * YRPP * W;
                 *reinterpret_cast<v2f *>(p) = v2f{yreg[i].x, yreg[i].y};
                 *reinterpret_cast<v2f *>(p + 2) = v2f{yreg[i].z, yreg[i].w};
             }
-        }
-#pragma unroll
-        for (int i = 0; i < XNP; ++i) {
-            const u32 e = t + i * kThreads;
-            if (XQ % kThreads == 0 || e < XQ) {
-                const u32 q = e % XIQ, c = (e / XIQ) % 16, img = e / (XIQ * 16);
-                float *p = dXs + c * XP + 4 + img * XIMG;
+        } else {
+            const int ix = i - YNP;
+            if (Cfg::XROWS % XRPP == 0 || ix * XRPP + int(xrp) < Cfg::XROWS) {
                 if constexpr (Cfg::S == 1) {
-                    p += 4 * q;
-                    *reinterpret_cast<v2f *>(p) = v2f{xreg[i].x, xreg[i].y};
-                    *reinterpret_cast<v2f *>(p + 2) = v2f{xreg[i].z, xreg[i].w};
+                    float *p = dXs + xlds + (ix * XRPP + xrp) * W;
+                    *reinterpret_cast<v2f *>(p) = v2f{xreg[ix].x, xreg[ix].y};
+                    *reinterpret_cast<v2f *>(p + 2) = v2f{xreg[ix].z, xreg[ix].w};
                 } else {
-                    // de-interleave: staged row j = q / XRQ has row parity j % 2 and plane row j / 2; the quad's
-                    // even columns go to the column-parity-0 plane, its odd columns to the column-parity-1 plane
-                    const u32 j = q / XRQ, qq = q % XRQ;
-                    p += (j & 1) * 2 * Cfg::PL + (j >> 1) * W + 2 * qq;
-                    *reinterpret_cast<v2f *>(p) = v2f{xreg[i].x, xreg[i].z};
-                    *reinterpret_cast<v2f *>(p + Cfg::PL) = v2f{xreg[i].y, xreg[i].w};
+                    // de-interleave: staged row j has row parity j % 2 and plane row j / 2; the quad's even columns go
+                    // to the column-parity-0 plane, its odd columns to the column-parity-1 plane
+                    const u32 j = ix * XRPP + xrp;
+                    float *p = dXs + xlds + (j & 1) * 2 * Cfg::PL + (j >> 1) * W;
+                    *reinterpret_cast<v2f *>(p) = v2f{xreg[ix].x, xreg[ix].z};
+                    *reinterpret_cast<v2f *>(p + Cfg::PL) = v2f{xreg[ix].y, xreg[ix].w};
                 }
             }
         }
     };
+    constexpr int NITEM = YNP + XNP;
 
     // leading / trailing pad floats of every X plane stay zero (they are read, multiplied by a zeroed dY value)
     for (u32 e = t; e < 2u * 16 * 8; e += kThreads) {
@@ -178,7 +181,11 @@ __global__ void __launch_bounds__(kThreads, Cfg::OCC) wgrad3x3_kernel(WgradArgs 
 #pragma unroll
     for (int k = 0; k < 9; ++k) acc[k] = v4f{0.f, 0.f, 0.f, 0.f};
 
-    auto compute = [&](const float *cy, const float *cx) {
+    // One tile: NSTEP MFMA steps. The LDS stores of the next tile's staged data (its global loads were issued before
+    // this call) are spread over the last steps, one item per step, so they issue in the shadow of the MFMAs instead
+    // of forming a store burst between tiles.
+    constexpr int FIRST_STORE_STEP = NSTEP > NITEM ? NSTEP - NITEM : 0;
+    auto compute = [&](const float *cy, const float *cx, float *ny, float *nx) {
         const float *py = cy + ybase, *px = cx + xbase;
         float av[2], bv[2][9];
         auto read_step = [&](int s, int slot) {
@@ -190,7 +197,6 @@ __global__ void __launch_bounds__(kThreads, Cfg::OCC) wgrad3x3_kernel(WgradArgs 
 #pragma unroll
         for (int s = 0; s < NSTEP; ++s) {
             if (s + 1 < NSTEP) read_step(s + 1, (s + 1) & 1);
-            __builtin_amdgcn_sched_barrier(0);
             const float am = av[s & 1];
             // lanes on dY column 0 contribute nothing to the fw = 0 taps; at stride 1 lanes on column W-1 nothing to fw = 2
             const float a0 = ((4 * s) % W == 0) ? (kq == 0 ? 0.f : am) : am;
@@ -198,6 +204,19 @@ __global__ void __launch_bounds__(kThreads, Cfg::OCC) wgrad3x3_kernel(WgradArgs 
 #pragma unroll
             for (int k = 0; k < 9; ++k)
                 acc[k] = __builtin_amdgcn_mfma_f32_16x16x4f32(k % 3 == 0 ? a0 : (k % 3 == 2 ? a2 : am), bv[s & 1][k], acc[k], 0, 0, 0);
+            if (s >= FIRST_STORE_STEP) {
+                // items per step: all remaining ones on the last step if there are more items than steps
+                const int first = s - FIRST_STORE_STEP, last = (s == NSTEP - 1) ? NITEM : first + 1;
+#pragma unroll
+                for (int i = first; i < last; ++i) commit_item(i, ny, nx);
+            }
+            // issue order inside the step: one MFMA, then one of the next step's LDS reads, and so on, so the matrix
+            // pipe never waits for the read burst; the fence keeps the steps themselves in order
+#pragma unroll
+            for (int k = 0; k < 9; ++k) {
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // MFMA
+                __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // DS read
+            }
             __builtin_amdgcn_sched_barrier(0);
         }
     };
@@ -205,34 +224,50 @@ __global__ void __launch_bounds__(kThreads, Cfg::OCC) wgrad3x3_kernel(WgradArgs 
     // ---- main loop over this split's tiles (double-buffered) ------------------------------------------------
     if (t_begin < t_end) {
         fetch(t_begin);
-        commit(smem, smem + Cfg::Y_SIZE);
+#pragma unroll
+        for (int i = 0; i < NITEM; ++i) commit_item(i, smem, smem + Cfg::Y_SIZE);
     }
     __syncthreads();
     for (u32 tile = t_begin; tile < t_end; ++tile) {
         const u32 b = (tile - t_begin) & 1;
-        const bool more = tile + 1 < t_end;
-        if (more) fetch(tile + 1);
-        compute(smem + b * Cfg::BUF, smem + b * Cfg::BUF + Cfg::Y_SIZE);
-        if (more) commit(smem + (b ^ 1) * Cfg::BUF, smem + (b ^ 1) * Cfg::BUF + Cfg::Y_SIZE);
+        // After the last tile nothing new was fetched: the stores inside compute() then rewrite stale registers into the
+        // idle buffer, which nothing reads before the reduction scratch overwrites it.
+        if (tile + 1 < t_end) fetch(tile + 1);
+        float *cur = smem + b * Cfg::BUF, *nxt = smem + (b ^ 1) * Cfg::BUF;
+        compute(cur, cur + Cfg::Y_SIZE, nxt, nxt + Cfg::Y_SIZE);
         __syncthreads();
     }
 
     // ---- sum the 4 waves' accumulators in wave order, write this (pair, split) block --------------------------
-    float *red = smem;  // [wave][tap][lane][4]
+    // Pass 1: every wave parks its 9 tiles in LDS as [wave][tap][lane][4]. Pass 2: thread t sums the 4 waves for
+    // element (lane = t/4, r = t%4) of each tap (consecutive threads read consecutive floats: no bank conflicts) and
+    // writes the sums back transposed to [oc][ic][tap], the order dW has in memory. Pass 3: coalesced store.
+    float *red = smem;                 // [wave][tap][lane][4]  (4*9*256 floats)
+    float *tr = smem + 4 * 9 * 256;    // [oc 16][ic 16][tap 9] (2304 floats)
 #pragma unroll
     for (int k = 0; k < 9; ++k) *reinterpret_cast<v4f *>(red + ((wave * 9 + k) * 64 + lane) * 4) = acc[k];
     __syncthreads();
+    {
+        const u32 l2 = t >> 2, r = t & 3;
+        const u32 oc = 4 * (l2 >> 4) + r, ic = l2 & 15;
+#pragma unroll
+        for (int k = 0; k < 9; ++k) {
+            float sum = red[k * 256 + t];
+#pragma unroll
+            for (int w = 1; w < 4; ++w) sum += red[(w * 9 + k) * 256 + t];
+            tr[(oc * 16 + ic) * 9 + k] = sum;
+        }
+    }
+    __syncthreads();
     const size_t count = size_t(a.OC) * a.IC * 9;
     float *out = a.out + size_t(z) * count * (a.accumulate ? 0 : 1);
-    for (u32 e = t; e < 16 * 16 * 9; e += kThreads) {
-        const u32 oc = e / 144, ic = (e % 144) / 9, tap = e % 9;
-        if (ob * 16 + oc >= a.OC || ib * 16 + ic >= a.IC) continue;
-        const u32 src = (tap * 64 + (oc / 4) * 16 + ic) * 4 + (oc % 4);
-        float s = red[src];
 #pragma unroll
-        for (int w = 1; w < 4; ++w) s += red[w * 9 * 64 * 4 + src];
-        float *dst = out + (size_t(ob * 16 + oc) * a.IC + ib * 16 + ic) * 9 + tap;
-        *dst = a.accumulate ? *dst + s : s;
+    for (int i = 0; i < 9; ++i) {
+        const u32 e = t + i * kThreads;       // e = oc*144 + ic*9 + tap
+        const u32 oc = e / 144, rest = e % 144;  // rest = ic*9 + tap: contiguous in dW for one oc
+        if (ob * 16 + oc >= a.OC || ib * 16 + rest / 9 >= a.IC) continue;
+        float *dst = out + (size_t(ob * 16 + oc) * a.IC + ib * 16) * 9 + rest;
+        *dst = a.accumulate ? *dst + tr[e] : tr[e];
     }
 }
 
