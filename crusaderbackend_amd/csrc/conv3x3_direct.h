@@ -1,4 +1,4 @@
-// Direct 3x3 / pad 1 convolution for gfx950, stride 1 or 2: forward and data gradient in one template.
+// Direct 3x3 / pad 1 convolution for gfx950, stride 1 or 2 (and 1x1 / stride 1): forward and data gradient in one template.
 //
 // A workgroup (4 wave64) owns ROWS rows of a "pixel grid" of one image and OCT output channels. The grid is the
 // output image for the forward pass and for the stride-1 data gradient; for the stride-2 data gradient it is the
@@ -32,9 +32,12 @@ namespace crb {
 
 // NBUF_ = 2: double-buffered chunk pipeline (any C_IN). NBUF_ = 1: the whole contraction is one chunk (C_IN <= CI),
 // half the LDS, so more workgroups fit on a CU and overlap each other's staging.
-template <int W_, int ROWS_, int CI_, int OCT_, int PBW_, int OBW_, bool DGRAD_, int OCC_, int NBUF_ = 2, int S_ = 1>
+// FS_ = 3: 3x3 filter with pad 1. FS_ = 1: 1x1 filter, no padding, stride 1 (one tap, no halo) — the bottleneck layers,
+// which are bandwidth-bound: same staging and MFMA mapping, the contraction is just the channel chunk.
+template <int W_, int ROWS_, int CI_, int OCT_, int PBW_, int OBW_, bool DGRAD_, int OCC_, int NBUF_ = 2, int S_ = 1, int FS_ = 3>
 struct DirectCfg {
     static constexpr int W = W_, ROWS = ROWS_, CI = CI_, OCT = OCT_, PBW = PBW_, OBW = OBW_, OCC = OCC_, NBUF = NBUF_, S = S_;
+    static constexpr int FS = FS_, NT = FS_ * FS_;  // filter size, taps
     static constexpr bool DGRAD = DGRAD_;
     static constexpr bool DG2 = DGRAD && S == 2;  // stride-2 data gradient (4 parity classes)
     static constexpr bool FW2 = !DGRAD && S == 2; // stride-2 forward
@@ -46,9 +49,9 @@ struct DirectCfg {
     static constexpr int NOBW = NOB / OBW;        // wave groups along channels
     // staged input: row width, row count, the input row LDS row 0 holds (ROW0_MUL*r0 + ROW0_ADD for first grid row r0)
     static constexpr int SW = FW2 ? 2 * W : W;
-    static constexpr int XR = DG2 ? ROWS + 1 : S * (ROWS - 1) + 3;
+    static constexpr int XR = FS == 1 ? ROWS : (DG2 ? ROWS + 1 : S * (ROWS - 1) + 3);
     static constexpr int ROW0_MUL = FW2 ? 2 : 1;
-    static constexpr int ROW0_ADD = DG2 ? 0 : -1;
+    static constexpr int ROW0_ADD = (DG2 || FS == 1) ? 0 : -1;
     static constexpr int PSTEP = FW2 ? 2 : 1;     // LDS distance of neighbouring grid pixels
     static constexpr int XS = SW + 8;  // LDS row stride: 3 pad, left halo, SW interior (16-byte aligned), right halo, 3 pad
     // channel plane stride (floats): the four lane groups (lane/16) of a fragment read sit one plane apart;
@@ -56,17 +59,18 @@ struct DirectCfg {
     static constexpr int XP_MIN = XR * XS;
     static constexpr int XP_RES = W == 8 ? 8 : 16;
     static constexpr int XP = XP_MIN + ((XP_RES - XP_MIN % 32) + 32) % 32;
-    static constexpr int NSTEP = CI * 9 / 4;      // MFMA steps per chunk
+    static constexpr int NSTEP = CI * NT / 4;     // MFMA steps per chunk
     static constexpr int CQ = CI / 4;             // steps per tap
     static constexpr int MPS = PBW * OBW;         // MFMAs per step
     static constexpr int PF = (8 / MPS) < 1 ? 1 : ((8 / MPS) > 4 ? 4 : (8 / MPS));  // read-ahead (steps)
     static constexpr int CIP = CI + 1;            // k index of (tap, channel) in a filter row is tap*CIP + channel: odd tap stride
-    static constexpr int WSTR_MIN = 9 * CIP;      // filter row stride == 2 mod 4: the 32 lanes of a half-wave (16 rows x 2 k) hit distinct banks
+    static constexpr int WSTR_MIN = NT * CIP;      // filter row stride == 2 mod 4: the 32 lanes of a half-wave (16 rows x 2 k) hit distinct banks
     static constexpr int WSTR = WSTR_MIN + ((2 - WSTR_MIN % 4) + 4) % 4;
     static constexpr int X_SIZE = CI * XP;
     static constexpr int W_SIZE = OCT * WSTR;
     static_assert(W == 8 || W == 16 || W == 32, "grid width");
     static_assert(S == 1 || S == 2, "stride");
+    static_assert(FS == 3 || (FS == 1 && S == 1), "1x1 filters are handled at stride 1 only");
     static_assert(TP % 16 == 0 && NPB % PBW == 0 && NOB % OBW == 0 && NPBW * NOBW == 4, "wave tiling must use 4 waves");
     static_assert((PBW * 16) % W == 0 || PBW == 1, "a wave's pixel blocks must start on a row boundary");
     static_assert(CI % 4 == 0, "chunk channel count");
@@ -74,6 +78,7 @@ struct DirectCfg {
     // LDS offset of tap (fh, fw) relative to the lane's pixel base (which points one float left of the pixel)
     static constexpr int tap_off(int tap) {
         const int fh = tap / 3, fw = tap % 3;
+        if (FS == 1) return 1;  // the pixel itself: interior starts one float past the lane's base
         if (DG2) return (fh == 0 ? 1 : 0) * XS + (fw == 0 ? 1 : 0) + 1;
         if (DGRAD) return (2 - fh) * XS + (2 - fw);
         return fh * XS + fw;
@@ -125,7 +130,8 @@ __global__ void __launch_bounds__(kThreads, Cfg::OCC) conv3x3_kernel(DirectArgs 
     constexpr int WQ = OCT * CI;
     constexpr int WNP = (WQ + kThreads - 1) / kThreads;
     v4f xreg[XNP];
-    float wreg[WNP * 9];
+    constexpr int NT = Cfg::NT;
+    float wreg[WNP * NT];
 
     auto fetch = [&](u32 c0) {
 #pragma unroll
@@ -146,16 +152,16 @@ __global__ void __launch_bounds__(kThreads, Cfg::OCC) conv3x3_kernel(DirectArgs 
             // forward: lanes run over chunk channels c (filter row j = e / CI): W[oc0 + j][c0 + c][0..8]
             // dgrad:   lanes run over filter rows j (gradient channel c = e / OCT): W[c0 + c][oc0 + j][0..8]
             const u32 j = Cfg::DGRAD ? e % OCT : e / CI, c = Cfg::DGRAD ? e / OCT : e % CI;
-            const float *src = Cfg::DGRAD ? a.Wt + ((size_t(c0) + c) * a.C_OUT + oc0 + j) * 9
-                                          : a.Wt + ((size_t(oc0) + j) * a.C_IN + c0 + c) * 9;
+            const float *src = Cfg::DGRAD ? a.Wt + ((size_t(c0) + c) * a.C_OUT + oc0 + j) * NT
+                                          : a.Wt + ((size_t(oc0) + j) * a.C_IN + c0 + c) * NT;
             // channels past the tensor's extent (ragged last chunk / last channel tile) are staged as zeros
             const bool ok = (WQ % kThreads == 0 || e < WQ) && c0 + c < a.C_IN && oc0 + j < a.C_OUT;
             if (ok) {  // one branch around the 9 contiguous loads keeps them mergeable into wide loads
 #pragma unroll
-                for (int tap = 0; tap < 9; ++tap) wreg[i * 9 + tap] = src[tap];
+                for (int tap = 0; tap < NT; ++tap) wreg[i * NT + tap] = src[tap];
             } else {
 #pragma unroll
-                for (int tap = 0; tap < 9; ++tap) wreg[i * 9 + tap] = 0.f;
+                for (int tap = 0; tap < NT; ++tap) wreg[i * NT + tap] = 0.f;
             }
         }
     };
@@ -175,7 +181,7 @@ __global__ void __launch_bounds__(kThreads, Cfg::OCC) conv3x3_kernel(DirectArgs 
             if (WQ % kThreads == 0 || e < WQ) {
                 const u32 j = Cfg::DGRAD ? e % OCT : e / CI, c = Cfg::DGRAD ? e / OCT : e % CI;
 #pragma unroll
-                for (int tap = 0; tap < 9; ++tap) dW[j * WSTR + tap * Cfg::CIP + c] = wreg[i * 9 + tap];
+                for (int tap = 0; tap < NT; ++tap) dW[j * WSTR + tap * Cfg::CIP + c] = wreg[i * NT + tap];
             }
         }
     };

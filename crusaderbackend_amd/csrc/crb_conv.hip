@@ -152,6 +152,52 @@ static int try_direct(const float *Wt, const float *X, float *Y, const float *bi
     return CRB_OK;
 }
 
+// Direct kernel configurations for 1x1 / stride 1 / no padding layers <W, ROWS, CI, OCT, PBW, OBW, DGRAD, OCC, NBUF, S, FS=1>.
+// The output-channel tile is the widest of 64 / 48 / 32 / 16 that wastes at most a quarter of its channels and still
+// yields enough workgroups for the chip; if none does, the batched GEMM forms run instead.
+template <bool DG>
+static int try_pointwise(const float *Wt, const float *X, float *Y, const float *bias, u32 N, u32 C_IN, u32 C_OUT, u32 gH, u32 gW,
+                         u32 relu, hipStream_t s, const char *what, bool &done) {
+    done = true;
+    if ((gW != 32 && gW != 16 && gW != 8) || gH % 8 != 0) {  // every configuration below tiles rows by 8 or 4
+        done = false;
+        return CRB_OK;
+    }
+    const u32 tiles = N * (gH / 8);
+    auto good = [&](u32 oct) {
+        const u32 nt = ceil_div(C_OUT, oct);
+        return nt * oct * 3 <= C_OUT * 4 + 3 * 15 && tiles * nt >= 192;  // <= 25 % padding (one ragged 16-block allowed)
+    };
+#define CRB_TRY(...)                                                                                          \
+    if (direct_fits<DirectCfg<__VA_ARGS__>>(C_IN, gH, gW))                                                     \
+        return launch_direct<DirectCfg<__VA_ARGS__>>(Wt, X, Y, bias, N, C_IN, C_OUT, gH, gH, relu, s, what);
+    // long contractions with few workgroups: half-height tiles, so two workgroups share a CU and one multiplies while
+    // the other waits for its next channel chunk
+    const bool half = C_IN > 64 && tiles * ceil_div(C_OUT, 48u) < 512;
+    if (gW == 32) {
+        if (half && good(48)) { CRB_TRY(32, 4, 16, 48, 2, 3, DG, 2, 2, 1, 1) }
+        if (half && good(64)) { CRB_TRY(32, 4, 16, 64, 2, 4, DG, 2, 2, 1, 1) }
+        if (good(64)) { CRB_TRY(32, 8, 16, 64, 4, 4, DG, 2, 2, 1, 1) }
+        if (good(48)) { CRB_TRY(32, 8, 16, 48, 4, 3, DG, 2, 2, 1, 1) }
+        if (good(32)) { CRB_TRY(32, 8, 16, 32, 4, 2, DG, 2, 2, 1, 1) }
+        if (good(16)) { CRB_TRY(32, 8, 16, 16, 4, 1, DG, 2, 2, 1, 1) }
+    } else if (gW == 16) {
+        if (half && good(48)) { CRB_TRY(16, 4, 16, 48, 1, 3, DG, 2, 2, 1, 1) }
+        if (good(64)) { CRB_TRY(16, 8, 16, 64, 2, 4, DG, 2, 2, 1, 1) }
+        if (good(48)) { CRB_TRY(16, 8, 16, 48, 2, 3, DG, 2, 2, 1, 1) }
+        if (good(32)) { CRB_TRY(16, 8, 16, 32, 2, 2, DG, 2, 2, 1, 1) }
+        if (good(16)) { CRB_TRY(16, 8, 16, 16, 2, 1, DG, 2, 2, 1, 1) }
+    } else {
+        if (good(64)) { CRB_TRY(8, 8, 16, 64, 1, 4, DG, 2, 2, 1, 1) }
+        if (good(48)) { CRB_TRY(8, 8, 16, 48, 1, 3, DG, 2, 2, 1, 1) }
+        if (good(32)) { CRB_TRY(8, 8, 16, 32, 1, 2, DG, 2, 2, 1, 1) }
+        if (good(16)) { CRB_TRY(8, 8, 16, 16, 1, 1, DG, 2, 2, 1, 1) }
+    }
+#undef CRB_TRY
+    done = false;
+    return CRB_OK;
+}
+
 // 1x1 / stride 1 / no padding: per image Y[n] (OC x HW) = W (OC x IC) * X[n] (IC x HW) on the native layout, i.e. the
 // batched forms of the GEMM family (forward NN with a per-row bias, data gradient TN, weight gradient accumulate-NT).
 static bool pointwise_shape(const crb_conv_geom *g) {
@@ -240,6 +286,12 @@ int crb_conv_fwd(const float *W, const float *X, float *Y, const float *bias_or_
     NchwEpi e{Y, bias_or_null, g->OC, g->OH * g->OW, (flags & CRB_FLAG_RELU) ? u32(EPI_RELU) : 0u,
               FastDiv(g->OH * g->OW), 0u};
     hipStream_t s = hipStream_t(stream);
+    if (pointwise_shape(g) && aligned16(X) && aligned16(Y)) {
+        bool done;
+        int st = try_pointwise<false>(W, X, Y, bias_or_null, g->N, g->IC, g->OC, g->OH, g->OW, flags & CRB_FLAG_RELU, s,
+                                      "crb_conv_fwd", done);
+        if (done) return st;
+    }
     if (pointwise_shape(g))
         return gemm_nn_rowbias(W, X, Y, g->OC, g->IH * g->IW, g->IC, g->N, bias_or_null,
                                (flags & CRB_FLAG_RELU) ? u32(EPI_RELU) : 0u, s, "crb_conv_fwd");
@@ -262,6 +314,12 @@ int crb_conv_fwd(const float *W, const float *X, float *Y, const float *bias_or_
 int crb_conv_dgrad(const float *W, const float *dY, float *dX, const crb_conv_geom *g, void *stream) {
     if (!W || !dY || !dX) return fail(CRB_ENULL, "crb_conv_dgrad: null operand");
     if (int st = check_geom("crb_conv_dgrad", g)) return st;
+    if (pointwise_shape(g) && aligned16(dY) && aligned16(dX)) {
+        bool done;
+        int st = try_pointwise<true>(W, dY, dX, nullptr, g->N, g->OC, g->IC, g->OH, g->OW, 0, hipStream_t(stream),
+                                     "crb_conv_dgrad", done);
+        if (done) return st;
+    }
     if (pointwise_shape(g))
         return gemm_tn_batched(W, dY, dX, g->IC, g->IH * g->IW, g->OC, g->N, hipStream_t(stream), "crb_conv_dgrad");
     if (aligned16(dY) && aligned16(dX) && (direct_shape(g, 1) || direct_shape(g, 2))) {

@@ -53,14 +53,34 @@ static int check_dims(const char *what, u32 M, u32 N, u32 K, u32 batch) {
     return CRB_OK;
 }
 
-// column sums of a (rows x cols) row-major matrix: out[c] += sum_r in[r*cols + c], ascending r.
+// column sums of a (rows x cols) row-major matrix: out[c] += sum_r in[r*cols + c]. 32 columns x 8 row-lanes per
+// workgroup; a row-lane sums rows lane, lane+8, ... with 4 independent running sums, the 8 lanes are combined through
+// LDS in lane order (fixed association: bit-reproducible).
 __global__ void __launch_bounds__(256) colsum_accum_kernel(const float *__restrict__ in, float *__restrict__ out,
                                                            u32 rows, u32 cols) {
-    const u32 c = blockIdx.x * 256 + threadIdx.x;
-    if (c >= cols) return;
-    float s = 0.0f;
-    for (u32 r = 0; r < rows; ++r) s += in[size_t(r) * cols + c];
-    out[c] += s;
+    __shared__ float red[8][32];
+    const u32 o = threadIdx.x % 32, g = threadIdx.x / 32;
+    const u32 c = blockIdx.x * 32 + o;
+    float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
+    if (c < cols) {
+        const float *p = in + c;
+        u32 r = g;
+        for (; r + 24 < rows; r += 32) {
+            s0 += p[size_t(r) * cols];
+            s1 += p[size_t(r + 8) * cols];
+            s2 += p[size_t(r + 16) * cols];
+            s3 += p[size_t(r + 24) * cols];
+        }
+        for (; r < rows; r += 8) s0 += p[size_t(r) * cols];
+    }
+    red[g][o] = (s0 + s1) + (s2 + s3);
+    __syncthreads();
+    if (g == 0 && c < cols) {
+        float r = red[0][o];
+#pragma unroll
+        for (int k = 1; k < 8; ++k) r += red[k][o];
+        out[c] += r;
+    }
 }
 
 static int gemm_nn(const float *A, const float *B, float *C, u32 M, u32 N, u32 K, u32 batch, const float *col_bias,
@@ -181,7 +201,7 @@ int crb_linear_wgrad(const float *dY, const float *X, float *dW, float *dB, uint
     // dW (OUT x IN) += dY^T (dY stored batch x OUT) * X (batch x IN)
     if (int st = gemm_tn(dY, X, dW, OUT, IN, batch, 1, EPI_ACCUM, s, "crb_linear_wgrad")) return st;
     if (dB) {
-        hipLaunchKernelGGL(colsum_accum_kernel, dim3(ceil_div(OUT, 256)), dim3(256), 0, s, dY, dB, batch, OUT);
+        hipLaunchKernelGGL(colsum_accum_kernel, dim3(ceil_div(OUT, 32)), dim3(256), 0, s, dY, dB, batch, OUT);
         return check_launch("crb_linear_wgrad(dB)");
     }
     return CRB_OK;

@@ -252,3 +252,16 @@ STRIDE2 = [
 @pytest.mark.parametrize("N,IC,IH,IW,OC", STRIDE2)
 def test_conv3x3_stride2_direct(dev, N, IC, IH, IW, OC):
     run_layer(dev, N, IC, IH, IW, OC, 3, 3, 2, 2, 1, 1, bias=True, seed=21)
+
+
+# 1x1 / stride 1 / no padding: direct staged kernel for widths 32/16/8 with rows divisible by 8, batched GEMM forms otherwise
+POINTWISE = [(3, 24, 32, 32, 48), (2, 204, 32, 32, 48), (2, 108, 16, 16, 48), (4, 330, 8, 8, 48), (2, 7, 16, 16, 5),
+             (2, 64, 32, 32, 64), (2, 17, 8, 8, 33), (2, 16, 12, 16, 16), (2, 16, 8, 12, 16), (1, 40, 24, 32, 70),
+             # batches large enough to pass the workgroup-count gate of the staged 1x1 kernel
+             (64, 204, 32, 32, 48), (64, 24, 32, 32, 48), (64, 108, 16, 16, 48), (96, 70, 16, 16, 130), (64, 150, 8, 8, 48),
+             (128, 37, 8, 8, 64), (48, 80, 32, 32, 20)]
+
+
+@pytest.mark.parametrize("N,IC,H,W,OC", POINTWISE)
+def test_conv1x1_paths(dev, N, IC, H, W, OC):
+    run_layer(dev, N, IC, H, W, OC, 1, 1, 1, 1, 0, 0, bias=True, seed=31)
