@@ -88,6 +88,19 @@ class Layer:
         return (("fwd", self.fwd), ("dgrad", self.dgrad), ("wgrad", self.wgrad))
 
 
+# HBM bytes one call moves (read + written, all kernels of the call), from the FETCH_SIZE and WRITE_SIZE hardware
+# counters of this workload under rocprofv3 --pmc, scaled by what the same counters read for a copy kernel of known
+# size (`--calibrate`): FETCH_SIZE x2.00, WRITE_SIZE x1.00. A property of the kernels' access pattern, not of a run;
+# the counter summaries are kept under profiles/.
+MEASURED_HBM_BYTES = {
+    "L1_16-16@32.fwd": 18.51e6, "L1_16-16@32.dgrad": 18.51e6, "L1_16-16@32.wgrad": 22.25e6,
+    "L2_32-32@16.fwd": 11.95e6, "L2_32-32@16.dgrad": 11.95e6, "L2_32-32@16.wgrad": 13.34e6,
+    "L3_64-64@8.fwd": 5.47e6, "L3_64-64@8.dgrad": 5.46e6, "L3_64-64@8.wgrad": 9.38e6,
+    "T1_16-32s2.fwd": 13.12e6, "T1_16-32s2.dgrad": 13.35e6, "T1_16-32s2.wgrad": 17.57e6,
+    "T2_32-64s2.fwd": 6.99e6, "T2_32-64s2.dgrad": 6.96e6, "T2_32-64s2.wgrad": 11.33e6,
+}
+
+
 def event_time_ms(torch, fn, reps, warm=3):
     """Average duration of `fn` (ms) over `reps` back-to-back launches between two events on the launch stream."""
     for _ in range(warm):
@@ -101,14 +114,15 @@ def event_time_ms(torch, fn, reps, warm=3):
     return e0.elapsed_time(e1) / reps
 
 
-def cpu_baseline(layers_spec):
-    """CPU oracle on a bounded sample: the same step at batch 64 (half of the images), all host cores capped at 16."""
+def cpu_baseline(layers_spec, min_seconds=10.0):
+    """CPU oracle on the same workload: whole ResNet-56 conv steps at the real batch, repeated until `min_seconds` of
+    CPU work have been timed (at least one step), all host cores capped at 16."""
     import numpy as np
 
     from oracle import seblas_oracle as orc
 
     threads = min(os.cpu_count() or 1, 16)
-    nb = 64
+    nb = BATCH
     rng = np.random.default_rng(0)
     work = []
     flops = 0.0
@@ -117,19 +131,22 @@ def cpu_baseline(layers_spec):
         X = rng.standard_normal((nb, IC, H, H)).astype(np.float32)
         W = (rng.standard_normal((OC, IC, 3, 3)) * math.sqrt(2.0 / (IC * 9))).astype(np.float32)
         dY = rng.standard_normal((nb, OC, OH, OH)).astype(np.float32)
-        work.append((X, W, dY, H, s, mult))
+        work.append((X, W, dY, np.zeros_like(W), H, s, mult))
         flops += 3 * mult * 2.0 * nb * OC * OH * OH * IC * 9
+    steps, dt = 0, 0.0
     t0 = time.perf_counter()
-    for (X, W, dY, H, s, mult) in work:
-        for _ in range(mult):
-            orc.conv(W, X, None, s, s, 1, 1, threads=threads)
-            orc.convDerive(W, dY, (H, H), s, s, 1, 1, threads=threads)
-            orc.convError(dY, X, np.zeros_like(W), s, s, 1, 1, threads=threads)
-    dt = time.perf_counter() - t0
+    while steps == 0 or dt < min_seconds:
+        for (X, W, dY, dW, H, s, mult) in work:
+            for _ in range(mult):
+                orc.conv(W, X, None, s, s, 1, 1, threads=threads)
+                orc.convDerive(W, dY, (H, H), s, s, 1, 1, threads=threads)
+                orc.convError(dY, X, dW, s, s, 1, 1, threads=threads)
+        steps += 1
+        dt = time.perf_counter() - t0
     return {
-        "value": flops / dt / 1e12, "unit": "TFLOP/s", "cores": threads, "kind": "port",
-        "images_per_s": nb / dt, "seconds": dt,
-        "sample": f"one full ResNet-56 conv step (fwd+dgrad+wgrad, all 56 layers) at batch {nb} instead of {BATCH}, "
+        "value": flops * steps / dt / 1e12, "unit": "TFLOP/s", "cores": threads, "kind": "port",
+        "images_per_s": nb * steps / dt, "seconds": dt,
+        "sample": f"{steps} full ResNet-56 conv steps (fwd+dgrad+wgrad, all 56 layers) at batch {nb}, "
                   f"fp32 loop oracle, {threads} threads",
     }
 
@@ -195,7 +212,9 @@ def main():
     d = per[dom]
     roofline = {
         "bound": "mfma", "kernel": dom, "achieved": d["tflops"], "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s",
-        "frac": d["tflops"] / PEAK_FP32_MFMA_TFLOPS, "traffic": None,
+        "frac": d["tflops"] / PEAK_FP32_MFMA_TFLOPS, "traffic": MEASURED_HBM_BYTES.get(dom),
+        "traffic_unit": "bytes per launch (FETCH_SIZE x2.00 + WRITE_SIZE x1.00, rocprofv3 --pmc)",
+        "algorithmic_bytes": d["bytes"],
         "flops_per_launch": d["flops"], "avg_launch_ms": d["ms"],
         "share_of_step": d["ms"] * d["mult"] / sum(v["ms"] * v["mult"] for v in per.values()),
     }

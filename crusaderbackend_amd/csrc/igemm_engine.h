@@ -334,10 +334,60 @@ static __global__ void __launch_bounds__(256) splitk_reduce_kernel(const float *
     }
 }
 
+// Same reduction with 16-byte loads: OL lanes cover 4 * OL consecutive results of one slice (a full 128-byte line
+// or more), 256 / OL lanes walk the slices.  Needs count % 4 == 0 and 16-byte aligned pointers.
+template <int OL>
+static __global__ void __launch_bounds__(256) splitk_reduce_vec_kernel(const float *__restrict__ partial, float *__restrict__ C,
+                                                                       u32 count, u32 splits, ReduceEpi e, FastDiv bdiv) {
+    constexpr u32 ZL = 256 / OL, OUTS = 4 * OL;
+    __shared__ float red[ZL][OUTS + 4];
+    const u32 o = threadIdx.x % OL, g = threadIdx.x / OL;
+    const u32 i = blockIdx.x * OUTS + 4 * o;
+    float4 s0 = make_float4(0.f, 0.f, 0.f, 0.f), s1 = s0;
+    if (i < count) {
+        const float *p = partial + i;
+        u32 zz = g;
+        for (; zz + ZL < splits; zz += 2 * ZL) {
+            const float4 a = *reinterpret_cast<const float4 *>(p + size_t(zz) * count);
+            const float4 b = *reinterpret_cast<const float4 *>(p + size_t(zz + ZL) * count);
+            s0.x += a.x, s0.y += a.y, s0.z += a.z, s0.w += a.w;
+            s1.x += b.x, s1.y += b.y, s1.z += b.z, s1.w += b.w;
+        }
+        if (zz < splits) {
+            const float4 a = *reinterpret_cast<const float4 *>(p + size_t(zz) * count);
+            s0.x += a.x, s0.y += a.y, s0.z += a.z, s0.w += a.w;
+        }
+    }
+    *reinterpret_cast<float4 *>(&red[g][4 * o]) = make_float4(s0.x + s1.x, s0.y + s1.y, s0.z + s1.z, s0.w + s1.w);
+    __syncthreads();
+    const u32 j = blockIdx.x * OUTS + threadIdx.x;
+    if (threadIdx.x < OUTS && j < count) {
+        float r = red[0][threadIdx.x];
+#pragma unroll
+        for (u32 k = 1; k < ZL; ++k) r += red[k][threadIdx.x];
+        if (e.bias) r += e.bias[bdiv.div(j) % e.bias_mod];
+        if (e.flags & EPI_ACCUM) r += C[j];
+        if (e.flags & EPI_RELU) r = r > 0.f ? r : 0.f;
+        C[j] = r;
+    }
+}
+
 inline int launch_splitk_reduce(const float *partial, float *C, u32 count, u32 splits, ReduceEpi e, hipStream_t s,
                                 const char *what) {
     FastDiv bdiv(e.bias_div ? e.bias_div : 1);
     if (!e.bias_mod) e.bias_mod = 1;
+    if (count % 4 == 0 && reinterpret_cast<uintptr_t>(partial) % 16 == 0) {
+        // slice lanes ~ splits / 2, so every lane has at least two independent loads in flight
+        if (splits >= 64)
+            hipLaunchKernelGGL(splitk_reduce_vec_kernel<8>, dim3(ceil_div(count, 32)), dim3(256), 0, s, partial, C, count, splits, e, bdiv);
+        else if (splits >= 32)
+            hipLaunchKernelGGL(splitk_reduce_vec_kernel<16>, dim3(ceil_div(count, 64)), dim3(256), 0, s, partial, C, count, splits, e, bdiv);
+        else if (splits >= 16 || count < 256u * 512u)
+            hipLaunchKernelGGL(splitk_reduce_vec_kernel<32>, dim3(ceil_div(count, 128)), dim3(256), 0, s, partial, C, count, splits, e, bdiv);
+        else
+            hipLaunchKernelGGL(splitk_reduce_vec_kernel<64>, dim3(ceil_div(count, 256)), dim3(256), 0, s, partial, C, count, splits, e, bdiv);
+        return check_launch(what);
+    }
     // enough workgroups to cover the chip even when the result is small
     if (count >= 32u * 512u)
         hipLaunchKernelGGL(splitk_reduce_kernel<32>, dim3(ceil_div(count, 32)), dim3(256), 0, s, partial, C, count, splits, e, bdiv);
