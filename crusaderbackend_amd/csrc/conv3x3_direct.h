@@ -39,6 +39,9 @@ struct DirectCfg {
     static constexpr int W = W_, ROWS = ROWS_, CI = CI_, OCT = OCT_, PBW = PBW_, OBW = OBW_, OCC = OCC_, NBUF = NBUF_, S = S_;
     static constexpr int FS = FS_, NT = FS_ * FS_;  // filter size, taps
     static constexpr bool DGRAD = DGRAD_;
+    // W = 4: the grid is a 4x4 image and a tile is ROWS / 4 whole images stacked, each staged with its own halo rows
+    static constexpr bool MI = W_ == 4;
+    static constexpr int IMGS = MI ? ROWS_ / 4 : 1;
     static constexpr bool DG2 = DGRAD && S == 2;  // stride-2 data gradient (4 parity classes)
     static constexpr bool FW2 = !DGRAD && S == 2; // stride-2 forward
     static constexpr int NPH = DG2 ? 4 : 1;       // accumulator sets per MFMA tile
@@ -49,7 +52,7 @@ struct DirectCfg {
     static constexpr int NOBW = NOB / OBW;        // wave groups along channels
     // staged input: row width, row count, the input row LDS row 0 holds (ROW0_MUL*r0 + ROW0_ADD for first grid row r0)
     static constexpr int SW = FW2 ? 2 * W : W;
-    static constexpr int XR = FS == 1 ? ROWS : (DG2 ? ROWS + 1 : S * (ROWS - 1) + 3);
+    static constexpr int XR = MI ? IMGS * 6 : (FS == 1 ? ROWS : (DG2 ? ROWS + 1 : S * (ROWS - 1) + 3));
     static constexpr int ROW0_MUL = FW2 ? 2 : 1;
     static constexpr int ROW0_ADD = (DG2 || FS == 1) ? 0 : -1;
     static constexpr int PSTEP = FW2 ? 2 : 1;     // LDS distance of neighbouring grid pixels
@@ -68,7 +71,8 @@ struct DirectCfg {
     static constexpr int WSTR = WSTR_MIN + ((2 - WSTR_MIN % 4) + 4) % 4;
     static constexpr int X_SIZE = CI * XP;
     static constexpr int W_SIZE = OCT * WSTR;
-    static_assert(W == 8 || W == 16 || W == 32, "grid width");
+    static_assert(W == 4 || W == 8 || W == 16 || W == 32, "grid width");
+    static_assert(!MI || (S == 1 && FS == 3 && ROWS % 4 == 0), "stacked 4x4 images: 3x3 stride 1 only");
     static_assert(S == 1 || S == 2, "stride");
     static_assert(FS == 3 || (FS == 1 && S == 1), "1x1 filters are handled at stride 1 only");
     static_assert(TP % 16 == 0 && NPB % PBW == 0 && NOB % OBW == 0 && NPBW * NOBW == 4, "wave tiling must use 4 waves");
@@ -85,7 +89,10 @@ struct DirectCfg {
     }
     // parity class 2*py + px of dX that tap (fh, fw) contributes to (stride-2 data gradient), else 0
     static constexpr int tap_phase(int tap) { return DG2 ? (tap / 3 == 1 ? 0 : 2) + (tap % 3 == 1 ? 0 : 1) : 0; }
-    static constexpr int pix_off(int q) { return (q / W) * PSTEP * XS + (q % W) * PSTEP; }
+    static constexpr int pix_off(int q) {
+        if (MI) return ((q / 16) * 6 + (q % 16) / 4) * XS + q % 4;  // image q/16 of the stack, 6 staged rows each
+        return (q / W) * PSTEP * XS + (q % W) * PSTEP;
+    }
 };
 
 struct DirectArgs {
@@ -96,7 +103,8 @@ struct DirectArgs {
     u32 C_IN, C_OUT;
     u32 in_H;           // rows of the staged tensor
     u32 grid_H;         // rows of the pixel grid
-    u32 tiles_per_img, oc_tiles, tiles_total;  // tiles_total = N * tiles_per_img
+    u32 tiles_per_img, oc_tiles, tiles_total;  // tiles_total = N * tiles_per_img (stacked 4x4 images: ceil(N / IMGS))
+    u32 n_images;
     u32 relu;
 };
 
@@ -115,8 +123,8 @@ __global__ void __launch_bounds__(kThreads, Cfg::OCC) conv3x3_kernel(DirectArgs 
     const u32 oct = slot % a.oc_tiles;
     const u32 rest = (slot / a.oc_tiles) * kXcds + xcd;
     if (rest >= a.tiles_total) return;
-    const u32 tile = rest % a.tiles_per_img;
-    const u32 n = rest / a.tiles_per_img;
+    const u32 tile = Cfg::MI ? 0 : rest % a.tiles_per_img;
+    const u32 n = Cfg::MI ? rest * Cfg::IMGS : rest / a.tiles_per_img;  // (first) image of this tile
     const int r0 = int(tile) * ROWS;  // first grid row of this tile
     const int srow0 = Cfg::ROW0_MUL * r0 + Cfg::ROW0_ADD;  // input row held by LDS row 0
     const u32 oc0 = oct * OCT;
@@ -140,9 +148,11 @@ __global__ void __launch_bounds__(kThreads, Cfg::OCC) conv3x3_kernel(DirectArgs 
             v4f v = {0.f, 0.f, 0.f, 0.f};
             if (XQ % kThreads == 0 || e < XQ) {
                 const u32 q = e % (SW / 4), lr = (e / (SW / 4)) % XR, c = e / ((SW / 4) * XR);
-                const int row = srow0 + int(lr);
-                if (row >= 0 && row < int(a.in_H) && c0 + c < a.C_IN)
-                    v = *reinterpret_cast<const v4f *>(a.X + (size_t(n) * a.C_IN + c0 + c) * in_HW + u32(row) * SW + 4 * q);
+                // stacked images: staged row lr is row lr % 6 - 1 of image lr / 6 (rows -1 and 4 are its halo)
+                const int row = Cfg::MI ? int(lr % 6) - 1 : srow0 + int(lr);
+                const u32 img = Cfg::MI ? n + lr / 6 : n;
+                if (row >= 0 && row < int(a.in_H) && c0 + c < a.C_IN && (!Cfg::MI || img < a.n_images))
+                    v = *reinterpret_cast<const v4f *>(a.X + (size_t(img) * a.C_IN + c0 + c) * in_HW + u32(row) * SW + 4 * q);
             }
             xreg[i] = v;
         }
@@ -269,7 +279,9 @@ __global__ void __launch_bounds__(kThreads, Cfg::OCC) conv3x3_kernel(DirectArgs 
 #pragma unroll
         for (int p = 0; p < PBW; ++p) {
             const int q = (wp * PBW + p) * 16 + 4 * kq;
-            const u32 gy = u32(r0 + q / W), gx = u32(q % W);
+            const u32 gy = Cfg::MI ? u32((q % 16) / 4) : u32(r0 + q / W), gx = u32(q % W);
+            const u32 img = Cfg::MI ? n + u32(q / 16) : n;
+            if (Cfg::MI && img >= a.n_images) continue;
             if constexpr (Cfg::DG2) {
                 // grid pixel (gy, gx..gx+3) -> dX rows 2gy, 2gy+1, columns 2gx .. 2gx+7 (column parities interleaved)
                 float *base = a.Y + ((size_t(n) * a.C_OUT + oc) * (2 * a.grid_H) + 2 * gy) * (2 * W) + 2 * gx;
@@ -286,7 +298,7 @@ __global__ void __launch_bounds__(kThreads, Cfg::OCC) conv3x3_kernel(DirectArgs 
                     v.x = v.x > 0.f ? v.x : 0.f, v.y = v.y > 0.f ? v.y : 0.f;
                     v.z = v.z > 0.f ? v.z : 0.f, v.w = v.w > 0.f ? v.w : 0.f;
                 }
-                *reinterpret_cast<v4f *>(a.Y + ((size_t(n) * a.C_OUT + oc) * a.grid_H + gy) * W + gx) = v;
+                *reinterpret_cast<v4f *>(a.Y + ((size_t(img) * a.C_OUT + oc) * a.grid_H + gy) * W + gx) = v;
             }
         }
     }
@@ -296,6 +308,7 @@ __global__ void __launch_bounds__(kThreads, Cfg::OCC) conv3x3_kernel(DirectArgs 
 // (grid_H, grid_W) = extent of the pixel grid: the output image, or dY for the stride-2 data gradient.
 template <class Cfg>
 inline bool direct_fits(u32 C_IN, u32 grid_H, u32 grid_W) {
+    if (Cfg::MI) return grid_W == 4 && grid_H == 4 && (Cfg::NBUF == 1 ? C_IN <= u32(Cfg::CI) : true);
     return grid_W == u32(Cfg::W) && grid_H % Cfg::ROWS == 0 && (Cfg::NBUF == 1 ? C_IN <= u32(Cfg::CI) : true);
 }
 
@@ -305,9 +318,10 @@ inline int launch_direct(const float *Wt, const float *X, float *Y, const float 
     DirectArgs a;
     a.Wt = Wt, a.X = X, a.Y = Y, a.bias = bias;
     a.C_IN = C_IN, a.C_OUT = C_OUT, a.grid_H = grid_H, a.in_H = in_H;
-    a.tiles_per_img = grid_H / Cfg::ROWS;
+    a.tiles_per_img = Cfg::MI ? 1 : grid_H / Cfg::ROWS;
     a.oc_tiles = ceil_div(C_OUT, u32(Cfg::OCT));
-    a.tiles_total = N * a.tiles_per_img;
+    a.tiles_total = Cfg::MI ? ceil_div(N, u32(Cfg::IMGS)) : N * a.tiles_per_img;
+    a.n_images = N;
     a.relu = relu;
     const uint64_t wgs = uint64_t(ceil_div(a.tiles_total, kXcds)) * kXcds * a.oc_tiles;  // padded to whole XCD rounds
     if (wgs > 0x7fffffffull) return fail(CRB_EINVAL_SHAPE, "%s: launch grid too large", what);

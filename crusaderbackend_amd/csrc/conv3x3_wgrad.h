@@ -23,13 +23,15 @@
 
 namespace crb {
 
-// W_: dY width; TR_: dY rows per image per tile; TI_: images per tile; S_: stride.
+// W_: dY width; TR_: dY rows per image per tile; TI_: images per tile (more than 4: whole small images, TI/4 per wave);
+// S_: stride.
 template <int W_, int TR_, int TI_, int OCC_, int S_ = 1>
 struct WgradCfg {
     static constexpr int W = W_, TR = TR_, TI = TI_, OCC = OCC_, S = S_;
-    static constexpr int WPI = 4 / TI;         // waves per image of the tile
-    static constexpr int RW = TR / WPI;        // rows per wave
-    static constexpr int KW = RW * W;          // pixels per wave per tile
+    static constexpr int WPI = TI >= 4 ? 1 : 4 / TI;  // waves per image of the tile
+    static constexpr int IPW = TI >= 4 ? TI / 4 : 1;  // images per wave (small images: TR is the whole image height)
+    static constexpr int RW = TR / WPI;        // rows per wave (per image)
+    static constexpr int KW = IPW * RW * W;    // pixels per wave per tile
     static constexpr int NSTEP = KW / 4;       // MFMA steps per wave per tile
     static constexpr int YIMG = TR * W;        // dY floats per image per plane
     static constexpr int PL = (TR + 1) * W;    // stride 2: one parity plane (halo row above + TR rows)
@@ -43,7 +45,11 @@ struct WgradCfg {
     static constexpr int BUF = Y_SIZE + X_SIZE;      // one staging buffer (floats)
     static constexpr int RED_SIZE = 4 * 9 * 256 + 2304;  // cross-wave reduction scratch (floats), reuses the staging space
     static constexpr int SMEM = 2 * BUF > RED_SIZE ? 2 * BUF : RED_SIZE;
-    static_assert(TI == 1 || TI == 2 || TI == 4, "images per tile");
+    static_assert(TI == 1 || TI == 2 || TI == 4 || TI == 8 || TI == 16, "images per tile");
+    static_assert(IPW == 1 || S == 1, "several images per wave: stride 1 only");
+    // X offset of MFMA step s of a wave's pixel run: the dY run is flat across the wave's images, the X planes of
+    // consecutive images are XIMG apart (they carry halo rows)
+    static constexpr int x_off(int s) { return IPW == 1 ? 4 * s : (4 * s / YIMG) * XIMG + (4 * s) % YIMG; }
     static_assert(TR % WPI == 0 && KW % 4 == 0, "rows must split evenly over the waves");
     static_assert(S == 1 || S == 2, "stride");
     // LDS offset of tap (fh, fw) relative to the lane's X base (which already carries the 4 leading pad floats)
@@ -173,7 +179,7 @@ __global__ void __launch_bounds__(kThreads, Cfg::OCC) wgrad3x3_kernel(WgradArgs 
     // ---- per-lane fragment addressing ---------------------------------------------------------------------
     const int lane = t & 63, wave = t >> 6;
     const int li = lane & 15, kq = lane >> 4;
-    const int img_w = wave / Cfg::WPI, row_w = (wave % Cfg::WPI) * Cfg::RW;
+    const int img_w = (wave / Cfg::WPI) * Cfg::IPW, row_w = (wave % Cfg::WPI) * Cfg::RW;
     const int ybase = li * YP + kq + img_w * YIMG + row_w * W;
     const int xbase = li * XP + kq + 4 + img_w * XIMG + row_w * W;  // +4: leading pad floats
 
@@ -191,7 +197,7 @@ __global__ void __launch_bounds__(kThreads, Cfg::OCC) wgrad3x3_kernel(WgradArgs 
         auto read_step = [&](int s, int slot) {
             av[slot] = py[4 * s];
 #pragma unroll
-            for (int k = 0; k < 9; ++k) bv[slot][k] = px[4 * s + Cfg::tap_off(k)];
+            for (int k = 0; k < 9; ++k) bv[slot][k] = px[Cfg::x_off(s) + Cfg::tap_off(k)];
         };
         read_step(0, 0);
 #pragma unroll
@@ -279,6 +285,7 @@ struct WgradDirectPlan {
 template <class Cfg>
 inline bool wgrad_direct_fits(u32 N, u32 IC, u32 OC, u32 H, u32 Wd) {
     (void)IC, (void)OC;  // ragged channel blocks are zero-filled
+    if (Cfg::IPW > 1 && H != u32(Cfg::TR)) return false;  // a wave's pixel run must cover whole images
     return Wd == u32(Cfg::W) && H % Cfg::TR == 0 && N % Cfg::TI == 0;
 }
 

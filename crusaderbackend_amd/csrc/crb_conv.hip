@@ -131,6 +131,13 @@ static int try_direct(const float *Wt, const float *X, float *Y, const float *bi
             if (C_IN > 8) { CRB_TRY(8, 8, 16, 16, 1, 1, DG, 2, 2, 1) }
             CRB_TRY(8, 8, 8, 16, 1, 1, DG, 2, 2, 1)
             CRB_TRY(8, 4, 8, 32, 1, 1, DG, 2, 2, 1)
+        } else if (gW == 4) {  // 4x4 images, four stacked per tile
+            // too few four-image tiles for the chip: two images per tile
+            if (C_OUT > 32 && C_IN > 8 && ceil_div(N, 4u) * ceil_div(C_OUT, 64u) < 192) { CRB_TRY(4, 8, 16, 64, 1, 2, DG, 2, 2, 1) }
+            if (C_OUT > 32 && C_IN > 8) { CRB_TRY(4, 16, 16, 64, 1, 4, DG, 2, 2, 1) }
+            if (C_OUT > 16 && C_IN > 8) { CRB_TRY(4, 16, 16, 32, 1, 2, DG, 2, 2, 1) }
+            if (C_IN > 8) { CRB_TRY(4, 16, 16, 16, 1, 1, DG, 2, 2, 1) }
+            CRB_TRY(4, 16, 8, 16, 1, 1, DG, 2, 2, 1)
         }
     } else {
         if (gW == 32) {
@@ -234,6 +241,9 @@ static bool wgrad_direct(const crb_conv_geom *g, bool run, const float *dY, cons
         if (g->OW == 8)
             return wgrad_cfg<WgradCfg<8, 8, 4, 2, 1>>(g, run, dY, X, dW, ws, s, plan, status) ||
                    wgrad_cfg<WgradCfg<8, 8, 2, 2, 1>>(g, run, dY, X, dW, ws, s, plan, status);
+        if (g->OW == 4)  // 4x4 images: 8 (or 4) whole images per tile
+            return wgrad_cfg<WgradCfg<4, 4, 8, 2, 1>>(g, run, dY, X, dW, ws, s, plan, status) ||
+                   wgrad_cfg<WgradCfg<4, 4, 4, 2, 1>>(g, run, dY, X, dW, ws, s, plan, status);
     } else if (direct_shape(g, 2)) {
         if (g->OW == 32) return wgrad_cfg<WgradCfg<32, 4, 1, 1, 2>>(g, run, dY, X, dW, ws, s, plan, status);
         if (g->OW == 16) return wgrad_cfg<WgradCfg<16, 8, 1, 1, 2>>(g, run, dY, X, dW, ws, s, plan, status);
