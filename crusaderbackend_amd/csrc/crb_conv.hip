@@ -217,6 +217,11 @@ static bool direct_shape(const crb_conv_geom *g, u32 stride) {
            g->IH == stride * g->OH && g->IW == stride * g->OW;
 }
 
+// 3x3 / pad 1 / stride 1 on 2x2 images: dense products over (channel, pixel) pairs (gemm_internal.h)
+static bool tiny2x2_shape(const crb_conv_geom *g) {
+    return direct_shape(g, 1) && g->IH == 2 && g->IW == 2 && uint64_t(g->OC) * g->IC * 16 <= 0x7fffffffull;
+}
+
 // ---- direct 3x3 / pad 1 weight gradient (stride 1 and 2) ---------------------------------------------------------
 // One entry per configuration <W, TR, TI, OCC>; `run` = false only computes the plan (workspace size).
 constexpr u32 kWgradTargetWgs = 256;  // one workgroup per CU: pairs x splits
@@ -305,6 +310,8 @@ int crb_conv_fwd(const float *W, const float *X, float *Y, const float *bias_or_
     if (pointwise_shape(g))
         return gemm_nn_rowbias(W, X, Y, g->OC, g->IH * g->IW, g->IC, g->N, bias_or_null,
                                (flags & CRB_FLAG_RELU) ? u32(EPI_RELU) : 0u, s, "crb_conv_fwd");
+    if (tiny2x2_shape(g) && aligned16(X) && aligned16(Y))
+        return conv2x2_fwd(W, X, Y, bias_or_null, g->N, g->IC, g->OC, (flags & CRB_FLAG_RELU) ? u32(EPI_RELU) : 0u, s, "crb_conv_fwd");
     if (aligned16(X) && aligned16(Y) && (direct_shape(g, 1) || direct_shape(g, 2))) {
         bool done;
         int st = g->sH == 1 ? try_direct<false, 1>(W, X, Y, bias_or_null, g->N, g->IC, g->OC, g->OH, g->OW, g->IH,
@@ -332,6 +339,8 @@ int crb_conv_dgrad(const float *W, const float *dY, float *dX, const crb_conv_ge
     }
     if (pointwise_shape(g))
         return gemm_tn_batched(W, dY, dX, g->IC, g->IH * g->IW, g->OC, g->N, hipStream_t(stream), "crb_conv_dgrad");
+    if (tiny2x2_shape(g) && aligned16(dY) && aligned16(dX))
+        return conv2x2_dgrad(W, dY, dX, g->N, g->IC, g->OC, hipStream_t(stream), "crb_conv_dgrad");
     if (aligned16(dY) && aligned16(dX) && (direct_shape(g, 1) || direct_shape(g, 2))) {
         bool done;
         // the pixel grid and the staged tensor are dY in both cases (at stride 1 dY and dX have the same extent)
@@ -360,6 +369,7 @@ int crb_conv_dgrad(const float *W, const float *dY, float *dX, const crb_conv_ge
 size_t crb_conv_wgrad_workspace_bytes(const crb_conv_geom *g) {
     if (check_geom("crb_conv_wgrad_workspace_bytes", g)) return 0;
     if (pointwise_shape(g)) return 0;  // accumulate-NT GEMM form; its split scratch comes from the library arena
+    if (tiny2x2_shape(g)) return size_t(g->OC) * g->IC * 16 * sizeof(float);  // (oc, p) x (ic, p') product before the tap fold
     {
         WgradDirectPlan dp;
         int st = 0;
@@ -375,6 +385,18 @@ int crb_conv_wgrad(const float *dY, const float *X, float *dW, const crb_conv_ge
     if (int st = check_geom("crb_conv_wgrad", g)) return st;
     hipStream_t s = hipStream_t(stream);
     if (pointwise_shape(g)) return crb_sgemm_nta(dY, X, dW, g->OC, g->IC, g->IH * g->IW, g->N, stream);
+    if (tiny2x2_shape(g) && aligned16(dY) && aligned16(X)) {
+        const size_t need = size_t(g->OC) * g->IC * 16 * sizeof(float);
+        float *G = static_cast<float *>(workspace);
+        if (G) {
+            if (workspace_bytes < need || !aligned16(G))
+                return fail(CRB_EWORKSPACE, "crb_conv_wgrad: workspace %zu bytes < required %zu (or not 16-byte aligned)", workspace_bytes, need);
+        } else {
+            G = static_cast<float *>(arena_get(need));
+            if (!G) return fail(CRB_EHIP, "crb_conv_wgrad: cannot allocate %zu bytes of scratch", need);
+        }
+        return conv2x2_wgrad(dY, X, dW, G, g->N, g->IC, g->OC, s, "crb_conv_wgrad");
+    }
     if (aligned16(dY) && aligned16(X)) {
         WgradDirectPlan dp;
         int st = CRB_OK;

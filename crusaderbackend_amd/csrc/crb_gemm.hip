@@ -26,7 +26,8 @@ static int run_cfg(const AOp &a, const BOp &b, const RowMajorEpi &e, u32 M, u32 
     RowMajorEpi pe{ws, nullptr, N, M * N, 0u};
     if (int st = launch_igemm<Cfg>(a, b, pe, M, N, K, sp.splits, 1, sp.k_per_z, s, what)) return st;
     if (e.row_bias) return launch_splitk_reduce(ws, e.C, M * N, sp.splits, ReduceEpi{e.row_bias, N, M, e.flags}, s, what);
-    return launch_splitk_reduce(ws, e.C, M * N, sp.splits, ReduceEpi{e.col_bias, 1, N, e.flags}, s, what);
+    return launch_splitk_reduce(ws, e.C, M * N, sp.splits, ReduceEpi{e.col_bias, 1u << e.col_bias_shift, N >> e.col_bias_shift, e.flags},
+                                s, what);
 }
 
 template <class AOp, class BOp>
@@ -121,6 +122,61 @@ static int gemm_nt(const float *A, const float *B, float *C, u32 M, u32 N, u32 K
     MatK<false> a{A, M, K, 0};
     MatK<false> b{B, N, K, 0};
     return run_tiles(a, b, e, M, N, K, 1, s, what);
+}
+
+// ---- 3x3 / pad 1 / stride 1 convolution of 2x2 images as dense products over (channel, pixel) pairs -------------------
+// X, Y, dY, dX are then plain row-major matrices: N x (C*4).
+
+int conv2x2_fwd(const float *W, const float *X, float *Y, const float *bias, u32 N, u32 IC, u32 OC, u32 flags, hipStream_t s,
+                const char *what) {
+    // Y (N x OC*4) = X (N x IC*4) * Wp^T, bias per group of 4 columns
+    RowMajorEpi e{Y, bias, OC * 4, 0, flags};
+    e.col_bias_shift = 2;
+    MatK<true> a{X, N, IC * 4, 0};
+    TapPairs b{W, OC * 4, IC, true};
+    return run_tiles(a, b, e, N, OC * 4, IC * 4, 1, s, what);
+}
+
+int conv2x2_dgrad(const float *W, const float *dY, float *dX, u32 N, u32 IC, u32 OC, hipStream_t s, const char *what) {
+    // dX (N x IC*4) = dY (N x OC*4) * Wp
+    RowMajorEpi e{dX, nullptr, IC * 4, 0, 0u};
+    MatK<true> a{dY, N, OC * 4, 0};
+    TapPairs b{W, IC * 4, IC, false};
+    return run_tiles(a, b, e, N, IC * 4, OC * 4, 1, s, what);
+}
+
+// dW[oc][ic][tap] += sum over the (p, p') pairs that meet in that tap of G[oc*4 + p][ic*4 + p'] (1, 2 or 4 pairs per tap)
+__global__ void __launch_bounds__(256) conv2x2_fold_kernel(const float *__restrict__ G, float *__restrict__ dW, u32 OC, u32 IC) {
+    const u32 i = blockIdx.x * 256 + threadIdx.x;  // (oc, ic) pair
+    if (i >= OC * IC) return;
+    const u32 oc = i / IC, ic = i % IC;
+    float acc[9];
+#pragma unroll
+    for (int t = 0; t < 9; ++t) acc[t] = 0.f;
+#pragma unroll
+    for (int p = 0; p < 4; ++p) {
+        const v4f g = *reinterpret_cast<const v4f *>(G + (size_t(oc) * 4 + p) * (IC * 4) + ic * 4);
+        const int o = 4 - 3 * (p >> 1) - (p & 1);
+        acc[o + 0] += g.x, acc[o + 1] += g.y, acc[o + 3] += g.z, acc[o + 4] += g.w;
+    }
+    float *dst = dW + size_t(i) * 9;
+#pragma unroll
+    for (int t = 0; t < 9; ++t) dst[t] += acc[t];
+}
+
+int conv2x2_wgrad(const float *dY, const float *X, float *dW, float *G, u32 N, u32 IC, u32 OC, hipStream_t s, const char *what) {
+    // G (OC*4 x IC*4, caller's scratch) = dY^T * X over the batch, then folded into the 9 taps
+    const u32 M = OC * 4, Nc = IC * 4;
+    RowMajorEpi e{G, nullptr, Nc, 0, 0u};
+    MatR<true> a{dY, M, M, 0};
+    MatR<true> b{X, Nc, Nc, 0};
+    // G may be the library's scratch arena, so the contraction is never split here
+    const uint64_t tiles_l = uint64_t(ceil_div(M, 128)) * ceil_div(Nc, 128);
+    int st = tiles_l >= 128 ? launch_igemm<CfgLarge>(a, b, e, M, Nc, N, 1, 0, N, s, what)
+                            : launch_igemm<CfgSmall>(a, b, e, M, Nc, N, 1, 0, N, s, what);
+    if (st) return st;
+    hipLaunchKernelGGL(conv2x2_fold_kernel, dim3(ceil_div(OC * IC, 256)), dim3(256), 0, s, G, dW, OC, IC);
+    return check_launch(what);
 }
 
 int gemm_nn_rowbias(const float *A, const float *B, float *C, u32 M, u32 N, u32 K, u32 batch, const float *row_bias, u32 flags,

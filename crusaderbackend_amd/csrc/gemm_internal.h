@@ -9,4 +9,11 @@ int gemm_nn_rowbias(const float *A, const float *B, float *C, u32 M, u32 N, u32 
                     hipStream_t s, const char *what);
 // For nd < batch: C[nd] (M x N) = A^T * B[nd], A stored K x M.
 int gemm_tn_batched(const float *A, const float *B, float *C, u32 M, u32 N, u32 K, u32 batch, hipStream_t s, const char *what);
+// 3x3 / pad 1 / stride 1 convolution on 2x2 images (every input pixel reaches every output pixel through one tap):
+// dense products over (channel, pixel) pairs. All tensors 16-byte aligned. dW is accumulated.
+int conv2x2_fwd(const float *W, const float *X, float *Y, const float *bias, u32 N, u32 IC, u32 OC, u32 flags, hipStream_t s,
+                const char *what);
+int conv2x2_dgrad(const float *W, const float *dY, float *dX, u32 N, u32 IC, u32 OC, hipStream_t s, const char *what);
+// G: scratch of OC*4 x IC*4 floats.
+int conv2x2_wgrad(const float *dY, const float *X, float *dW, float *G, u32 N, u32 IC, u32 OC, hipStream_t s, const char *what);
 }  // namespace crb

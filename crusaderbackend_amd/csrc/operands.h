@@ -121,6 +121,39 @@ struct SepK {
     }
 };
 
+// ---- 3x3 / pad 1 / stride 1 filters seen from a 2x2 image --------------------------------------------------------
+// On a 2x2 image every input pixel p' = (y', x') reaches every output pixel p = (y, x) through exactly one tap,
+// (fh, fw) = (y' - y + 1, x' - x + 1), so the convolution is a dense product over (channel, pixel) pairs with
+//   Wp[oc*4 + p][ic*4 + p'] = W[oc][ic][tap],  tap = 3*fh + fw = (4 - 3y - x) + (3y' + x'):
+// the filter offset separates into an output-side and an input-side part. This operand presents W in that form.
+// element(row, k) = base[side(row) + side(k)], side(i) = (i / 4)*stride + (out ? 4 - 3*((i/2)%2) - i%2 : 3*((i/2)%2) + i%2).
+// rows_out = true: rows are (oc, p) pairs and k runs over (ic, p') (forward); false: the roles are swapped (data gradient).
+struct TapPairs {
+    static constexpr bool kKFast = true, kVec = false;
+    const float *base;
+    u32 rows;
+    u32 IC;  // input channels of the forward convolution
+    bool rows_out;
+    struct RowS {
+        u32 off;
+        bool ok;
+    };
+    struct KS {
+        u32 off;
+        bool ok;
+    };
+    __device__ __forceinline__ void bind(u32) {}
+    __device__ __forceinline__ u32 side(u32 i, bool out) const {
+        const u32 y = (i >> 1) & 1, x = i & 1;
+        return out ? (i >> 2) * IC * 9 + 4 - 3 * y - x : (i >> 2) * 9 + 3 * y + x;
+    }
+    __device__ __forceinline__ RowS prep_row(u32 row) const { return {side(row, rows_out), row < rows}; }
+    __device__ __forceinline__ KS prep_k(u32 k, u32 klimit) const { return {side(k, !rows_out), k < klimit}; }
+    __device__ __forceinline__ float fetch(const RowS &r, const KS &k) const {
+        return (r.ok && k.ok) ? base[r.off + k.off] : 0.0f;
+    }
+};
+
 // ---- implicit im2col gather ---------------------------------------------------------------------------
 // value(pixel j = (n, oh, ow), tap t = (ic, fh, fw)) = X[n, ic, oh*sH - pH + fh, ow*sW - pW + fw], 0 outside.
 struct Im2col {
@@ -233,6 +266,7 @@ struct RowMajorEpi {
     const float *col_bias;
     u32 ld, zstride, flags;
     const float *row_bias = nullptr;
+    u32 col_bias_shift = 0;  // column c takes col_bias[c >> shift] (groups of 2^shift columns share a bias)
     struct ColS {
         u32 col;
         float bias;
@@ -241,7 +275,7 @@ struct RowMajorEpi {
     __device__ __forceinline__ void bind(u32 z) { C += size_t(z) * zstride; }
     __device__ __forceinline__ ColS prep_col(u32 col, u32 ncols) const {
         const bool ok = col < ncols;
-        return {col, (ok && col_bias) ? col_bias[col] : 0.0f, ok};
+        return {col, (ok && col_bias) ? col_bias[col >> col_bias_shift] : 0.0f, ok};
     }
     __device__ __forceinline__ void store(u32 row, const ColS &c, float v) const {
         if (!c.ok) return;

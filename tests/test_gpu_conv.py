@@ -234,9 +234,19 @@ def test_conv3x3_direct_configs(dev, N, IC, H, W, OC):
     run_layer(dev, N, IC, H, W, OC, 3, 3, 1, 1, 1, 1, bias=True, seed=11)
 
 
+# 3x3 / pad 1 / stride 1 on 2x2 images: dense products over (channel, pixel) pairs. (N, IC, OC)
+TINY2 = [(3, 5, 7), (128, 64, 48), (2, 1, 1), (7, 33, 130), (130, 20, 16), (64, 128, 96)]
+
+
+@pytest.mark.parametrize("N,IC,OC", TINY2)
+def test_conv3x3_on_2x2_images(dev, N, IC, OC):
+    run_layer(dev, N, IC, 2, 2, OC, 3, 3, 1, 1, 1, 1, bias=True, seed=41)
+    run_layer(dev, N, IC, 2, 2, OC, 3, 3, 1, 1, 1, 1, bias=False, seed=42, ws=True)
+
+
 def test_conv_relu_flag(dev):
     capi, orc = _capi(), _oracle()
-    for (N, IC, H, OC) in [(2, 16, 32, 16), (2, 5, 9, 7)]:  # direct path and implicit-GEMM path
+    for (N, IC, H, OC) in [(2, 16, 32, 16), (2, 5, 9, 7), (9, 6, 2, 5)]:  # direct, implicit-GEMM and 2x2-image paths
         g = capi.ConvGeom.make(N, IC, H, H, OC, 3, 3, 1, 1, 1, 1)
         X, W, b = normal(1, N, IC, H, H), he_normal(2, OC, IC, 3, 3), normal(3, OC)
         Y = _nan(dev, N, OC, H, H)
