@@ -406,7 +406,7 @@ inline SplitPlan plan_split(u32 M, u32 N, u32 K, u32 BM, u32 BN, u32 BK, u32 zdi
     SplitPlan p{1, K};
     const uint64_t tiles = uint64_t(ceil_div(M, BM)) * ceil_div(N, BN) * zdim;
     if (zdim != 1 || tiles >= 160) return p;
-    u32 want = u32(ceil_div(256u, u32(tiles)));
+    u32 want = u32(ceil_div(512u, u32(tiles)));
     const u32 max_by_k = K / (8 * BK) ? K / (8 * BK) : 1;  // keep at least 8 slabs per slice
     if (want > max_by_k) want = max_by_k;
     if (want <= 1) return p;
