@@ -101,6 +101,20 @@ MEASURED_HBM_BYTES = {
 }
 
 
+def device_clock_khz():
+    """Peak engine clock of device 0 in kHz (hipDeviceAttributeClockRate), 0 if the runtime cannot be asked."""
+    import ctypes
+
+    try:
+        hip = ctypes.CDLL("libamdhip64.so")
+        v = ctypes.c_int(0)
+        if hip.hipDeviceGetAttribute(ctypes.byref(v), 5, 0) == 0:  # 5 = hipDeviceAttributeClockRate
+            return v.value
+    except OSError:
+        pass
+    return 0
+
+
 def event_time_ms(torch, fn, reps, warm=3):
     """Average duration of `fn` (ms) over `reps` back-to-back launches between two events on the launch stream."""
     for _ in range(warm):
@@ -229,6 +243,8 @@ def main():
     gemm_tflops = 2.0 * n ** 3 / gemm_ms / 1e9
     del A, B, C
 
+    clock_khz = device_clock_khz()
+
     out = {
         "metric": "fp32 conv TFLOP/s, ResNet-56 conv layers fwd+dgrad+wgrad (also % FP32 MFMA peak, images/s in extra)",
         "value": tflops, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -247,7 +263,9 @@ def main():
             "sgemm_4096_frac_peak": gemm_tflops / PEAK_FP32_MFMA_TFLOPS,
             "per_kernel": {k: {"ms": round(v["ms"], 5), "tflops": round(v["tflops"], 2), "gbs": round(v["gbs"], 1)}
                            for k, v in per.items()},
-            "device": props.name, "cus": props.multi_processor_count,
+            "device": props.name, "cus": props.multi_processor_count, "clock_mhz": clock_khz / 1e3,
+            # 256 flop per clock per CU on the fp32 matrix pipe, at the peak clock the device reports
+            "peak_from_reported_clock_tflops": props.multi_processor_count * clock_khz * 1e3 * 256 / 1e12,
         },
     }
     if not args.no_cpu:

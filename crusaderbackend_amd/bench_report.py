@@ -9,6 +9,7 @@ import math
 PEAK_TF = 157.3
 PEAK_GBS = 8000.0
 RIDGE = PEAK_TF * 1e3 / PEAK_GBS  # flop per byte
+COLD_FOOTPRINT = 640e6  # bytes of distinct operands cycled through for the cold-cache figures
 
 
 def _entry(name, ms, flops, nbytes):
@@ -35,9 +36,32 @@ def run(torch, capi, dev, event_time_ms, Layer):
     def conv_entries(key, specs, batch, bias):
         for i, (name, IC, H, OC, F, s, p) in enumerate(specs):
             L = Layer(torch, capi, dev, name, IC, H, OC, s, 1, seed=100 + i, batch=batch, F=F, pad=p, bias=bias)
+            entries = {}
             for pname, fn in L.passes():
                 reps = 30 if L.flops < 2e9 else 10
-                out[key].append(_entry(f"{name}.{pname}", event_time_ms(torch, fn, reps=reps), L.flops, L.bytes[pname]))
+                entries[pname] = _entry(f"{name}.{pname}", event_time_ms(torch, fn, reps=reps), L.flops, L.bytes[pname])
+                out[key].append(entries[pname])
+            # Bandwidth-bound shapes also get a cold-cache figure: the same call cycled over enough distinct buffer sets
+            # (>= 640 MB in total, beyond L2 and the 256 MB memory-side cache) that no launch finds its operands cached.
+            if any(e["bound"] == "hbm" for e in entries.values()):
+                per_set = max(L.bytes.values())
+                copies = min(int(COLD_FOOTPRINT // per_set) + 1, 64)
+                ring = [L] + [Layer(torch, capi, dev, name, IC, H, OC, s, 1, seed=100 + i, batch=batch, F=F, pad=p, bias=bias)
+                              for _ in range(copies - 1)]
+                for pname in entries:
+                    fns = [dict(R.passes())[pname] for R in ring]
+                    state = {"i": 0}
+
+                    def cyc():
+                        fns[state["i"] % len(fns)]()
+                        state["i"] += 1
+
+                    ms = event_time_ms(torch, cyc, reps=2 * len(fns), warm=len(fns))
+                    e = entries[pname]
+                    e["us_cold"] = round(ms * 1e3, 2)
+                    e["gbs_cold"] = round(L.bytes[pname] / ms / 1e6, 1)
+                    e["cold_sets"] = len(fns)
+                del ring
             del L
             torch.cuda.empty_cache()
 
@@ -100,8 +124,10 @@ def run(torch, capi, dev, event_time_ms, Layer):
 def to_markdown(rep):
     lines = []
     for key in ("gemm", "resnet56", "vgg16", "densenet", "dense"):
-        lines += [f"### {key}", "", "| shape.pass | us | GFLOP | MB | AI | TFLOP/s | GB/s | bound | fraction of roofline |", "|---|---|---|---|---|---|---|---|---|"]
+        lines += [f"### {key}", "", "| shape.pass | us | GFLOP | MB | AI | TFLOP/s | GB/s | bound | fraction of roofline | cold-cache us | cold GB/s |",
+                  "|---|---|---|---|---|---|---|---|---|---|---|"]
         for e in rep[key]:
-            lines.append(f"| {e['name']} | {e['us']} | {e['gflop']} | {e['mbytes']} | {e['ai']} | {e['tflops']} | {e['gbs']} | {e['bound']} | {e['frac'] * 100:.1f} % |")
+            cold = f"{e['us_cold']} | {e['gbs_cold']}" if "us_cold" in e else " | "
+            lines.append(f"| {e['name']} | {e['us']} | {e['gflop']} | {e['mbytes']} | {e['ai']} | {e['tflops']} | {e['gbs']} | {e['bound']} | {e['frac'] * 100:.1f} % | {cold} |")
         lines.append("")
     return "\n".join(lines)
