@@ -55,6 +55,17 @@ SIGNATURES = {
     "crb_conv_bias_grad": (ctypes.c_int, [_ptr, _ptr, _u32, _u32, _u32, _ptr]),
     "crb_tensor_add_inplace": (ctypes.c_int, [_ptr, _ptr, _u32, _ptr]),
     "crb_tensor_fill": (ctypes.c_int, [_ptr, ctypes.c_float, _u32, _ptr]),
+    "crb_tensor_sub_inplace": (ctypes.c_int, [_ptr, _ptr, _u32, _ptr]),
+    "crb_tensor_scale_inplace": (ctypes.c_int, [_ptr, ctypes.c_float, _u32, _ptr]),
+    "crb_relu_fwd": (ctypes.c_int, [_ptr, _ptr, _u32, _ptr]),
+    "crb_relu_bwd": (ctypes.c_int, [_ptr, _ptr, _ptr, _u32, _ptr]),
+    "crb_maxpool_fwd": (ctypes.c_int, [_ptr, _ptr, _ptr, _u32, _u32, _u32, _u32, _u32, _u32, _u32, _ptr]),
+    "crb_maxpool_bwd": (ctypes.c_int, [_ptr, _ptr, _ptr, _u32, _u32, _u32, _u32, _u32, _u32, _u32, _ptr]),
+    "crb_softmax": (ctypes.c_int, [_ptr, _ptr, _u32, _u32, _ptr]),
+    "crb_cross_entropy_grad": (ctypes.c_int, [_ptr, _ptr, _ptr, _u32, _ptr]),
+    "crb_cross_entropy_scratch_floats": (_u32, [_u32]),
+    "crb_cross_entropy_loss": (ctypes.c_int, [_ptr, _ptr, _ptr, _u32, _ptr, _u32, _ptr]),
+    "crb_momentum_apply": (ctypes.c_int, [_ptr, _ptr, _ptr, _u32, ctypes.c_float, ctypes.c_float, ctypes.c_float, _ptr]),
 }
 
 _lib = None
@@ -154,3 +165,49 @@ def tensor_add_inplace(a, b, count, stream=None):
 
 def tensor_fill(a, value, count, stream=None):
     check(load().crb_tensor_fill(_p(a), value, count, _stream(stream)))
+
+
+def tensor_sub_inplace(a, b, count, stream=None):
+    check(load().crb_tensor_sub_inplace(_p(a), _p(b), count, _stream(stream)))
+
+
+def tensor_scale_inplace(a, factor, count, stream=None):
+    check(load().crb_tensor_scale_inplace(_p(a), factor, count, _stream(stream)))
+
+
+def relu_fwd(X, Y, count, stream=None):
+    check(load().crb_relu_fwd(_p(X), _p(Y), count, _stream(stream)))
+
+
+def relu_bwd(X, dY, dX, count, stream=None):
+    check(load().crb_relu_bwd(_p(X), _p(dY), _p(dX), count, _stream(stream)))
+
+
+def maxpool_fwd(X, Y, record, planes, IH, IW, sH, sW, rH, rW, stream=None):
+    check(load().crb_maxpool_fwd(_p(X), _p(Y), _p(record), planes, IH, IW, sH, sW, rH, rW, _stream(stream)))
+
+
+def maxpool_bwd(dX, dY, record, planes, IH, IW, sH, sW, rH, rW, stream=None):
+    check(load().crb_maxpool_bwd(_p(dX), _p(dY), _p(record), planes, IH, IW, sH, sW, rH, rW, _stream(stream)))
+
+
+def softmax(A, out, rows, step, stream=None):
+    check(load().crb_softmax(_p(A), _p(out), rows, step, _stream(stream)))
+
+
+def cross_entropy_grad(Y, labels, dY, count, stream=None):
+    check(load().crb_cross_entropy_grad(_p(Y), _p(labels), _p(dY), count, _stream(stream)))
+
+
+def cross_entropy_scratch_floats(count):
+    return int(load().crb_cross_entropy_scratch_floats(count))
+
+
+def cross_entropy_loss(Y, labels, scratch, loss_out, count, stream=None):
+    """`loss_out`: one-element device tensor; `scratch`: device tensor of cross_entropy_scratch_floats(count) floats or None."""
+    n = 0 if scratch is None else scratch.numel()
+    check(load().crb_cross_entropy_loss(_p(Y), _p(labels), _p(scratch), n, _p(loss_out), count, _stream(stream)))
+
+
+def momentum_apply(X, G, M, count, lr, beta, decay=1.0, stream=None):
+    check(load().crb_momentum_apply(_p(X), _p(G), _p(M), count, lr, beta, decay, _stream(stream)))

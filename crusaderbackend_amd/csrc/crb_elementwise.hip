@@ -1,0 +1,414 @@
+// Elementwise and small reduction operators that sit between the GEMM / convolution calls of a training step:
+// ReLU and its gradient, max pooling (non-overlapping windows) and its gradient, row softmax, cross-entropy value and
+// gradient, in-place subtract / scale, and the momentum update with weight decay.
+// All are HBM-bound streaming kernels: 16-byte accesses where alignment allows, grid-stride loops, and reductions
+// with a fixed association (bit-reproducible, no atomics).
+#include "igemm_engine.h"
+
+namespace crb {
+
+static inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+static u32 stream_grid(u32 count) {
+    u32 blocks = ceil_div(ceil_div(count, 4), 256);
+    return blocks < 1 ? 1 : (blocks > 4096 ? 4096 : blocks);
+}
+
+// out[i] = f(in0[i], in1[i]) over `count` floats; quads when `vec`, scalars for the tail / unaligned buffers.
+// (no __restrict__: the in-place forms pass the same buffer as input and output)
+template <class F>
+__global__ void __launch_bounds__(256) map2_kernel(const float *a, const float *b, float *o,
+                                                   u32 count, u32 vec, F f) {
+    const u32 stride = gridDim.x * 256;
+    u32 i = blockIdx.x * 256 + threadIdx.x;
+    if (vec) {
+        const u32 nq = count / 4;
+        for (u32 q = i; q < nq; q += stride) {
+            const v4f x = reinterpret_cast<const v4f *>(a)[q];
+            const v4f y = b ? reinterpret_cast<const v4f *>(b)[q] : v4f{0.f, 0.f, 0.f, 0.f};
+            reinterpret_cast<v4f *>(o)[q] = v4f{f(x.x, y.x), f(x.y, y.y), f(x.z, y.z), f(x.w, y.w)};
+        }
+        for (u32 r = nq * 4 + i; r < count; r += stride) o[r] = f(a[r], b ? b[r] : 0.f);
+    } else {
+        for (; i < count; i += stride) o[i] = f(a[i], b ? b[i] : 0.f);
+    }
+}
+
+struct ReluF {
+    __device__ float operator()(float x, float) const { return x > 0.f ? x : 0.f; }
+};
+struct ReluGradF {  // (x, dy) -> dx
+    __device__ float operator()(float x, float dy) const { return x > 0.f ? dy : 0.f; }
+};
+struct SubF {
+    __device__ float operator()(float a, float b) const { return a - b; }
+};
+struct ScaleF {
+    float s;
+    __device__ float operator()(float a, float) const { return a * s; }
+};
+
+template <class F>
+static int launch_map2(const float *a, const float *b, float *o, u32 count, F f, hipStream_t s, const char *what) {
+    const u32 vec = aligned16(a) && aligned16(o) && (!b || aligned16(b));
+    hipLaunchKernelGGL((map2_kernel<F>), dim3(stream_grid(count)), dim3(256), 0, s, a, b, o, count, vec, f);
+    return check_launch(what);
+}
+
+// ---- max pooling, windows rH x rW, stride = window ------------------------------------------------------------------
+// One thread per window. X plane IH x IW; record plane RH x RW = (OH*rH) x (OW*rW). The first maximum in row-major
+// window order wins (strict '>', start value -1e15).
+__global__ void __launch_bounds__(256) maxpool_fwd_kernel(const float *__restrict__ X, float *__restrict__ Y, float *__restrict__ rec,
+                                                          u32 windows, u32 IH, u32 IW, u32 rH, u32 rW, FastDiv ow_div,
+                                                          FastDiv oh_div) {
+    const u32 w = blockIdx.x * 256 + threadIdx.x;
+    if (w >= windows) return;
+    u32 t, ow, p, oh;
+    ow_div.divmod(w, t, ow);
+    oh_div.divmod(t, p, oh);
+    const u32 OH = oh_div.d, OW = ow_div.d;
+    const float *x = X + (size_t(p) * IH + oh * rH) * IW + ow * rW;
+    float best = -1e15f;
+    u32 bi = 0, bj = 0;
+    for (u32 i = 0; i < rH; ++i)
+        for (u32 j = 0; j < rW; ++j) {
+            const float v = x[i * IW + j];
+            if (v > best) best = v, bi = i, bj = j;
+        }
+    float *r = rec + (size_t(p) * OH * rH + oh * rH) * (OW * rW) + ow * rW;
+    for (u32 i = 0; i < rH; ++i)
+        for (u32 j = 0; j < rW; ++j) r[i * (OW * rW) + j] = (i == bi && j == bj) ? 1.f : 0.f;
+    Y[w] = best;
+}
+
+// 2x2 windows on rows of even length with 16-byte aligned planes: one thread per pair of horizontally adjacent
+// windows, i.e. one quad of each of the two input rows.
+__global__ void __launch_bounds__(256) maxpool2x2_fwd_kernel(const float *__restrict__ X, float *__restrict__ Y,
+                                                             float *__restrict__ rec, u32 pairs, u32 IW, FastDiv qdiv) {
+    const u32 e = blockIdx.x * 256 + threadIdx.x;  // (plane*OH + oh, quad)
+    if (e >= pairs) return;
+    u32 row, q;
+    qdiv.divmod(e, row, q);
+    const float *x = X + size_t(row) * 2 * IW + 4 * q;
+    const v4f a = *reinterpret_cast<const v4f *>(x), b = *reinterpret_cast<const v4f *>(x + IW);
+    v4f ra = {0.f, 0.f, 0.f, 0.f}, rb = ra;
+    float y[2];
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+        const float v00 = h ? a.z : a.x, v01 = h ? a.w : a.y, v10 = h ? b.z : b.x, v11 = h ? b.w : b.y;
+        float best = -1e15f;
+        int k = 0;
+        if (v00 > best) best = v00, k = 0;
+        if (v01 > best) best = v01, k = 1;
+        if (v10 > best) best = v10, k = 2;
+        if (v11 > best) best = v11, k = 3;
+        y[h] = best;
+        if (h == 0) ra.x = k == 0, ra.y = k == 1, rb.x = k == 2, rb.y = k == 3;
+        else ra.z = k == 0, ra.w = k == 1, rb.z = k == 2, rb.w = k == 3;
+    }
+    float *r = rec + size_t(row) * 2 * IW + 4 * q;  // record has the extent of X here (IH, IW even)
+    *reinterpret_cast<v4f *>(r) = ra;
+    *reinterpret_cast<v4f *>(r + IW) = rb;
+    *reinterpret_cast<v2f *>(Y + size_t(row) * (IW / 2) + 2 * q) = v2f{y[0], y[1]};
+}
+
+// One thread per window: the first maximum of the record window receives dY, the rest of the window 0; the used
+// record entry is cleared.
+__global__ void __launch_bounds__(256) maxpool_bwd_kernel(float *__restrict__ dX, const float *__restrict__ dY, float *__restrict__ rec,
+                                                          u32 windows, u32 IH, u32 IW, u32 rH, u32 rW, FastDiv ow_div,
+                                                          FastDiv oh_div) {
+    const u32 w = blockIdx.x * 256 + threadIdx.x;
+    if (w >= windows) return;
+    u32 t, ow, p, oh;
+    ow_div.divmod(w, t, ow);
+    oh_div.divmod(t, p, oh);
+    const u32 OH = oh_div.d, OW = ow_div.d;
+    float *r = rec + (size_t(p) * OH * rH + oh * rH) * (OW * rW) + ow * rW;
+    float best = -1e15f;
+    u32 bi = 0, bj = 0;
+    for (u32 i = 0; i < rH; ++i)
+        for (u32 j = 0; j < rW; ++j) {
+            const float v = r[i * (OW * rW) + j];
+            if (v > best) best = v, bi = i, bj = j;
+        }
+    const float g = dY[w];
+    float *x = dX + (size_t(p) * IH + oh * rH) * IW + ow * rW;
+    for (u32 i = 0; i < rH; ++i)
+        for (u32 j = 0; j < rW; ++j) x[i * IW + j] = (i == bi && j == bj) ? g : 0.f;
+    r[bi * (OW * rW) + bj] = 0.f;
+}
+
+__global__ void __launch_bounds__(256) maxpool2x2_bwd_kernel(float *__restrict__ dX, const float *__restrict__ dY,
+                                                             float *__restrict__ rec, u32 pairs, u32 IW, FastDiv qdiv) {
+    const u32 e = blockIdx.x * 256 + threadIdx.x;
+    if (e >= pairs) return;
+    u32 row, q;
+    qdiv.divmod(e, row, q);
+    float *r = rec + size_t(row) * 2 * IW + 4 * q;
+    v4f ra = *reinterpret_cast<const v4f *>(r), rb = *reinterpret_cast<const v4f *>(r + IW);
+    const v2f g = *reinterpret_cast<const v2f *>(dY + size_t(row) * (IW / 2) + 2 * q);
+    v4f xa = {0.f, 0.f, 0.f, 0.f}, xb = xa;
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+        const float v00 = h ? ra.z : ra.x, v01 = h ? ra.w : ra.y, v10 = h ? rb.z : rb.x, v11 = h ? rb.w : rb.y;
+        float best = -1e15f;
+        int k = 0;
+        if (v00 > best) best = v00, k = 0;
+        if (v01 > best) best = v01, k = 1;
+        if (v10 > best) best = v10, k = 2;
+        if (v11 > best) best = v11, k = 3;
+        const float gv = h ? g.y : g.x;
+        if (h == 0) {
+            xa.x = k == 0 ? gv : 0.f, xa.y = k == 1 ? gv : 0.f, xb.x = k == 2 ? gv : 0.f, xb.y = k == 3 ? gv : 0.f;
+            if (k == 0) ra.x = 0.f; else if (k == 1) ra.y = 0.f; else if (k == 2) rb.x = 0.f; else rb.y = 0.f;
+        } else {
+            xa.z = k == 0 ? gv : 0.f, xa.w = k == 1 ? gv : 0.f, xb.z = k == 2 ? gv : 0.f, xb.w = k == 3 ? gv : 0.f;
+            if (k == 0) ra.z = 0.f; else if (k == 1) ra.w = 0.f; else if (k == 2) rb.z = 0.f; else rb.w = 0.f;
+        }
+    }
+    float *x = dX + size_t(row) * 2 * IW + 4 * q;
+    *reinterpret_cast<v4f *>(x) = xa;
+    *reinterpret_cast<v4f *>(x + IW) = xb;
+    *reinterpret_cast<v4f *>(r) = ra;
+    *reinterpret_cast<v4f *>(r + IW) = rb;
+}
+
+// ---- block-wide reductions with a fixed association (256 threads) ------------------------------------------------------
+template <bool MAX>
+__device__ __forceinline__ float block_reduce(float v, float *sh) {
+    const u32 t = threadIdx.x;
+    sh[t] = v;
+    __syncthreads();
+#pragma unroll
+    for (u32 s = 128; s > 0; s >>= 1) {
+        if (t < s) sh[t] = MAX ? (sh[t] > sh[t + s] ? sh[t] : sh[t + s]) : sh[t] + sh[t + s];
+        __syncthreads();
+    }
+    const float r = sh[0];
+    __syncthreads();
+    return r;
+}
+
+// Row softmax: out = exp(a - max) / (sum exp(a - max) + 1e-10). One workgroup per row (any row length).
+__global__ void __launch_bounds__(256) softmax_rows_kernel(const float *__restrict__ A, float *__restrict__ out, u32 step) {
+    __shared__ float sh[256];
+    const float *a = A + size_t(blockIdx.x) * step;
+    float *o = out + size_t(blockIdx.x) * step;
+    float mx = -1e15f;
+    for (u32 i = threadIdx.x; i < step; i += 256) mx = a[i] > mx ? a[i] : mx;
+    mx = block_reduce<true>(mx, sh);
+    float sum = 0.f;
+    for (u32 i = threadIdx.x; i < step; i += 256) {
+        const float e = expf(a[i] - mx);
+        o[i] = e;
+        sum += e;
+    }
+    sum = block_reduce<false>(sum, sh);
+    const float den = sum + 1e-10f;
+    for (u32 i = threadIdx.x; i < step; i += 256) o[i] = o[i] / den;
+}
+
+// Short rows (step <= 64): one wave per row, 4 rows per workgroup, lanes reduced with cross-lane shuffles in a
+// fixed butterfly order.
+__global__ void __launch_bounds__(256) softmax_short_kernel(const float *__restrict__ A, float *__restrict__ out, u32 rows, u32 step) {
+    const u32 row = blockIdx.x * 4 + threadIdx.x / 64, lane = threadIdx.x % 64;
+    if (row >= rows) return;
+    const bool on = lane < step;
+    const float v = on ? A[size_t(row) * step + lane] : -1e15f;
+    float mx = v;
+#pragma unroll
+    for (int m = 32; m > 0; m >>= 1) {
+        const float other = __shfl_xor(mx, m, 64);
+        mx = other > mx ? other : mx;
+    }
+    const float e = on ? expf(v - mx) : 0.f;
+    float sum = e;
+#pragma unroll
+    for (int m = 32; m > 0; m >>= 1) sum += __shfl_xor(sum, m, 64);
+    if (on) out[size_t(row) * step + lane] = e / (sum + 1e-10f);
+}
+
+// ---- cross-entropy value: sum of -log(y + 1e-10) * label --------------------------------------------------------------
+// Stage 1: workgroup b sums elements b*chunk .. (b+1)*chunk - 1 (thread-strided, then the fixed tree) into part[b].
+// Stage 2 (or the only stage when one workgroup covers everything): sums part[] the same way into *loss.
+__global__ void __launch_bounds__(256) ce_partial_kernel(const float *__restrict__ Y, const float *__restrict__ L,
+                                                         float *__restrict__ part, u32 count, u32 chunk) {
+    __shared__ float sh[256];
+    const u32 lo = blockIdx.x * chunk, hi = lo + chunk < count ? lo + chunk : count;
+    float s = 0.f;
+    for (u32 i = lo + threadIdx.x; i < hi; i += 256) s += -logf(Y[i] + 1e-10f) * L[i];
+    s = block_reduce<false>(s, sh);
+    if (threadIdx.x == 0) part[blockIdx.x] = s;
+}
+
+__global__ void __launch_bounds__(256) sum_small_kernel(const float *__restrict__ part, float *__restrict__ out, u32 n) {
+    __shared__ float sh[256];
+    float s = 0.f;
+    for (u32 i = threadIdx.x; i < n; i += 256) s += part[i];
+    s = block_reduce<false>(s, sh);
+    if (threadIdx.x == 0) out[0] = s;
+}
+
+// ---- momentum step with weight decay -------------------------------------------------------------------------------------
+// x = x*decay; m = beta*m + (1-beta)*g; x -= lr*m; g = 0. Every product and sum is rounded on its own (no fused
+// multiply-add), as when decay and update run as separate kernels.
+__device__ __forceinline__ void momentum1(float &x, float &g, float &m, float lr, float beta, float omb, float decay) {
+#pragma clang fp contract(off)
+    const float xd = x * decay;
+    const float mn = beta * m + omb * g;
+    x = xd - lr * mn;
+    m = mn;
+    g = 0.f;
+}
+
+__global__ void __launch_bounds__(256) momentum_kernel(float *__restrict__ X, float *__restrict__ G, float *__restrict__ M, u32 count,
+                                                       u32 vec, float lr, float beta, float omb, float decay) {
+    const u32 stride = gridDim.x * 256;
+    u32 i = blockIdx.x * 256 + threadIdx.x;
+    if (vec) {
+        const u32 nq = count / 4;
+        for (u32 q = i; q < nq; q += stride) {
+            const v4f xv = reinterpret_cast<v4f *>(X)[q], gv = reinterpret_cast<v4f *>(G)[q], mv = reinterpret_cast<v4f *>(M)[q];
+            float x[4] = {xv.x, xv.y, xv.z, xv.w}, g[4] = {gv.x, gv.y, gv.z, gv.w}, m[4] = {mv.x, mv.y, mv.z, mv.w};
+#pragma unroll
+            for (int k = 0; k < 4; ++k) momentum1(x[k], g[k], m[k], lr, beta, omb, decay);
+            reinterpret_cast<v4f *>(X)[q] = v4f{x[0], x[1], x[2], x[3]};
+            reinterpret_cast<v4f *>(G)[q] = v4f{g[0], g[1], g[2], g[3]};
+            reinterpret_cast<v4f *>(M)[q] = v4f{m[0], m[1], m[2], m[3]};
+        }
+        for (u32 r = nq * 4 + i; r < count; r += stride) momentum1(X[r], G[r], M[r], lr, beta, omb, decay);
+    } else {
+        for (; i < count; i += stride) momentum1(X[i], G[i], M[i], lr, beta, omb, decay);
+    }
+}
+
+static int check_pool(const char *what, u32 planes, u32 IH, u32 IW, u32 sH, u32 sW, u32 rH, u32 rW) {
+    if (!planes || !IH || !IW || !sH || !sW || !rH || !rW) return fail(CRB_EINVAL_SHAPE, "%s: zero dimension", what);
+    if (sH != rH || sW != rW)
+        return fail(CRB_EINVAL_SHAPE, "%s: only non-overlapping windows (stride == range) are supported, got stride %ux%u range %ux%u",
+                    what, sH, sW, rH, rW);
+    if (IH < rH || IW < rW) return fail(CRB_EINVAL_SHAPE, "%s: window larger than the input", what);
+    if (uint64_t(planes) * IH * IW > 0x7fffffffull) return fail(CRB_EINVAL_SHAPE, "%s: tensor exceeds 2^31 elements", what);
+    return CRB_OK;
+}
+
+}  // namespace crb
+
+using namespace crb;
+
+extern "C" {
+
+int crb_relu_fwd(const float *X, float *Y, uint32_t count, void *stream) {
+    if (!X || !Y) return fail(CRB_ENULL, "crb_relu_fwd: null operand");
+    if (!count) return fail(CRB_EINVAL_SHAPE, "crb_relu_fwd: zero size");
+    return launch_map2(X, nullptr, Y, count, ReluF{}, hipStream_t(stream), "crb_relu_fwd");
+}
+
+int crb_relu_bwd(const float *X, const float *dY, float *dX, uint32_t count, void *stream) {
+    if (!X || !dY || !dX) return fail(CRB_ENULL, "crb_relu_bwd: null operand");
+    if (!count) return fail(CRB_EINVAL_SHAPE, "crb_relu_bwd: zero size");
+    return launch_map2(X, dY, dX, count, ReluGradF{}, hipStream_t(stream), "crb_relu_bwd");
+}
+
+int crb_maxpool_fwd(const float *X, float *Y, float *record, uint32_t planes, uint32_t IH, uint32_t IW, uint32_t sH, uint32_t sW,
+                    uint32_t rH, uint32_t rW, void *stream) {
+    if (!X || !Y || !record) return fail(CRB_ENULL, "crb_maxpool_fwd: null operand");
+    if (int st = check_pool("crb_maxpool_fwd", planes, IH, IW, sH, sW, rH, rW)) return st;
+    const u32 OH = IH / rH, OW = IW / rW;
+    hipStream_t s = hipStream_t(stream);
+    if (rH == 2 && rW == 2 && IH % 2 == 0 && IW % 4 == 0 && aligned16(X) && aligned16(record) && aligned16(Y)) {
+        const u32 pairs = planes * OH * (IW / 4);
+        hipLaunchKernelGGL(maxpool2x2_fwd_kernel, dim3(ceil_div(pairs, 256)), dim3(256), 0, s, X, Y, record, pairs, IW, FastDiv(IW / 4));
+        return check_launch("crb_maxpool_fwd");
+    }
+    const u32 windows = planes * OH * OW;
+    hipLaunchKernelGGL(maxpool_fwd_kernel, dim3(ceil_div(windows, 256)), dim3(256), 0, s, X, Y, record, windows, IH, IW, rH, rW,
+                       FastDiv(OW), FastDiv(OH));
+    return check_launch("crb_maxpool_fwd");
+}
+
+int crb_maxpool_bwd(float *dX, const float *dY, float *record, uint32_t planes, uint32_t IH, uint32_t IW, uint32_t sH, uint32_t sW,
+                    uint32_t rH, uint32_t rW, void *stream) {
+    if (!dX || !dY || !record) return fail(CRB_ENULL, "crb_maxpool_bwd: null operand");
+    if (int st = check_pool("crb_maxpool_bwd", planes, IH, IW, sH, sW, rH, rW)) return st;
+    const u32 OH = IH / rH, OW = IW / rW;
+    hipStream_t s = hipStream_t(stream);
+    if (rH == 2 && rW == 2 && IH % 2 == 0 && IW % 4 == 0 && aligned16(dX) && aligned16(record) && aligned16(dY)) {
+        const u32 pairs = planes * OH * (IW / 4);
+        hipLaunchKernelGGL(maxpool2x2_bwd_kernel, dim3(ceil_div(pairs, 256)), dim3(256), 0, s, dX, dY, record, pairs, IW, FastDiv(IW / 4));
+        return check_launch("crb_maxpool_bwd");
+    }
+    if (OH * rH != IH || OW * rW != IW) {  // rows / columns no window covers receive no gradient
+        if (int st = crb_tensor_fill(dX, 0.f, planes * IH * IW, stream)) return st;
+    }
+    const u32 windows = planes * OH * OW;
+    hipLaunchKernelGGL(maxpool_bwd_kernel, dim3(ceil_div(windows, 256)), dim3(256), 0, s, dX, dY, record, windows, IH, IW, rH, rW,
+                       FastDiv(OW), FastDiv(OH));
+    return check_launch("crb_maxpool_bwd");
+}
+
+int crb_softmax(const float *A, float *out, uint32_t rows, uint32_t step, void *stream) {
+    if (!A || !out) return fail(CRB_ENULL, "crb_softmax: null operand");
+    if (!rows || !step) return fail(CRB_EINVAL_SHAPE, "crb_softmax: zero dimension");
+    if (uint64_t(rows) * step > 0x7fffffffull) return fail(CRB_EINVAL_SHAPE, "crb_softmax: tensor exceeds 2^31 elements");
+    hipStream_t s = hipStream_t(stream);
+    if (step <= 64)
+        hipLaunchKernelGGL(softmax_short_kernel, dim3(ceil_div(rows, 4)), dim3(256), 0, s, A, out, rows, step);
+    else
+        hipLaunchKernelGGL(softmax_rows_kernel, dim3(rows), dim3(256), 0, s, A, out, step);
+    return check_launch("crb_softmax");
+}
+
+int crb_cross_entropy_grad(const float *Y, const float *labels, float *dY, uint32_t count, void *stream) {
+    if (!Y || !labels || !dY) return fail(CRB_ENULL, "crb_cross_entropy_grad: null operand");
+    if (!count) return fail(CRB_EINVAL_SHAPE, "crb_cross_entropy_grad: zero size");
+    return launch_map2(Y, labels, dY, count, SubF{}, hipStream_t(stream), "crb_cross_entropy_grad");
+}
+
+uint32_t crb_cross_entropy_scratch_floats(uint32_t count) {
+    const u32 blocks = ceil_div(count, 4096u);
+    return blocks > 1024 ? 1024 : blocks;
+}
+
+int crb_cross_entropy_loss(const float *Y, const float *labels, float *scratch, uint32_t scratch_floats, float *loss_out,
+                           uint32_t count, void *stream) {
+    if (!Y || !labels || !loss_out) return fail(CRB_ENULL, "crb_cross_entropy_loss: null operand");
+    if (!count) return fail(CRB_EINVAL_SHAPE, "crb_cross_entropy_loss: zero size");
+    hipStream_t s = hipStream_t(stream);
+    const u32 blocks = crb_cross_entropy_scratch_floats(count);
+    if (blocks == 1) {
+        hipLaunchKernelGGL(ce_partial_kernel, dim3(1), dim3(256), 0, s, Y, labels, loss_out, count, count);
+        return check_launch("crb_cross_entropy_loss");
+    }
+    if (!scratch) return fail(CRB_ENULL, "crb_cross_entropy_loss: null scratch");
+    if (scratch_floats < blocks)
+        return fail(CRB_EWORKSPACE, "crb_cross_entropy_loss: scratch of %u floats < required %u", scratch_floats, blocks);
+    const u32 chunk = ceil_div(count, blocks);
+    hipLaunchKernelGGL(ce_partial_kernel, dim3(blocks), dim3(256), 0, s, Y, labels, scratch, count, chunk);
+    if (int st = check_launch("crb_cross_entropy_loss")) return st;
+    hipLaunchKernelGGL(sum_small_kernel, dim3(1), dim3(256), 0, s, scratch, loss_out, blocks);
+    return check_launch("crb_cross_entropy_loss");
+}
+
+int crb_tensor_sub_inplace(float *a, const float *b, uint32_t count, void *stream) {
+    if (!a || !b) return fail(CRB_ENULL, "crb_tensor_sub_inplace: null operand");
+    if (!count) return fail(CRB_EINVAL_SHAPE, "crb_tensor_sub_inplace: zero size");
+    return launch_map2(a, b, a, count, SubF{}, hipStream_t(stream), "crb_tensor_sub_inplace");
+}
+
+int crb_tensor_scale_inplace(float *a, float factor, uint32_t count, void *stream) {
+    if (!a) return fail(CRB_ENULL, "crb_tensor_scale_inplace: null operand");
+    if (!count) return fail(CRB_EINVAL_SHAPE, "crb_tensor_scale_inplace: zero size");
+    return launch_map2(a, nullptr, a, count, ScaleF{factor}, hipStream_t(stream), "crb_tensor_scale_inplace");
+}
+
+int crb_momentum_apply(float *X, float *G, float *M, uint32_t count, float lr, float beta, float decay, void *stream) {
+    if (!X || !G || !M) return fail(CRB_ENULL, "crb_momentum_apply: null operand");
+    if (!count) return fail(CRB_EINVAL_SHAPE, "crb_momentum_apply: zero size");
+    const u32 vec = aligned16(X) && aligned16(G) && aligned16(M);
+    hipLaunchKernelGGL(momentum_kernel, dim3(stream_grid(count)), dim3(256), 0, hipStream_t(stream), X, G, M, count, vec, lr, beta,
+                       1.0f - beta, decay);
+    return check_launch("crb_momentum_apply");
+}
+
+}  // extern "C"

@@ -149,6 +149,54 @@ int crb_tensor_add_inplace(float *a, const float *b, uint32_t count, void *strea
 /* Replaces the device branch of seblas::Tensor::constFill (Tensor.cu:294-304, 638-657): a[i] = value. */
 int crb_tensor_fill(float *a, float value, uint32_t count, void *stream);
 
+/* Replaces the device branch of seblas::Tensor::operator-(Tensor*) (Tensor.cu:485-506): a[i] -= b[i], in place. */
+int crb_tensor_sub_inplace(float *a, const float *b, uint32_t count, void *stream);
+
+/* Replaces the device branch of seblas::Tensor::operator*(float) (Tensor.cu:596-617): a[i] *= factor, in place.
+ * The optimizers use it for L2 weight decay, `*A->A * (1 - L2)` (seann/optimizers/Optimizers.cu:10,18). */
+int crb_tensor_scale_inplace(float *a, float factor, uint32_t count, void *stream);
+
+/* Elementwise and reduction operators of a training step (the callers around the GEMM / conv path) ----------- */
+
+/* Replaces seblas::relu (seblas/operations/cuActivation.cu:268-280; kernels :14-19, :28-39): Y = max(X, 0). */
+int crb_relu_fwd(const float *X, float *Y, uint32_t count, void *stream);
+
+/* Replaces seblas::reluGradFast (cuActivation.cu:296-308; kernels :54-59, :61-76): dX = X > 0 ? dY : 0. */
+int crb_relu_bwd(const float *X, const float *dY, float *dX, uint32_t count, void *stream);
+
+/* Replaces seblas::maxPool (seblas/operations/cuPool.cu:135-143; kernel :8-40). X: planes x IH x IW (planes = n*c),
+ * Y: planes x IH/rH x IW/rW, record: planes x (IH/rH)*rH x (IW/rW)*rW. Y = window maximum (first maximum in row-major
+ * window order, start value -1e15); record = 1 at that element, 0 elsewhere in the window (the reference writes
+ * only the 1 and relies on the rest being 0). Only stride == range (non-overlapping windows), the one case the
+ * reference's plane-offset arithmetic addresses correctly; anything else returns CRB_EINVAL_SHAPE. */
+int crb_maxpool_fwd(const float *X, float *Y, float *record, uint32_t planes, uint32_t IH, uint32_t IW, uint32_t sH,
+                    uint32_t sW, uint32_t rH, uint32_t rW, void *stream);
+
+/* Replaces seblas::maxPoolBack (cuPool.cu:145-151; kernel :42-70): per window, the element holding the first maximum
+ * of `record` receives dY and that record entry is cleared. Every other element of dX is written as 0 (the reference
+ * leaves them untouched, i.e. at the 0 the gradient tensor was created with). */
+int crb_maxpool_bwd(float *dX, const float *dY, float *record, uint32_t planes, uint32_t IH, uint32_t IW, uint32_t sH,
+                    uint32_t sW, uint32_t rH, uint32_t rW, void *stream);
+
+/* Replaces seblas::softmax (seblas/operations/cuReduce.cu:296-357; kernel :98-146): for each of `rows` consecutive
+ * groups of `step` elements, out = exp(a - max) / (sum exp(a - max) + 1e-10). Any step; no buffer needed. */
+int crb_softmax(const float *A, float *out, uint32_t rows, uint32_t step, void *stream);
+
+/* Replaces seblas::crossEntropyLoss (seblas/operations/cuLoss.cu:231-234): dY = Y - labels. */
+int crb_cross_entropy_grad(const float *Y, const float *labels, float *dY, uint32_t count, void *stream);
+
+/* Replaces seblas::crossEntropyCalc (cuLoss.cu:220-228; kernel :31-37): *loss_out (device) = sum over all elements of
+ * -log(Y + 1e-10) * label, summed in a fixed order. `scratch` must hold crb_cross_entropy_scratch_floats(count)
+ * floats (the reference's `buf`, which has Y's size, always does); it may be null when that is 1. */
+uint32_t crb_cross_entropy_scratch_floats(uint32_t count);
+int crb_cross_entropy_loss(const float *Y, const float *labels, float *scratch, uint32_t scratch_floats, float *loss_out,
+                           uint32_t count, void *stream);
+
+/* Replaces seann::Momentum::apply (seann/optimizers/Optimizers.cu:16-22) = weight decay `A *= decay` followed by
+ * seblas::momentumApply (seblas/operations/cuOptim.cu:259-272; kernels :38-46, :48-73), in one pass:
+ *   x = x*decay;  m = beta*m + (1-beta)*g;  x -= lr*m;  g = 0.   decay = 1 - L2 for weights, 1 otherwise. */
+int crb_momentum_apply(float *X, float *G, float *M, uint32_t count, float lr, float beta, float decay, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

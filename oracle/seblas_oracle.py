@@ -162,3 +162,93 @@ def convBias(Y, bias):
     HW = int(np.prod(out.shape[2:]))
     load().oracle_convBias(_ptr(out), _ptr(_f32(bias)), _u32(N), _u32(C), _u32(HW))
     return out
+
+
+# ---- elementwise / reduction operators (oracle/seblas_oracle_ew.c) -------------------------------------------------
+def relu(X):
+    X = _f32(X)
+    Y = np.empty_like(X)
+    load().oracle_relu(_ptr(X), _ptr(Y), _u32(X.size))
+    return Y
+
+
+def reluGradFast(X, dY):
+    X, dY = _f32(X), _f32(dY)
+    dX = np.empty_like(X)
+    load().oracle_reluGradFast(_ptr(X), _ptr(dY), _ptr(dX), _u32(X.size))
+    return dX
+
+
+def maxPool(X, rH, rW):
+    """X (N,C,IH,IW) -> (Y (N,C,IH//rH,IW//rW), record (N,C,OH*rH,OW*rW))."""
+    X = _f32(X)
+    N, C, IH, IW = X.shape
+    OH, OW = IH // rH, IW // rW
+    Y = np.empty((N, C, OH, OW), np.float32)
+    rec = np.empty((N, C, OH * rH, OW * rW), np.float32)
+    load().oracle_maxPool(_ptr(X), _ptr(Y), _ptr(rec), _u32(N * C), _u32(IH), _u32(IW), _u32(rH), _u32(rW))
+    return Y, rec
+
+
+def maxPoolBack(dY, record, in_hw, rH, rW):
+    """Returns (dX, record after the pass); `record` is not modified."""
+    dY, rec = _f32(dY), _f32(record).copy()
+    N, C = dY.shape[:2]
+    IH, IW = in_hw
+    dX = np.empty((N, C, IH, IW), np.float32)
+    load().oracle_maxPoolBack(_ptr(dX), _ptr(dY), _ptr(rec), _u32(N * C), _u32(IH), _u32(IW), _u32(rH), _u32(rW))
+    return dX, rec
+
+
+def softmax(A, step):
+    A = _f32(A)
+    assert A.size % step == 0
+    out = np.empty_like(A)
+    load().oracle_softmax(_ptr(A), _ptr(out), _u32(A.size // step), _u32(step))
+    return out
+
+
+def crossEntropyLoss(Y, labels):
+    Y, labels = _f32(Y), _f32(labels)
+    dY = np.empty_like(Y)
+    load().oracle_crossEntropyLoss(_ptr(Y), _ptr(labels), _ptr(dY), _u32(Y.size))
+    return dY
+
+
+def crossEntropyCalc(Y, labels):
+    Y, labels = _f32(Y), _f32(labels)
+    fn = load().oracle_crossEntropyCalc
+    fn.restype = ctypes.c_float
+    return float(fn(_ptr(Y), _ptr(labels), _u32(Y.size)))
+
+
+def tensorAdd(A, B):
+    A, B = _f32(A).copy(), _f32(B)
+    load().oracle_tensorAdd(_ptr(A), _ptr(B), _u32(A.size))
+    return A
+
+
+def tensorSub(A, B):
+    A, B = _f32(A).copy(), _f32(B)
+    load().oracle_tensorSub(_ptr(A), _ptr(B), _u32(A.size))
+    return A
+
+
+def tensorScale(A, s):
+    A = _f32(A).copy()
+    load().oracle_tensorScale(_ptr(A), ctypes.c_float(s), _u32(A.size))
+    return A
+
+
+def constFill(A, v):
+    A = _f32(A).copy()
+    load().oracle_constFill(_ptr(A), ctypes.c_float(v), _u32(A.size))
+    return A
+
+
+def momentumApply(X, G, M, lr, beta, decay=1.0):
+    """Returns the updated (X, G, M); the arguments are not modified."""
+    X, G, M = _f32(X).copy(), _f32(G).copy(), _f32(M).copy()
+    load().oracle_momentumApply(_ptr(X), _ptr(G), _ptr(M), _u32(X.size), ctypes.c_float(lr), ctypes.c_float(beta),
+                                ctypes.c_float(decay))
+    return X, G, M

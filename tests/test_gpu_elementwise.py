@@ -1,0 +1,160 @@
+"""GPU parity of the elementwise / reduction operators (through the C ABI) against the CPU oracle.
+
+Bit-exact where the operator only selects, copies or performs individually rounded float operations (ReLU, pooling,
+subtract, scale, fill, momentum); within stated tolerances where device exp/log and the summation order differ
+(softmax: 1e-5 relative; cross-entropy value: 1e-5*sqrt(count) relative).
+"""
+import numpy as np
+import pytest
+
+from tests.util import normal, to_dev, to_np
+
+pytestmark = pytest.mark.gpu
+
+
+def _capi():
+    from crusaderbackend_amd import capi
+    return capi
+
+
+def _oracle():
+    from oracle import seblas_oracle
+    return seblas_oracle
+
+
+def _nan(dev, *shape):
+    import torch
+    return torch.full(shape, float("nan"), dtype=torch.float32, device=dev)
+
+
+SIZES = [1, 3, 4, 255, 1024, 4099, 128 * 64 * 32 * 32]
+
+
+@pytest.mark.parametrize("n", SIZES)
+def test_relu_forward_and_gradient(dev, n):
+    capi, orc = _capi(), _oracle()
+    x, dy = normal(1, n), normal(2, n)
+    x[::7] = 0.0
+    X, dY = to_dev(x, dev), to_dev(dy, dev)
+    Y, dX = _nan(dev, n), _nan(dev, n)
+    capi.relu_fwd(X, Y, n)
+    capi.relu_bwd(X, dY, dX, n)
+    assert np.array_equal(to_np(Y), orc.relu(x))
+    assert np.array_equal(to_np(dX), orc.reluGradFast(x, dy))
+
+
+def test_relu_unaligned_views(dev):
+    capi, orc = _capi(), _oracle()
+    n = 1001
+    x, dy = normal(3, n + 1), normal(4, n + 1)
+    X, dY, Y = to_dev(x, dev)[1:], to_dev(dy, dev)[1:], _nan(dev, n + 1)[1:]  # 4-byte aligned only
+    capi.relu_fwd(X, Y, n)
+    assert np.array_equal(to_np(Y), orc.relu(x[1:]))
+    capi.relu_bwd(X, dY, Y, n)
+    assert np.array_equal(to_np(Y), orc.reluGradFast(x[1:], dy[1:]))
+
+
+# (N, C, IH, IW, r): the VGG pooling stages (2x2 on 32/16/8/4/2) at reduced batch, the full first stage, windows
+# other than 2x2, extents the window does not divide, rows whose length defeats the 16-byte path
+POOL = [(4, 64, 32, 32, 2), (4, 128, 16, 16, 2), (4, 256, 8, 8, 2), (4, 512, 4, 4, 2), (4, 512, 2, 2, 2),
+        (128, 64, 32, 32, 2), (2, 3, 9, 9, 3), (2, 5, 7, 5, 2), (3, 2, 6, 6, 2), (1, 1, 4, 8, 4), (2, 3, 8, 10, 2)]
+
+
+@pytest.mark.parametrize("N,C,IH,IW,r", POOL)
+def test_maxpool_forward_and_gradient(dev, N, C, IH, IW, r):
+    capi, orc = _capi(), _oracle()
+    x = normal(5, N, C, IH, IW)
+    x[0, 0, :r, :r] = 1.5  # a window of ties: the first element must win
+    OH, OW = IH // r, IW // r
+    Yr, rec_r = orc.maxPool(x, r, r)
+    X, Y, rec = to_dev(x, dev), _nan(dev, N, C, OH, OW), _nan(dev, N, C, OH * r, OW * r)
+    capi.maxpool_fwd(X, Y, rec, N * C, IH, IW, r, r, r, r)
+    assert np.array_equal(to_np(Y), Yr)
+    assert np.array_equal(to_np(rec), rec_r)
+    dy = normal(6, N, C, OH, OW)
+    dXr, rec_after = orc.maxPoolBack(dy, rec_r, (IH, IW), r, r)
+    dX = _nan(dev, N, C, IH, IW)
+    capi.maxpool_bwd(dX, to_dev(dy, dev), rec, N * C, IH, IW, r, r, r, r)
+    assert np.array_equal(to_np(dX), dXr)
+    assert np.array_equal(to_np(rec), rec_after)
+
+
+def test_maxpool_rejects_overlapping_windows(dev):
+    capi = _capi()
+    X, Y, rec = _nan(dev, 1, 1, 8, 8), _nan(dev, 1, 1, 3, 3), _nan(dev, 1, 1, 9, 9)
+    with pytest.raises(capi.CrbError, match="non-overlapping"):
+        capi.maxpool_fwd(X, Y, rec, 1, 8, 8, 2, 2, 3, 3)
+    with pytest.raises(capi.CrbError, match="zero"):
+        capi.maxpool_fwd(X, Y, rec, 0, 8, 8, 2, 2, 2, 2)
+
+
+@pytest.mark.parametrize("rows,step", [(128, 10), (1, 1), (7, 64), (5, 65), (33, 1000), (3, 1025), (2, 5000), (4096, 10)])
+def test_softmax(dev, rows, step):
+    capi, orc = _capi(), _oracle()
+    a = normal(7, rows, step) * 3
+    out = _nan(dev, rows, step)
+    capi.softmax(to_dev(a, dev), out, rows, step)
+    ref = orc.softmax(a, step)
+    got = to_np(out)
+    assert np.all(np.isfinite(got))
+    np.testing.assert_allclose(got, ref, rtol=1e-5, atol=1e-12)
+    np.testing.assert_allclose(got.sum(axis=1), 1.0, rtol=1e-5)
+
+
+@pytest.mark.parametrize("rows,classes", [(128, 10), (1, 1), (37, 1000), (2048, 100)])
+def test_cross_entropy_value_and_gradient(dev, rows, classes):
+    import torch
+    capi, orc = _capi(), _oracle()
+    n = rows * classes
+    y = orc.softmax(normal(8, rows, classes), classes)
+    labels = np.eye(classes, dtype=np.float32)[np.random.default_rng(9).integers(0, classes, rows)]
+    Y, L = to_dev(y, dev), to_dev(labels, dev)
+    dY = _nan(dev, rows, classes)
+    capi.cross_entropy_grad(Y, L, dY, n)
+    assert np.array_equal(to_np(dY), orc.crossEntropyLoss(y, labels))
+    need = capi.cross_entropy_scratch_floats(n)
+    scratch = torch.empty(max(need, 1), dtype=torch.float32, device=dev)
+    loss = _nan(dev, 1)
+    capi.cross_entropy_loss(Y, L, scratch, loss, n)
+    ref = orc.crossEntropyCalc(y, labels)
+    assert abs(float(to_np(loss)[0]) - ref) <= 1e-5 * np.sqrt(n) * abs(ref) + 1e-6
+    again = _nan(dev, 1)
+    capi.cross_entropy_loss(Y, L, scratch, again, n)
+    assert to_np(again)[0] == to_np(loss)[0]  # fixed summation order
+    if need > 1:
+        with pytest.raises(capi.CrbError, match="scratch"):
+            capi.cross_entropy_loss(Y, L, scratch[:1], loss, n)
+
+
+@pytest.mark.parametrize("n", [1, 5, 1024, 4099, 512 * 512 * 9])
+def test_sub_scale_and_momentum(dev, n):
+    capi, orc = _capi(), _oracle()
+    a, b = normal(10, n), normal(11, n)
+    A = to_dev(a, dev)
+    capi.tensor_sub_inplace(A, to_dev(b, dev), n)
+    assert np.array_equal(to_np(A), orc.tensorSub(a, b))
+    A = to_dev(a, dev)
+    capi.tensor_scale_inplace(A, 0.9995, n)
+    assert np.array_equal(to_np(A), orc.tensorScale(a, np.float32(0.9995)))
+
+    x, g, m = normal(12, n), normal(13, n), normal(14, n)
+    for decay in (1.0, 1.0 - 5e-4):
+        X, G, M = to_dev(x, dev), to_dev(g, dev), to_dev(m, dev)
+        capi.momentum_apply(X, G, M, n, 0.01, 0.9, decay)
+        xr, gr, mr = orc.momentumApply(x, g, m, 0.01, 0.9, decay)
+        assert np.array_equal(to_np(M), mr)
+        assert np.array_equal(to_np(X), xr)
+        assert not to_np(G).any() and not gr.any()
+
+
+def test_null_and_zero_arguments(dev):
+    capi = _capi()
+    X = _nan(dev, 8)
+    with pytest.raises(capi.CrbError):
+        capi.relu_fwd(X, None, 8)
+    with pytest.raises(capi.CrbError):
+        capi.relu_fwd(X, X, 0)
+    with pytest.raises(capi.CrbError):
+        capi.softmax(X, X, 0, 8)
+    with pytest.raises(capi.CrbError):
+        capi.momentum_apply(X, None, X, 8, 0.1, 0.9)
