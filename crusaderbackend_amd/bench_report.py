@@ -110,6 +110,47 @@ def run(torch, capi, dev, event_time_ms, Layer):
     out["dense"].append(_entry("sgemm tall-skinny 32768x64x576", event_time_ms(torch, lambda: capi.sgemm_nn(A, B, C, M, N, K), 20),
                                2.0 * M * N * K, 4.0 * (M * K + K * N + M * N)))
 
+    # elementwise / reduction operators at the sizes the VGG-16 step runs them (all bandwidth-bound; flops counted as 0)
+    out["elementwise"] = []
+
+    def ew(name, fn, nbytes, reps=30):
+        ms = event_time_ms(torch, fn, reps=reps)
+        out["elementwise"].append({"name": name, "us": round(ms * 1e3, 2), "gflop": 0.0, "mbytes": round(nbytes / 1e6, 2), "ai": 0.0,
+                                   "tflops": 0.0, "gbs": round(nbytes / ms / 1e6, 1), "bound": "hbm",
+                                   "frac": round(nbytes / ms / 1e6 / PEAK_GBS, 4)})
+
+    for (C, H) in ((64, 32), (256, 8)):
+        n = 128 * C * H * H
+        X, Y, dY = rnd(n), torch.empty(n, device=dev), rnd(n)
+        ew(f"relu 128x{C}x{H}x{H}", lambda: capi.relu_fwd(X, Y, n), 8.0 * n)
+        ew(f"reluGradFast 128x{C}x{H}x{H}", lambda: capi.relu_bwd(X, dY, Y, n), 12.0 * n)
+        P, rec = torch.empty(n // 4, device=dev), torch.empty(n, device=dev)
+        ew(f"maxPool 2x2 128x{C}x{H}x{H}", lambda: capi.maxpool_fwd(X, P, rec, 128 * C, H, H, 2, 2, 2, 2), 4.0 * (2 * n + n // 4))
+        ew(f"maxPoolBack 2x2 128x{C}x{H}x{H}", lambda: capi.maxpool_bwd(Y, P, rec, 128 * C, H, H, 2, 2, 2, 2), 4.0 * (3 * n + n // 4))
+        del X, Y, dY, P, rec
+    n = 512 * 512 * 9
+    Wt, G, M = rnd(n), rnd(n), rnd(n)
+    ew("momentumApply + decay 512x512x3x3", lambda: capi.momentum_apply(Wt, G, M, n, 0.01, 0.9, 0.9995), 24.0 * n)
+    A, S, L = rnd(128, 10), torch.empty(128, 10, device=dev), torch.zeros(128, 10, device=dev)
+    loss = torch.empty(1, device=dev)
+    ew("softmax 128x10", lambda: capi.softmax(A, S, 128, 10), 8.0 * 1280)
+    ew("crossEntropyCalc 128x10", lambda: capi.cross_entropy_loss(S, L, None, loss, 1280), 8.0 * 1280)
+    del Wt, G, M
+
+    # config 3 end to end: the whole training step (every operator, real data flow, momentum update), batch 128
+    from .vgg16_step import Vgg16Step
+    net = Vgg16Step(torch, capi, dev, batch=128)
+    step_ms = event_time_ms(torch, net.step, reps=10, warm=3)
+    fwd_ms = event_time_ms(torch, net.forward, reps=10, warm=2)
+    bwd_ms = event_time_ms(torch, net.backward, reps=10, warm=2)
+    upd_ms = event_time_ms(torch, net.update, reps=10, warm=2)
+    out["vgg16_full_step"] = {"us": round(step_ms * 1e3, 1), "forward_us": round(fwd_ms * 1e3, 1), "backward_us": round(bwd_ms * 1e3, 1),
+                              "update_us": round(upd_ms * 1e3, 1), "conv_fc_gflop": round(net.flops / 1e9, 2),
+                              "tflops": round(net.flops / step_ms / 1e9, 2), "images_per_s": round(128 / step_ms * 1e3, 1),
+                              "frac_fp32_mfma_peak": round(net.flops / step_ms / 1e9 / PEAK_TF, 4)}
+    del net
+    torch.cuda.empty_cache()
+
     # summary lines
     def total(key, suffix=None):
         es = [e for e in out[key] if suffix is None or e["name"].endswith(suffix)]
@@ -117,13 +158,16 @@ def run(torch, capi, dev, event_time_ms, Layer):
                 "tflops": round(sum(e["gflop"] for e in es) / max(sum(e["us"] for e in es), 1e-9) * 1e3, 2)}
 
     out["summary"] = {"vgg16_conv_fc_train_step": total("vgg16"), "vgg16_fwd": total("vgg16", ".fwd"),
+                      "vgg16_full_train_step": out["vgg16_full_step"],
                       "peak_fp32_mfma_tflops": PEAK_TF, "peak_hbm_gbs": PEAK_GBS, "ridge_flop_per_byte": round(RIDGE, 2)}
     return out
 
 
 def to_markdown(rep):
     lines = []
-    for key in ("gemm", "resnet56", "vgg16", "densenet", "dense"):
+    for key in ("gemm", "resnet56", "vgg16", "densenet", "dense", "elementwise"):
+        if key not in rep:
+            continue
         lines += [f"### {key}", "", "| shape.pass | us | GFLOP | MB | AI | TFLOP/s | GB/s | bound | fraction of roofline | cold-cache us | cold GB/s |",
                   "|---|---|---|---|---|---|---|---|---|---|---|"]
         for e in rep[key]:

@@ -267,14 +267,64 @@ __global__ void __launch_bounds__(256) conv_bias_kernel(float *__restrict__ Y, c
     Y[i] += bias[plane % C];
 }
 
-// One workgroup per channel: dB[c] += sum over (n, hw) of dY[n,c,hw]; fixed-order tree reduction in LDS.
-__global__ void __launch_bounds__(256) conv_bias_grad_kernel(const float *__restrict__ dY, float *__restrict__ dB, u32 N,
-                                                             u32 C, u32 HW) {
+// Bias gradient dB[c] += sum over (n, hw) of dY[n,c,hw], in two passes with a fixed association (bit-reproducible).
+// Pass 1 views dY as a (N x C*HW) matrix and sums its columns over a slice of the rows: a workgroup covers 64 columns
+// (16 lanes x 4 floats, whole 256-byte row segments) with 16 row-lanes, or 32 columns x 8 row-lanes with scalar loads when
+// the matrix is not 16-byte friendly; the row-lanes are combined through LDS in lane order. part[slice][column].
+template <bool VEC>
+__global__ void __launch_bounds__(256) bias_grad_colsum_kernel(const float *__restrict__ in, float *__restrict__ part, u32 rows,
+                                                               u32 cols, u32 rows_per_slice) {
+    constexpr u32 CL = VEC ? 16 : 32, RL = 256 / CL, W = VEC ? 4 : 1;
+    __shared__ float red[RL][CL * W + 4];
+    const u32 o = threadIdx.x % CL, g = threadIdx.x / CL;
+    const u32 c = (blockIdx.x * CL + o) * W;
+    const u32 r0 = blockIdx.y * rows_per_slice, r1 = r0 + rows_per_slice < rows ? r0 + rows_per_slice : rows;
+    float acc[2][W];
+#pragma unroll
+    for (u32 k = 0; k < W; ++k) acc[0][k] = acc[1][k] = 0.f;
+    if (c < cols) {
+        const float *p = in + c;
+        u32 r = r0 + g;
+        for (; r + RL < r1; r += 2 * RL) {
+            if constexpr (VEC) {
+                const v4f a = *reinterpret_cast<const v4f *>(p + size_t(r) * cols);
+                const v4f b = *reinterpret_cast<const v4f *>(p + size_t(r + RL) * cols);
+                acc[0][0] += a.x, acc[0][1] += a.y, acc[0][2] += a.z, acc[0][3] += a.w;
+                acc[1][0] += b.x, acc[1][1] += b.y, acc[1][2] += b.z, acc[1][3] += b.w;
+            } else {
+                acc[0][0] += p[size_t(r) * cols];
+                acc[1][0] += p[size_t(r + RL) * cols];
+            }
+        }
+        if (r < r1) {
+            if constexpr (VEC) {
+                const v4f a = *reinterpret_cast<const v4f *>(p + size_t(r) * cols);
+                acc[0][0] += a.x, acc[0][1] += a.y, acc[0][2] += a.z, acc[0][3] += a.w;
+            } else {
+                acc[0][0] += p[size_t(r) * cols];
+            }
+        }
+    }
+#pragma unroll
+    for (u32 k = 0; k < W; ++k) red[g][o * W + k] = acc[0][k] + acc[1][k];
+    __syncthreads();
+    const u32 j = blockIdx.x * CL * W + threadIdx.x;
+    if (threadIdx.x < CL * W && j < cols) {
+        float v = red[0][threadIdx.x];
+#pragma unroll
+        for (u32 k = 1; k < RL; ++k) v += red[k][threadIdx.x];
+        part[size_t(blockIdx.y) * cols + j] = v;
+    }
+}
+
+// Pass 2: one workgroup per channel folds its HW columns of every slice: dB[c] += sum_{slice, hw} part[slice][c*HW + hw].
+__global__ void __launch_bounds__(256) bias_grad_fold_kernel(const float *__restrict__ part, float *__restrict__ dB, u32 HW, u32 cols,
+                                                             u32 slices) {
     __shared__ float red[256];
     const u32 c = blockIdx.x;
-    float s = 0.0f;
-    for (u32 n = 0; n < N; ++n) {
-        const float *p = dY + (size_t(n) * C + c) * HW;
+    float s = 0.f;
+    for (u32 sl = 0; sl < slices; ++sl) {
+        const float *p = part + size_t(sl) * cols + c * HW;
         for (u32 i = threadIdx.x; i < HW; i += 256) s += p[i];
     }
     red[threadIdx.x] = s;
@@ -443,7 +493,24 @@ int crb_conv_bias_grad(const float *dY, float *dB, uint32_t N, uint32_t C, uint3
     if (!N || !C || !HW) return fail(CRB_EINVAL_SHAPE, "crb_conv_bias_grad: zero dimension");
     if (uint64_t(N) * C * HW > 0x7fffffffull)
         return fail(CRB_EINVAL_SHAPE, "crb_conv_bias_grad: tensor exceeds 2^31 elements");
-    hipLaunchKernelGGL(conv_bias_grad_kernel, dim3(C), dim3(256), 0, hipStream_t(stream), dY, dB, N, C, HW);
+    hipStream_t s = hipStream_t(stream);
+    const u32 cols = C * HW;
+    const bool vec = cols % 4 == 0 && aligned16(dY);
+    const u32 col_wgs = ceil_div(cols, vec ? 64u : 32u);
+    // rows are cut into slices until the grid covers the chip (at least 16 rows per slice)
+    u32 slices = col_wgs >= 512 ? 1 : ceil_div(512u, col_wgs);
+    if (slices > ceil_div(N, 16u)) slices = ceil_div(N, 16u);
+    const u32 rows_per_slice = ceil_div(N, slices);
+    slices = ceil_div(N, rows_per_slice);
+    const size_t need = size_t(slices) * cols * sizeof(float);
+    float *part = static_cast<float *>(arena_get(need));
+    if (!part) return fail(CRB_EHIP, "crb_conv_bias_grad: cannot allocate %zu bytes of scratch", need);
+    if (vec)
+        hipLaunchKernelGGL(bias_grad_colsum_kernel<true>, dim3(col_wgs, slices), dim3(256), 0, s, dY, part, N, cols, rows_per_slice);
+    else
+        hipLaunchKernelGGL(bias_grad_colsum_kernel<false>, dim3(col_wgs, slices), dim3(256), 0, s, dY, part, N, cols, rows_per_slice);
+    if (int st = check_launch("crb_conv_bias_grad")) return st;
+    hipLaunchKernelGGL(bias_grad_fold_kernel, dim3(C), dim3(256), 0, s, part, dB, HW, cols, slices);
     return check_launch("crb_conv_bias_grad");
 }
 

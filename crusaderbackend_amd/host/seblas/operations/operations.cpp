@@ -133,4 +133,79 @@ Tensor *convBias(Tensor *Y, Tensor *biases) {
     return Y;
 }
 
+// ---- elementwise / reduction operators ---------------------------------------------------------------------------------
+
+Tensor *relu(Tensor *X, Tensor *Y) {
+    require(X->dims.size == Y->dims.size, "relu: element counts differ");
+    finish(crb_relu_fwd(X->elements, Y->elements, X->dims.size, nullptr), __FILE__, __LINE__);  // cuActivation.cu:268-280
+    return Y;
+}
+
+Tensor *reluGradFast(Tensor *X, Tensor *dY, Tensor *dX) {
+    require(X->dims.size == dY->dims.size && X->dims.size == dX->dims.size, "reluGradFast: element counts differ");
+    finish(crb_relu_bwd(X->elements, dY->elements, dX->elements, X->dims.size, nullptr), __FILE__, __LINE__);  // :296-308
+    return dX;
+}
+
+static void requirePool(const char *what, Tensor *X, Tensor *Y, Tensor *record, uint32 sH, uint32 sW, uint32 rH, uint32 rW) {
+    require(sH && sW && rH && rW, what);
+    require(X->dims.h >= rH - sH && X->dims.w >= rW - sW, what);
+    require((X->dims.h - (rH - sH)) / sH == Y->dims.h, what);  // cuPool.cu:136
+    require((X->dims.w - (rW - sW)) / sW == Y->dims.w, what);  // :137
+    require(X->dims.n == Y->dims.n && X->dims.c == Y->dims.c, what);
+    require(record->dims.size == uint64_t(X->dims.n) * X->dims.c * Y->dims.h * rH * Y->dims.w * rW, what);  // MaxPool2D.cuh:47-51
+}
+
+void maxPool(Tensor *X, Tensor *Y, Tensor *record, uint32 strideH, uint32 strideW, uint32 rangeH, uint32 rangeW) {
+    requirePool("maxPool: shapes do not satisfy the pooling relationship", X, Y, record, strideH, strideW, rangeH, rangeW);
+    finish(crb_maxpool_fwd(X->elements, Y->elements, record->elements, X->dims.n * X->dims.c, X->dims.h, X->dims.w, strideH,
+                           strideW, rangeH, rangeW, nullptr),
+           __FILE__, __LINE__);
+}
+
+void maxPoolBack(Tensor *dX, Tensor *dY, Tensor *record, uint32 strideH, uint32 strideW, uint32 rangeH, uint32 rangeW) {
+    requirePool("maxPoolBack: shapes do not satisfy the pooling relationship", dX, dY, record, strideH, strideW, rangeH, rangeW);
+    finish(crb_maxpool_bwd(dX->elements, dY->elements, record->elements, dX->dims.n * dX->dims.c, dX->dims.h, dX->dims.w,
+                           strideH, strideW, rangeH, rangeW, nullptr),
+           __FILE__, __LINE__);
+}
+
+Tensor *softmax(Tensor *A, Tensor *out, Tensor *buffer, uint32 step) {
+    (void)buffer;
+    require(step != 0 && A->dims.size % step == 0, "softmax: size is not a multiple of step");  // cuReduce.cu:297
+    require(out->dims.size == A->dims.size, "softmax: element counts differ");                   // :298
+    finish(crb_softmax(A->elements, out->elements, A->dims.size / step, step, nullptr), __FILE__, __LINE__);
+    return out;
+}
+
+void crossEntropyLoss(Parameter *Y, Tensor *labels) {
+    require(Y->A->dims.size == labels->dims.size, "crossEntropyLoss: element counts differ");
+    finish(crb_cross_entropy_grad(Y->A->elements, labels->elements, Y->dA->elements, Y->A->dims.size, nullptr), __FILE__,
+           __LINE__);  // cuLoss.cu:231-234
+}
+
+float crossEntropyCalc(Parameter *Y, Tensor *labels, Tensor *buf) {
+    const uint32 n = Y->A->dims.size;
+    require(n == labels->dims.size, "crossEntropyCalc: element counts differ");
+    const uint32 need = crb_cross_entropy_scratch_floats(n);
+    require(buf != nullptr && buf->dims.size >= need + 1, "crossEntropyCalc: buf too small");
+    float *out = buf->elements + (buf->dims.size - 1);  // partial sums at the front, the total in the last element
+    finish(crb_cross_entropy_loss(Y->A->elements, labels->elements, buf->elements, buf->dims.size - 1, out, n, nullptr),
+           __FILE__, __LINE__);
+    float loss = 0.f;
+    if (hipMemcpy(&loss, out, sizeof(float), hipMemcpyDeviceToHost) != hipSuccess) assertHip(__FILE__, __LINE__);
+    return loss;
+}
+
+void momentumApply(Tensor *X, Tensor *Xgrad, Tensor *V, float LEARNING_RATE, float MOMENTUM) {
+    momentumApplyDecay(X, Xgrad, V, LEARNING_RATE, MOMENTUM, 0.0f);
+}
+
+void momentumApplyDecay(Tensor *X, Tensor *Xgrad, Tensor *V, float LEARNING_RATE, float MOMENTUM, float L2) {
+    require(X->dims.size == Xgrad->dims.size && X->dims.size == V->dims.size, "momentumApply: element counts differ");
+    finish(crb_momentum_apply(X->elements, Xgrad->elements, V->elements, X->dims.size, LEARNING_RATE, MOMENTUM, 1.0f - L2,
+                              nullptr),
+           __FILE__, __LINE__);  // cuOptim.cu:259-272
+}
+
 }  // namespace seblas

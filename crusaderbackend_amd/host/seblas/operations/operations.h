@@ -30,4 +30,22 @@ Tensor *convDerive(Tensor *A, Tensor *B, Tensor *C, int strideH, int strideW, in
 // reference does (cuConv.cu:805).
 Tensor *convError(Tensor *A, Tensor *B, Tensor *C, int strideH, int strideW, int padH, int padW);
 Tensor *convBias(Tensor *Y, Tensor *biases);
+
+// ---- the elementwise / reduction operators a training step runs between those calls -------------------------------
+// cuActivation.cuh:13,18
+Tensor *relu(Tensor *X, Tensor *Y);
+Tensor *reluGradFast(Tensor *X, Tensor *dY, Tensor *dX);
+// cuPool.cuh:13-17. Non-overlapping windows only (stride == range); see include/crusader_hip.h.
+void maxPool(Tensor *X, Tensor *Y, Tensor *record, uint32 strideH, uint32 strideW, uint32 rangeH, uint32 rangeW);
+void maxPoolBack(Tensor *dX, Tensor *dY, Tensor *record, uint32 strideH, uint32 strideW, uint32 rangeH, uint32 rangeW);
+// cuReduce.cuh:44. `buffer` is accepted for signature compatibility and never used (may be null).
+Tensor *softmax(Tensor *A, Tensor *out, Tensor *buffer, uint32 step);
+// cuLoss.cuh:18,20. crossEntropyLoss: Y->dA = Y->A - labels. crossEntropyCalc: sum of -log(Y->A + 1e-10)*label; `buf`
+// is device scratch (the reference passes a tensor of Y's size; its last element receives the sum before the copy back).
+void crossEntropyLoss(Parameter *Y, Tensor *labels);
+float crossEntropyCalc(Parameter *Y, Tensor *labels, Tensor *buf);
+// cuOptim.cuh:16. V is the momentum buffer; Xgrad is cleared by the step.
+void momentumApply(Tensor *X, Tensor *Xgrad, Tensor *V, float LEARNING_RATE, float MOMENTUM);
+// Optimizers.cu:16-22 in one pass: X *= (1 - L2) then momentumApply. No separate counterpart in the reference.
+void momentumApplyDecay(Tensor *X, Tensor *Xgrad, Tensor *V, float LEARNING_RATE, float MOMENTUM, float L2);
 }  // namespace seblas

@@ -145,6 +145,28 @@ Tensor *Tensor::operator+(Tensor *other) {
     return this;
 }
 
+Tensor *Tensor::operator-(Tensor *other) {
+    require(dims.size == other->dims.size, "Tensor::operator-: element counts differ");
+    require(deviceId == other->deviceId, "Tensor::operator-: tensors live on different devices");
+    if (deviceId == -1) {
+        for (uint32 i = 0; i < dims.size; ++i) elements[i] -= other->elements[i];
+        return this;
+    }
+    throwOnStatus(crb_tensor_sub_inplace(elements, other->elements, dims.size, nullptr), __FILE__, __LINE__);
+    assertHip(__FILE__, __LINE__);
+    return this;
+}
+
+Tensor *Tensor::operator*(float factor) {
+    if (deviceId == -1) {
+        for (uint32 i = 0; i < dims.size; ++i) elements[i] *= factor;
+        return this;
+    }
+    throwOnStatus(crb_tensor_scale_inplace(elements, factor, dims.size, nullptr), __FILE__, __LINE__);
+    assertHip(__FILE__, __LINE__);
+    return this;
+}
+
 Tensor *Tensor::constFill(float val) {
     if (deviceId == -1) {
         for (uint32 i = 0; i < dims.size; ++i) elements[i] = val;

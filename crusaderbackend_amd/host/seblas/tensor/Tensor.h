@@ -80,6 +80,9 @@ public:
     // 462-483,638-657): in-place `*this += *other`, and fill. Device tensors run on the GPU.
     Tensor *operator+(Tensor *other);
     Tensor *constFill(float val);
+    // `*this -= *other` (Tensor.cu:485-506: the loss gradient) and `*this *= factor` (Tensor.cu:596-617: weight decay)
+    Tensor *operator-(Tensor *other);
+    Tensor *operator*(float factor);
     // Host-generated N(mean, stddev) from a fixed-seed mt19937 (the reference's wall-clock-seeded cuRAND
     // stream, Tensor.cu:306-322,667-683, is deliberately not reproduced).
     Tensor *randNormal(float mean, float stddev, uint32 seed = 0x5eb1a5u);

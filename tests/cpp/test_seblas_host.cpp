@@ -25,6 +25,14 @@ void oracle_convDerive(const float *, const float *, float *, uint32_t, uint32_t
                        uint32_t, uint32_t, uint32_t, uint32_t, uint32_t, uint32_t, uint32_t, int);
 void oracle_convError(const float *, const float *, float *, uint32_t, uint32_t, uint32_t, uint32_t, uint32_t, uint32_t,
                       uint32_t, uint32_t, uint32_t, uint32_t, uint32_t, uint32_t, uint32_t, int);
+void oracle_relu(const float *, float *, uint32_t);
+void oracle_reluGradFast(const float *, const float *, float *, uint32_t);
+void oracle_maxPool(const float *, float *, float *, uint32_t, uint32_t, uint32_t, uint32_t, uint32_t);
+void oracle_maxPoolBack(float *, const float *, float *, uint32_t, uint32_t, uint32_t, uint32_t, uint32_t);
+void oracle_softmax(const float *, float *, uint32_t, uint32_t);
+void oracle_crossEntropyLoss(const float *, const float *, float *, uint32_t);
+float oracle_crossEntropyCalc(const float *, const float *, uint32_t);
+void oracle_momentumApply(float *, float *, float *, uint32_t, float, float, float);
 }
 
 using namespace seblas;
@@ -237,11 +245,85 @@ static void gpu_tests() {
     }
 }
 
+// The elementwise / reduction operators through the seblas signatures: relu -> maxPool -> softmax -> cross-entropy and
+// back, then a momentum step, each against the CPU oracle (bit-exact except where exp/log and summation order differ).
+static void gpu_elementwise_tests() {
+    const uint32_t N = 6, C = 5, H = 8, W = 8, n = N * C * H * W;
+    auto x = randn(n, 21), dy = randn(n, 22);
+    Tensor *X = push(shape4(N, C, H, W), x), *Y = Tensor::create(N, C, H, W), *dY = push(shape4(N, C, H, W), dy);
+    Tensor *dX = Tensor::create(N, C, H, W);
+    CHECK(relu(X, Y) == Y);
+    std::vector<float> ry(n), rdx(n);
+    oracle_relu(x.data(), ry.data(), n);
+    CHECK(pull(Y) == ry);
+    CHECK(reluGradFast(X, dY, dX) == dX);
+    oracle_reluGradFast(x.data(), dy.data(), rdx.data(), n);
+    CHECK(pull(dX) == rdx);
+
+    // pooling: record has the MaxPool2D operand's shape (MaxPool2D.cuh:47-51)
+    Tensor *P = Tensor::create(N, C, H / 2, W / 2), *rec = Tensor::create(N, C, H, W);
+    maxPool(Y, P, rec, 2, 2, 2, 2);
+    std::vector<float> rp(n / 4), rrec(n), rback(n);
+    oracle_maxPool(ry.data(), rp.data(), rrec.data(), N * C, H, W, 2, 2);
+    CHECK(pull(P) == rp);
+    CHECK(pull(rec) == rrec);
+    auto dp = randn(n / 4, 23);
+    Tensor *dP = push(shape4(N, C, H / 2, W / 2), dp);
+    maxPoolBack(dX, dP, rec, 2, 2, 2, 2);
+    oracle_maxPoolBack(rback.data(), dp.data(), rrec.data(), N * C, H, W, 2, 2);
+    CHECK(pull(dX) == rback);
+    CHECK(pull(rec) == rrec);  // both cleared
+    CHECK(throws_invalid([&] { maxPool(Y, P, rec, 2, 2, 3, 3); }));   // shape relationship (cuPool.cu:136-137)
+    CHECK(throws_invalid([&] { maxPool(Y, Y, rec, 2, 2, 2, 2); }));
+
+    // softmax over rows of 10, cross-entropy value and gradient
+    const uint32_t rows = 16, classes = 10;
+    auto z = randn(rows * classes, 24, 2.0f);
+    std::vector<float> lab(rows * classes, 0.f);
+    for (uint32_t r = 0; r < rows; ++r) lab[r * classes + (r * 7) % classes] = 1.f;
+    seann::Parameter *S = seann::Parameter::create(rows, 1, classes, 1);
+    Tensor *Z = push(shape4(rows, 1, classes, 1), z), *L = push(shape4(rows, 1, classes, 1), lab);
+    CHECK(softmax(Z, S->A, nullptr, classes) == S->A);
+    std::vector<float> rs(rows * classes), rg(rows * classes);
+    oracle_softmax(z.data(), rs.data(), rows, classes);
+    compare("seblas::softmax", pull(S->A), rs, 1);
+    auto s_gpu = pull(S->A);
+    crossEntropyLoss(S, L);
+    oracle_crossEntropyLoss(s_gpu.data(), lab.data(), rg.data(), rows * classes);
+    CHECK(pull(S->dA) == rg);
+    Tensor *buf = Tensor::create(rows, 1, classes, 1);
+    const float loss = crossEntropyCalc(S, L, buf), rloss = oracle_crossEntropyCalc(s_gpu.data(), lab.data(), rows * classes);
+    CHECK(std::fabs(loss - rloss) <= 1e-5f * std::fabs(rloss) * std::sqrt(float(rows * classes)));
+    CHECK(throws_invalid([&] { softmax(Z, S->A, nullptr, 7); }));  // cuReduce.cu:297
+
+    // Tensor arithmetic used by the loss and the optimizer, then one momentum step with weight decay
+    auto a = randn(1000, 25), b = randn(1000, 26), m = randn(1000, 27);
+    Tensor *A = push(shape4(1000, 1), a), *B = push(shape4(1000, 1), b), *M = push(shape4(1000, 1), m);
+    CHECK((*A - B) == A);
+    auto ra = a;
+    for (size_t i = 0; i < ra.size(); ++i) ra[i] = a[i] - b[i];
+    CHECK(pull(A) == ra);
+    CHECK((*A * 0.5f) == A);
+    for (auto &v : ra) v *= 0.5f;
+    CHECK(pull(A) == ra);
+    auto rb = b, rm = m;
+    momentumApplyDecay(A, B, M, 0.01f, 0.9f, 5e-4f);
+    oracle_momentumApply(ra.data(), rb.data(), rm.data(), 1000, 0.01f, 0.9f, 1.0f - 5e-4f);
+    CHECK(pull(A) == ra);
+    CHECK(pull(M) == rm);
+    CHECK(pull(B) == rb);  // gradient cleared
+    momentumApply(A, B, M, 0.01f, 0.9f);
+    oracle_momentumApply(ra.data(), rb.data(), rm.data(), 1000, 0.01f, 0.9f, 1.0f);
+    CHECK(pull(A) == ra);
+}
+
 int main(int argc, char **argv) {
     const bool gpu = argc > 1 && std::strcmp(argv[1], "gpu") == 0;
     try {
-        if (gpu)
+        if (gpu) {
             gpu_tests();
+            gpu_elementwise_tests();
+        }
         else
             host_tests();
     } catch (const std::exception &e) {

@@ -189,6 +189,20 @@ def test_conv_shape_errors(dev):
     assert st == capi.CRB_EWORKSPACE
 
 
+# (N, C, H, W): the VGG stages at reduced / full batch, shapes with C*H*W not a multiple of 4, one row, many rows
+@pytest.mark.parametrize("N,C,H,W", [(128, 64, 32, 32), (128, 512, 2, 2), (128, 512, 1, 1), (37, 5, 7, 9), (1, 3, 5, 5),
+                                     (300, 2, 3, 3), (16, 48, 8, 8), (2, 1, 1, 1), (64, 12, 16, 16)])
+def test_conv_bias_grad(dev, N, C, H, W):
+    capi = _capi()
+    dY0, dB0 = normal(1, N, C, H, W), normal(2, C)
+    dB, dY = to_dev(dB0, dev), to_dev(dY0, dev)
+    capi.conv_bias_grad(dY, dB, N, C, H * W)
+    assert_close(to_np(dB), dB0 + dY0.astype(np.float64).sum(axis=(0, 2, 3)), N * H * W, "conv bias grad")
+    again = to_dev(dB0, dev)
+    capi.conv_bias_grad(dY, again, N, C, H * W)
+    assert np.array_equal(to_np(again), to_np(dB))  # fixed summation order
+
+
 def test_bias_grad_and_tensor_helpers(dev):
     import torch
     capi = _capi()
