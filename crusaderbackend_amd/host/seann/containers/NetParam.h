@@ -1,16 +1,11 @@
-// seann::NetParam — a trainable Parameter (weights or biases) as the conv/linear operands hold it
-// (seann/containers/NetParam.cuh:20-116). The reference pairs it with an Optimizer; optimizers are outside
-// this build, so `opt` is an opaque pointer that the operands pass through untouched, and the gradient
-// zeroing the reference's optimizers perform after every apply (seblas/operations/cuOptim.cu:65-71) is
-// available as zeroGrad().
+// seann::NetParam — a trainable Parameter (weights or biases) paired with its optimizer, as the operands hold it
+// (seann/containers/NetParam.cuh:20-56). `info` may be null (no optimizer: update() is then a no-op), which is how
+// the operands are used when only forward / gradients are wanted.
 #pragma once
-#include "../../seblas/tensor/Parameter.h"
+#include "../optimizers/Optimizers.h"
 
 namespace seann {
 using namespace seblas;
-
-struct Optimizer;      // not part of this build
-struct OptimizerInfo;  // not part of this build
 
 class NetParam {
 public:
@@ -19,12 +14,26 @@ public:
     bool isWeight = false;
 
     template <typename... Args>
-    explicit NetParam(OptimizerInfo *, Args &&...args) { A = Parameter::create(std::forward<Args>(args)...); }
+    explicit NetParam(OptimizerInfo *info, Args &&...args) {
+        A = Parameter::create(std::forward<Args>(args)...);
+        if (info) opt = info->create(A);
+    }
     NetParam(Parameter *A, Optimizer *opt) : A(A), opt(opt) {}
+    NetParam(Parameter *A, OptimizerInfo *info) : A(A) { opt = info ? info->create(A) : nullptr; }
 
     NetParam *setWeight() {
         isWeight = true;
+        if (opt) opt->isWeight = true;
         return this;
+    }
+    void setWeightDecay(float weightDecay) const {
+        if (opt) opt->L2 = weightDecay;
+    }
+    void update() const {
+        if (opt) opt->apply();
+    }
+    void batchUpdate() const {
+        if (opt) opt->batchApply();
     }
     Tensor *data() const { return A->A; }
     Tensor *grad() const { return A->dA; }

@@ -1,0 +1,44 @@
+// seann::Sequential — the linear container that owns the operand list, wires each operand's input to its predecessor's
+// output and drives forward / backward / update (seann/containers/Sequential.{cuh,cu}). Dataset-driven `train`,
+// checkpointing and logging are outside this build.
+#pragma once
+#include <initializer_list>
+#include <vector>
+
+#include "../operands/OperandBase.h"
+
+namespace seann {
+
+typedef void (*LossFunc)(Parameter *, Tensor *);
+typedef float (*LossFuncCalc)(Parameter *, Tensor *, Tensor *);
+
+class Sequential {
+public:
+    Parameter *netX;
+    Parameter *netY{};
+    LossFunc loss{};
+    LossFuncCalc lossFW{};
+    std::vector<OperandBase *> operands;
+    uint32 OPERAND_COUNT;
+
+    Sequential(shape4 inputShape, std::initializer_list<OperandBase *> list) : operands(list), OPERAND_COUNT(uint32(list.size())) {
+        netX = Parameter::create(inputShape);
+    }
+    Sequential(shape4 inputShape, const std::vector<OperandBase *> &list) : operands(list), OPERAND_COUNT(uint32(list.size())) {
+        netX = Parameter::create(inputShape);
+    }
+
+    void waive() const;                     // bind prev/next and inputs along the chain
+    void construct(OptimizerInfo *info);    // create every operand's tensors, then bind
+    void setLoss(LossFunc lossFunc, LossFuncCalc lossFWD) { loss = lossFunc, lossFW = lossFWD; }
+    void randInit() const;
+    Tensor *forward() const;
+    Tensor *forward(Tensor *X) const;
+    Tensor *inferenceForward() const;
+    Tensor *inferenceForward(Tensor *X) const;
+    Tensor *backward(Tensor *label) const;  // loss gradient, then xGrads + paramGrads from last to first
+    void learn() const;
+    void learnBatch() const;
+    void zeroGrads() const;
+};
+}  // namespace seann

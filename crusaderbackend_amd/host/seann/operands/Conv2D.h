@@ -29,6 +29,14 @@ public:
     void paramGrads() override;
     void randFillNetParams() override;
     void zeroGrads() override;
+    void updateParams() override {  // Conv2D.cu:31-34
+        filter->update();
+        if (WITH_BIAS) bias->update();
+    }
+    void batchUpdateParams() override {
+        filter->batchUpdate();
+        if (WITH_BIAS) bias->batchUpdate();
+    }
     uint32 OPERAND_ID() override { return OPR_SEBLAS_CONV2D; }
 };
 }  // namespace seann

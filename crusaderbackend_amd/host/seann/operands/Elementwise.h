@@ -1,0 +1,84 @@
+// The parameter-free operands of a CIFAR-style network: ReLU, MaxPool2D, Softmax — each a thin call into the seblas
+// operator of the same name, with the reference's members and gradient bookkeeping (the reserve gradient a shortcut
+// may have deposited in Y->dAReserve is folded into Y->dA first and cleared afterwards).
+// seann/operands/seblas/activate/ReLU.{cuh,cu}, pooling/MaxPool2D.{cuh,cu}, Softmax.{cuh,cu}.
+#pragma once
+#include "OperandBase.h"
+
+#define OPR_SEBLAS_RELU 0xa002
+#define OPR_SEBLAS_MAXPOOL2D 0xb003
+#define OPR_SEBLAS_SOFTMAX 0x0003
+
+namespace seann {
+
+class ParamFreeOperand : public OperandBase {
+public:
+    void paramGrads() override {}
+    void randFillNetParams() override {}
+    void zeroGrads() override {}
+
+protected:
+    void foldReserve() const { *Y->dA + Y->dAReserve; }
+    void clearReserve() const { Y->dAReserve->constFill(0); }
+};
+
+class ReLU : public ParamFreeOperand {
+public:
+    uint32 INPUT_SIZE{};
+    uint32 PARALELL_SIZE{};
+    std::string info() override { return "ReLU          { " + std::to_string(INPUT_SIZE / PARALELL_SIZE) + " }"; }
+    void initNetParams(OptimizerInfo *, shape4 inShape) override {  // ReLU.cuh:27-32
+        INPUT_SIZE = inShape.size;
+        PARALELL_SIZE = inShape.n;
+        X = Parameter::declare(inShape);
+        Y = Parameter::create(inShape);
+    }
+    void forward() override { relu(X->A, Y->A); }  // ReLU.cu:8-10
+    void xGrads() override {                         // ReLU.cu:13-17
+        foldReserve();
+        reluGradFast(X->A, Y->dA, X->dA);
+        clearReserve();
+    }
+    uint32 OPERAND_ID() override { return OPR_SEBLAS_RELU; }
+};
+
+class MaxPool2D : public ParamFreeOperand {
+public:
+    Tensor *record{};
+    uint32 strideH, strideW, rangeH, rangeW;
+    MaxPool2D(uint32 strideH, uint32 strideW, uint32 rangeH, uint32 rangeW)
+        : strideH(strideH), strideW(strideW), rangeH(rangeH), rangeW(rangeW) {}
+    std::string info() override { return "MaxPool2D     { " + X->A->dims.toString() + ", " + Y->A->dims.toString() + " }"; }
+    void initNetParams(OptimizerInfo *, shape4 inShape) override {  // MaxPool2D.cuh:42-51
+        X = Parameter::declare(inShape);
+        Y = Parameter::create(inShape.n, inShape.c, inShape.h / strideH, inShape.w / strideW);
+        record = Tensor::create(inShape.n, inShape.c, ((inShape.h - (rangeH - strideH)) / strideH) * rangeH,
+                                ((inShape.w - (rangeW - strideW)) / strideW) * rangeW);
+    }
+    void forward() override { maxPool(X->A, Y->A, record, strideH, strideW, rangeH, rangeW); }  // MaxPool2D.cu:12-14
+    void xGrads() override {                                                                     // MaxPool2D.cu:16-20
+        foldReserve();
+        maxPoolBack(X->dA, Y->dA, record, strideH, strideW, rangeH, rangeW);
+        clearReserve();
+    }
+    uint32 OPERAND_ID() override { return OPR_SEBLAS_MAXPOOL2D; }
+};
+
+// Output probabilities; the loss function writes Y->dA = Y->A - labels, which is already the gradient with respect to
+// the softmax input, so xGrads only passes it on (Softmax.cu:12-18).
+class Softmax : public ParamFreeOperand {
+public:
+    std::string info() override { return "Softmax       { " + std::to_string(Y->A->dims.size / Y->A->dims.n) + " }"; }
+    void initNetParams(OptimizerInfo *, shape4 inShape) override {
+        X = Parameter::declare(inShape);
+        Y = Parameter::create(inShape);
+    }
+    void forward() override { softmax(X->A, Y->A, nullptr, Y->A->dims.size / Y->A->dims.n); }  // Softmax.cu:8-10
+    void xGrads() override {
+        foldReserve();
+        Y->dA->copyToD2D(X->dA);
+        clearReserve();
+    }
+    uint32 OPERAND_ID() override { return OPR_SEBLAS_SOFTMAX; }
+};
+}  // namespace seann

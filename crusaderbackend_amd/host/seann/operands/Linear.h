@@ -26,6 +26,14 @@ public:
     void xGrads() override;
     void randFillNetParams() override;
     void zeroGrads() override;
+    void updateParams() override {  // Linear.cu:25-28
+        weights->update();
+        biases->update();
+    }
+    void batchUpdateParams() override {
+        weights->batchUpdate();
+        biases->batchUpdate();
+    }
     uint32 OPERAND_ID() override { return OPR_SEBLAS_LINEAR; }
 };
 }  // namespace seann

@@ -1,7 +1,6 @@
-// seann::OperandBase — the operand plugin interface of the reference (seann/operands/OperandBase.cuh:16-108),
-// restricted to what the conv / linear operands of this build implement: forward / xGrads / paramGrads,
-// parameter initialisation and graph wiring. Optimizer application and checkpoint encoding are outside
-// this build; their virtuals are kept with empty defaults so operand code reads like the reference's.
+// seann::OperandBase — the operand plugin interface of the reference (seann/operands/OperandBase.cuh:16-108):
+// forward / xGrads / paramGrads, parameter initialisation, optimizer application and graph wiring. Checkpoint
+// encoding is outside this build.
 #pragma once
 #include <string>
 
@@ -27,6 +26,7 @@ public:
     virtual void batchUpdateParams() {}
     virtual void initNetParams(OptimizerInfo *info, shape4 inShape) = 0;
     virtual void randFillNetParams() = 0;
+    virtual void postWaiveInit(OptimizerInfo *) {}  // second construction pass, after the chain is bound
     virtual void inferenceForward() { forward(); }
     virtual void zeroGrads() = 0;
     virtual std::string info() = 0;
@@ -35,6 +35,8 @@ public:
     void bindPrev(OperandBase *p) { prev = p; }
     void bindNext(OperandBase *n) { next = n; }
     void bindInput(Parameter *prevY) const { X->inherit(prevY); }
+    OperandBase *tracePrev() const { return prev; }
+    OperandBase *traceNext() const { return next; }
     OperandBase *tracePrev(uint32 ago) { return ago == 0 ? this : prev->tracePrev(ago - 1); }
     OperandBase *traceNext(uint32 dist) { return dist == 0 ? this : next->traceNext(dist - 1); }
 };

@@ -1,0 +1,44 @@
+// seann::ShortcutEndpoint — the pair of markers that delimit a residual connection in a Sequential
+// (seann/operands/controlling/ShortcutEndpoint.{cuh,cu}). The opening endpoint (isContainer = false) forwards its input
+// unchanged; the closing endpoint (isContainer = true, same uuid) adds to the main path either the opening endpoint's
+// output (identity shortcut) or the output of its own branch operands applied to it (projection shortcut). Backward, the
+// closing endpoint hands its output gradient to the branch (or, for the identity, to the opening endpoint's reserve
+// gradient), and the opening endpoint folds that reserve into the gradient it passes further back.
+#pragma once
+#include <initializer_list>
+#include <vector>
+
+#include "OperandBase.h"
+
+#define OPR_CTRL_SHORTCUTENDPOINT_BEG 0xf002
+#define OPR_CTRL_SHORTCUTENDPOINT_END 0xf003
+
+namespace seann {
+
+class ShortcutEndpoint : public OperandBase {
+public:
+    bool isContainer;
+    ShortcutEndpoint *other{};
+    std::vector<OperandBase *> branchOperands;
+    uint32 operandCount = 0;
+    uint32 uuid;
+
+    ShortcutEndpoint(bool isContainer, uint32 uuid, std::initializer_list<OperandBase *> operands)
+        : isContainer(isContainer), uuid(uuid) {
+        if (isContainer) branchOperands.assign(operands.begin(), operands.end());
+        operandCount = uint32(branchOperands.size());
+    }
+
+    void initNetParams(OptimizerInfo *info, shape4 inShape) override;
+    void postWaiveInit(OptimizerInfo *info) override;
+    void forward() override;
+    void xGrads() override;
+    void paramGrads() override;
+    void updateParams() override;
+    void batchUpdateParams() override;
+    void randFillNetParams() override;
+    void zeroGrads() override;
+    std::string info() override { return "ShortcutEndpoint { " + std::to_string(operandCount) + " }"; }
+    uint32 OPERAND_ID() override { return isContainer ? OPR_CTRL_SHORTCUTENDPOINT_END : OPR_CTRL_SHORTCUTENDPOINT_BEG; }
+};
+}  // namespace seann

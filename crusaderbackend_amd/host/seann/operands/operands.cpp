@@ -2,11 +2,15 @@
 #include <hip/hip_runtime_api.h>
 
 #include <cmath>
+#include <stdexcept>
 
 #include "../../../../include/crusader_hip.h"
 #include "../../seblas/assist/HipAssert.h"
+#include "../containers/Sequential.h"
 #include "Conv2D.h"
+#include "Elementwise.h"
 #include "Linear.h"
+#include "ShortcutEndpoint.h"
 
 namespace seann {
 
@@ -36,7 +40,7 @@ void Conv2D::paramGrads() {  // Conv2D.cu:24-29; the bias gradient is the per-ch
         const shape4 &d = Y->dA->dims;
         throwOnStatus(crb_conv_bias_grad(Y->dA->elements, bias->grad()->elements, d.n, d.c, d.h * d.w, nullptr), __FILE__,
                       __LINE__);
-        if (hipStreamSynchronize(nullptr) != hipSuccess) assertHip(__FILE__, __LINE__);
+        if (isBlocking() && hipStreamSynchronize(nullptr) != hipSuccess) assertHip(__FILE__, __LINE__);
     }
 }
 
@@ -79,6 +83,152 @@ void Linear::randFillNetParams() {  // Linear.cu:42-46
 void Linear::zeroGrads() {
     weights->zeroGrad();
     biases->zeroGrad();
+}
+
+// ---- ShortcutEndpoint (seann/operands/controlling/ShortcutEndpoint.cu) ---------------------------------------------------
+void ShortcutEndpoint::initNetParams(OptimizerInfo *, shape4 inShape) {  // :8-11
+    X = Parameter::declare(inShape);
+    Y = Parameter::create(inShape);
+}
+
+void ShortcutEndpoint::postWaiveInit(OptimizerInfo *inf) {  // :13-55
+    if (isContainer) {
+        OperandBase *tracer = tracePrev();
+        while (tracer && (tracer->OPERAND_ID() != OPR_CTRL_SHORTCUTENDPOINT_BEG || static_cast<ShortcutEndpoint *>(tracer)->uuid != uuid))
+            tracer = tracer->tracePrev();
+        if (!tracer) throw std::invalid_argument("ShortcutEndpoint: no opening endpoint with this uuid");
+        other = static_cast<ShortcutEndpoint *>(tracer);
+        if (operandCount > 0) {
+            branchOperands[0]->initNetParams(inf, other->Y->A->dims);
+            for (uint32 i = 1; i < operandCount; i++) branchOperands[i]->initNetParams(inf, branchOperands[i - 1]->Y->A->dims);
+            if (!(branchOperands[operandCount - 1]->Y->A->dims == Y->A->dims))
+                throw std::invalid_argument("ShortcutEndpoint: branch output shape differs from the main path");
+            branchOperands[0]->bindPrev(other);
+            branchOperands[0]->bindInput(other->Y);
+            branchOperands[0]->X->dA = other->Y->dAReserve;  // the branch's input gradient lands in the reserve
+            for (uint32 i = 1; i < operandCount; i++) {
+                branchOperands[i]->bindPrev(branchOperands[i - 1]);
+                branchOperands[i]->bindInput(branchOperands[i - 1]->Y);
+            }
+            for (uint32 i = 0; i < operandCount; i++) branchOperands[i]->postWaiveInit(inf);
+        }
+    } else {
+        OperandBase *tracer = traceNext();
+        while (tracer && (tracer->OPERAND_ID() != OPR_CTRL_SHORTCUTENDPOINT_END || static_cast<ShortcutEndpoint *>(tracer)->uuid != uuid))
+            tracer = tracer->traceNext();
+        if (!tracer) throw std::invalid_argument("ShortcutEndpoint: no closing endpoint with this uuid");
+        other = static_cast<ShortcutEndpoint *>(tracer);
+    }
+}
+
+void ShortcutEndpoint::forward() {  // :57-74
+    X->A->copyToD2D(Y->A);
+    if (isContainer) {
+        if (operandCount > 0) {
+            for (uint32 i = 0; i < operandCount; i++) branchOperands[i]->forward();
+            *Y->A + branchOperands[operandCount - 1]->Y->A;
+        } else {
+            *Y->A + other->Y->A;  // identity shortcut
+        }
+    }
+}
+
+void ShortcutEndpoint::xGrads() {  // :76-99
+    if (isContainer) {
+        if (operandCount > 0) {
+            Y->dA->copyToD2D(branchOperands[operandCount - 1]->Y->dA);
+            for (int i = int(operandCount) - 1; i >= 0; i--) branchOperands[i]->xGrads();
+        } else {
+            Y->dA->copyToD2D(other->Y->dAReserve);
+        }
+    } else {
+        *Y->dA + Y->dAReserve;
+        Y->dAReserve->constFill(0);
+    }
+    Y->dA->copyToD2D(X->dA);
+}
+
+void ShortcutEndpoint::paramGrads() {
+    for (OperandBase *op : branchOperands) op->paramGrads();
+}
+void ShortcutEndpoint::updateParams() {
+    for (OperandBase *op : branchOperands) op->updateParams();
+}
+void ShortcutEndpoint::batchUpdateParams() {
+    for (OperandBase *op : branchOperands) op->batchUpdateParams();
+}
+void ShortcutEndpoint::randFillNetParams() {
+    for (OperandBase *op : branchOperands) op->randFillNetParams();
+}
+void ShortcutEndpoint::zeroGrads() {
+    for (OperandBase *op : branchOperands) op->zeroGrads();
+}
+
+// ---- Sequential (seann/containers/Sequential.cu:10-103) -----------------------------------------------------------------
+void Sequential::waive() const {
+    for (uint32 i = 1; i < OPERAND_COUNT; i++) {
+        operands[i]->bindPrev(operands[i - 1]);
+        operands[i]->bindInput(operands[i - 1]->Y);
+    }
+    for (uint32 i = 0; i + 1 < OPERAND_COUNT; i++) operands[i]->bindNext(operands[i + 1]);
+}
+
+void Sequential::construct(OptimizerInfo *info) {
+    if (OPERAND_COUNT == 0) throw std::invalid_argument("Sequential: no operands");
+    for (uint32 i = 0; i < OPERAND_COUNT; i++) {
+        operands[i]->initNetParams(info, i == 0 ? netX->A->dims : operands[i - 1]->Y->A->dims);
+        operands[i]->operandID = i;
+    }
+    operands[0]->X->inherit(netX);
+    netY = Parameter::declare(operands[OPERAND_COUNT - 1]->Y->A->dims)->inherit(operands[OPERAND_COUNT - 1]->Y);
+    waive();
+    for (uint32 i = 0; i < OPERAND_COUNT; i++) operands[i]->postWaiveInit(info);
+}
+
+void Sequential::randInit() const {
+    for (OperandBase *op : operands) op->randFillNetParams();
+}
+
+Tensor *Sequential::forward() const {
+    for (OperandBase *op : operands) op->forward();
+    return netY->A;
+}
+
+Tensor *Sequential::forward(Tensor *X) const {
+    X->copyToD2D(netX->A);
+    return forward();
+}
+
+Tensor *Sequential::inferenceForward() const {
+    for (OperandBase *op : operands) op->inferenceForward();
+    return netY->A;
+}
+
+Tensor *Sequential::inferenceForward(Tensor *X) const {
+    X->copyToD2D(netX->A);
+    return inferenceForward();
+}
+
+Tensor *Sequential::backward(Tensor *label) const {
+    if (!loss) throw std::invalid_argument("Sequential::backward: no loss function set");
+    loss(netY, label);
+    for (int i = int(OPERAND_COUNT) - 1; i >= 0; i--) {
+        operands[i]->xGrads();
+        operands[i]->paramGrads();
+    }
+    return netX->dA;
+}
+
+void Sequential::learn() const {
+    for (OperandBase *op : operands) op->updateParams();
+}
+
+void Sequential::learnBatch() const {
+    for (OperandBase *op : operands) op->batchUpdateParams();
+}
+
+void Sequential::zeroGrads() const {
+    for (OperandBase *op : operands) op->zeroGrads();
 }
 
 }  // namespace seann

@@ -15,10 +15,14 @@ static void require(bool ok, const char *what) {
     if (!ok) throw std::invalid_argument(what);
 }
 
+static bool g_blocking = true;
+void setBlocking(bool blocking) { g_blocking = blocking; }
+bool isBlocking() { return g_blocking; }
+
 // every reference op ends with cudaDeviceSynchronize(); assertCuda(...)
 static void finish(int status, const char *file, int line) {
     throwOnStatus(status, file, line);
-    if (hipStreamSynchronize(nullptr) != hipSuccess) assertHip(file, line);
+    if (g_blocking && hipStreamSynchronize(nullptr) != hipSuccess) assertHip(file, line);
     assertHip(file, line);
 }
 

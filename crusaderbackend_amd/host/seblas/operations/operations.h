@@ -12,6 +12,12 @@
 #include "../tensor/Tensor.h"
 
 namespace seblas {
+// The reference blocks the host after every operator (cudaDeviceSynchronize), and so does this layer by default.
+// A caller that issues a whole step on the default stream and synchronises once can switch that off; device errors
+// then surface at its own synchronisation point. No counterpart in the reference.
+void setBlocking(bool blocking);
+bool isBlocking();
+
 // cuGEMM.cu:1649-1714
 Tensor *sgemm(Tensor *A, Tensor *B, Tensor *C);     // C[n] = A * B[n]
 Tensor *sgemmTN(Tensor *A, Tensor *B, Tensor *C);   // C[n] = A^T * B[n]

@@ -2,6 +2,8 @@
 // shape-error translation, which all happen before any device work). Mode "gpu" drives the reference-shaped API
 // end to end on the device — Tensor::create / copy / seblas::conv ... / seann::Conv2D, Linear — and checks results
 // against the CPU oracle (linked here as the checker only).
+#include <hip/hip_runtime_api.h>
+
 #include <cmath>
 #include <cstdio>
 #include <cstring>
@@ -11,7 +13,10 @@
 
 #include "../../crusaderbackend_amd/csrc/crb_common.h"
 #include "../../crusaderbackend_amd/host/seann/operands/Conv2D.h"
+#include "../../crusaderbackend_amd/host/seann/containers/Sequential.h"
+#include "../../crusaderbackend_amd/host/seann/operands/Elementwise.h"
 #include "../../crusaderbackend_amd/host/seann/operands/Linear.h"
+#include "../../crusaderbackend_amd/host/seann/operands/ShortcutEndpoint.h"
 
 extern "C" {
 void oracle_sgemm(const float *, const float *, float *, uint32_t, uint32_t, uint32_t, uint32_t, int);
@@ -317,12 +322,156 @@ static void gpu_elementwise_tests() {
     CHECK(pull(A) == ra);
 }
 
+// seann::Sequential with residual connections (identity and projection shortcuts), the parameter-free operands and the
+// momentum optimizer: one training step through the container, and the same step written out by hand with the seblas
+// operators on separate tensors. Both run the same deterministic kernels, so every tensor must agree bit for bit; that
+// pins the graph wiring (input aliasing, reserve gradients of the shortcuts, update order), not the arithmetic, which the
+// operator tests pin. The forward result is also checked against the CPU oracle.
+static Tensor *clone(Tensor *t) {
+    Tensor *c = Tensor::create(t->dims);
+    t->copyToD2D(c);
+    return c;
+}
+
+static void gpu_sequential_tests() {
+    using namespace seann;
+    const uint32_t N = 4;
+    auto *c1 = new Conv2D(shape4(8, 3, 3, 3), 1, 1, 1, 1, true);
+    auto *c2 = new Conv2D(shape4(8, 8, 3, 3), 1, 1, 1, 1, true);
+    auto *c3 = new Conv2D(shape4(8, 8, 3, 3), 1, 1, 1, 1, false);
+    auto *c4 = new Conv2D(shape4(16, 8, 3, 3), 2, 2, 1, 1, true);
+    auto *cp = new Conv2D(shape4(16, 8, 1, 1), 2, 2, 0, 0, false);  // projection shortcut
+    auto *fc = new Linear(10);
+    OPTIMIZER_MOMENTUM opt(0.05f, 0.9f);
+    Sequential net(shape4(N, 3, 8, 8),
+                   {c1, new ReLU(), new MaxPool2D(2, 2, 2, 2),
+                    new ShortcutEndpoint(false, 1, {}), c2, new ReLU(), c3, new ShortcutEndpoint(true, 1, {}), new ReLU(),
+                    new ShortcutEndpoint(false, 2, {}), c4, new ShortcutEndpoint(true, 2, {cp}), new ReLU(),
+                    fc, new Softmax()});
+    net.construct(&opt);
+    net.setLoss(crossEntropyLoss, crossEntropyCalc);
+    net.randInit();
+    CHECK(net.netY->A->dims.size == N * 10);
+    CHECK(c4->Y->A->dims == shape4(N, 16, 2, 2) && cp->Y->A->dims == shape4(N, 16, 2, 2));
+
+    auto x = randn(N * 3 * 8 * 8, 31);
+    std::vector<float> lab(N * 10, 0.f);
+    for (uint32_t n = 0; n < N; ++n) lab[n * 10 + (3 * n + 1) % 10] = 1.f;
+    Tensor *X = push(shape4(N, 3, 8, 8), x), *L = push(shape4(N, 1, 10, 1), lab);
+
+    // copies of the initial parameters for the hand-written step
+    Tensor *w1 = clone(c1->filter->data()), *b1 = clone(c1->bias->data()), *w2 = clone(c2->filter->data()),
+           *b2 = clone(c2->bias->data()), *w3 = clone(c3->filter->data()), *w4 = clone(c4->filter->data()),
+           *b4 = clone(c4->bias->data()), *wp = clone(cp->filter->data()), *wf = clone(fc->weights->data()),
+           *bf = clone(fc->biases->data());
+
+    net.forward(X);
+    net.backward(L);
+    Tensor *lossBuf = Tensor::create(net.netY->A->dims);
+    const float loss = net.lossFW(net.netY, L, lossBuf);
+    auto g_w1 = pull(c1->filter->grad()), g_b1 = pull(c1->bias->grad()), g_w3 = pull(c3->filter->grad()),
+         g_wp = pull(cp->filter->grad()), g_wf = pull(fc->weights->grad()), g_dx = pull(net.netX->dA);
+    auto probs = pull(net.netY->A);
+    net.learn();
+
+    // ---- the same step by hand ----
+    auto T = [&](uint32_t c, uint32_t h) { return Tensor::create(N, c, h, h); };
+    Tensor *z1 = T(8, 8), *a1 = T(8, 8), *p1 = T(8, 4), *rec = T(8, 8), *z2 = T(8, 4), *a2 = T(8, 4), *z3 = T(8, 4), *s1 = T(8, 4),
+           *a3 = T(8, 4), *z4 = T(16, 2), *zp = T(16, 2), *s2 = T(16, 2), *a4 = T(16, 2);
+    Tensor *zf = Tensor::create(N, 1, 10, 1);
+    seblas::Parameter *P = seblas::Parameter::create(N, 1, 10, 1);
+    conv(w1, X, z1, 1, 1, 1, 1, b1);
+    relu(z1, a1);
+    maxPool(a1, p1, rec, 2, 2, 2, 2);
+    conv(w2, p1, z2, 1, 1, 1, 1, b2);
+    relu(z2, a2);
+    conv(w3, a2, z3, 1, 1, 1, 1, nullptr);
+    z3->copyToD2D(s1);
+    *s1 + p1;  // identity shortcut
+    relu(s1, a3);
+    conv(w4, a3, z4, 2, 2, 1, 1, b4);
+    conv(wp, a3, zp, 2, 2, 0, 0, nullptr);
+    z4->copyToD2D(s2);
+    *s2 + zp;  // projection shortcut
+    relu(s2, a4);
+    Tensor *a4flat = Tensor::declare(N, 1, 64, 1)->attach(a4);
+    linear(a4flat, wf, bf, zf);
+    softmax(zf, P->A, nullptr, 10);
+    CHECK(pull(P->A) == probs);
+    {   // forward against the CPU oracle (first convolution + ReLU + pooling, then the final probabilities sum to 1)
+        std::vector<float> rz(N * 8 * 64), ra(N * 8 * 64), rp(N * 8 * 16), rr(N * 8 * 64);
+        auto hw1 = pull(w1), hb1 = pull(b1);
+        oracle_conv(hw1.data(), x.data(), rz.data(), hb1.data(), N, 3, 8, 8, 8, 3, 3, 8, 8, 1, 1, 1, 1, 2);
+        oracle_relu(rz.data(), ra.data(), N * 8 * 64);
+        oracle_maxPool(ra.data(), rp.data(), rr.data(), N * 8, 8, 8, 2, 2);
+        compare("Sequential: conv+relu+pool", pull(p1), rp, 27);
+        for (uint32_t n = 0; n < N; ++n) {
+            float sum = 0.f;
+            for (int k = 0; k < 10; ++k) sum += probs[n * 10 + k];
+            CHECK(std::fabs(sum - 1.f) < 1e-5f);
+        }
+    }
+    crossEntropyLoss(P, L);
+    CHECK(crossEntropyCalc(P, L, Tensor::create(N, 1, 10, 1)) == loss);
+    // backward
+    Tensor *dwf = Tensor::create(wf->dims), *dbf = Tensor::create(bf->dims), *da4 = Tensor::create(N, 1, 64, 1);
+    linearXGrad(P->dA, wf, da4);
+    linearParamGrad(P->dA, a4flat, dwf, dbf);
+    CHECK(pull(dwf) == g_wf);
+    Tensor *ds2 = T(16, 2), *da3 = T(8, 4), *da3p = T(8, 4), *dwp = Tensor::create(wp->dims), *dw4 = Tensor::create(w4->dims);
+    reluGradFast(s2, Tensor::declare(N, 16, 2, 2)->attach(da4), ds2);
+    convDerive(wp, ds2, da3p, 2, 2, 0, 0);  // projection branch
+    convError(ds2, a3, dwp, 2, 2, 0, 0);
+    CHECK(pull(dwp) == g_wp);
+    convDerive(w4, ds2, da3, 2, 2, 1, 1);  // main branch
+    convError(ds2, a3, dw4, 2, 2, 1, 1);
+    *da3 + da3p;
+    Tensor *ds1 = T(8, 4), *da2 = T(8, 4), *dz2 = T(8, 4), *dp1 = T(8, 4), *dw3 = Tensor::create(w3->dims), *dw2 = Tensor::create(w2->dims);
+    reluGradFast(s1, da3, ds1);
+    convDerive(w3, ds1, da2, 1, 1, 1, 1);
+    convError(ds1, a2, dw3, 1, 1, 1, 1);
+    CHECK(pull(dw3) == g_w3);
+    reluGradFast(z2, da2, dz2);
+    convDerive(w2, dz2, dp1, 1, 1, 1, 1);
+    convError(dz2, p1, dw2, 1, 1, 1, 1);
+    *dp1 + ds1;  // identity shortcut: the block input also receives the block output's gradient
+    Tensor *da1 = T(8, 8), *dz1 = T(8, 8), *dx = Tensor::create(N, 3, 8, 8), *dw1 = Tensor::create(w1->dims), *db1 = Tensor::create(b1->dims);
+    maxPoolBack(da1, dp1, rec, 2, 2, 2, 2);
+    reluGradFast(z1, da1, dz1);
+    convDerive(w1, dz1, dx, 1, 1, 1, 1);
+    convError(dz1, X, dw1, 1, 1, 1, 1);
+    CHECK(crb_conv_bias_grad(dz1->elements, db1->elements, N, 8, 64, nullptr) == 0);
+    CHECK(pull(dw1) == g_w1);
+    CHECK(pull(db1) == g_b1);
+    CHECK(pull(dx) == g_dx);
+    // update: weights decay with the optimizer's default L2, biases do not
+    Tensor *m1 = Tensor::create(w1->dims), *mb1 = Tensor::create(b1->dims), *mf = Tensor::create(wf->dims);
+    momentumApplyDecay(w1, dw1, m1, 0.05f, 0.9f, 0.0001f);
+    momentumApplyDecay(b1, db1, mb1, 0.05f, 0.9f, 0.0f);
+    momentumApplyDecay(wf, dwf, mf, 0.05f, 0.9f, 0.0001f);
+    CHECK(pull(w1) == pull(c1->filter->data()));
+    CHECK(pull(b1) == pull(c1->bias->data()));
+    CHECK(pull(wf) == pull(fc->weights->data()));
+    for (float v : pull(c1->filter->grad())) CHECK(v == 0.f);  // gradients are cleared by the step
+    // a second forward after the update runs and changes the loss
+    net.forward(X);
+    CHECK(net.lossFW(net.netY, L, lossBuf) != loss);
+    // the non-blocking mode gives the same numbers
+    setBlocking(false);
+    net.forward(X);
+    net.backward(L);
+    CHECK(hipDeviceSynchronize() == hipSuccess);
+    setBlocking(true);
+    CHECK(throws_invalid([&] { Sequential bad(shape4(1, 3, 8, 8), {new ShortcutEndpoint(true, 9, {})}); bad.construct(nullptr); }));
+}
+
 int main(int argc, char **argv) {
     const bool gpu = argc > 1 && std::strcmp(argv[1], "gpu") == 0;
     try {
         if (gpu) {
             gpu_tests();
             gpu_elementwise_tests();
+            gpu_sequential_tests();
         }
         else
             host_tests();
