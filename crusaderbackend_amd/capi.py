@@ -56,6 +56,8 @@ SIGNATURES = {
     "crb_tensor_add_inplace": (ctypes.c_int, [_ptr, _ptr, _u32, _ptr]),
     "crb_tensor_fill": (ctypes.c_int, [_ptr, ctypes.c_float, _u32, _ptr]),
     "crb_tensor_sub_inplace": (ctypes.c_int, [_ptr, _ptr, _u32, _ptr]),
+    "crb_tensor_copy": (ctypes.c_int, [_ptr, _ptr, _u32, _ptr]),
+    "crb_tensor_add_clear": (ctypes.c_int, [_ptr, _ptr, _u32, _ptr]),
     "crb_tensor_scale_inplace": (ctypes.c_int, [_ptr, ctypes.c_float, _u32, _ptr]),
     "crb_relu_fwd": (ctypes.c_int, [_ptr, _ptr, _u32, _ptr]),
     "crb_relu_bwd": (ctypes.c_int, [_ptr, _ptr, _ptr, _u32, _ptr]),
@@ -65,6 +67,10 @@ SIGNATURES = {
     "crb_cross_entropy_grad": (ctypes.c_int, [_ptr, _ptr, _ptr, _u32, _ptr]),
     "crb_cross_entropy_scratch_floats": (_u32, [_u32]),
     "crb_cross_entropy_loss": (ctypes.c_int, [_ptr, _ptr, _ptr, _u32, _ptr, _u32, _ptr]),
+    "crb_momentum_apply_multi": (ctypes.c_int, [_ptr, _u32, _u32, _ptr]),
+    "crb_batchnorm_fwd": (ctypes.c_int, [_ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _u32, _u32, _ptr]),
+    "crb_batchnorm_bwd": (ctypes.c_int, [_ptr, _ptr, _ptr, _ptr, _u32, _u32, _ptr]),
+    "crb_batchnorm_param_grads": (ctypes.c_int, [_ptr, _ptr, _ptr, _ptr, _u32, _u32, _ptr]),
     "crb_momentum_apply": (ctypes.c_int, [_ptr, _ptr, _ptr, _u32, ctypes.c_float, ctypes.c_float, ctypes.c_float, _ptr]),
 }
 
@@ -211,3 +217,44 @@ def cross_entropy_loss(Y, labels, scratch, loss_out, count, stream=None):
 
 def momentum_apply(X, G, M, count, lr, beta, decay=1.0, stream=None):
     check(load().crb_momentum_apply(_p(X), _p(G), _p(M), count, lr, beta, decay, _stream(stream)))
+
+
+def batchnorm_fwd(X, beta, gamma, mean, var, Y, xHat, N, F, stream=None):
+    check(load().crb_batchnorm_fwd(_p(X), _p(beta), _p(gamma), _p(mean), _p(var), _p(Y), _p(xHat), N, F, _stream(stream)))
+
+
+def batchnorm_bwd(dY, gamma, X, dX, N, F, stream=None):
+    check(load().crb_batchnorm_bwd(_p(dY), _p(gamma), _p(X), _p(dX), N, F, _stream(stream)))
+
+
+def batchnorm_param_grads(dY, xHat, dGamma, dBeta, N, F, stream=None):
+    check(load().crb_batchnorm_param_grads(_p(dY), _p(xHat), _p(dGamma), _p(dBeta), N, F, _stream(stream)))
+
+
+def tensor_copy(dst, src, count, stream=None):
+    check(load().crb_tensor_copy(_p(dst), _p(src), count, _stream(stream)))
+
+
+def tensor_add_clear(a, b, count, stream=None):
+    check(load().crb_tensor_add_clear(_p(a), _p(b), count, _stream(stream)))
+
+
+class MomentumItem(ctypes.Structure):
+    """Mirror of ``crb_momentum_item``."""
+
+    _fields_ = [("X", ctypes.c_void_p), ("G", ctypes.c_void_p), ("M", ctypes.c_void_p), ("count", _u32),
+                ("lr", ctypes.c_float), ("beta", ctypes.c_float), ("decay", ctypes.c_float)]
+
+
+def momentum_table(torch, dev, entries):
+    """entries: (X, G, M, lr, beta, decay) tuples of device tensors / floats -> (device byte tensor holding the table, n,
+    largest count). The tensors must stay alive as long as the table is used."""
+    arr = (MomentumItem * len(entries))()
+    for i, (X, G, M, lr, beta, decay) in enumerate(entries):
+        arr[i] = MomentumItem(X.data_ptr(), G.data_ptr(), M.data_ptr(), X.numel(), lr, beta, decay)
+    raw = torch.frombuffer(bytearray(bytes(arr)), dtype=torch.uint8).to(dev)
+    return raw, len(entries), max(e[0].numel() for e in entries)
+
+
+def momentum_apply_multi(table, n_items, max_count, stream=None):
+    check(load().crb_momentum_apply_multi(_p(table), n_items, max_count, _stream(stream)))

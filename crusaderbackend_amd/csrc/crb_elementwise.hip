@@ -1,6 +1,6 @@
 // Elementwise and small reduction operators that sit between the GEMM / convolution calls of a training step:
 // ReLU and its gradient, max pooling (non-overlapping windows) and its gradient, row softmax, cross-entropy value and
-// gradient, in-place subtract / scale, and the momentum update with weight decay.
+// gradient, in-place subtract / scale, the momentum update with weight decay, and per-feature batch normalisation.
 // All are HBM-bound streaming kernels: 16-byte accesses where alignment allows, grid-stride loops, and reductions
 // with a fixed association (bit-reproducible, no atomics).
 #include "igemm_engine.h"
@@ -282,6 +282,209 @@ __global__ void __launch_bounds__(256) momentum_kernel(float *__restrict__ X, fl
     }
 }
 
+// ---- batch normalisation per feature over the batch -------------------------------------------------------------------
+// X viewed as N x F. A workgroup owns FL consecutive features and splits the samples over G = 256 / FL lane groups: group
+// g takes samples g, g+G, ...; per-feature sums are combined through LDS in group order (fixed association). FL is 64
+// (256-byte row segments) when that already yields enough workgroups for the chip, else 32 or 16, which also shortens
+// each thread's sample loop. A thread keeps up to kBnCache of its samples in registers (N <= G * kBnCache: every tensor is
+// then read from memory once, with all loads of a sweep in flight together); beyond that it re-reads them.
+constexpr int kBnCache = 16;
+
+template <int FL>
+struct BnGeom {
+    static constexpr u32 G = 256 / FL;
+    u32 fl, g, f;
+    bool on;
+    __device__ __forceinline__ BnGeom(u32 F) : fl(threadIdx.x % FL), g(threadIdx.x / FL), f(blockIdx.x * FL + fl), on(f < F) {}
+    // sum of v over the G lane groups of feature fl, in group order
+    __device__ __forceinline__ float reduce(float v, float (*red)[FL]) const {
+        __syncthreads();  // the previous use of `red` is over
+        red[g][fl] = v;
+        __syncthreads();
+        float r = red[0][fl];
+#pragma unroll
+        for (u32 k = 1; k < G; ++k) r += red[k][fl];
+        return r;
+    }
+};
+
+template <int FL>
+__global__ void __launch_bounds__(256) batchnorm_fwd_kernel(const float *__restrict__ X, const float *__restrict__ beta,
+                                                            const float *__restrict__ gamma, float *__restrict__ mean,
+                                                            float *__restrict__ var, float *__restrict__ Y, float *__restrict__ xHat,
+                                                            u32 N, u32 F) {
+    constexpr u32 G = 256 / FL;
+    __shared__ float red[G][FL];
+    const BnGeom<FL> t(F);
+    const bool cached = N <= G * kBnCache;
+    const float *x = X + (t.on ? t.f : 0);
+    float xv[kBnCache];
+    float s = 0.f;
+    if (cached) {
+#pragma unroll
+        for (int i = 0; i < kBnCache; ++i) {
+            const u32 n = t.g + G * i;
+            xv[i] = (t.on && n < N) ? x[size_t(n) * F] : 0.f;
+        }
+#pragma unroll
+        for (int i = 0; i < kBnCache; ++i) s += xv[i];
+    } else if (t.on) {
+        for (u32 n = t.g; n < N; n += G) s += x[size_t(n) * F];
+    }
+    const float m = t.reduce(s, red) / float(N);
+    float q = 0.f;
+    if (cached) {
+#pragma unroll
+        for (int i = 0; i < kBnCache; ++i) {
+            const float d = xv[i] - m;
+            q += (t.g + G * i < N) ? d * d : 0.f;
+        }
+    } else if (t.on) {
+        for (u32 n = t.g; n < N; n += G) {
+            const float d = x[size_t(n) * F] - m;
+            q += d * d;
+        }
+    }
+    const float v = t.reduce(q, red) / float(N);
+    if (!t.on) return;
+    const float inv = 1.0f / sqrtf(v + 1e-8f), ga = gamma[t.f], be = beta[t.f];
+    if (cached) {
+#pragma unroll
+        for (int i = 0; i < kBnCache; ++i) {
+            const u32 n = t.g + G * i;
+            if (n < N) {
+                const float xh = (xv[i] - m) * inv;
+                xHat[size_t(n) * F + t.f] = xh;
+                Y[size_t(n) * F + t.f] = xh * ga + be;
+            }
+        }
+    } else {
+        for (u32 n = t.g; n < N; n += G) {
+            const float xh = (x[size_t(n) * F] - m) * inv;
+            xHat[size_t(n) * F + t.f] = xh;
+            Y[size_t(n) * F + t.f] = xh * ga + be;
+        }
+    }
+    if (t.g == 0) mean[t.f] = m, var[t.f] = v;
+}
+
+template <int FL>
+__global__ void __launch_bounds__(256) batchnorm_bwd_kernel(const float *__restrict__ dY, const float *__restrict__ gamma,
+                                                            const float *__restrict__ X, float *__restrict__ dX, u32 N, u32 F) {
+    constexpr u32 G = 256 / FL;
+    __shared__ float red[G][FL];
+    const BnGeom<FL> t(F);
+    const bool cached = N <= G * kBnCache;
+    const float *x = X + (t.on ? t.f : 0), *dy = dY + (t.on ? t.f : 0);
+    float xv[kBnCache], dv[kBnCache];
+    float s = 0.f;
+    if (cached) {
+#pragma unroll
+        for (int i = 0; i < kBnCache; ++i) {
+            const u32 n = t.g + G * i;
+            const bool ok = t.on && n < N;
+            xv[i] = ok ? x[size_t(n) * F] : 0.f;
+            dv[i] = ok ? dy[size_t(n) * F] : 0.f;
+        }
+#pragma unroll
+        for (int i = 0; i < kBnCache; ++i) s += xv[i];
+    } else if (t.on) {
+        for (u32 n = t.g; n < N; n += G) s += x[size_t(n) * F];
+    }
+    const float m = t.reduce(s, red) / float(N);
+    // one sweep for the remaining sums: sum d^2, sum dy*d, sum dy, sum d  (d = x - mean)
+    float q = 0.f, sdd = 0.f, sdy = 0.f, sd = 0.f;
+    if (cached) {
+#pragma unroll
+        for (int i = 0; i < kBnCache; ++i) {
+            const bool ok = t.g + G * i < N;
+            const float d = ok ? xv[i] - m : 0.f;
+            q += d * d, sdd += dv[i] * d, sdy += dv[i], sd += d;
+        }
+    } else if (t.on) {
+        for (u32 n = t.g; n < N; n += G) {
+            const float d = x[size_t(n) * F] - m, e = dy[size_t(n) * F];
+            q += d * d, sdd += e * d, sdy += e, sd += d;
+        }
+    }
+    const float v = t.reduce(q, red) / float(N);
+    const float Sdd = t.reduce(sdd, red), Sdy = t.reduce(sdy, red), Sd = t.reduce(sd, red);
+    if (!t.on) return;
+    const float inv = 1.0f / sqrtf(v + 1e-8f), ga = gamma[t.f], invN = 1.0f / float(N);
+    const float dVar = ga * Sdd * -0.5f * inv * inv * inv;
+    const float dMean = ga * Sdy * -inv + dVar * (-2.0f * Sd) * invN;
+    if (cached) {
+#pragma unroll
+        for (int i = 0; i < kBnCache; ++i) {
+            const u32 n = t.g + G * i;
+            if (n < N) dX[size_t(n) * F + t.f] = dv[i] * ga * inv + dVar * (xv[i] - m) * 2.0f * invN + dMean * invN;
+        }
+    } else {
+        for (u32 n = t.g; n < N; n += G)
+            dX[size_t(n) * F + t.f] = dy[size_t(n) * F] * ga * inv + dVar * (x[size_t(n) * F] - m) * 2.0f * invN + dMean * invN;
+    }
+}
+
+template <int FL>
+__global__ void __launch_bounds__(256) batchnorm_param_grads_kernel(const float *__restrict__ dY, const float *__restrict__ xHat,
+                                                                    float *__restrict__ dGamma, float *__restrict__ dBeta, u32 N, u32 F) {
+    constexpr u32 G = 256 / FL;
+    __shared__ float red[G][FL];
+    const BnGeom<FL> t(F);
+    float db = 0.f, dg = 0.f;
+    if (t.on) {
+        const float *dy = dY + t.f, *xh = xHat + t.f;
+        u32 n = t.g;
+        for (; n + 3 * G < N; n += 4 * G) {  // four independent samples in flight
+            const float e0 = dy[size_t(n) * F], e1 = dy[size_t(n + G) * F], e2 = dy[size_t(n + 2 * G) * F], e3 = dy[size_t(n + 3 * G) * F];
+            const float h0 = xh[size_t(n) * F], h1 = xh[size_t(n + G) * F], h2 = xh[size_t(n + 2 * G) * F], h3 = xh[size_t(n + 3 * G) * F];
+            db += (e0 + e1) + (e2 + e3);
+            dg += (e0 * h0 + e1 * h1) + (e2 * h2 + e3 * h3);
+        }
+        for (; n < N; n += G) {
+            const float e = dy[size_t(n) * F];
+            db += e;
+            dg += e * xh[size_t(n) * F];
+        }
+    }
+    const float DB = t.reduce(db, red), DG = t.reduce(dg, red);
+    if (t.on && t.g == 0) dBeta[t.f] = DB, dGamma[t.f] = DG;
+}
+
+// features per workgroup: the widest of 64 / 32 / 16 that still gives at least 512 workgroups (16 if none does)
+static u32 bn_features_per_wg(u32 F) { return F >= 64 * 512 ? 64 : (F >= 32 * 512 ? 32 : 16); }
+
+static int check_bn(const char *what, u32 N, u32 F) {
+    if (!N || !F) return fail(CRB_EINVAL_SHAPE, "%s: zero dimension", what);
+    if (uint64_t(N) * F > 0x7fffffffull) return fail(CRB_EINVAL_SHAPE, "%s: tensor exceeds 2^31 elements", what);
+    return CRB_OK;
+}
+
+// The momentum step over a table of parameter tensors in one launch: blockIdx.y selects the item, the blocks of a row
+// stride over its elements. Same arithmetic as momentum_kernel.
+__global__ void __launch_bounds__(256) momentum_multi_kernel(const crb_momentum_item *__restrict__ items) {
+    const crb_momentum_item it = items[blockIdx.y];
+    const float omb = 1.0f - it.beta;
+    const u32 stride = gridDim.x * 256;
+    u32 i = blockIdx.x * 256 + threadIdx.x;
+    const bool vec = ((reinterpret_cast<uintptr_t>(it.X) | reinterpret_cast<uintptr_t>(it.G) | reinterpret_cast<uintptr_t>(it.M)) & 15u) == 0;
+    if (vec) {
+        const u32 nq = it.count / 4;
+        for (u32 q = i; q < nq; q += stride) {
+            const v4f xv = reinterpret_cast<v4f *>(it.X)[q], gv = reinterpret_cast<v4f *>(it.G)[q], mv = reinterpret_cast<v4f *>(it.M)[q];
+            float x[4] = {xv.x, xv.y, xv.z, xv.w}, g[4] = {gv.x, gv.y, gv.z, gv.w}, m[4] = {mv.x, mv.y, mv.z, mv.w};
+#pragma unroll
+            for (int k = 0; k < 4; ++k) momentum1(x[k], g[k], m[k], it.lr, it.beta, omb, it.decay);
+            reinterpret_cast<v4f *>(it.X)[q] = v4f{x[0], x[1], x[2], x[3]};
+            reinterpret_cast<v4f *>(it.G)[q] = v4f{g[0], g[1], g[2], g[3]};
+            reinterpret_cast<v4f *>(it.M)[q] = v4f{m[0], m[1], m[2], m[3]};
+        }
+        for (u32 r = nq * 4 + i; r < it.count; r += stride) momentum1(it.X[r], it.G[r], it.M[r], it.lr, it.beta, omb, it.decay);
+    } else {
+        for (; i < it.count; i += stride) momentum1(it.X[i], it.G[i], it.M[i], it.lr, it.beta, omb, it.decay);
+    }
+}
+
 static int check_pool(const char *what, u32 planes, u32 IH, u32 IW, u32 sH, u32 sW, u32 rH, u32 rW) {
     if (!planes || !IH || !IW || !sH || !sW || !rH || !rW) return fail(CRB_EINVAL_SHAPE, "%s: zero dimension", what);
     if (sH != rH || sW != rW)
@@ -402,6 +605,44 @@ int crb_tensor_scale_inplace(float *a, float factor, uint32_t count, void *strea
     return launch_map2(a, nullptr, a, count, ScaleF{factor}, hipStream_t(stream), "crb_tensor_scale_inplace");
 }
 
+int crb_batchnorm_fwd(const float *X, const float *beta, const float *gamma, float *mean, float *var, float *Y, float *xHat,
+                      uint32_t N, uint32_t F, void *stream) {
+    if (!X || !beta || !gamma || !mean || !var || !Y || !xHat) return fail(CRB_ENULL, "crb_batchnorm_fwd: null operand");
+    if (int st = check_bn("crb_batchnorm_fwd", N, F)) return st;
+    hipStream_t s = hipStream_t(stream);
+    switch (bn_features_per_wg(F)) {
+        case 64: hipLaunchKernelGGL(batchnorm_fwd_kernel<64>, dim3(ceil_div(F, 64)), dim3(256), 0, s, X, beta, gamma, mean, var, Y, xHat, N, F); break;
+        case 32: hipLaunchKernelGGL(batchnorm_fwd_kernel<32>, dim3(ceil_div(F, 32)), dim3(256), 0, s, X, beta, gamma, mean, var, Y, xHat, N, F); break;
+        default: hipLaunchKernelGGL(batchnorm_fwd_kernel<16>, dim3(ceil_div(F, 16)), dim3(256), 0, s, X, beta, gamma, mean, var, Y, xHat, N, F);
+    }
+    return check_launch("crb_batchnorm_fwd");
+}
+
+int crb_batchnorm_bwd(const float *dY, const float *gamma, const float *X, float *dX, uint32_t N, uint32_t F, void *stream) {
+    if (!dY || !gamma || !X || !dX) return fail(CRB_ENULL, "crb_batchnorm_bwd: null operand");
+    if (int st = check_bn("crb_batchnorm_bwd", N, F)) return st;
+    hipStream_t s = hipStream_t(stream);
+    switch (bn_features_per_wg(F)) {
+        case 64: hipLaunchKernelGGL(batchnorm_bwd_kernel<64>, dim3(ceil_div(F, 64)), dim3(256), 0, s, dY, gamma, X, dX, N, F); break;
+        case 32: hipLaunchKernelGGL(batchnorm_bwd_kernel<32>, dim3(ceil_div(F, 32)), dim3(256), 0, s, dY, gamma, X, dX, N, F); break;
+        default: hipLaunchKernelGGL(batchnorm_bwd_kernel<16>, dim3(ceil_div(F, 16)), dim3(256), 0, s, dY, gamma, X, dX, N, F);
+    }
+    return check_launch("crb_batchnorm_bwd");
+}
+
+int crb_batchnorm_param_grads(const float *dY, const float *xHat, float *dGamma, float *dBeta, uint32_t N, uint32_t F,
+                              void *stream) {
+    if (!dY || !xHat || !dGamma || !dBeta) return fail(CRB_ENULL, "crb_batchnorm_param_grads: null operand");
+    if (int st = check_bn("crb_batchnorm_param_grads", N, F)) return st;
+    hipStream_t s = hipStream_t(stream);
+    switch (bn_features_per_wg(F)) {
+        case 64: hipLaunchKernelGGL(batchnorm_param_grads_kernel<64>, dim3(ceil_div(F, 64)), dim3(256), 0, s, dY, xHat, dGamma, dBeta, N, F); break;
+        case 32: hipLaunchKernelGGL(batchnorm_param_grads_kernel<32>, dim3(ceil_div(F, 32)), dim3(256), 0, s, dY, xHat, dGamma, dBeta, N, F); break;
+        default: hipLaunchKernelGGL(batchnorm_param_grads_kernel<16>, dim3(ceil_div(F, 16)), dim3(256), 0, s, dY, xHat, dGamma, dBeta, N, F);
+    }
+    return check_launch("crb_batchnorm_param_grads");
+}
+
 int crb_momentum_apply(float *X, float *G, float *M, uint32_t count, float lr, float beta, float decay, void *stream) {
     if (!X || !G || !M) return fail(CRB_ENULL, "crb_momentum_apply: null operand");
     if (!count) return fail(CRB_EINVAL_SHAPE, "crb_momentum_apply: zero size");
@@ -409,6 +650,16 @@ int crb_momentum_apply(float *X, float *G, float *M, uint32_t count, float lr, f
     hipLaunchKernelGGL(momentum_kernel, dim3(stream_grid(count)), dim3(256), 0, hipStream_t(stream), X, G, M, count, vec, lr, beta,
                        1.0f - beta, decay);
     return check_launch("crb_momentum_apply");
+}
+
+int crb_momentum_apply_multi(const crb_momentum_item *items_on_device, uint32_t n_items, uint32_t max_count, void *stream) {
+    if (!items_on_device) return fail(CRB_ENULL, "crb_momentum_apply_multi: null table");
+    if (!n_items || !max_count) return fail(CRB_EINVAL_SHAPE, "crb_momentum_apply_multi: empty table");
+    if (n_items > 65535u) return fail(CRB_EINVAL_SHAPE, "crb_momentum_apply_multi: more than 65535 items");
+    u32 bx = ceil_div(ceil_div(max_count, 4), 256);
+    bx = bx > 64 ? 64 : bx;
+    hipLaunchKernelGGL(momentum_multi_kernel, dim3(bx, n_items), dim3(256), 0, hipStream_t(stream), items_on_device);
+    return check_launch("crb_momentum_apply_multi");
 }
 
 }  // extern "C"

@@ -1,4 +1,4 @@
-// Elementwise helpers the conv/linear operands call around the hot path: in-place add and constant fill.
+// Elementwise helpers the operands call around the hot path: in-place add, add-and-clear, copy and constant fill.
 // Pure streaming kernels (HBM-bound): 16-byte accesses when the buffer is 16-byte aligned, grid-stride loop.
 #include "igemm_engine.h"
 
@@ -33,6 +33,36 @@ __global__ void __launch_bounds__(256) fill_kernel(float *__restrict__ a, float 
     }
 }
 
+// a[i] += b[i]; b[i] = 0 — folds a side gradient into the main one and clears it, in one pass.
+__global__ void __launch_bounds__(256) add_clear_kernel(float *__restrict__ a, float *__restrict__ b, u32 count, u32 vec) {
+    const u32 stride = gridDim.x * 256;
+    u32 i = blockIdx.x * 256 + threadIdx.x;
+    if (vec) {
+        const u32 nq = count / 4;
+        v4f *a4 = reinterpret_cast<v4f *>(a), *b4 = reinterpret_cast<v4f *>(b);
+        const v4f z = {0.f, 0.f, 0.f, 0.f};
+        for (u32 q = i; q < nq; q += stride) {
+            a4[q] = a4[q] + b4[q];
+            b4[q] = z;
+        }
+        for (u32 r = nq * 4 + i; r < count; r += stride) a[r] += b[r], b[r] = 0.f;
+    } else {
+        for (; i < count; i += stride) a[i] += b[i], b[i] = 0.f;
+    }
+}
+
+__global__ void __launch_bounds__(256) copy_kernel(float *__restrict__ dst, const float *__restrict__ src, u32 count, u32 vec) {
+    const u32 stride = gridDim.x * 256;
+    u32 i = blockIdx.x * 256 + threadIdx.x;
+    if (vec) {
+        const u32 nq = count / 4;
+        for (u32 q = i; q < nq; q += stride) reinterpret_cast<v4f *>(dst)[q] = reinterpret_cast<const v4f *>(src)[q];
+        for (u32 r = nq * 4 + i; r < count; r += stride) dst[r] = src[r];
+    } else {
+        for (; i < count; i += stride) dst[i] = src[i];
+    }
+}
+
 static u32 stream_grid(u32 count) {
     u32 blocks = ceil_div(ceil_div(count, 4), 256);
     return blocks < 1 ? 1 : (blocks > 4096 ? 4096 : blocks);
@@ -50,6 +80,24 @@ int crb_tensor_add_inplace(float *a, const float *b, uint32_t count, void *strea
     const u32 vec = ((reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b)) & 15u) == 0;
     hipLaunchKernelGGL(add_inplace_kernel, dim3(stream_grid(count)), dim3(256), 0, hipStream_t(stream), a, b, count, vec);
     return check_launch("crb_tensor_add_inplace");
+}
+
+int crb_tensor_add_clear(float *a, float *b, uint32_t count, void *stream) {
+    if (!a || !b) return fail(CRB_ENULL, "crb_tensor_add_clear: null operand");
+    if (!count) return fail(CRB_EINVAL_SHAPE, "crb_tensor_add_clear: zero size");
+    if (a == b) return fail(CRB_EINVAL_SHAPE, "crb_tensor_add_clear: operands alias");
+    const u32 vec = ((reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b)) & 15u) == 0;
+    hipLaunchKernelGGL(add_clear_kernel, dim3(stream_grid(count)), dim3(256), 0, hipStream_t(stream), a, b, count, vec);
+    return check_launch("crb_tensor_add_clear");
+}
+
+int crb_tensor_copy(float *dst, const float *src, uint32_t count, void *stream) {
+    if (!dst || !src) return fail(CRB_ENULL, "crb_tensor_copy: null operand");
+    if (!count) return fail(CRB_EINVAL_SHAPE, "crb_tensor_copy: zero size");
+    if (dst == src) return CRB_OK;
+    const u32 vec = ((reinterpret_cast<uintptr_t>(dst) | reinterpret_cast<uintptr_t>(src)) & 15u) == 0;
+    hipLaunchKernelGGL(copy_kernel, dim3(stream_grid(count)), dim3(256), 0, hipStream_t(stream), dst, src, count, vec);
+    return check_launch("crb_tensor_copy");
 }
 
 int crb_tensor_fill(float *a, float value, uint32_t count, void *stream) {

@@ -18,18 +18,27 @@
 
 using namespace seann;
 
+static bool g_fused = false;  // use Sequential::learnFused
+
+static void learn(Sequential &net) {
+    if (g_fused)
+        net.learnFused();
+    else
+        net.learn();
+}
+
 static double time_steps(Sequential &net, Tensor *X, Tensor *L, int steps) {
     for (int i = 0; i < 2; ++i) {  // warm-up
         net.forward(X);
         net.backward(L);
-        net.learn();
+        learn(net);
     }
     (void)hipDeviceSynchronize();
     const auto t0 = std::chrono::steady_clock::now();
     for (int i = 0; i < steps; ++i) {
         net.forward(X);
         net.backward(L);
-        net.learn();
+        learn(net);
     }
     (void)hipDeviceSynchronize();
     return std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - t0).count() / steps;
@@ -84,12 +93,19 @@ int main(int argc, char **argv) {
     const double ms_blocking = time_steps(net, X, L, steps);
     setBlocking(false);
     const double ms_async = time_steps(net, X, L, steps);
+    // the same network with the two optional shortcuts: reserve folds pruned, one launch for all momentum updates
+    net.pruneReserveFolds();
+    g_fused = true;
+    const double ms_fast = time_steps(net, X, L, steps);
+    g_fused = false;
     setBlocking(true);
     net.forward(X);
     const float loss = net.lossFW(net.netY, L, lossBuf);
     std::printf("{\"workload\": \"VGG-16 CIFAR training step through seann::Sequential (C++ host layer)\", \"batch\": %u, "
                 "\"steps\": %d, \"ms_per_step_blocking\": %.3f, \"ms_per_step_nonblocking\": %.3f, \"conv_fc_gflop\": %.2f, "
-                "\"tflops_nonblocking\": %.2f, \"images_per_s_nonblocking\": %.1f, \"loss_after\": %.4f}\n",
-                batch, steps, ms_blocking, ms_async, flops / 1e9, flops / ms_async / 1e9, batch / ms_async * 1e3, double(loss));
+                "\"tflops_nonblocking\": %.2f, \"images_per_s_nonblocking\": %.1f, \"ms_per_step_pruned_fused\": %.3f, "
+                "\"tflops_pruned_fused\": %.2f, \"images_per_s_pruned_fused\": %.1f, \"loss_after\": %.4f}\n",
+                batch, steps, ms_blocking, ms_async, flops / 1e9, flops / ms_async / 1e9, batch / ms_async * 1e3, ms_fast,
+                flops / ms_fast / 1e9, batch / ms_fast * 1e3, double(loss));
     return 0;
 }

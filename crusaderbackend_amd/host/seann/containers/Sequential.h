@@ -40,5 +40,17 @@ public:
     void learn() const;
     void learnBatch() const;
     void zeroGrads() const;
+
+    // Two optional shortcuts with no counterpart in the reference; results are unchanged.
+    // pruneReserveFolds: after construct(), stop folding Y->dAReserve into Y->dA in the xGrads of operands into whose
+    // reserve no operand of this network deposits anything (only shortcut endpoints do). An operand type of your own that
+    // writes another operand's reserve must increment that operand's `reserveWriters` in its postWaiveInit.
+    void pruneReserveFolds() const;
+    // learnFused: the momentum step of every parameter in one kernel launch instead of one launch per parameter.
+    void learnFused();
+
+private:
+    void *fusedTable = nullptr;    // device copy of the parameter table used by learnFused
+    std::vector<char> fusedHost;   // its host image, to detect changed rates
 };
 }  // namespace seann

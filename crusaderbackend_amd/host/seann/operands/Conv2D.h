@@ -37,6 +37,10 @@ public:
         filter->batchUpdate();
         if (WITH_BIAS) bias->batchUpdate();
     }
+    void collectNetParams(std::vector<NetParam *> &out) override {
+        out.push_back(filter);
+        if (WITH_BIAS) out.push_back(bias);
+    }
     uint32 OPERAND_ID() override { return OPR_SEBLAS_CONV2D; }
 };
 }  // namespace seann

@@ -1,5 +1,5 @@
-// The parameter-free operands of a CIFAR-style network: ReLU, MaxPool2D, Softmax — each a thin call into the seblas
-// operator of the same name, with the reference's members and gradient bookkeeping (the reserve gradient a shortcut
+// The operands of a CIFAR-style network besides convolution and dense layers: ReLU, MaxPool2D, BatchNorm, Softmax — each
+// a thin call into the seblas operator of the same name, with the reference's members and gradient bookkeeping (the reserve gradient a shortcut
 // may have deposited in Y->dAReserve is folded into Y->dA first and cleared afterwards).
 // seann/operands/seblas/activate/ReLU.{cuh,cu}, pooling/MaxPool2D.{cuh,cu}, Softmax.{cuh,cu}.
 #pragma once
@@ -7,7 +7,8 @@
 
 #define OPR_SEBLAS_RELU 0xa002
 #define OPR_SEBLAS_MAXPOOL2D 0xb003
-#define OPR_SEBLAS_SOFTMAX 0x0003
+#define OPR_SEBLAS_SOFTMAX 0x0005
+#define OPR_SEBLAS_BATCHNORM 0x0003
 
 namespace seann {
 
@@ -17,9 +18,6 @@ public:
     void randFillNetParams() override {}
     void zeroGrads() override {}
 
-protected:
-    void foldReserve() const { *Y->dA + Y->dAReserve; }
-    void clearReserve() const { Y->dAReserve->constFill(0); }
 };
 
 class ReLU : public ParamFreeOperand {
@@ -37,7 +35,6 @@ public:
     void xGrads() override {                         // ReLU.cu:13-17
         foldReserve();
         reluGradFast(X->A, Y->dA, X->dA);
-        clearReserve();
     }
     uint32 OPERAND_ID() override { return OPR_SEBLAS_RELU; }
 };
@@ -59,9 +56,58 @@ public:
     void xGrads() override {                                                                     // MaxPool2D.cu:16-20
         foldReserve();
         maxPoolBack(X->dA, Y->dA, record, strideH, strideW, rangeH, rangeW);
-        clearReserve();
     }
     uint32 OPERAND_ID() override { return OPR_SEBLAS_MAXPOOL2D; }
+};
+
+// Batch normalisation with per-feature statistics and trainable beta / gamma of one sample's shape
+// (seann/operands/seblas/BatchNorm.{cuh,cu}). paramGrads gives gamma the gradient of gamma and beta the gradient of beta
+// (the reference passes the two tensors to batchNormParamGrads in swapped order, BatchNorm.cu:24).
+class BatchNorm : public OperandBase {
+public:
+    NetParam *beta{};
+    NetParam *gamma{};
+    Tensor *mean{};
+    Tensor *variance{};
+    Tensor *xHatP{};
+    std::string info() override { return "BatchNorm"; }
+    void initNetParams(OptimizerInfo *info, shape4 inShape) override {  // BatchNorm.cuh:27-37
+        shape4 paramShape = {1, inShape.c, inShape.h, inShape.w};
+        beta = new NetParam(info, paramShape);
+        gamma = new NetParam(info, paramShape);
+        mean = Tensor::create(paramShape);
+        variance = Tensor::create(paramShape);
+        xHatP = Tensor::create(inShape);
+        X = Parameter::declare(inShape);
+        Y = Parameter::create(inShape);
+    }
+    void randFillNetParams() override {  // BatchNorm.cu:8-11
+        beta->data()->constFill(0.0f);
+        gamma->data()->constFill(1.0f);
+    }
+    void forward() override { batchNorm(X->A, beta->data(), gamma->data(), mean, variance, Y->A, xHatP); }
+    void xGrads() override {  // BatchNorm.cu:17-21
+        foldReserve();
+        batchNormGrad(Y->dA, gamma->data(), X->A, X->dA);
+    }
+    void paramGrads() override { batchNormParamGrads(Y->dA, xHatP, gamma->grad(), beta->grad()); }
+    void updateParams() override {
+        beta->update();
+        gamma->update();
+    }
+    void batchUpdateParams() override {
+        beta->batchUpdate();
+        gamma->batchUpdate();
+    }
+    void zeroGrads() override {
+        beta->zeroGrad();
+        gamma->zeroGrad();
+    }
+    void collectNetParams(std::vector<NetParam *> &out) override {
+        out.push_back(beta);
+        out.push_back(gamma);
+    }
+    uint32 OPERAND_ID() override { return OPR_SEBLAS_BATCHNORM; }
 };
 
 // Output probabilities; the loss function writes Y->dA = Y->A - labels, which is already the gradient with respect to
@@ -77,7 +123,6 @@ public:
     void xGrads() override {
         foldReserve();
         Y->dA->copyToD2D(X->dA);
-        clearReserve();
     }
     uint32 OPERAND_ID() override { return OPR_SEBLAS_SOFTMAX; }
 };

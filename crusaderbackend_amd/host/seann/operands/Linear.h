@@ -34,6 +34,10 @@ public:
         weights->batchUpdate();
         biases->batchUpdate();
     }
+    void collectNetParams(std::vector<NetParam *> &out) override {
+        out.push_back(weights);
+        out.push_back(biases);
+    }
     uint32 OPERAND_ID() override { return OPR_SEBLAS_LINEAR; }
 };
 }  // namespace seann

@@ -3,6 +3,7 @@
 // encoding is outside this build.
 #pragma once
 #include <string>
+#include <vector>
 
 #include "../../seblas/operations/operations.h"
 #include "../containers/NetParam.h"
@@ -16,6 +17,10 @@ public:
     OperandBase *prev = nullptr;
     OperandBase *next = nullptr;
     uint32 operandID = 0;
+    // Operands that deposit a gradient in this operand's Y->dAReserve (shortcut endpoints) count themselves here;
+    // pruneReserveFolds() switches the fold off where nobody does. Until it is called every operand folds, as in the reference.
+    uint32 reserveWriters = 0;
+    bool foldReserveEnabled = true;
 
     virtual ~OperandBase() = default;
 
@@ -31,6 +36,15 @@ public:
     virtual void zeroGrads() = 0;
     virtual std::string info() = 0;
     virtual uint32 OPERAND_ID() { return 0x0000; }
+
+    virtual void collectNetParams(std::vector<NetParam *> &) {}  // every trainable parameter, for a fused update
+    virtual void pruneReserveFolds() { foldReserveEnabled = reserveWriters > 0; }
+
+    // Y->dA += Y->dAReserve and the reserve is cleared, in one pass (the reference clears it after the gradient call, which
+    // never reads it): the first thing every xGrads does
+    void foldReserve() const {
+        if (foldReserveEnabled) Y->dA->addAndClear(Y->dAReserve);
+    }
 
     void bindPrev(OperandBase *p) { prev = p; }
     void bindNext(OperandBase *n) { next = n; }

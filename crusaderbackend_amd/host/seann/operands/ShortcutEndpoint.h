@@ -38,6 +38,13 @@ public:
     void batchUpdateParams() override;
     void randFillNetParams() override;
     void zeroGrads() override;
+    void collectNetParams(std::vector<NetParam *> &out) override {
+        for (OperandBase *op : branchOperands) op->collectNetParams(out);
+    }
+    void pruneReserveFolds() override {
+        OperandBase::pruneReserveFolds();
+        for (OperandBase *op : branchOperands) op->pruneReserveFolds();
+    }
     std::string info() override { return "ShortcutEndpoint { " + std::to_string(operandCount) + " }"; }
     uint32 OPERAND_ID() override { return isContainer ? OPR_CTRL_SHORTCUTENDPOINT_END : OPR_CTRL_SHORTCUTENDPOINT_BEG; }
 };

@@ -2,6 +2,7 @@
 #include <hip/hip_runtime_api.h>
 
 #include <cmath>
+#include <cstring>
 #include <stdexcept>
 
 #include "../../../../include/crusader_hip.h"
@@ -29,9 +30,8 @@ void Conv2D::forward() {  // Conv2D.cu:8-16
 }
 
 void Conv2D::xGrads() {  // Conv2D.cu:18-22
-    *Y->dA + Y->dAReserve;
+    foldReserve();
     convDerive(filter->data(), Y->dA, X->dA, int(strideH), int(strideW), int(padH), int(padW));
-    Y->dAReserve->constFill(0);
 }
 
 void Conv2D::paramGrads() {  // Conv2D.cu:24-29; the bias gradient is the per-channel sum of dY
@@ -69,9 +69,8 @@ void Linear::forward() { linear(X->A, weights->data(), biases->data(), Y->A); } 
 void Linear::paramGrads() { linearParamGrad(Y->dA, X->A, weights->grad(), biases->grad()); }  // :21-23
 
 void Linear::xGrads() {  // Linear.cu:35-40
-    *Y->dA + Y->dAReserve;
+    foldReserve();
     linearXGrad(Y->dA, weights->data(), X->dA);
-    Y->dAReserve->constFill(0);
 }
 
 void Linear::randFillNetParams() {  // Linear.cu:42-46
@@ -98,6 +97,7 @@ void ShortcutEndpoint::postWaiveInit(OptimizerInfo *inf) {  // :13-55
             tracer = tracer->tracePrev();
         if (!tracer) throw std::invalid_argument("ShortcutEndpoint: no opening endpoint with this uuid");
         other = static_cast<ShortcutEndpoint *>(tracer);
+        other->reserveWriters++;  // identity: this endpoint's xGrads copies into it; projection: the branch's input gradient is it
         if (operandCount > 0) {
             branchOperands[0]->initNetParams(inf, other->Y->A->dims);
             for (uint32 i = 1; i < operandCount; i++) branchOperands[i]->initNetParams(inf, branchOperands[i - 1]->Y->A->dims);
@@ -142,8 +142,7 @@ void ShortcutEndpoint::xGrads() {  // :76-99
             Y->dA->copyToD2D(other->Y->dAReserve);
         }
     } else {
-        *Y->dA + Y->dAReserve;
-        Y->dAReserve->constFill(0);
+        foldReserve();
     }
     Y->dA->copyToD2D(X->dA);
 }
@@ -229,6 +228,44 @@ void Sequential::learnBatch() const {
 
 void Sequential::zeroGrads() const {
     for (OperandBase *op : operands) op->zeroGrads();
+}
+
+void Sequential::pruneReserveFolds() const {
+    for (OperandBase *op : operands) op->pruneReserveFolds();
+}
+
+// All parameters in one kernel launch. The device table of (weights, gradient, momentum, rates) is built on the first
+// call and rebuilt when a rate changed; any optimizer other than Momentum makes this fall back to learn().
+void Sequential::learnFused() {
+    std::vector<NetParam *> params;
+    for (OperandBase *op : operands) op->collectNetParams(params);
+    std::vector<crb_momentum_item> items;
+    uint32 maxCount = 0;
+    for (NetParam *p : params) {
+        auto *m = dynamic_cast<Momentum *>(p->opt);
+        if (!m) {
+            learn();
+            return;
+        }
+        const uint32 count = p->data()->dims.size;
+        items.push_back({p->data()->elements, p->grad()->elements, m->m->elements, count, m->LEARNING_RATE, m->BETA,
+                         m->isWeight ? 1.0f - m->L2 : 1.0f});
+        maxCount = count > maxCount ? count : maxCount;
+    }
+    if (items.empty()) return;
+    const size_t bytes = items.size() * sizeof(crb_momentum_item);
+    if (fusedHost.size() != bytes || std::memcmp(fusedHost.data(), items.data(), bytes) != 0) {
+        if (fusedTable && fusedHost.size() != bytes) {
+            (void)hipFree(fusedTable);
+            fusedTable = nullptr;
+        }
+        if (!fusedTable && hipMalloc(&fusedTable, bytes) != hipSuccess) assertHip(__FILE__, __LINE__);
+        if (hipMemcpy(fusedTable, items.data(), bytes, hipMemcpyHostToDevice) != hipSuccess) assertHip(__FILE__, __LINE__);
+        fusedHost.assign(reinterpret_cast<const char *>(items.data()), reinterpret_cast<const char *>(items.data()) + bytes);
+    }
+    throwOnStatus(crb_momentum_apply_multi(static_cast<const crb_momentum_item *>(fusedTable), uint32(items.size()), maxCount, nullptr),
+                  __FILE__, __LINE__);
+    if (isBlocking() && hipStreamSynchronize(nullptr) != hipSuccess) assertHip(__FILE__, __LINE__);
 }
 
 }  // namespace seann

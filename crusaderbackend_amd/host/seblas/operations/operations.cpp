@@ -15,14 +15,10 @@ static void require(bool ok, const char *what) {
     if (!ok) throw std::invalid_argument(what);
 }
 
-static bool g_blocking = true;
-void setBlocking(bool blocking) { g_blocking = blocking; }
-bool isBlocking() { return g_blocking; }
-
 // every reference op ends with cudaDeviceSynchronize(); assertCuda(...)
 static void finish(int status, const char *file, int line) {
     throwOnStatus(status, file, line);
-    if (g_blocking && hipStreamSynchronize(nullptr) != hipSuccess) assertHip(file, line);
+    if (isBlocking() && hipStreamSynchronize(nullptr) != hipSuccess) assertHip(file, line);
     assertHip(file, line);
 }
 
@@ -199,6 +195,35 @@ float crossEntropyCalc(Parameter *Y, Tensor *labels, Tensor *buf) {
     float loss = 0.f;
     if (hipMemcpy(&loss, out, sizeof(float), hipMemcpyDeviceToHost) != hipSuccess) assertHip(__FILE__, __LINE__);
     return loss;
+}
+
+Tensor *batchNorm(Tensor *X, Tensor *beta, Tensor *gamma, Tensor *mean, Tensor *var, Tensor *Y, Tensor *xHat) {
+    require(X->dims.n == Y->dims.n && X->dims.size == Y->dims.size, "batchNorm: X and Y differ");  // cuBatchNorm.cu:162-163
+    const uint32 F = X->dims.size / X->dims.n;
+    require(xHat->dims.size == X->dims.size, "batchNorm: xHat size");
+    require(beta->dims.size == F && gamma->dims.size == F && mean->dims.size == F && var->dims.size == F,
+            "batchNorm: beta / gamma / mean / var must hold one value per feature");
+    finish(crb_batchnorm_fwd(X->elements, beta->elements, gamma->elements, mean->elements, var->elements, Y->elements,
+                             xHat->elements, X->dims.n, F, nullptr),
+           __FILE__, __LINE__);
+    return Y;
+}
+
+Tensor *batchNormGrad(Tensor *dY, Tensor *gamma, Tensor *X, Tensor *dX) {
+    require(dY->dims.n == X->dims.n && dY->dims.size == X->dims.size, "batchNormGrad: dY and X differ");  // :177-178
+    require(dX->dims.size == X->dims.size, "batchNormGrad: dX size");
+    const uint32 F = X->dims.size / X->dims.n;
+    require(gamma->dims.size == F, "batchNormGrad: gamma must hold one value per feature");
+    finish(crb_batchnorm_bwd(dY->elements, gamma->elements, X->elements, dX->elements, X->dims.n, F, nullptr), __FILE__, __LINE__);
+    return dX;
+}
+
+void batchNormParamGrads(Tensor *dY, Tensor *xHat, Tensor *dGamma, Tensor *dBeta) {
+    require(dY->dims.n == xHat->dims.n && dY->dims.size == xHat->dims.size, "batchNormParamGrads: dY and xHat differ");  // :191-192
+    const uint32 F = dY->dims.size / dY->dims.n;
+    require(dGamma->dims.size == F && dBeta->dims.size == F, "batchNormParamGrads: one value per feature");
+    finish(crb_batchnorm_param_grads(dY->elements, xHat->elements, dGamma->elements, dBeta->elements, dY->dims.n, F, nullptr),
+           __FILE__, __LINE__);
 }
 
 void momentumApply(Tensor *X, Tensor *Xgrad, Tensor *V, float LEARNING_RATE, float MOMENTUM) {

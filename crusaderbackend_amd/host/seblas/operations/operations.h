@@ -12,12 +12,6 @@
 #include "../tensor/Tensor.h"
 
 namespace seblas {
-// The reference blocks the host after every operator (cudaDeviceSynchronize), and so does this layer by default.
-// A caller that issues a whole step on the default stream and synchronises once can switch that off; device errors
-// then surface at its own synchronisation point. No counterpart in the reference.
-void setBlocking(bool blocking);
-bool isBlocking();
-
 // cuGEMM.cu:1649-1714
 Tensor *sgemm(Tensor *A, Tensor *B, Tensor *C);     // C[n] = A * B[n]
 Tensor *sgemmTN(Tensor *A, Tensor *B, Tensor *C);   // C[n] = A^T * B[n]
@@ -50,6 +44,12 @@ Tensor *softmax(Tensor *A, Tensor *out, Tensor *buffer, uint32 step);
 // is device scratch (the reference passes a tensor of Y's size; its last element receives the sum before the copy back).
 void crossEntropyLoss(Parameter *Y, Tensor *labels);
 float crossEntropyCalc(Parameter *Y, Tensor *labels, Tensor *buf);
+// cuBatchNorm.cuh: per-feature batch normalisation (a feature = one (c,h,w) position; statistics over n). beta, gamma,
+// mean, var have the shape of one sample. batchNormParamGrads overwrites dGamma / dBeta. Any batch size (the reference
+// asserts n <= 96).
+Tensor *batchNorm(Tensor *X, Tensor *beta, Tensor *gamma, Tensor *mean, Tensor *var, Tensor *Y, Tensor *xHat);
+Tensor *batchNormGrad(Tensor *dY, Tensor *gamma, Tensor *X, Tensor *dX);
+void batchNormParamGrads(Tensor *dY, Tensor *xHat, Tensor *dGamma, Tensor *dBeta);
 // cuOptim.cuh:16. V is the momentum buffer; Xgrad is cleared by the step.
 void momentumApply(Tensor *X, Tensor *Xgrad, Tensor *V, float LEARNING_RATE, float MOMENTUM);
 // Optimizers.cu:16-22 in one pass: X *= (1 - L2) then momentumApply. No separate counterpart in the reference.

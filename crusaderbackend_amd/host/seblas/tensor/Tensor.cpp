@@ -117,7 +117,12 @@ static Tensor *copy(const Tensor *src, Tensor *dst, hipMemcpyKind kind) {
 }
 Tensor *Tensor::copyToH2D(Tensor *onDevice) const { return copy(this, onDevice, hipMemcpyHostToDevice); }
 Tensor *Tensor::copyToD2H(Tensor *onHost) const { return copy(this, onHost, hipMemcpyDeviceToHost); }
-Tensor *Tensor::copyToD2D(Tensor *onDevice) const { return copy(this, onDevice, hipMemcpyDeviceToDevice); }
+Tensor *Tensor::copyToD2D(Tensor *onDevice) const {  // a kernel on the default stream, so the host need not stall
+    require(dims.size == onDevice->dims.size, "Tensor::copyToD2D: element counts differ");
+    throwOnStatus(crb_tensor_copy(onDevice->elements, elements, dims.size, nullptr), __FILE__, __LINE__);
+    if (isBlocking() && hipStreamSynchronize(nullptr) != hipSuccess) assertHip(__FILE__, __LINE__);
+    return onDevice;
+}
 Tensor *Tensor::copyToH2H(Tensor *onHost) const { return copy(this, onHost, hipMemcpyHostToHost); }
 
 Tensor *Tensor::attach(Tensor *other) {
@@ -141,6 +146,22 @@ Tensor *Tensor::operator+(Tensor *other) {
         return this;
     }
     throwOnStatus(crb_tensor_add_inplace(elements, other->elements, dims.size, nullptr), __FILE__, __LINE__);
+    assertHip(__FILE__, __LINE__);
+    return this;
+}
+
+static bool g_blocking = true;
+void setBlocking(bool blocking) { g_blocking = blocking; }
+bool isBlocking() { return g_blocking; }
+
+Tensor *Tensor::addAndClear(Tensor *other) {
+    require(dims.size == other->dims.size, "Tensor::addAndClear: element counts differ");
+    require(deviceId == other->deviceId, "Tensor::addAndClear: tensors live on different devices");
+    if (deviceId == -1) {
+        for (uint32 i = 0; i < dims.size; ++i) elements[i] += other->elements[i], other->elements[i] = 0.f;
+        return this;
+    }
+    throwOnStatus(crb_tensor_add_clear(elements, other->elements, dims.size, nullptr), __FILE__, __LINE__);
     assertHip(__FILE__, __LINE__);
     return this;
 }

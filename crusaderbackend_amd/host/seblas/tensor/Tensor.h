@@ -80,6 +80,9 @@ public:
     // 462-483,638-657): in-place `*this += *other`, and fill. Device tensors run on the GPU.
     Tensor *operator+(Tensor *other);
     Tensor *constFill(float val);
+    // `*this += *other; *other = 0` in one pass: what every operand's xGrads does with its reserve gradient
+    // (`*Y->dA + Y->dAReserve` ... `Y->dAReserve->constFill(0)`, e.g. seann/operands/seblas/Conv2D.cu:19,21).
+    Tensor *addAndClear(Tensor *other);
     // `*this -= *other` (Tensor.cu:485-506: the loss gradient) and `*this *= factor` (Tensor.cu:596-617: weight decay)
     Tensor *operator-(Tensor *other);
     Tensor *operator*(float factor);
@@ -90,4 +93,9 @@ public:
 
     float get(uint32 offset) const;
 };
+// The reference blocks the host after every operator and every device copy (cudaDeviceSynchronize / cudaMemcpy), and so
+// does this layer by default. A caller that issues a whole step on the default stream and synchronises once can switch
+// that off; device errors then surface at its own synchronisation point. No counterpart in the reference.
+void setBlocking(bool blocking);
+bool isBlocking();
 }  // namespace seblas

@@ -149,6 +149,15 @@ int crb_tensor_add_inplace(float *a, const float *b, uint32_t count, void *strea
 /* Replaces the device branch of seblas::Tensor::constFill (Tensor.cu:294-304, 638-657): a[i] = value. */
 int crb_tensor_fill(float *a, float value, uint32_t count, void *stream);
 
+/* Device-to-device copy on `stream`: dst[i] = src[i]. Stands in for the cudaMemcpy(..., cudaMemcpyDeviceToDevice) of
+ * seblas::Tensor::copyToD2D (seblas/tensor/Tensor.cu:435-440) and of the shortcut operand
+ * (seann/operands/controlling/ShortcutEndpoint.cu:59-60,80-81,96-97) without stalling the host. */
+int crb_tensor_copy(float *dst, const float *src, uint32_t count, void *stream);
+
+/* a[i] += b[i]; b[i] = 0. The pair every operand's xGrads performs around its gradient call — `*Y->dA + Y->dAReserve`
+ * ... `Y->dAReserve->constFill(0)` (e.g. seann/operands/seblas/Conv2D.cu:19,21) — in one pass. The two must not alias. */
+int crb_tensor_add_clear(float *a, float *b, uint32_t count, void *stream);
+
 /* Replaces the device branch of seblas::Tensor::operator-(Tensor*) (Tensor.cu:485-506): a[i] -= b[i], in place. */
 int crb_tensor_sub_inplace(float *a, const float *b, uint32_t count, void *stream);
 
@@ -196,6 +205,33 @@ int crb_cross_entropy_loss(const float *Y, const float *labels, float *scratch, 
  * seblas::momentumApply (seblas/operations/cuOptim.cu:259-272; kernels :38-46, :48-73), in one pass:
  *   x = x*decay;  m = beta*m + (1-beta)*g;  x -= lr*m;  g = 0.   decay = 1 - L2 for weights, 1 otherwise. */
 int crb_momentum_apply(float *X, float *G, float *M, uint32_t count, float lr, float beta, float decay, void *stream);
+
+/* The same step for a whole table of parameter tensors in ONE launch (a network has hundreds of small ones and a launch
+ * per tensor is then launch-bound). `items_on_device` is a device array of n_items entries, built and kept by the caller;
+ * max_count = the largest `count` in it. No counterpart in the reference, which launches per parameter
+ * (seann/containers/Sequential.cu:93-97 -> updateParams -> Optimizer::apply). Arithmetic identical to crb_momentum_apply. */
+typedef struct crb_momentum_item {
+    float *X, *G, *M;
+    uint32_t count;
+    float lr, beta, decay;
+} crb_momentum_item;
+int crb_momentum_apply_multi(const crb_momentum_item *items_on_device, uint32_t n_items, uint32_t max_count, void *stream);
+
+/* Batch normalisation with per-feature statistics: X is N x F, F = c*h*w, and each of the F positions is normalised
+ * over the N samples (biased variance, eps 1e-8); beta, gamma, mean, var hold F floats.
+ * Replaces seblas::batchNorm (seblas/operations/cuBatchNorm.cu:158-173; kernel :13-60): Y = xHat*gamma + beta, and
+ * mean, var, xHat are stored. The reference's N <= 96 limit (:9,164) does not apply. */
+int crb_batchnorm_fwd(const float *X, const float *beta, const float *gamma, float *mean, float *var, float *Y, float *xHat,
+                      uint32_t N, uint32_t F, void *stream);
+
+/* Replaces seblas::batchNormGrad (cuBatchNorm.cu:176-188; kernel :62-125): dX from dY, gamma and X (statistics are
+ * recomputed from X, as in the reference). */
+int crb_batchnorm_bwd(const float *dY, const float *gamma, const float *X, float *dX, uint32_t N, uint32_t F, void *stream);
+
+/* Replaces seblas::batchNormParamGrads (cuBatchNorm.cu:190-202; kernel :127-148): dBeta = sum_n dY, dGamma = sum_n dY*xHat.
+ * Both are overwritten, not accumulated. */
+int crb_batchnorm_param_grads(const float *dY, const float *xHat, float *dGamma, float *dBeta, uint32_t N, uint32_t F,
+                              void *stream);
 
 #ifdef __cplusplus
 }

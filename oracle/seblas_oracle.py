@@ -252,3 +252,31 @@ def momentumApply(X, G, M, lr, beta, decay=1.0):
     load().oracle_momentumApply(_ptr(X), _ptr(G), _ptr(M), _u32(X.size), ctypes.c_float(lr), ctypes.c_float(beta),
                                 ctypes.c_float(decay))
     return X, G, M
+
+
+def batchNorm(X, beta, gamma):
+    """X (N, ...) -> (Y, xHat, mean, var); statistics per feature (every position after the batch axis) over N."""
+    X = _f32(X)
+    N, F = X.shape[0], X.size // X.shape[0]
+    Y, xHat = np.empty_like(X), np.empty_like(X)
+    mean, var = np.empty(F, np.float32), np.empty(F, np.float32)
+    load().oracle_batchNorm(_ptr(X), _ptr(_f32(beta).ravel()), _ptr(_f32(gamma).ravel()), _ptr(mean), _ptr(var), _ptr(Y),
+                            _ptr(xHat), _u32(N), _u32(F))
+    return Y, xHat, mean, var
+
+
+def batchNormGrad(dY, gamma, X):
+    dY, X = _f32(dY), _f32(X)
+    N, F = X.shape[0], X.size // X.shape[0]
+    dX = np.empty_like(X)
+    load().oracle_batchNormGrad(_ptr(dY), _ptr(_f32(gamma).ravel()), _ptr(X), _ptr(dX), _u32(N), _u32(F))
+    return dX
+
+
+def batchNormParamGrads(dY, xHat):
+    """Returns (dGamma, dBeta), each with F values."""
+    dY, xHat = _f32(dY), _f32(xHat)
+    N, F = dY.shape[0], dY.size // dY.shape[0]
+    dG, dB = np.empty(F, np.float32), np.empty(F, np.float32)
+    load().oracle_batchNormParamGrads(_ptr(dY), _ptr(xHat), _ptr(dG), _ptr(dB), _u32(N), _u32(F))
+    return dG, dB

@@ -1,7 +1,7 @@
 /*
  * seblas_oracle_ew.c — CPU fp32 restatement of the elementwise / reduction operators that surround the
  * GEMM and convolution path in a training step: ReLU, max pooling, softmax, cross-entropy, the in-place
- * tensor arithmetic and the momentum update.
+ * tensor arithmetic, the momentum update and per-feature batch normalisation.
  *
  * THIS IS TEST INFRASTRUCTURE, NOT PRODUCT CODE (same rule as seblas_oracle.c): only the test-suite, the
  * smoke check and the benchmark's cpu_baseline leg may load it.
@@ -18,6 +18,8 @@
  *                         the loss through the softmax (finite differences)
  *   tensor add/sub/scale/fill   numpy
  *   momentumApply         closed form after k steps with a constant gradient; numpy float64 recurrence
+ *   batchNorm*            torch-CPU batch_norm (training mode) and its autograd in float64; xHat has zero mean and unit
+ *                         variance per feature; finite differences
  * No function here is "parity unpinned".
  */
 #include <math.h>
@@ -151,5 +153,87 @@ void oracle_momentumApply(float *X, float *G, float *M, u32 n, float lr, float b
         X[i] = x - step;
         M[i] = m;
         G[i] = 0.0f;
+    }
+}
+
+/* ---- batch normalisation over the batch dimension, per feature -----------------------------------------------------
+ * A "feature" is one (c, h, w) position: X is viewed as N x F with F = C*H*W, and every column is normalised with its
+ * own statistics over the N samples (seblas/operations/cuBatchNorm.cu:13-60: one thread per feature index, loop over
+ * depth = sample). beta, gamma, mean, var hold F values. Pinned in tests/test_oracle_elementwise.py by torch-CPU
+ * batch_norm (training mode, eps 1e-8) on the N x F view in float64, its autograd for all three gradients, the
+ * zero-mean / unit-variance property of xHat, and finite differences. */
+
+/* batchNorm (cuBatchNorm.cu:13-60, host :158-173): mean = sum/N, var = sum (x-mean)^2 / N (biased),
+ * xHat = (x - mean) / sqrt(var + 1e-8), Y = xHat*gamma + beta; mean, var and xHat are stored. The reference asserts
+ * N <= 96 (its shared-memory staging, :9,164); that limit does not exist here. */
+void oracle_batchNorm(const float *X, const float *beta, const float *gamma, float *mean, float *var, float *Y,
+                      float *xHat, u32 N, u32 F) {
+    for (u32 f = 0; f < F; ++f) {
+        float m = 0.0f, v = 0.0f;
+        for (u32 n = 0; n < N; ++n) m += X[(size_t)n * F + f];
+        m /= (float)N;
+        for (u32 n = 0; n < N; ++n) {
+            const float d = X[(size_t)n * F + f] - m;
+            v += d * d;
+        }
+        v /= (float)N;
+        const float inv = 1.0f / sqrtf(v + 1e-8f);
+        for (u32 n = 0; n < N; ++n) {
+            const float xh = (X[(size_t)n * F + f] - m) * inv;
+            xHat[(size_t)n * F + f] = xh;
+            Y[(size_t)n * F + f] = xh * gamma[f] + beta[f];
+        }
+        mean[f] = m;
+        var[f] = v;
+    }
+}
+
+/* batchNormGrad (cuBatchNorm.cu:62-125, host :176-188): statistics are recomputed from X, then with dxHat = dY*gamma
+ *   dVar  = sum dxHat*(x-mean) * -0.5*(var+1e-8)^(-3/2)
+ *   dMean = sum dxHat * -1/sqrt(var+1e-8)  +  dVar * sum(-2(x-mean)) / N
+ *   dX    = dxHat/sqrt(var+1e-8) + dVar*2(x-mean)/N + dMean/N. */
+void oracle_batchNormGrad(const float *dY, const float *gamma, const float *X, float *dX, u32 N, u32 F) {
+    for (u32 f = 0; f < F; ++f) {
+        float m = 0.0f, v = 0.0f;
+        for (u32 n = 0; n < N; ++n) m += X[(size_t)n * F + f];
+        m /= (float)N;
+        for (u32 n = 0; n < N; ++n) {
+            const float d = X[(size_t)n * F + f] - m;
+            v += d * d;
+        }
+        v /= (float)N;
+        const float inv = 1.0f / sqrtf(v + 1e-8f);
+        const float g = gamma[f];
+        float dVar = 0.0f, dMean = 0.0f, temp = 0.0f;
+        for (u32 n = 0; n < N; ++n) {
+            const float d = X[(size_t)n * F + f] - m;
+            const float dxh = dY[(size_t)n * F + f] * g;
+            dVar += dxh * d * -0.5f * inv * inv * inv;
+            dMean += dxh * -inv;
+            temp += -2.0f * d;
+        }
+        dMean += dVar * temp / (float)N;
+        for (u32 n = 0; n < N; ++n) {
+            const float d = X[(size_t)n * F + f] - m;
+            const float dxh = dY[(size_t)n * F + f] * g;
+            dX[(size_t)n * F + f] = dxh * inv + dVar * d * 2.0f / (float)N + dMean / (float)N;
+        }
+    }
+}
+
+/* batchNormParamGrads (cuBatchNorm.cu:127-148, host :190-202): dBeta = sum dY, dGamma = sum dY*xHat; both OVERWRITE.
+ * (The BatchNorm operand of the reference passes the two output tensors in swapped order,
+ * seann/operands/seblas/BatchNorm.cu:24 against cuBatchNorm.cu:190, so its beta receives dGamma and its gamma dBeta;
+ * that slip is not reproduced: here dGamma is the gradient of gamma.) */
+void oracle_batchNormParamGrads(const float *dY, const float *xHat, float *dGamma, float *dBeta, u32 N, u32 F) {
+    for (u32 f = 0; f < F; ++f) {
+        float db = 0.0f, dg = 0.0f;
+        for (u32 n = 0; n < N; ++n) {
+            const float dy = dY[(size_t)n * F + f];
+            db += dy;
+            dg += dy * xHat[(size_t)n * F + f];
+        }
+        dBeta[f] = db;
+        dGamma[f] = dg;
     }
 }

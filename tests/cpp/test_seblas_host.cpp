@@ -38,6 +38,9 @@ void oracle_softmax(const float *, float *, uint32_t, uint32_t);
 void oracle_crossEntropyLoss(const float *, const float *, float *, uint32_t);
 float oracle_crossEntropyCalc(const float *, const float *, uint32_t);
 void oracle_momentumApply(float *, float *, float *, uint32_t, float, float, float);
+void oracle_batchNorm(const float *, const float *, const float *, float *, float *, float *, float *, uint32_t, uint32_t);
+void oracle_batchNormGrad(const float *, const float *, const float *, float *, uint32_t, uint32_t);
+void oracle_batchNormParamGrads(const float *, const float *, float *, float *, uint32_t, uint32_t);
 }
 
 using namespace seblas;
@@ -301,6 +304,36 @@ static void gpu_elementwise_tests() {
     CHECK(std::fabs(loss - rloss) <= 1e-5f * std::fabs(rloss) * std::sqrt(float(rows * classes)));
     CHECK(throws_invalid([&] { softmax(Z, S->A, nullptr, 7); }));  // cuReduce.cu:297
 
+    // seann::BatchNorm: forward, xGrads, paramGrads (gamma's gradient lands in gamma, beta's in beta)
+    {
+        const uint32_t bn = 24, bc = 3, bh = 5, F = bc * bh * bh;
+        seann::BatchNorm op;
+        op.initNetParams(nullptr, shape4(bn, bc, bh, bh));
+        seann::Parameter *src = seann::Parameter::create(bn, bc, bh, bh);
+        op.bindInput(src);
+        op.randFillNetParams();
+        auto bx = randn(bn * F, 41, 2.0f), bdy = randn(bn * F, 42), bg = randn(F, 43), bb = randn(F, 44);
+        for (auto &v : bg) v += 1.0f;
+        push(src->A->dims, bx)->copyToD2D(src->A);
+        push(op.gamma->data()->dims, bg)->copyToD2D(op.gamma->data());
+        push(op.beta->data()->dims, bb)->copyToD2D(op.beta->data());
+        push(op.Y->dA->dims, bdy)->copyToD2D(op.Y->dA);
+        op.forward();
+        std::vector<float> rY(bn * F), rxh(bn * F), rm(F), rv(F), rdx(bn * F), rdg(F), rdb(F);
+        oracle_batchNorm(bx.data(), bb.data(), bg.data(), rm.data(), rv.data(), rY.data(), rxh.data(), bn, F);
+        compare("BatchNorm::forward", pull(op.Y->A), rY, bn * 16);
+        compare("BatchNorm mean", pull(op.mean), rm, bn * 16);
+        op.xGrads();
+        oracle_batchNormGrad(bdy.data(), bg.data(), bx.data(), rdx.data(), bn, F);
+        compare("BatchNorm::xGrads", pull(src->dA), rdx, bn * 64);
+        op.paramGrads();
+        auto xh_gpu = pull(op.xHatP);
+        oracle_batchNormParamGrads(bdy.data(), xh_gpu.data(), rdg.data(), rdb.data(), bn, F);
+        compare("BatchNorm dGamma", pull(op.gamma->grad()), rdg, bn * 16);
+        compare("BatchNorm dBeta", pull(op.beta->grad()), rdb, bn * 16);
+        CHECK(throws_invalid([&] { batchNorm(src->A, op.beta->data(), op.gamma->data(), op.mean, op.variance, op.Y->A, op.mean); }));
+    }
+
     // Tensor arithmetic used by the loss and the optimizer, then one momentum step with weight decay
     auto a = randn(1000, 25), b = randn(1000, 26), m = randn(1000, 27);
     Tensor *A = push(shape4(1000, 1), a), *B = push(shape4(1000, 1), b), *M = push(shape4(1000, 1), m);
@@ -456,6 +489,29 @@ static void gpu_sequential_tests() {
     // a second forward after the update runs and changes the loss
     net.forward(X);
     CHECK(net.lossFW(net.netY, L, lossBuf) != loss);
+    // the two optional shortcuts change nothing: prune the reserve folds, update all parameters in one launch
+    {
+        auto before_w = pull(c2->filter->data());
+        net.forward(X);
+        net.backward(L);
+        auto g_plain = pull(c2->filter->grad()), dx_plain = pull(net.netX->dA), gp_plain = pull(cp->filter->grad());
+        net.zeroGrads();
+        net.pruneReserveFolds();
+        net.forward(X);
+        net.backward(L);
+        CHECK(pull(c2->filter->grad()) == g_plain);
+        CHECK(pull(cp->filter->grad()) == gp_plain);
+        CHECK(pull(net.netX->dA) == dx_plain);
+        // fused update against the per-parameter update on a copy of the state
+        Tensor *wc = clone(c2->filter->data()), *gc = clone(c2->filter->grad());
+        Tensor *mc = clone(static_cast<Momentum *>(c2->filter->opt)->m);
+        momentumApplyDecay(wc, gc, mc, 0.05f, 0.9f, 0.0001f);
+        net.learnFused();
+        CHECK(pull(c2->filter->data()) == pull(wc));
+        CHECK(pull(static_cast<Momentum *>(c2->filter->opt)->m) == pull(mc));
+        for (float v : pull(fc->biases->grad())) CHECK(v == 0.f);
+        CHECK(pull(c2->filter->data()) != before_w);
+    }
     // the non-blocking mode gives the same numbers
     setBlocking(false);
     net.forward(X);

@@ -158,3 +158,59 @@ def test_null_and_zero_arguments(dev):
         capi.softmax(X, X, 0, 8)
     with pytest.raises(capi.CrbError):
         capi.momentum_apply(X, None, X, 8, 0.1, 0.9)
+
+
+# (N, C, H, W): the ResNet-56 stages at its archived batch of 64, batches beyond the register cache (N > 128), a batch of
+# one, feature counts that are not multiples of 64
+@pytest.mark.parametrize("N,C,H,W", [(64, 16, 32, 32), (64, 32, 16, 16), (64, 64, 8, 8), (128, 8, 4, 4), (200, 3, 5, 5),
+                                     (1, 4, 3, 3), (7, 1, 1, 1), (96, 5, 7, 3), (129, 2, 8, 8), (300, 2, 3, 3), (4, 32, 32, 32),
+                                     (70, 32, 32, 32)])
+def test_batchnorm(dev, N, C, H, W):
+    capi, orc = _capi(), _oracle()
+    F = C * H * W
+    x = normal(20, N, C, H, W) * 1.5 + 0.3
+    gamma, beta, dy = normal(21, F) + 1.0, normal(22, F), normal(23, N, C, H, W)
+    Yr, xhr, mr, vr = orc.batchNorm(x, beta, gamma)
+    X, G, B = to_dev(x, dev), to_dev(gamma, dev), to_dev(beta, dev)
+    Y, xh, m, v = _nan(dev, N, C, H, W), _nan(dev, N, C, H, W), _nan(dev, F), _nan(dev, F)
+    capi.batchnorm_fwd(X, B, G, m, v, Y, xh, N, F)
+    # tolerance: sums over N samples in a different order; values are O(1)
+    tol = 1e-5 * np.sqrt(max(N, 1))
+    np.testing.assert_allclose(to_np(m), mr, rtol=0, atol=tol * 2)
+    np.testing.assert_allclose(to_np(v), vr, rtol=tol * 4, atol=tol)
+    if N > 1:  # with one sample var = 0 and xHat = 0/sqrt(1e-8) amplifies rounding of x - mean = 0 exactly: still 0
+        np.testing.assert_allclose(to_np(xh), xhr, rtol=0, atol=tol * 8)
+        np.testing.assert_allclose(to_np(Y), Yr, rtol=0, atol=tol * 16)
+    else:
+        assert not to_np(xh).any() and np.array_equal(to_np(Y).ravel(), np.tile(beta, N))
+    dXr = orc.batchNormGrad(dy, gamma, x)
+    dX = _nan(dev, N, C, H, W)
+    dY = to_dev(dy, dev)
+    capi.batchnorm_bwd(dY, G, X, dX, N, F)
+    scale = max(float(np.abs(dXr).max()), 1.0)
+    np.testing.assert_allclose(to_np(dX), dXr, rtol=0, atol=tol * 32 * scale if N > 1 else 1e30)
+    dGr, dBr = orc.batchNormParamGrads(dy, xhr)
+    dG, dB = _nan(dev, F), _nan(dev, F)
+    capi.batchnorm_param_grads(dY, to_dev(xhr, dev), dG, dB, N, F)
+    np.testing.assert_allclose(to_np(dB), dBr, rtol=0, atol=tol * 8)
+    np.testing.assert_allclose(to_np(dG), dGr, rtol=0, atol=tol * 16)
+    again = _nan(dev, N, C, H, W)
+    capi.batchnorm_bwd(dY, G, X, again, N, F)
+    assert np.array_equal(to_np(again), to_np(dX))  # fixed summation order
+
+
+def test_momentum_multi_matches_single(dev):
+    import torch
+    capi, orc = _capi(), _oracle()
+    sizes = [1, 16, 144, 2304, 4099, 36864, 65]
+    host = [(normal(50 + i, n), normal(60 + i, n), normal(70 + i, n)) for i, n in enumerate(sizes)]
+    tens = [tuple(to_dev(a, dev) for a in h) for h in host]
+    # one unaligned view in the table
+    base = [to_dev(np.concatenate([[0], a]).astype(np.float32), dev) for a in host[-1]]
+    tens[-1] = tuple(b[1:] for b in base)
+    entries = [(X, G, M, 0.01 * (i + 1), 0.9, 1.0 - 5e-4 * (i % 2)) for i, (X, G, M) in enumerate(tens)]
+    table, n, mx = capi.momentum_table(torch, dev, entries)
+    capi.momentum_apply_multi(table, n, mx)
+    for i, ((x, g, m), (X, G, M)) in enumerate(zip(host, tens)):
+        xr, gr, mr = orc.momentumApply(x, g, m, np.float32(0.01 * (i + 1)), 0.9, np.float32(1.0 - 5e-4 * (i % 2)))
+        assert np.array_equal(to_np(X), xr) and np.array_equal(to_np(M), mr) and not to_np(G).any()

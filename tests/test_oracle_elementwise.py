@@ -136,3 +136,52 @@ def test_momentum_closed_form_and_recurrence():
         x64 = x64 * (1 - 5e-4) - lr * m64
     np.testing.assert_allclose(m, m64, rtol=1e-5, atol=1e-7)
     np.testing.assert_allclose(x, x64, rtol=1e-5, atol=1e-6)
+
+
+@pytest.mark.parametrize("shape", [(8, 3, 4, 4), (64, 2, 3, 5), (2, 7, 1, 1), (130, 1, 2, 2)])
+def test_batchnorm_against_torch(shape):
+    import torch
+    import torch.nn.functional as F
+
+    N, feat = shape[0], int(np.prod(shape[1:]))
+    x = rnd(30, *shape) * 2 + 0.5
+    gamma, beta = rnd(31, feat) + 1.0, rnd(32, feat)
+    dy = rnd(33, *shape)
+    Y, xHat, mean, var = orc.batchNorm(x, beta, gamma)
+    xt = torch.tensor(x.reshape(N, feat), dtype=torch.float64, requires_grad=True)
+    gt = torch.tensor(gamma, dtype=torch.float64, requires_grad=True)
+    bt = torch.tensor(beta, dtype=torch.float64, requires_grad=True)
+    yt = F.batch_norm(xt, None, None, weight=gt, bias=bt, training=True, eps=1e-8)
+    np.testing.assert_allclose(Y.reshape(N, feat), yt.detach().numpy(), rtol=2e-5, atol=2e-5)
+    np.testing.assert_allclose(mean, x.reshape(N, feat).astype(np.float64).mean(axis=0), rtol=1e-5, atol=1e-6)
+    np.testing.assert_allclose(var, x.reshape(N, feat).astype(np.float64).var(axis=0), rtol=1e-4, atol=1e-7)  # biased
+    # xHat: zero mean, unit (biased) variance per feature
+    np.testing.assert_allclose(xHat.reshape(N, feat).mean(axis=0), 0, atol=1e-5)
+    np.testing.assert_allclose(xHat.reshape(N, feat).astype(np.float64).var(axis=0), 1, rtol=1e-4)
+    yt.backward(torch.tensor(dy.reshape(N, feat), dtype=torch.float64))
+    dX = orc.batchNormGrad(dy, gamma, x)
+    scale = np.abs(xt.grad.numpy()).max()
+    np.testing.assert_allclose(dX.reshape(N, feat), xt.grad.numpy(), rtol=1e-3, atol=2e-5 * max(scale, 1))
+    dG, dB = orc.batchNormParamGrads(dy, xHat)
+    np.testing.assert_allclose(dG, gt.grad.numpy(), rtol=1e-4, atol=1e-4)
+    np.testing.assert_allclose(dB, bt.grad.numpy(), rtol=1e-5, atol=1e-5)
+
+
+def test_batchnorm_gradient_finite_differences():
+    N, feat = 5, 3
+    x = rnd(34, N, feat).astype(np.float64)
+    gamma, beta, dy = rnd(35, feat) + 1.0, rnd(36, feat), rnd(37, N, feat)
+
+    def f(xx):  # scalar objective <Y, dy> in float64
+        m, v = xx.mean(axis=0), xx.var(axis=0)
+        return float((((xx - m) / np.sqrt(v + 1e-8) * gamma + beta) * dy).sum())
+
+    g = np.zeros_like(x)
+    h = 1e-5
+    for i in range(N):
+        for j in range(feat):
+            xp, xm = x.copy(), x.copy()
+            xp[i, j] += h
+            xm[i, j] -= h
+            g[i, j] = (f(xp) - f(xm)) / (2 * h)
+    np.testing.assert_allclose(orc.batchNormGrad(dy, gamma, x.astype(np.float32)), g, rtol=2e-3, atol=2e-4)
