@@ -58,6 +58,9 @@ SIGNATURES = {
     "crb_tensor_sub_inplace": (ctypes.c_int, [_ptr, _ptr, _u32, _ptr]),
     "crb_tensor_copy": (ctypes.c_int, [_ptr, _ptr, _u32, _ptr]),
     "crb_tensor_add_clear": (ctypes.c_int, [_ptr, _ptr, _u32, _ptr]),
+    "crb_tensor_add": (ctypes.c_int, [_ptr, _ptr, _ptr, _u32, _ptr]),
+    "crb_tensor_add_clear_copy": (ctypes.c_int, [_ptr, _ptr, _ptr, _u32, _ptr]),
+    "crb_tensor_copy2": (ctypes.c_int, [_ptr, _ptr, _ptr, _u32, _ptr]),
     "crb_tensor_scale_inplace": (ctypes.c_int, [_ptr, ctypes.c_float, _u32, _ptr]),
     "crb_relu_fwd": (ctypes.c_int, [_ptr, _ptr, _u32, _ptr]),
     "crb_relu_bwd": (ctypes.c_int, [_ptr, _ptr, _ptr, _u32, _ptr]),
@@ -258,3 +261,15 @@ def momentum_table(torch, dev, entries):
 
 def momentum_apply_multi(table, n_items, max_count, stream=None):
     check(load().crb_momentum_apply_multi(_p(table), n_items, max_count, _stream(stream)))
+
+
+def tensor_add(dst, a, b, count, stream=None):
+    check(load().crb_tensor_add(_p(dst), _p(a), _p(b), count, _stream(stream)))
+
+
+def tensor_add_clear_copy(dst, a, b, count, stream=None):
+    check(load().crb_tensor_add_clear_copy(_p(dst), _p(a), _p(b), count, _stream(stream)))
+
+
+def tensor_copy2(dst1, dst2, src, count, stream=None):
+    check(load().crb_tensor_copy2(_p(dst1), _p(dst2), _p(src), count, _stream(stream)))

@@ -63,9 +63,45 @@ __global__ void __launch_bounds__(256) copy_kernel(float *__restrict__ dst, cons
     }
 }
 
+// Three-operand streaming forms used by the residual-connection operand. MODE 0: d = a + b. MODE 1: a += b; b = 0; d = a.
+// MODE 2: d = a; b = a (one source, two destinations).
+template <int MODE>
+__global__ void __launch_bounds__(256) tri_kernel(float *d, float *a, float *b, u32 count, u32 vec) {
+    const u32 stride = gridDim.x * 256;
+    u32 i = blockIdx.x * 256 + threadIdx.x;
+    auto one = [&](auto *pd, auto *pa, auto *pb, u32 k, auto zero) {
+        if (MODE == 0) {
+            pd[k] = pa[k] + pb[k];
+        } else if (MODE == 1) {
+            const auto v = pa[k] + pb[k];
+            pa[k] = v, pb[k] = zero, pd[k] = v;
+        } else {
+            const auto v = pa[k];
+            pd[k] = v, pb[k] = v;
+        }
+    };
+    if (vec) {
+        const u32 nq = count / 4;
+        const v4f z4 = {0.f, 0.f, 0.f, 0.f};
+        for (u32 q = i; q < nq; q += stride) one(reinterpret_cast<v4f *>(d), reinterpret_cast<v4f *>(a), reinterpret_cast<v4f *>(b), q, z4);
+        for (u32 r = nq * 4 + i; r < count; r += stride) one(d, a, b, r, 0.f);
+    } else {
+        for (; i < count; i += stride) one(d, a, b, i, 0.f);
+    }
+}
+
 static u32 stream_grid(u32 count) {
     u32 blocks = ceil_div(ceil_div(count, 4), 256);
     return blocks < 1 ? 1 : (blocks > 4096 ? 4096 : blocks);
+}
+
+template <int MODE>
+static int launch_tri(float *d, float *a, float *b, uint32_t count, void *stream, const char *what) {
+    if (!d || !a || !b) return fail(CRB_ENULL, "%s: null operand", what);
+    if (!count) return fail(CRB_EINVAL_SHAPE, "%s: zero size", what);
+    const u32 vec = ((reinterpret_cast<uintptr_t>(d) | reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b)) & 15u) == 0;
+    hipLaunchKernelGGL((tri_kernel<MODE>), dim3(stream_grid(count)), dim3(256), 0, hipStream_t(stream), d, a, b, count, vec);
+    return check_launch(what);
 }
 
 }  // namespace crb
@@ -98,6 +134,19 @@ int crb_tensor_copy(float *dst, const float *src, uint32_t count, void *stream) 
     const u32 vec = ((reinterpret_cast<uintptr_t>(dst) | reinterpret_cast<uintptr_t>(src)) & 15u) == 0;
     hipLaunchKernelGGL(copy_kernel, dim3(stream_grid(count)), dim3(256), 0, hipStream_t(stream), dst, src, count, vec);
     return check_launch("crb_tensor_copy");
+}
+
+int crb_tensor_add(float *dst, const float *a, const float *b, uint32_t count, void *stream) {
+    return launch_tri<0>(dst, const_cast<float *>(a), const_cast<float *>(b), count, stream, "crb_tensor_add");
+}
+
+int crb_tensor_add_clear_copy(float *dst, float *a, float *b, uint32_t count, void *stream) {
+    if (a == b || dst == b) return fail(CRB_EINVAL_SHAPE, "crb_tensor_add_clear_copy: operands alias");
+    return launch_tri<1>(dst, a, b, count, stream, "crb_tensor_add_clear_copy");
+}
+
+int crb_tensor_copy2(float *dst1, float *dst2, const float *src, uint32_t count, void *stream) {
+    return launch_tri<2>(dst1, const_cast<float *>(src), dst2, count, stream, "crb_tensor_copy2");
 }
 
 int crb_tensor_fill(float *a, float value, uint32_t count, void *stream) {

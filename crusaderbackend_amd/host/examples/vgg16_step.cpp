@@ -93,8 +93,8 @@ int main(int argc, char **argv) {
     const double ms_blocking = time_steps(net, X, L, steps);
     setBlocking(false);
     const double ms_async = time_steps(net, X, L, steps);
-    // the same network with the two optional shortcuts: reserve folds pruned, one launch for all momentum updates
-    net.pruneReserveFolds();
+    // the same network with the optional shortcuts: streamlined graph, one launch for all momentum updates
+    net.streamline();
     g_fused = true;
     const double ms_fast = time_steps(net, X, L, steps);
     g_fused = false;

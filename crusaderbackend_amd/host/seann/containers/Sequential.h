@@ -41,11 +41,14 @@ public:
     void learnBatch() const;
     void zeroGrads() const;
 
-    // Two optional shortcuts with no counterpart in the reference; results are unchanged.
+    // Optional shortcuts with no counterpart in the reference; results are unchanged.
     // pruneReserveFolds: after construct(), stop folding Y->dAReserve into Y->dA in the xGrads of operands into whose
     // reserve no operand of this network deposits anything (only shortcut endpoints do). An operand type of your own that
     // writes another operand's reserve must increment that operand's `reserveWriters` in its postWaiveInit.
     void pruneReserveFolds() const;
+    // streamline: pruneReserveFolds plus letting every opening shortcut endpoint's output value alias its input (it only
+    // passes it on), which removes one device copy per residual block from the forward pass.
+    void streamline() const;
     // learnFused: the momentum step of every parameter in one kernel launch instead of one launch per parameter.
     void learnFused();
 

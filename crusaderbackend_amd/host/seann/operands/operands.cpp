@@ -121,30 +121,39 @@ void ShortcutEndpoint::postWaiveInit(OptimizerInfo *inf) {  // :13-55
     }
 }
 
-void ShortcutEndpoint::forward() {  // :57-74
-    X->A->copyToD2D(Y->A);
-    if (isContainer) {
-        if (operandCount > 0) {
-            for (uint32 i = 0; i < operandCount; i++) branchOperands[i]->forward();
-            *Y->A + branchOperands[operandCount - 1]->Y->A;
-        } else {
-            *Y->A + other->Y->A;  // identity shortcut
-        }
+static void launched(int status, const char *file, int line) {
+    throwOnStatus(status, file, line);
+    if (isBlocking() && hipStreamSynchronize(nullptr) != hipSuccess) assertHip(file, line);
+}
+
+void ShortcutEndpoint::forward() {  // :57-74: Y = X for the opening endpoint, Y = X + shortcut for the closing one
+    const uint32 n = X->A->dims.size;
+    if (!isContainer) {
+        if (Y->A->elements != X->A->elements) X->A->copyToD2D(Y->A);  // aliased by Sequential::streamline()
+        return;
     }
+    for (uint32 i = 0; i < operandCount; i++) branchOperands[i]->forward();
+    Tensor *shortcut = operandCount > 0 ? branchOperands[operandCount - 1]->Y->A : other->Y->A;
+    launched(crb_tensor_add(Y->A->elements, X->A->elements, shortcut->elements, n, nullptr), __FILE__, __LINE__);
 }
 
 void ShortcutEndpoint::xGrads() {  // :76-99
+    const uint32 n = X->A->dims.size;
     if (isContainer) {
         if (operandCount > 0) {
-            Y->dA->copyToD2D(branchOperands[operandCount - 1]->Y->dA);
+            // projection: the branch gets a copy of the gradient, as does the main path
+            launched(crb_tensor_copy2(X->dA->elements, branchOperands[operandCount - 1]->Y->dA->elements, Y->dA->elements, n, nullptr),
+                     __FILE__, __LINE__);
             for (int i = int(operandCount) - 1; i >= 0; i--) branchOperands[i]->xGrads();
         } else {
-            Y->dA->copyToD2D(other->Y->dAReserve);
+            // identity: the opening endpoint's reserve gets a copy of the gradient, as does the main path
+            launched(crb_tensor_copy2(X->dA->elements, other->Y->dAReserve->elements, Y->dA->elements, n, nullptr), __FILE__, __LINE__);
         }
+    } else if (foldReserveEnabled) {
+        launched(crb_tensor_add_clear_copy(X->dA->elements, Y->dA->elements, Y->dAReserve->elements, n, nullptr), __FILE__, __LINE__);
     } else {
-        foldReserve();
+        Y->dA->copyToD2D(X->dA);
     }
-    Y->dA->copyToD2D(X->dA);
 }
 
 void ShortcutEndpoint::paramGrads() {
@@ -232,6 +241,35 @@ void Sequential::zeroGrads() const {
 
 void Sequential::pruneReserveFolds() const {
     for (OperandBase *op : operands) op->pruneReserveFolds();
+}
+
+void Sequential::streamline() const {
+    pruneReserveFolds();
+    if (hipDeviceSynchronize() != hipSuccess) assertHip(__FILE__, __LINE__);  // buffers are released below: nothing may be in flight
+    for (uint32 i = 0; i + 1 < OPERAND_COUNT; i++) {
+        OperandBase *op = operands[i];
+        if (op->OPERAND_ID() != OPR_CTRL_SHORTCUTENDPOINT_BEG) continue;
+        if (op->Y->A->elements == op->X->A->elements) continue;
+        // The opening endpoint only passes its input on: its output value takes over the input's storage. Every tensor that
+        // was bound to the old output buffer holds a copy of its address (Tensor::attach copies the pointer), so the
+        // consumers are re-attached before anything can run: the next operand of the chain and, for a projection
+        // shortcut, the first operand of the closing endpoint's branch.
+        auto *beg = static_cast<ShortcutEndpoint *>(op);
+        op->Y->A->destroy();
+        op->Y->A->attach(op->X->A);
+        operands[i + 1]->X->A->attach(op->Y->A);
+        if (beg->other && beg->other->operandCount > 0) beg->other->branchOperands[0]->X->A->attach(op->Y->A);
+    }
+    // no operand may be left reading a buffer other than its producer's
+    for (uint32 i = 1; i < OPERAND_COUNT; i++) {
+        if (operands[i]->X->A->elements != operands[i - 1]->Y->A->elements)
+            throw std::runtime_error("Sequential::streamline: an operand's input is not its predecessor's output");
+        if (operands[i]->OPERAND_ID() == OPR_CTRL_SHORTCUTENDPOINT_END) {
+            auto *end = static_cast<ShortcutEndpoint *>(operands[i]);
+            if (end->operandCount > 0 && end->branchOperands[0]->X->A->elements != end->other->Y->A->elements)
+                throw std::runtime_error("Sequential::streamline: a shortcut branch's input is not the opening endpoint's output");
+        }
+    }
 }
 
 // All parameters in one kernel launch. The device table of (weights, gradient, momentum, rates) is built on the first

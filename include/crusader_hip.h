@@ -158,6 +158,14 @@ int crb_tensor_copy(float *dst, const float *src, uint32_t count, void *stream);
  * ... `Y->dAReserve->constFill(0)` (e.g. seann/operands/seblas/Conv2D.cu:19,21) — in one pass. The two must not alias. */
 int crb_tensor_add_clear(float *a, float *b, uint32_t count, void *stream);
 
+/* Fused forms of the copies and adds the shortcut operand performs (seann/operands/controlling/ShortcutEndpoint.cu):
+ *   crb_tensor_add:             dst = a + b           (forward of the closing endpoint, :59-73: copy then add; dst may be a)
+ *   crb_tensor_add_clear_copy:  a += b; b = 0; dst = a (backward of the opening endpoint, :92-97: fold the reserve, copy on)
+ *   crb_tensor_copy2:           dst1 = src; dst2 = src (backward of an identity closing endpoint, :88-89,96-97: two copies) */
+int crb_tensor_add(float *dst, const float *a, const float *b, uint32_t count, void *stream);
+int crb_tensor_add_clear_copy(float *dst, float *a, float *b, uint32_t count, void *stream);
+int crb_tensor_copy2(float *dst1, float *dst2, const float *src, uint32_t count, void *stream);
+
 /* Replaces the device branch of seblas::Tensor::operator-(Tensor*) (Tensor.cu:485-506): a[i] -= b[i], in place. */
 int crb_tensor_sub_inplace(float *a, const float *b, uint32_t count, void *stream);
 

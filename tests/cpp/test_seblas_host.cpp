@@ -496,7 +496,7 @@ static void gpu_sequential_tests() {
         net.backward(L);
         auto g_plain = pull(c2->filter->grad()), dx_plain = pull(net.netX->dA), gp_plain = pull(cp->filter->grad());
         net.zeroGrads();
-        net.pruneReserveFolds();
+        net.streamline();
         net.forward(X);
         net.backward(L);
         CHECK(pull(c2->filter->grad()) == g_plain);

@@ -41,3 +41,22 @@ def test_vgg16_sequential_example_trains(dev):
     assert losses[-1] < losses[0]
     out = json.loads(r.stdout.strip().splitlines()[-1])
     assert out["batch"] == 16 and out["ms_per_step_nonblocking"] > 0 and out["ms_per_step_blocking"] >= out["ms_per_step_nonblocking"] * 0.8
+
+
+@pytest.mark.gpu
+def test_resnet56_sequential_example_runs(dev):
+    """The archived ResNet-56 topology (59 convolutions, 57 batch norms, 28 residual blocks) through seann::Sequential:
+    plain, non-blocking and streamlined + fused-update modes all run and the loss of a repeated batch goes down."""
+    import json
+    import re
+
+    exe = os.path.join(ROOT, "crusaderbackend_amd", "host", "examples", "bin", "resnet56_step")
+    assert os.path.exists(exe), f"{exe} missing: run `make -C crusaderbackend_amd/host`"
+    r = subprocess.run([exe, "16", "2", "trace"], capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0, r.stdout + r.stderr
+    losses = [float(m) for m in re.findall(r"loss/sample ([-0-9.naif]+)", r.stdout)]
+    assert len(losses) == 8 and all(l == l for l in losses)
+    assert min(losses[1:]) < losses[0]
+    out = json.loads(r.stdout.strip().splitlines()[-1])
+    assert out["operands"] == 230 and out["ms_per_step_pruned_fused"] > 0
+    assert out["loss_per_sample_after"] == out["loss_per_sample_after"]  # finite after the streamlined steps too
