@@ -165,12 +165,37 @@ def cpu_baseline(layers_spec, min_seconds=10.0):
     }
 
 
+def full_network_steps():
+    """The whole ResNet-56 / VGG-16 training steps (every operator, optimizer included) through the C++ seann host layer,
+    each run by its own example program as a child process BEFORE this process touches the GPU. Returns {} when the
+    programs are not built, when a profiler has already initialised the GPU in this process, or on any failure: the
+    figures are an extra, the benchmark does not depend on them."""
+    import subprocess
+
+    if any(k.startswith(("ROCPROF", "ROCP_", "ROCTRACER")) for k in os.environ):
+        return {}
+    out = {}
+    bindir = os.path.join(ROOT, "crusaderbackend_amd", "host", "examples", "bin")
+    for key, exe, argv in (("resnet56_full_step", "resnet56_step", ["128", "10"]), ("vgg16_full_step_cpp", "vgg16_step", ["128", "10"])):
+        path = os.path.join(bindir, exe)
+        if not os.path.exists(path):
+            continue
+        try:
+            r = subprocess.run([path] + argv, capture_output=True, text=True, timeout=120)
+            if r.returncode == 0:
+                out[key] = json.loads(r.stdout.strip().splitlines()[-1])
+        except (OSError, subprocess.SubprocessError, ValueError, IndexError):
+            pass
+    return out
+
+
 def main():
     args = parse()
     if args.gpus != 1:
         print("bench.py: this build targets one GPU per process and has no multi-GPU path; run with --gpus 1",
               file=sys.stderr)
         sys.exit(2)
+    full_net = {} if args.calibrate else full_network_steps()
     import torch
 
     from crusaderbackend_amd import capi
@@ -263,6 +288,7 @@ def main():
             "sgemm_4096_frac_peak": gemm_tflops / PEAK_FP32_MFMA_TFLOPS,
             "per_kernel": {k: {"ms": round(v["ms"], 5), "tflops": round(v["tflops"], 2), "gbs": round(v["gbs"], 1)}
                            for k, v in per.items()},
+            "full_network_steps_cpp_host": full_net,
             "device": props.name, "cus": props.multi_processor_count, "clock_mhz": clock_khz / 1e3,
             # 256 flop per clock per CU on the fp32 matrix pipe, at the peak clock the device reports
             "peak_from_reported_clock_tflops": props.multi_processor_count * clock_khz * 1e3 * 256 / 1e12,
