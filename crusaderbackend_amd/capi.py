@@ -72,7 +72,7 @@ SIGNATURES = {
     "crb_cross_entropy_loss": (ctypes.c_int, [_ptr, _ptr, _ptr, _u32, _ptr, _u32, _ptr]),
     "crb_momentum_apply_multi": (ctypes.c_int, [_ptr, _u32, _u32, _ptr]),
     "crb_batchnorm_fwd": (ctypes.c_int, [_ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _u32, _u32, _ptr]),
-    "crb_batchnorm_bwd": (ctypes.c_int, [_ptr, _ptr, _ptr, _ptr, _u32, _u32, _ptr]),
+    "crb_batchnorm_bwd": (ctypes.c_int, [_ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _u32, _u32, _ptr]),
     "crb_batchnorm_param_grads": (ctypes.c_int, [_ptr, _ptr, _ptr, _ptr, _u32, _u32, _ptr]),
     "crb_momentum_apply": (ctypes.c_int, [_ptr, _ptr, _ptr, _u32, ctypes.c_float, ctypes.c_float, ctypes.c_float, _ptr]),
 }
@@ -226,8 +226,8 @@ def batchnorm_fwd(X, beta, gamma, mean, var, Y, xHat, N, F, stream=None):
     check(load().crb_batchnorm_fwd(_p(X), _p(beta), _p(gamma), _p(mean), _p(var), _p(Y), _p(xHat), N, F, _stream(stream)))
 
 
-def batchnorm_bwd(dY, gamma, X, dX, N, F, stream=None):
-    check(load().crb_batchnorm_bwd(_p(dY), _p(gamma), _p(X), _p(dX), N, F, _stream(stream)))
+def batchnorm_bwd(dY, gamma, X, dX, N, F, dGamma=None, dBeta=None, stream=None):
+    check(load().crb_batchnorm_bwd(_p(dY), _p(gamma), _p(X), _p(dX), _p(dGamma), _p(dBeta), N, F, _stream(stream)))
 
 
 def batchnorm_param_grads(dY, xHat, dGamma, dBeta, N, F, stream=None):

@@ -370,7 +370,8 @@ __global__ void __launch_bounds__(256) batchnorm_fwd_kernel(const float *__restr
 
 template <int FL>
 __global__ void __launch_bounds__(256) batchnorm_bwd_kernel(const float *__restrict__ dY, const float *__restrict__ gamma,
-                                                            const float *__restrict__ X, float *__restrict__ dX, u32 N, u32 F) {
+                                                            const float *__restrict__ X, float *__restrict__ dX,
+                                                            float *__restrict__ dGamma, float *__restrict__ dBeta, u32 N, u32 F) {
     constexpr u32 G = 256 / FL;
     __shared__ float red[G][FL];
     const BnGeom<FL> t(F);
@@ -413,6 +414,8 @@ __global__ void __launch_bounds__(256) batchnorm_bwd_kernel(const float *__restr
     const float inv = 1.0f / sqrtf(v + 1e-8f), ga = gamma[t.f], invN = 1.0f / float(N);
     const float dVar = ga * Sdd * -0.5f * inv * inv * inv;
     const float dMean = ga * Sdy * -inv + dVar * (-2.0f * Sd) * invN;
+    // the parameter gradients fall out of the same sums: dBeta = sum dy, dGamma = sum dy*xHat = inv * sum dy*(x - mean)
+    if (dGamma && t.g == 0) dGamma[t.f] = Sdd * inv, dBeta[t.f] = Sdy;
     if (cached) {
 #pragma unroll
         for (int i = 0; i < kBnCache; ++i) {
@@ -618,14 +621,17 @@ int crb_batchnorm_fwd(const float *X, const float *beta, const float *gamma, flo
     return check_launch("crb_batchnorm_fwd");
 }
 
-int crb_batchnorm_bwd(const float *dY, const float *gamma, const float *X, float *dX, uint32_t N, uint32_t F, void *stream) {
+int crb_batchnorm_bwd(const float *dY, const float *gamma, const float *X, float *dX, float *dGamma_or_null, float *dBeta_or_null,
+                      uint32_t N, uint32_t F, void *stream) {
     if (!dY || !gamma || !X || !dX) return fail(CRB_ENULL, "crb_batchnorm_bwd: null operand");
+    if (!dGamma_or_null != !dBeta_or_null) return fail(CRB_ENULL, "crb_batchnorm_bwd: dGamma and dBeta go together");
+    float *dGamma = dGamma_or_null, *dBeta = dBeta_or_null;
     if (int st = check_bn("crb_batchnorm_bwd", N, F)) return st;
     hipStream_t s = hipStream_t(stream);
     switch (bn_features_per_wg(F)) {
-        case 64: hipLaunchKernelGGL(batchnorm_bwd_kernel<64>, dim3(ceil_div(F, 64)), dim3(256), 0, s, dY, gamma, X, dX, N, F); break;
-        case 32: hipLaunchKernelGGL(batchnorm_bwd_kernel<32>, dim3(ceil_div(F, 32)), dim3(256), 0, s, dY, gamma, X, dX, N, F); break;
-        default: hipLaunchKernelGGL(batchnorm_bwd_kernel<16>, dim3(ceil_div(F, 16)), dim3(256), 0, s, dY, gamma, X, dX, N, F);
+        case 64: hipLaunchKernelGGL(batchnorm_bwd_kernel<64>, dim3(ceil_div(F, 64)), dim3(256), 0, s, dY, gamma, X, dX, dGamma, dBeta, N, F); break;
+        case 32: hipLaunchKernelGGL(batchnorm_bwd_kernel<32>, dim3(ceil_div(F, 32)), dim3(256), 0, s, dY, gamma, X, dX, dGamma, dBeta, N, F); break;
+        default: hipLaunchKernelGGL(batchnorm_bwd_kernel<16>, dim3(ceil_div(F, 16)), dim3(256), 0, s, dY, gamma, X, dX, dGamma, dBeta, N, F);
     }
     return check_launch("crb_batchnorm_bwd");
 }

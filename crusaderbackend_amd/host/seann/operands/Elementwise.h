@@ -70,6 +70,7 @@ public:
     Tensor *mean{};
     Tensor *variance{};
     Tensor *xHatP{};
+    bool paramGradsDone = false;
     std::string info() override { return "BatchNorm"; }
     void initNetParams(OptimizerInfo *info, shape4 inShape) override {  // BatchNorm.cuh:27-37
         shape4 paramShape = {1, inShape.c, inShape.h, inShape.w};
@@ -85,12 +86,21 @@ public:
         beta->data()->constFill(0.0f);
         gamma->data()->constFill(1.0f);
     }
-    void forward() override { batchNorm(X->A, beta->data(), gamma->data(), mean, variance, Y->A, xHatP); }
+    void forward() override {
+        paramGradsDone = false;
+        batchNorm(X->A, beta->data(), gamma->data(), mean, variance, Y->A, xHatP);
+    }
+    // xGrads also produces the parameter gradients (they fall out of the same per-feature sums); the paramGrads call
+    // that follows it in Sequential::backward then has nothing left to do. Called on its own, paramGrads computes them.
     void xGrads() override {  // BatchNorm.cu:17-21
         foldReserve();
-        batchNormGrad(Y->dA, gamma->data(), X->A, X->dA);
+        batchNormGradAll(Y->dA, gamma->data(), X->A, X->dA, gamma->grad(), beta->grad());
+        paramGradsDone = true;
     }
-    void paramGrads() override { batchNormParamGrads(Y->dA, xHatP, gamma->grad(), beta->grad()); }
+    void paramGrads() override {
+        if (!paramGradsDone) batchNormParamGrads(Y->dA, xHatP, gamma->grad(), beta->grad());
+        paramGradsDone = false;
+    }
     void updateParams() override {
         beta->update();
         gamma->update();

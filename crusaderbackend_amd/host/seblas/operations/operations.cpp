@@ -214,7 +214,19 @@ Tensor *batchNormGrad(Tensor *dY, Tensor *gamma, Tensor *X, Tensor *dX) {
     require(dX->dims.size == X->dims.size, "batchNormGrad: dX size");
     const uint32 F = X->dims.size / X->dims.n;
     require(gamma->dims.size == F, "batchNormGrad: gamma must hold one value per feature");
-    finish(crb_batchnorm_bwd(dY->elements, gamma->elements, X->elements, dX->elements, X->dims.n, F, nullptr), __FILE__, __LINE__);
+    finish(crb_batchnorm_bwd(dY->elements, gamma->elements, X->elements, dX->elements, nullptr, nullptr, X->dims.n, F, nullptr),
+           __FILE__, __LINE__);
+    return dX;
+}
+
+Tensor *batchNormGradAll(Tensor *dY, Tensor *gamma, Tensor *X, Tensor *dX, Tensor *dGamma, Tensor *dBeta) {
+    require(dY->dims.n == X->dims.n && dY->dims.size == X->dims.size, "batchNormGradAll: dY and X differ");
+    require(dX->dims.size == X->dims.size, "batchNormGradAll: dX size");
+    const uint32 F = X->dims.size / X->dims.n;
+    require(gamma->dims.size == F && dGamma->dims.size == F && dBeta->dims.size == F, "batchNormGradAll: one value per feature");
+    finish(crb_batchnorm_bwd(dY->elements, gamma->elements, X->elements, dX->elements, dGamma->elements, dBeta->elements,
+                             X->dims.n, F, nullptr),
+           __FILE__, __LINE__);
     return dX;
 }
 

@@ -50,6 +50,9 @@ float crossEntropyCalc(Parameter *Y, Tensor *labels, Tensor *buf);
 Tensor *batchNorm(Tensor *X, Tensor *beta, Tensor *gamma, Tensor *mean, Tensor *var, Tensor *Y, Tensor *xHat);
 Tensor *batchNormGrad(Tensor *dY, Tensor *gamma, Tensor *X, Tensor *dX);
 void batchNormParamGrads(Tensor *dY, Tensor *xHat, Tensor *dGamma, Tensor *dBeta);
+// batchNormGrad and batchNormParamGrads in one pass over the data (no counterpart in the reference; same results up to
+// the rounding of xHat, which is recomputed instead of read back).
+Tensor *batchNormGradAll(Tensor *dY, Tensor *gamma, Tensor *X, Tensor *dX, Tensor *dGamma, Tensor *dBeta);
 // cuOptim.cuh:16. V is the momentum buffer; Xgrad is cleared by the step.
 void momentumApply(Tensor *X, Tensor *Xgrad, Tensor *V, float LEARNING_RATE, float MOMENTUM);
 // Optimizers.cu:16-22 in one pass: X *= (1 - L2) then momentumApply. No separate counterpart in the reference.

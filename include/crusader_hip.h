@@ -233,8 +233,11 @@ int crb_batchnorm_fwd(const float *X, const float *beta, const float *gamma, flo
                       uint32_t N, uint32_t F, void *stream);
 
 /* Replaces seblas::batchNormGrad (cuBatchNorm.cu:176-188; kernel :62-125): dX from dY, gamma and X (statistics are
- * recomputed from X, as in the reference). */
-int crb_batchnorm_bwd(const float *dY, const float *gamma, const float *X, float *dX, uint32_t N, uint32_t F, void *stream);
+ * recomputed from X, as in the reference). When dGamma / dBeta are given (both or neither) the parameter gradients are
+ * written too — they are by-products of the same sums (dBeta = sum dY, dGamma = sum dY*xHat) — which saves the separate
+ * crb_batchnorm_param_grads pass. */
+int crb_batchnorm_bwd(const float *dY, const float *gamma, const float *X, float *dX, float *dGamma_or_null, float *dBeta_or_null,
+                      uint32_t N, uint32_t F, void *stream);
 
 /* Replaces seblas::batchNormParamGrads (cuBatchNorm.cu:190-202; kernel :127-148): dBeta = sum_n dY, dGamma = sum_n dY*xHat.
  * Both are overwritten, not accumulated. */

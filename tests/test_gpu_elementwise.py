@@ -194,9 +194,12 @@ def test_batchnorm(dev, N, C, H, W):
     capi.batchnorm_param_grads(dY, to_dev(xhr, dev), dG, dB, N, F)
     np.testing.assert_allclose(to_np(dB), dBr, rtol=0, atol=tol * 8)
     np.testing.assert_allclose(to_np(dG), dGr, rtol=0, atol=tol * 16)
-    again = _nan(dev, N, C, H, W)
-    capi.batchnorm_bwd(dY, G, X, again, N, F)
+    again, dG2, dB2 = _nan(dev, N, C, H, W), _nan(dev, F), _nan(dev, F)
+    capi.batchnorm_bwd(dY, G, X, again, N, F, dGamma=dG2, dBeta=dB2)  # parameter gradients as by-products
     assert np.array_equal(to_np(again), to_np(dX))  # fixed summation order
+    np.testing.assert_allclose(to_np(dB2), dBr, rtol=0, atol=tol * 8)
+    if N > 1:
+        np.testing.assert_allclose(to_np(dG2), dGr, rtol=0, atol=tol * 32 * max(float(np.abs(dGr).max()), 1.0) / 8)
 
 
 def test_momentum_multi_matches_single(dev):
