@@ -26,6 +26,8 @@
 //     formulation would multiply are never touched. The two column parities held by a lane interleave into 8
 //     consecutive dX floats per row parity.
 #pragma once
+#include <type_traits>
+
 #include "igemm_engine.h"
 
 namespace crb {
@@ -34,10 +36,13 @@ namespace crb {
 // half the LDS, so more workgroups fit on a CU and overlap each other's staging.
 // FS_ = 3: 3x3 filter with pad 1. FS_ = 1: 1x1 filter, no padding, stride 1 (one tap, no halo) — the bottleneck layers,
 // which are bandwidth-bound: same staging and MFMA mapping, the contraction is just the channel chunk.
-template <int W_, int ROWS_, int CI_, int OCT_, int PBW_, int OBW_, bool DGRAD_, int OCC_, int NBUF_ = 2, int S_ = 1, int FS_ = 3>
+// PGS_ > 1 (single-chunk configurations only): a wave finishes its pixel blocks in PGS groups, one after the other, and
+// stores each group as soon as it is complete, so the stores of all groups but the last overlap the MFMAs of the next.
+template <int W_, int ROWS_, int CI_, int OCT_, int PBW_, int OBW_, bool DGRAD_, int OCC_, int NBUF_ = 2, int S_ = 1, int FS_ = 3, int PGS_ = 1>
 struct DirectCfg {
     static constexpr int W = W_, ROWS = ROWS_, CI = CI_, OCT = OCT_, PBW = PBW_, OBW = OBW_, OCC = OCC_, NBUF = NBUF_, S = S_;
     static constexpr int FS = FS_, NT = FS_ * FS_;  // filter size, taps
+    static constexpr int PGS = PGS_, PGC = PBW_ / PGS_;  // pixel-block groups per wave, blocks per group
     static constexpr bool DGRAD = DGRAD_;
     // W = 4: the grid is a 4x4 image and a tile is ROWS / 4 whole images stacked, each staged with its own halo rows
     static constexpr bool MI = W_ == 4;
@@ -65,7 +70,6 @@ struct DirectCfg {
     static constexpr int NSTEP = CI * NT / 4;     // MFMA steps per chunk
     static constexpr int CQ = CI / 4;             // steps per tap
     static constexpr int MPS = PBW * OBW;         // MFMAs per step
-    static constexpr int PF = (8 / MPS) < 1 ? 1 : ((8 / MPS) > 4 ? 4 : (8 / MPS));  // read-ahead (steps)
     static constexpr int CIP = CI + 1;            // k index of (tap, channel) in a filter row is tap*CIP + channel: odd tap stride
     static constexpr int WSTR_MIN = NT * CIP;      // filter row stride == 2 mod 4: the 32 lanes of a half-wave (16 rows x 2 k) hit distinct banks
     static constexpr int WSTR = WSTR_MIN + ((2 - WSTR_MIN % 4) + 4) % 4;
@@ -78,6 +82,7 @@ struct DirectCfg {
     static_assert(TP % 16 == 0 && NPB % PBW == 0 && NOB % OBW == 0 && NPBW * NOBW == 4, "wave tiling must use 4 waves");
     static_assert((PBW * 16) % W == 0 || PBW == 1, "a wave's pixel blocks must start on a row boundary");
     static_assert(CI % 4 == 0, "chunk channel count");
+    static_assert(PBW % PGS == 0 && (PGS == 1 || NBUF == 1), "pixel groups need a single-chunk configuration");
 
     // LDS offset of tap (fh, fw) relative to the lane's pixel base (which points one float left of the pixel)
     static constexpr int tap_off(int tap) {
@@ -220,15 +225,18 @@ __global__ void __launch_bounds__(kThreads, Cfg::OCC) conv3x3_kernel(DirectArgs 
 #pragma unroll
             for (int o = 0; o < OBW; ++o) acc[ph][p][o] = v4f{0.f, 0.f, 0.f, 0.f};
 
-    constexpr int PF = Cfg::PF, CQ = Cfg::CQ;
-    auto compute = [&](const float *cx, const float *cw) {
+    constexpr int CQ = Cfg::CQ;
+    // MFMAs of one chunk for the pixel blocks [P0, P0 + PC) of this wave
+    auto compute = [&](const float *cx, const float *cw, auto p0c, auto pcc) {
+        constexpr int P0 = decltype(p0c)::value, PC = decltype(pcc)::value;
+        constexpr int MPS = PC * OBW, PF = (8 / MPS) < 1 ? 1 : ((8 / MPS) > 4 ? 4 : (8 / MPS));  // read-ahead (steps)
         const float *px = cx + xbase, *pw = cw + wbase;
-        float av[PF + 1][PBW], bv[PF + 1][OBW];
+        float av[PF + 1][PC], bv[PF + 1][OBW];
         auto read_step = [&](int s, int slot) {
             const int tap = s / CQ, cq = s % CQ;
             const int xo = cq * 4 * XP + Cfg::tap_off(tap);
 #pragma unroll
-            for (int p = 0; p < PBW; ++p) av[slot][p] = px[xo + Cfg::pix_off(p * 16)];
+            for (int p = 0; p < PC; ++p) av[slot][p] = px[xo + Cfg::pix_off((P0 + p) * 16)];
 #pragma unroll
             for (int o = 0; o < OBW; ++o) bv[slot][o] = pw[o * 16 * WSTR + tap * Cfg::CIP + 4 * cq];
         };
@@ -240,11 +248,50 @@ __global__ void __launch_bounds__(kThreads, Cfg::OCC) conv3x3_kernel(DirectArgs 
             __builtin_amdgcn_sched_barrier(0);
             const int ph = Cfg::tap_phase(s / CQ);
 #pragma unroll
-            for (int p = 0; p < PBW; ++p)
+            for (int p = 0; p < PC; ++p)
 #pragma unroll
                 for (int o = 0; o < OBW; ++o)
-                    acc[ph][p][o] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[s % (PF + 1)][p], bv[s % (PF + 1)][o], acc[ph][p][o], 0, 0, 0);
+                    acc[ph][P0 + p][o] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[s % (PF + 1)][p], bv[s % (PF + 1)][o], acc[ph][P0 + p][o], 0, 0, 0);
             __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+    using std::integral_constant;
+    typedef integral_constant<int, 0> AllP0;
+    typedef integral_constant<int, PBW> AllPC;
+
+    // ---- epilogue for the pixel blocks [p_lo, p_lo + p_cnt): a lane holds 4 consecutive grid pixels of one output channel ----
+    auto store = [&](int p_lo, int p_cnt) {
+#pragma unroll
+        for (int o = 0; o < OBW; ++o) {
+            const u32 oc = oc0 + (wo * OBW + o) * 16 + li;
+            if (oc >= a.C_OUT) continue;
+            const float b = a.bias ? a.bias[oc] : 0.f;
+#pragma unroll
+            for (int p = 0; p < PBW; ++p) {
+                if (p < p_lo || p >= p_lo + p_cnt) continue;
+                const int q = (wp * PBW + p) * 16 + 4 * kq;
+                const u32 gy = Cfg::MI ? u32((q % 16) / 4) : u32(r0 + q / W), gx = u32(q % W);
+                const u32 img = Cfg::MI ? n + u32(q / 16) : n;
+                if (Cfg::MI && img >= a.n_images) continue;
+                if constexpr (Cfg::DG2) {
+                    // grid pixel (gy, gx..gx+3) -> dX rows 2gy, 2gy+1, columns 2gx .. 2gx+7 (column parities interleaved)
+                    float *base = a.Y + ((size_t(n) * a.C_OUT + oc) * (2 * a.grid_H) + 2 * gy) * (2 * W) + 2 * gx;
+#pragma unroll
+                    for (int py = 0; py < 2; ++py) {
+                        const v4f e = acc[2 * py][p][o], d = acc[2 * py + 1][p][o];  // px = 0, px = 1
+                        *reinterpret_cast<v4f *>(base + py * 2 * W) = v4f{e.x, d.x, e.y, d.y};
+                        *reinterpret_cast<v4f *>(base + py * 2 * W + 4) = v4f{e.z, d.z, e.w, d.w};
+                    }
+                } else {
+                    v4f v = acc[0][p][o];
+                    v.x += b, v.y += b, v.z += b, v.w += b;
+                    if (a.relu) {
+                        v.x = v.x > 0.f ? v.x : 0.f, v.y = v.y > 0.f ? v.y : 0.f;
+                        v.z = v.z > 0.f ? v.z : 0.f, v.w = v.w > 0.f ? v.w : 0.f;
+                    }
+                    *reinterpret_cast<v4f *>(a.Y + ((size_t(img) * a.C_OUT + oc) * a.grid_H + gy) * W + gx) = v;
+                }
+            }
         }
     };
 
@@ -252,56 +299,36 @@ __global__ void __launch_bounds__(kThreads, Cfg::OCC) conv3x3_kernel(DirectArgs 
     fetch(0);
     commit(sX[0], sW[0]);
     __syncthreads();
-    if constexpr (NBUF == 1) {
-        compute(sX[0], sW[0]);
+    if constexpr (NBUF == 1 && Cfg::PGS > 1) {
+        // group by group: the stores of a finished group drain while the next group's MFMAs run
+        auto group = [&](auto g) {
+            constexpr int G = decltype(g)::value;
+            compute(sX[0], sW[0], integral_constant<int, G * Cfg::PGC>{}, integral_constant<int, Cfg::PGC>{});
+            store(G * Cfg::PGC, Cfg::PGC);
+        };
+        group(integral_constant<int, 0>{});
+        if constexpr (Cfg::PGS > 1) group(integral_constant<int, 1>{});
+        if constexpr (Cfg::PGS > 2) group(integral_constant<int, 2>{});
+        if constexpr (Cfg::PGS > 3) group(integral_constant<int, 3>{});
+        return;
+    } else if constexpr (NBUF == 1) {
+        compute(sX[0], sW[0], AllP0{}, AllPC{});
     } else {
         const u32 nchunk = (a.C_IN + CI - 1) / CI;
         for (u32 ch = 0; ch < nchunk; ++ch) {
             const bool more = ch + 1 < nchunk;
             if (more) fetch((ch + 1) * CI);
             if (ch & 1) {
-                compute(sX[NBUF - 1], sW[NBUF - 1]);
+                compute(sX[NBUF - 1], sW[NBUF - 1], AllP0{}, AllPC{});
                 if (more) commit(sX[0], sW[0]);
             } else {
-                compute(sX[0], sW[0]);
+                compute(sX[0], sW[0], AllP0{}, AllPC{});
                 if (more) commit(sX[NBUF - 1], sW[NBUF - 1]);
             }
             __syncthreads();
         }
     }
-
-    // ---- epilogue: a lane holds 4 consecutive grid pixels of one output channel per tile ----------------------
-#pragma unroll
-    for (int o = 0; o < OBW; ++o) {
-        const u32 oc = oc0 + (wo * OBW + o) * 16 + li;
-        if (oc >= a.C_OUT) continue;
-        const float b = a.bias ? a.bias[oc] : 0.f;
-#pragma unroll
-        for (int p = 0; p < PBW; ++p) {
-            const int q = (wp * PBW + p) * 16 + 4 * kq;
-            const u32 gy = Cfg::MI ? u32((q % 16) / 4) : u32(r0 + q / W), gx = u32(q % W);
-            const u32 img = Cfg::MI ? n + u32(q / 16) : n;
-            if (Cfg::MI && img >= a.n_images) continue;
-            if constexpr (Cfg::DG2) {
-                // grid pixel (gy, gx..gx+3) -> dX rows 2gy, 2gy+1, columns 2gx .. 2gx+7 (column parities interleaved)
-                float *base = a.Y + ((size_t(n) * a.C_OUT + oc) * (2 * a.grid_H) + 2 * gy) * (2 * W) + 2 * gx;
-#pragma unroll
-                for (int py = 0; py < 2; ++py) {
-                    const v4f e = acc[2 * py][p][o], d = acc[2 * py + 1][p][o];  // px = 0, px = 1
-                    *reinterpret_cast<v4f *>(base + py * 2 * W) = v4f{e.x, d.x, e.y, d.y};
-                    *reinterpret_cast<v4f *>(base + py * 2 * W + 4) = v4f{e.z, d.z, e.w, d.w};
-                }
-            } else {
-                v4f v = acc[0][p][o];
-                v.x += b, v.y += b, v.z += b, v.w += b;
-                if (a.relu) {
-                    v.x = v.x > 0.f ? v.x : 0.f, v.y = v.y > 0.f ? v.y : 0.f;
-                    v.z = v.z > 0.f ? v.z : 0.f, v.w = v.w > 0.f ? v.w : 0.f;
-                }
-                *reinterpret_cast<v4f *>(a.Y + ((size_t(img) * a.C_OUT + oc) * a.grid_H + gy) * W + gx) = v;
-            }
-        }
-    }
+    store(0, PBW);
 }
 
 // Shape gate of one configuration. Channel counts need not divide CI / OCT: ragged chunks and tiles are zero-filled.

@@ -114,7 +114,7 @@ static int try_direct(const float *Wt, const float *X, float *Y, const float *bi
     // stride 1 when C_IN > 8, chunks of 8 otherwise (stride 2 stages wider / more rows per chunk)
     if constexpr (S == 1) {
         if (gW == 32) {
-            if (C_IN <= 16 && C_IN > 8 && C_OUT <= 16) { CRB_TRY(32, 8, 16, 16, 4, 1, DG, 2, 1, 1) }  // one LDS-resident chunk
+            if (C_IN <= 16 && C_IN > 8 && C_OUT <= 16) { CRB_TRY(32, 8, 16, 16, 4, 1, DG, 2, 1, 1, 3, 4) }  // one LDS-resident chunk
             if (C_OUT > 32) { CRB_TRY(32, 8, 8, 64, 4, 4, DG, 2, 2, 1) }
             if (C_OUT > 16) { CRB_TRY(32, 8, 8, 32, 4, 2, DG, 2, 2, 1) }
             CRB_TRY(32, 8, 8, 16, 4, 1, DG, 2, 2, 1)
