@@ -1,7 +1,10 @@
 // seann::NetParam — a trainable Parameter (weights or biases) paired with its optimizer, as the operands hold it
 // (seann/containers/NetParam.cuh:20-56). `info` may be null (no optimizer: update() is then a no-op), which is how
-// the operands are used when only forward / gradients are wanted.
+// the operands are used when only forward / gradients are wanted. The encode / decode members move the tensor between
+// device memory and a model file (NetParam.cuh:45-102) with one device copy per tensor instead of one per 400 values.
 #pragma once
+#include <fstream>
+
 #include "../optimizers/Optimizers.h"
 
 namespace seann {
@@ -35,6 +38,10 @@ public:
     void batchUpdate() const {
         if (opt) opt->batchApply();
     }
+    uint32 encodeNetParamInfo(std::fstream *fout, uint64 offset) const;  // dims n, c, h, w: 16 bytes
+    uint32 encodeNetParamData(std::fstream *fout, uint64 offset) const;  // raw float32 values
+    static NetParam *decodeNetParamInfo(std::fstream *fin, uint64 &offset, OptimizerInfo *info);
+    static NetParam *decodeNetParamData(std::fstream *fin, uint64 &offset, NetParam *param);
     Tensor *data() const { return A->A; }
     Tensor *grad() const { return A->dA; }
     void zeroGrad() const { A->dA->constFill(0); }

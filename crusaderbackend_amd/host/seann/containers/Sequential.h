@@ -1,6 +1,6 @@
 // seann::Sequential — the linear container that owns the operand list, wires each operand's input to its predecessor's
-// output and drives forward / backward / update (seann/containers/Sequential.{cuh,cu}). Dataset-driven `train`,
-// checkpointing and logging are outside this build.
+// output and drives forward / backward / update (seann/containers/Sequential.{cuh,cu}). Dataset-driven `train` and logging are
+// outside this build; seio::saveSequence / loadSequence write and read a network's model file.
 #pragma once
 #include <initializer_list>
 #include <vector>

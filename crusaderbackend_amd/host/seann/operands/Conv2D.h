@@ -42,5 +42,12 @@ public:
         if (WITH_BIAS) out.push_back(bias);
     }
     uint32 OPERAND_ID() override { return OPR_SEBLAS_CONV2D; }
+    // info: filter dims, strides, paddings, has-bias flag (36 bytes); params: filter, then bias (Conv2D.cu:59-80)
+    uint32 encodeInfo(std::fstream *fout, uint64 offset) override;
+    uint32 encodeNetParams(std::fstream *fout, uint64 offset) override;
+    uint32 getInfoEncodingSize() override { return sizeof(uint32) * 9; }
+    uint32 getNetParamsEncodingSize() override {
+        return uint32((filter->data()->dims.size + (WITH_BIAS ? bias->data()->dims.size : 0)) * sizeof(float));
+    }
 };
 }  // namespace seann

@@ -58,6 +58,8 @@ public:
         maxPoolBack(X->dA, Y->dA, record, strideH, strideW, rangeH, rangeW);
     }
     uint32 OPERAND_ID() override { return OPR_SEBLAS_MAXPOOL2D; }
+    uint32 encodeInfo(std::fstream *fout, uint64 offset) override;  // strides, ranges (MaxPool2D.cu:22-29)
+    uint32 getInfoEncodingSize() override { return sizeof(uint32) * 4; }
 };
 
 // Batch normalisation with per-feature statistics and trainable beta / gamma of one sample's shape
@@ -118,6 +120,10 @@ public:
         out.push_back(gamma);
     }
     uint32 OPERAND_ID() override { return OPR_SEBLAS_BATCHNORM; }
+    uint32 encodeNetParams(std::fstream *fout, uint64 offset) override;  // beta, then gamma (BatchNorm.cu:50-55)
+    uint32 getNetParamsEncodingSize() override {
+        return uint32(sizeof(float) * (beta->data()->dims.size + gamma->data()->dims.size));
+    }
 };
 
 // Output probabilities; the loss function writes Y->dA = Y->A - labels, which is already the gradient with respect to

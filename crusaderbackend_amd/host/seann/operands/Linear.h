@@ -39,5 +39,12 @@ public:
         out.push_back(biases);
     }
     uint32 OPERAND_ID() override { return OPR_SEBLAS_LINEAR; }
+    // info: OUTPUT_SIZE; params: weights, then biases (Linear.cu:62-75)
+    uint32 encodeInfo(std::fstream *fout, uint64 offset) override;
+    uint32 encodeNetParams(std::fstream *fout, uint64 offset) override;
+    uint32 getInfoEncodingSize() override { return sizeof(uint32); }
+    uint32 getNetParamsEncodingSize() override {
+        return uint32(sizeof(float) * (weights->data()->dims.size + biases->data()->dims.size));
+    }
 };
 }  // namespace seann

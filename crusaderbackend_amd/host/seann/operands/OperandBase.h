@@ -1,7 +1,8 @@
 // seann::OperandBase — the operand plugin interface of the reference (seann/operands/OperandBase.cuh:16-108):
-// forward / xGrads / paramGrads, parameter initialisation, optimizer application and graph wiring. Checkpoint
-// encoding is outside this build.
+// forward / xGrads / paramGrads, parameter initialisation, optimizer application, graph wiring and the operand's records
+// in a model file.
 #pragma once
+#include <fstream>
 #include <string>
 #include <vector>
 
@@ -36,6 +37,14 @@ public:
     virtual void zeroGrads() = 0;
     virtual std::string info() = 0;
     virtual uint32 OPERAND_ID() { return 0x0000; }
+
+    // Model-file records (OperandBase.cuh:102-108): the construction arguments ("info") and the trainable tensors
+    // ("net params") written at byte `offset` of the stream; each returns the number of bytes it wrote. Operands without
+    // arguments or parameters write nothing.
+    virtual uint32 encodeInfo(std::fstream *, uint64) { return 0; }
+    virtual uint32 encodeNetParams(std::fstream *, uint64) { return 0; }
+    virtual uint32 getInfoEncodingSize() { return 0; }
+    virtual uint32 getNetParamsEncodingSize() { return 0; }
 
     virtual void collectNetParams(std::vector<NetParam *> &) {}  // every trainable parameter, for a fused update
     virtual void pruneReserveFolds() { foldReserveEnabled = reserveWriters > 0; }

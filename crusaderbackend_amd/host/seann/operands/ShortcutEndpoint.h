@@ -28,6 +28,16 @@ public:
         if (isContainer) branchOperands.assign(operands.begin(), operands.end());
         operandCount = uint32(branchOperands.size());
     }
+    ShortcutEndpoint(bool isContainer, uint32 uuid, const std::vector<OperandBase *> &operands) : isContainer(isContainer), uuid(uuid) {
+        if (isContainer) branchOperands = operands;
+        operandCount = uint32(branchOperands.size());
+    }
+    ShortcutEndpoint(bool isContainer, uint32 uuid, OperandBase **operands, uint32 operandCount)
+        : ShortcutEndpoint(isContainer, uuid, std::vector<OperandBase *>(operands, operands + operandCount)) {}
+
+    // Set once the branch operands own their tensors (a model file's decoder creates and fills them before the chain is
+    // bound); postWaiveInit then binds them without creating them again.
+    bool branchInitialised = false;
 
     void initNetParams(OptimizerInfo *info, shape4 inShape) override;
     void postWaiveInit(OptimizerInfo *info) override;
@@ -47,5 +57,11 @@ public:
     }
     std::string info() override { return "ShortcutEndpoint { " + std::to_string(operandCount) + " }"; }
     uint32 OPERAND_ID() override { return isContainer ? OPR_CTRL_SHORTCUTENDPOINT_END : OPR_CTRL_SHORTCUTENDPOINT_BEG; }
+    // info: uuid, branch operand count, then for a closing endpoint the branch's type ids and infos; params: the branch's
+    // (ShortcutEndpoint.cu:151-177)
+    uint32 encodeInfo(std::fstream *fout, uint64 offset) override;
+    uint32 encodeNetParams(std::fstream *fout, uint64 offset) override;
+    uint32 getInfoEncodingSize() override;
+    uint32 getNetParamsEncodingSize() override;
 };
 }  // namespace seann

@@ -99,8 +99,13 @@ void ShortcutEndpoint::postWaiveInit(OptimizerInfo *inf) {  // :13-55
         other = static_cast<ShortcutEndpoint *>(tracer);
         other->reserveWriters++;  // identity: this endpoint's xGrads copies into it; projection: the branch's input gradient is it
         if (operandCount > 0) {
-            branchOperands[0]->initNetParams(inf, other->Y->A->dims);
-            for (uint32 i = 1; i < operandCount; i++) branchOperands[i]->initNetParams(inf, branchOperands[i - 1]->Y->A->dims);
+            if (!branchInitialised) {
+                branchOperands[0]->initNetParams(inf, other->Y->A->dims);
+                for (uint32 i = 1; i < operandCount; i++) branchOperands[i]->initNetParams(inf, branchOperands[i - 1]->Y->A->dims);
+                branchInitialised = true;
+            } else if (!(branchOperands[0]->X->A->dims == other->Y->A->dims)) {
+                throw std::invalid_argument("ShortcutEndpoint: branch was created for another input shape");
+            }
             if (!(branchOperands[operandCount - 1]->Y->A->dims == Y->A->dims))
                 throw std::invalid_argument("ShortcutEndpoint: branch output shape differs from the main path");
             branchOperands[0]->bindPrev(other);

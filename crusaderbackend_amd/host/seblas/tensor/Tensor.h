@@ -10,6 +10,7 @@
 
 namespace seblas {
 typedef uint32_t uint32;
+typedef uint64_t uint64;
 
 struct index4 {
     uint32 n = 0, c = 0, h = 0, w = 0;

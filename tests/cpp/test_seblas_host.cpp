@@ -1,12 +1,14 @@
 // Host-side tests of the C++ seblas / seann layer. Mode "host" needs no GPU (shape rules, exact division helper,
 // shape-error translation, which all happen before any device work). Mode "gpu" drives the reference-shaped API
 // end to end on the device — Tensor::create / copy / seblas::conv ... / seann::Conv2D, Linear — and checks results
-// against the CPU oracle (linked here as the checker only).
+// against the CPU oracle (linked here as the checker only). Mode "codec <dir>" writes, reads back and re-writes model
+// files in <dir> for the Python test that checks their bytes against the file-format restatement.
 #include <hip/hip_runtime_api.h>
 
 #include <cmath>
 #include <cstdio>
 #include <cstring>
+#include <fstream>
 #include <random>
 #include <stdexcept>
 #include <vector>
@@ -17,6 +19,7 @@
 #include "../../crusaderbackend_amd/host/seann/operands/Elementwise.h"
 #include "../../crusaderbackend_amd/host/seann/operands/Linear.h"
 #include "../../crusaderbackend_amd/host/seann/operands/ShortcutEndpoint.h"
+#include "../../crusaderbackend_amd/host/seio/modelcache/codec.h"
 
 extern "C" {
 void oracle_sgemm(const float *, const float *, float *, uint32_t, uint32_t, uint32_t, uint32_t, int);
@@ -521,9 +524,143 @@ static void gpu_sequential_tests() {
     CHECK(throws_invalid([&] { Sequential bad(shape4(1, 3, 8, 8), {new ShortcutEndpoint(true, 9, {})}); bad.construct(nullptr); }));
 }
 
+// ---- model files -------------------------------------------------------------------------------------------------------
+static void dump(const std::string &path, const std::vector<float> &v) {
+    std::ofstream f(path, std::ios::binary | std::ios::trunc);
+    f.write(reinterpret_cast<const char *>(v.data()), std::streamsize(v.size() * sizeof(float)));
+}
+
+static std::vector<float> slurp(const std::string &path) {
+    std::ifstream f(path, std::ios::binary | std::ios::ate);
+    std::vector<float> v(size_t(f.tellg()) / sizeof(float));
+    f.seekg(0);
+    f.read(reinterpret_cast<char *>(v.data()), std::streamsize(v.size() * sizeof(float)));
+    return v;
+}
+
+static bool file_exists(const std::string &path) { return bool(std::ifstream(path)); }
+
+static std::vector<float> all_params(const seann::Sequential &net) {
+    std::vector<seann::NetParam *> ps;
+    for (auto *op : net.operands) op->collectNetParams(ps);
+    std::vector<float> out;
+    for (auto *p : ps) {
+        auto v = pull(p->data());
+        out.insert(out.end(), v.begin(), v.end());
+    }
+    return out;
+}
+
+// A network with every operand type the file format carries here: saved, loaded, and the loaded copy must compute and
+// train exactly like the original. Files are left in `dir` for the byte-level check.
+static void codec_tests(const std::string &dir) {
+    using namespace seann;
+    const uint32_t N = 4;
+    auto build = [&] {
+        return new Sequential(shape4(N, 3, 8, 8),
+                              {new Conv2D(shape4(8, 3, 3, 3), 1, 1, 1, 1, true), new BatchNorm(), new ReLU(), new MaxPool2D(2, 2, 2, 2),
+                               new ShortcutEndpoint(false, 1, {}), new Conv2D(shape4(8, 8, 3, 3), 1, 1, 1, 1, false), new BatchNorm(),
+                               new ShortcutEndpoint(true, 1, {}), new ReLU(),
+                               new ShortcutEndpoint(false, 2, {}), new Conv2D(shape4(16, 8, 3, 3), 2, 2, 1, 1, true),
+                               new ShortcutEndpoint(true, 2, {new Conv2D(shape4(16, 8, 1, 1), 2, 2, 0, 0, false), new BatchNorm()}),
+                               new ReLU(), new Linear(10), new Softmax()});
+    };
+    OPTIMIZER_MOMENTUM opt(0.05f, 0.9f);
+    Sequential *net = build();
+    net->construct(&opt);
+    net->setLoss(crossEntropyLoss, crossEntropyCalc);
+    net->randInit();
+    {  // batch-norm parameters away from their 0 / 1 start so that their order in the file matters
+        std::vector<NetParam *> ps;
+        for (auto *op : net->operands) op->collectNetParams(ps);
+        uint32_t seed = 900;
+        for (auto *op : net->operands) {
+            auto give = [&](BatchNorm *bn) {
+                auto b = randn(bn->beta->data()->dims.size, seed++, 0.3f), g = randn(bn->gamma->data()->dims.size, seed++, 0.2f);
+                for (auto &v : g) v += 1.0f;
+                CHECK(hipMemcpy(bn->beta->data()->elements, b.data(), b.size() * 4, hipMemcpyHostToDevice) == hipSuccess);
+                CHECK(hipMemcpy(bn->gamma->data()->elements, g.data(), g.size() * 4, hipMemcpyHostToDevice) == hipSuccess);
+            };
+            if (auto *bn = dynamic_cast<BatchNorm *>(op)) give(bn);
+            if (auto *se = dynamic_cast<ShortcutEndpoint *>(op))
+                for (auto *b : se->branchOperands)
+                    if (auto *bn = dynamic_cast<BatchNorm *>(b)) give(bn);
+        }
+    }
+    auto x = randn(N * 3 * 8 * 8, 77);
+    std::vector<float> lab(N * 10, 0.f);
+    for (uint32_t n = 0; n < N; ++n) lab[n * 10 + (7 * n + 2) % 10] = 1.f;
+    Tensor *X = push(shape4(N, 3, 8, 8), x), *L = push(shape4(N, 1, 10, 1), lab);
+
+    const std::string fa = dir + "/a.crseq";
+    seio::saveSequence(fa.c_str(), net, 17);
+    dump(dir + "/a.params.f32", all_params(*net));
+    auto y1 = pull(net->forward(X));
+    dump(dir + "/a.x.f32", x);
+    dump(dir + "/a.y.f32", y1);
+
+    CHECK(seio::loadedEpochID(fa.c_str()) == 17);
+    Sequential *twin = seio::loadSequence(fa.c_str(), shape4(N, 3, 8, 8), &opt);
+    twin->setLoss(crossEntropyLoss, crossEntropyCalc);
+    CHECK(twin->OPERAND_COUNT == net->OPERAND_COUNT);
+    CHECK(all_params(*twin) == all_params(*net));
+    auto y2 = pull(twin->forward(X));
+    CHECK(y1 == y2);  // same kernels on the same values: identical bits
+    // one training step on both: the loaded network is wired for backward and update as well
+    net->backward(L), net->learn();
+    twin->forward(X), twin->backward(L), twin->learn();
+    CHECK(all_params(*twin) == all_params(*net));
+    CHECK(pull(net->forward(X)) == pull(twin->forward(X)));
+    // a second save of an unchanged network replaces the file with the same bytes
+    const std::string fa2 = dir + "/a2.crseq";
+    seio::saveSequence(fa2.c_str(), twin, 18);
+    seio::saveSequence(fa2.c_str(), twin, 18);
+    dump(dir + "/a2.params.f32", all_params(*twin));
+
+    // a file written by the format restatement: load, run, write again
+    const std::string fb = dir + "/b.crseq";
+    if (file_exists(fb)) {
+        auto shp = slurp(dir + "/b.shape.f32");  // n, c, h, w
+        shape4 in = shape4((uint32_t)shp[0], (uint32_t)shp[1], (uint32_t)shp[2], (uint32_t)shp[3]);
+        Sequential *b = seio::loadSequence(fb.c_str(), in, nullptr);
+        Tensor *BX = push(in, slurp(dir + "/b.x.f32"));
+        dump(dir + "/b.y.f32", pull(b->forward(BX)));
+        seio::saveSequence((dir + "/b2.crseq").c_str(), b, seio::loadedEpochID(fb.c_str()));
+    }
+
+    // malformed files are reported, not followed
+    auto throws_runtime = [&](const std::string &path) {
+        try {
+            seio::loadSequence(path.c_str(), shape4(N, 3, 8, 8), nullptr);
+        } catch (const std::runtime_error &) {
+            return true;
+        } catch (...) {
+            return false;
+        }
+        return false;
+    };
+    CHECK(throws_runtime(dir + "/does_not_exist.crseq"));
+    {
+        std::ifstream src(fa, std::ios::binary);
+        std::vector<char> bytes((std::istreambuf_iterator<char>(src)), std::istreambuf_iterator<char>());
+        std::ofstream(dir + "/truncated.crseq", std::ios::binary).write(bytes.data(), std::streamsize(bytes.size() - 40));
+        bytes[0] ^= 1;
+        std::ofstream(dir + "/badmagic.crseq", std::ios::binary).write(bytes.data(), std::streamsize(bytes.size()));
+    }
+    CHECK(throws_runtime(dir + "/truncated.crseq"));
+    CHECK(throws_runtime(dir + "/badmagic.crseq"));
+}
+
 int main(int argc, char **argv) {
     const bool gpu = argc > 1 && std::strcmp(argv[1], "gpu") == 0;
+    const bool codec = argc > 2 && std::strcmp(argv[1], "codec") == 0;
     try {
+        if (codec) {
+            setBlocking(true);
+            codec_tests(argv[2]);
+            std::printf("codec: %s\n", g_fail ? "FAILED" : "OK");
+            return g_fail ? 1 : 0;
+        }
         if (gpu) {
             gpu_tests();
             gpu_elementwise_tests();
