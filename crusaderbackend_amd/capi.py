@@ -75,6 +75,8 @@ SIGNATURES = {
     "crb_batchnorm_bwd": (ctypes.c_int, [_ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _u32, _u32, _ptr]),
     "crb_batchnorm_param_grads": (ctypes.c_int, [_ptr, _ptr, _ptr, _ptr, _u32, _u32, _ptr]),
     "crb_momentum_apply": (ctypes.c_int, [_ptr, _ptr, _ptr, _u32, ctypes.c_float, ctypes.c_float, ctypes.c_float, _ptr]),
+    "crb_images_from_bytes": (ctypes.c_int, [_ptr, _ptr, _u32, _u32, _u32, _u32, ctypes.c_int, ctypes.c_float, ctypes.c_float,
+                                             _ptr, _ptr]),
 }
 
 _lib = None
@@ -273,3 +275,25 @@ def tensor_add_clear_copy(dst, a, b, count, stream=None):
 
 def tensor_copy2(dst1, dst2, src, count, stream=None):
     check(load().crb_tensor_copy2(_p(dst1), _p(dst2), _p(src), count, _stream(stream)))
+
+
+NORM_NONE, NORM_UNIFORM, NORM_DISTRIBUTION = 0, 1, 2
+AUG_MIRROR, AUG_SHIFT = 1, 2
+
+
+class ImageAug(ctypes.Structure):
+    """Mirror of ``crb_image_aug``."""
+
+    _fields_ = [("dh", ctypes.c_int32), ("dw", ctypes.c_int32), ("flags", _u32)]
+
+
+def image_aug_table(torch, dev, entries):
+    """entries: (dh, dw, flags) per image -> device byte tensor holding the records."""
+    arr = (ImageAug * len(entries))()
+    for i, (dh, dw, flags) in enumerate(entries):
+        arr[i] = ImageAug(dh, dw, flags)
+    return torch.frombuffer(bytearray(bytes(arr)), dtype=torch.uint8).to(dev)
+
+
+def images_from_bytes(src, dst, images, channels, H, W, norm=NORM_NONE, p0=0.0, p1=1.0, aug=None, stream=None):
+    check(load().crb_images_from_bytes(_p(src), _p(dst), images, channels, H, W, norm, p0, p1, _p(aug), _stream(stream)))

@@ -244,6 +244,30 @@ int crb_batchnorm_bwd(const float *dY, const float *gamma, const float *X, float
 int crb_batchnorm_param_grads(const float *dY, const float *xHat, float *dGamma, float *dBeta, uint32_t N, uint32_t F,
                               void *stream);
 
+/* Dataset bytes to network input. src holds `images` images of `channels` planes of H x W byte pixels, as they lie in a
+ * dataset file; dst receives the same images as floats, normalised per image:
+ *   CRB_NORM_NONE          dst = (float) src                                  (seio/data/DataLoader.cu:34-36)
+ *   CRB_NORM_UNIFORM       (x - min) / (max - min) * (p1 - p0) + p0, p0 = desiredMin, p1 = desiredMax, with the extrema
+ *                          of channel k taken over channels 0..k of the image, as UniformNorm::apply computes them
+ *                          (seio/data/DataTransform.cu:29-44)
+ *   CRB_NORM_DISTRIBUTION  (x - mean) * p1 / sqrt(var + 1e-8) + p0, p0 = desiredMean, p1 = desiredVar, per channel,
+ *                          biased variance (DistribNorm::apply, DataTransform.cu:7-27)
+ * aug_on_device, when not null, holds one record per image (device memory): with CRB_AUG_MIRROR the image is mirrored
+ * along its width (the effect RandFlipW::apply is written for, seio/data/DataAugmentor.cu:64-104); with CRB_AUG_SHIFT the
+ * output pixel (h, w) is the (mirrored) pixel (h + dh, w + dw) where 0 < h + dh < H and 0 < w + dw < W and 0 elsewhere
+ * (RandCorp::apply, DataAugmentor.cu:26-62, comparisons as written there). Normalisation statistics are those of the
+ * whole stored image, as in the reference, where the transforms run before the augmentations (Dataset.cu:65-72).
+ * Replaces the per-image host loops of Dataset::genBatch (seio/data/Dataset.cu:63-85) and the float upload that follows
+ * them: the batch is uploaded as bytes and converted here. channels <= 64. */
+enum { CRB_NORM_NONE = 0, CRB_NORM_UNIFORM = 1, CRB_NORM_DISTRIBUTION = 2 };
+enum { CRB_AUG_MIRROR = 1, CRB_AUG_SHIFT = 2 };
+typedef struct crb_image_aug {
+    int32_t dh, dw;
+    uint32_t flags;
+} crb_image_aug;
+int crb_images_from_bytes(const uint8_t *src, float *dst, uint32_t images, uint32_t channels, uint32_t H, uint32_t W, int norm,
+                          float p0, float p1, const crb_image_aug *aug_on_device, void *stream);
+
 #ifdef __cplusplus
 }
 #endif
