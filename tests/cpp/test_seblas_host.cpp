@@ -2,7 +2,8 @@
 // shape-error translation, which all happen before any device work). Mode "gpu" drives the reference-shaped API
 // end to end on the device — Tensor::create / copy / seblas::conv ... / seann::Conv2D, Linear — and checks results
 // against the CPU oracle (linked here as the checker only). Mode "codec <dir>" writes, reads back and re-writes model
-// files in <dir> for the Python test that checks their bytes against the file-format restatement.
+// files in <dir> for the Python test that checks their bytes against the file-format restatement. Mode "data <dir>" reads
+// the dataset files the Python test put in <dir> through the seio data pipeline and leaves what it produced there.
 #include <hip/hip_runtime_api.h>
 
 #include <cmath>
@@ -19,6 +20,7 @@
 #include "../../crusaderbackend_amd/host/seann/operands/Elementwise.h"
 #include "../../crusaderbackend_amd/host/seann/operands/Linear.h"
 #include "../../crusaderbackend_amd/host/seann/operands/ShortcutEndpoint.h"
+#include "../../crusaderbackend_amd/host/seio/data/Dataset.h"
 #include "../../crusaderbackend_amd/host/seio/modelcache/codec.h"
 
 extern "C" {
@@ -651,6 +653,143 @@ static void codec_tests(const std::string &dir) {
     CHECK(throws_runtime(dir + "/badmagic.crseq"));
 }
 
+// ---- data pipeline ---------------------------------------------------------------------------------------------------------
+template <class T>
+static std::vector<T> slurp_as(const std::string &path) {
+    std::ifstream f(path, std::ios::binary | std::ios::ate);
+    std::vector<T> v(size_t(f.tellg()) / sizeof(T));
+    f.seekg(0);
+    f.read(reinterpret_cast<char *>(v.data()), std::streamsize(v.size() * sizeof(T)));
+    return v;
+}
+template <class T>
+static void dump_as(const std::string &path, const std::vector<T> &v) {
+    std::ofstream f(path, std::ios::binary | std::ios::trunc);
+    f.write(reinterpret_cast<const char *>(v.data()), std::streamsize(v.size() * sizeof(T)));
+}
+
+// draws come from a file, so that the Python side knows which records a batch holds
+struct ScriptedFetcher : public seio::DataFetcher {
+    std::vector<uint32_t> draws, taken;
+    size_t at = 0;
+    using seio::DataFetcher::DataFetcher;
+    uint32_t draw(uint32_t remaining) override {
+        uint32_t d = draws.at(at++) % remaining;
+        taken.push_back(d);
+        return d;
+    }
+};
+
+static void data_tests(const std::string &dir) {
+    using namespace seio;
+    // dataset of 20 records (3 x 8 x 8 pixels, 10 label values): 16 per epoch + 4 held out
+    const shape4 dataShape(3, 8, 8), labelShape(10, 1);
+    auto *loader = new CrdatLoader();
+    auto *fetcher = new ScriptedFetcher(dir, "set", 16, 4, loader, 1);
+    fetcher->draws = slurp_as<uint32_t>(dir + "/draws.u32");
+
+    // the reference's form of a record: host tensors of floats
+    Tensor *hx = Tensor::createHost(dataShape), *hl = Tensor::createHost(labelShape);
+    loader->loadData(hx, hl, dir.c_str(), "set", 7);
+    dump(dir + "/rec7.x.f32", std::vector<float>(hx->elements, hx->elements + hx->dims.size));
+    dump(dir + "/rec7.label.f32", std::vector<float>(hl->elements, hl->elements + hl->dims.size));
+    bool past_end = false;
+    try {
+        loader->loadData(hx, hl, dir.c_str(), "set", 20);
+    } catch (const std::out_of_range &) {
+        past_end = true;
+    }
+    CHECK(past_end);
+
+    Dataset *set = Dataset::construct(8, 4, 16, 10, dataShape, labelShape, 5);
+    set->setDataFetcher(fetcher);
+    set->setProcSteps({new UniformNorm()});
+    set->setAugmentSteps({new RandFlipW(4, dataShape, labelShape), new RandCorp(4, dataShape, labelShape, 2, 2)});
+    std::vector<uint32_t> order;
+    for (int b = 0; b < 3; b++) {
+        const size_t before = fetcher->taken.size();
+        if (b == 1)
+            set->genBatchAsync().join();
+        else
+            set->genBatch();
+        CHECK(fetcher->taken.size() == before + 8);
+        CHECK(set->batchID == uint32_t(b + 1) && set->epochID == uint32_t((b + 1) * 8 / 16));
+        std::vector<float> x, lab;
+        for (uint32_t i = 0; i < 2; i++) {
+            Data *mb = set->dataBatch[b % 2][i];
+            CHECK(mb->X->dims == shape4(4, 3, 8, 8) && mb->label->dims == shape4(4, 1, 10, 1));
+            auto vx = pull(mb->X), vl = pull(mb->label);
+            x.insert(x.end(), vx.begin(), vx.end());
+            lab.insert(lab.end(), vl.begin(), vl.end());
+        }
+        dump(dir + "/batch" + std::to_string(b) + ".x.f32", x);
+        dump(dir + "/batch" + std::to_string(b) + ".label.f32", lab);
+        std::vector<int32_t> aug;
+        for (const ImageAug &a : set->lastAugmentations()) aug.push_back(a.dh), aug.push_back(a.dw), aug.push_back(int32_t(a.flags));
+        dump_as(dir + "/batch" + std::to_string(b) + ".aug.i32", aug);
+    }
+    dump_as(dir + "/taken.u32", fetcher->taken);
+
+    // a second dataset without transform or augmentation, distribution scaling on a third; seeded random sampling
+    auto *plain = Dataset::construct(4, 2, 16, 1, dataShape, labelShape, 3);
+    auto *f2 = new ScriptedFetcher(dir, "set", 16, 4, new CrdatLoader(), 1);
+    f2->draws = {3, 3, 0, 0};
+    plain->setDataFetcher(f2);
+    plain->genBatch();
+    {
+        std::vector<float> x;
+        for (uint32_t i = 0; i < 2; i++) {
+            auto v = pull(plain->dataBatch[0][i]->X);
+            x.insert(x.end(), v.begin(), v.end());
+        }
+        dump(dir + "/plain.x.f32", x);
+    }
+    auto *dist = Dataset::construct(4, 4, 16, 1, dataShape, labelShape, 3);
+    auto *f3 = new ScriptedFetcher(dir, "set", 16, 4, new CrdatLoader(), 1);
+    f3->draws = {19, 0, 5, 5};
+    dist->setDataFetcher(f3);
+    dist->setProcSteps({new DistribNorm(0.5f, 0.25f)});
+    dist->genBatch();
+    dump(dir + "/dist.x.f32", pull(dist->dataBatch[0][0]->X));
+
+    // sampling without replacement with the built-in generator: the first 20 fetches visit every record once
+    DataFetcher rnd(dir, "set", 16, 4, new CrdatLoader(), 77);
+    std::vector<int> seen(20, 0);
+    for (int i = 0; i < 20; i++) seen[rnd.nextRecord()]++;
+    bool once = true;
+    for (int c : seen) once = once && c == 1;
+    CHECK(once && rnd.remainedData == 16);
+    std::vector<int> seen2(20, 0);
+    for (int i = 0; i < 16; i++) seen2[rnd.nextRecord()]++;
+    bool atmost = true;
+    for (int c : seen2) atmost = atmost && c <= 1;
+    CHECK(atmost);
+
+    // CIFAR-10 binary batches: two files of 6 records
+    CifarBinLoader cifar({dir + "/cifar_1.bin", dir + "/cifar_2.bin"}, 6);
+    Tensor *cx = Tensor::createHost(shape4(3, 32, 32)), *cl = Tensor::createHost(shape4(10, 1));
+    std::vector<float> cxs, cls;
+    for (uint32_t id : {0u, 5u, 6u, 11u, 3u}) {
+        cifar.loadData(cx, cl, "", "", id);
+        cxs.insert(cxs.end(), cx->elements, cx->elements + 3072);
+        cls.insert(cls.end(), cl->elements, cl->elements + 10);
+    }
+    dump(dir + "/cifar.x.f32", cxs);
+    dump(dir + "/cifar.label.f32", cls);
+    bool past = false;
+    try {
+        cifar.loadData(cx, cl, "", "", 12);
+    } catch (const std::out_of_range &) {
+        past = true;
+    }
+    CHECK(past);
+
+    // argument checks
+    CHECK(throws_invalid([&] { Dataset::construct(8, 3, 16, 1, dataShape, labelShape); }));
+    CHECK(throws_invalid([&] { Dataset::construct(32, 4, 16, 1, dataShape, labelShape); }));
+    CHECK(throws_invalid([&] { plain->setProcSteps({new UniformNorm(), new DistribNorm()}); }));
+}
+
 int main(int argc, char **argv) {
     const bool gpu = argc > 1 && std::strcmp(argv[1], "gpu") == 0;
     const bool codec = argc > 2 && std::strcmp(argv[1], "codec") == 0;
@@ -659,6 +798,12 @@ int main(int argc, char **argv) {
             setBlocking(true);
             codec_tests(argv[2]);
             std::printf("codec: %s\n", g_fail ? "FAILED" : "OK");
+            return g_fail ? 1 : 0;
+        }
+        if (argc > 2 && std::strcmp(argv[1], "data") == 0) {
+            setBlocking(true);
+            data_tests(argv[2]);
+            std::printf("data: %s\n", g_fail ? "FAILED" : "OK");
             return g_fail ? 1 : 0;
         }
         if (gpu) {
