@@ -136,6 +136,18 @@ def run(torch, capi, dev, event_time_ms, Layer):
     ew("softmax 128x10", lambda: capi.softmax(A, S, 128, 10), 8.0 * 1280)
     ew("crossEntropyCalc 128x10", lambda: capi.cross_entropy_loss(S, L, None, loss, 1280), 8.0 * 1280)
     del Wt, G, M
+    # dataset bytes -> network input, one batch of the archived CIFAR programs (6400 images): 1 byte read, 4 written per value
+    nimg = 6400
+    raw = torch.randint(0, 256, (nimg, 3, 32, 32), dtype=torch.uint8, device=dev)
+    Xf = torch.empty(nimg, 3, 32, 32, device=dev)
+    aug = capi.image_aug_table(torch, dev, [((i % 9) - 4, ((i // 9) % 9) - 4, i % 4) for i in range(nimg)])
+    nb = 5.0 * raw.numel()
+    ew("bytes->float 6400x3x32x32", lambda: capi.images_from_bytes(raw, Xf, nimg, 3, 32, 32), nb)
+    ew("bytes->float + UniformNorm 6400x3x32x32", lambda: capi.images_from_bytes(raw, Xf, nimg, 3, 32, 32, capi.NORM_UNIFORM, 0.0, 1.0), nb)
+    ew("bytes->float + DistribNorm 6400x3x32x32", lambda: capi.images_from_bytes(raw, Xf, nimg, 3, 32, 32, capi.NORM_DISTRIBUTION, 0.0, 1.0), nb)
+    ew("bytes->float + UniformNorm + mirror/shift 6400x3x32x32",
+       lambda: capi.images_from_bytes(raw, Xf, nimg, 3, 32, 32, capi.NORM_UNIFORM, 0.0, 1.0, aug=aug), nb)
+    del raw, Xf, aug
 
     # config 3 end to end: the whole training step (every operator, real data flow, momentum update), batch 128
     from .vgg16_step import Vgg16Step
