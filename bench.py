@@ -73,6 +73,8 @@ class Layer:
             "dgrad": 4.0 * (self.dY.numel() + self.W.numel() + self.dX.numel()),
             "wgrad": 4.0 * (self.dY.numel() + self.X.numel() + 2 * self.dW.numel()),
         }
+        # both gradients in one call: dY is read by both halves but counted once
+        self.bytes["bwd"] = 4.0 * (self.dY.numel() + self.W.numel() + self.dX.numel() + self.X.numel() + 2 * self.dW.numel())
         self.capi = capi
 
     def fwd(self):
@@ -84,8 +86,13 @@ class Layer:
     def wgrad(self):
         self.capi.conv_wgrad(self.dY, self.X, self.dW, self.g, workspace=self.ws)
 
+    def bwd(self):
+        self.capi.conv_bwd(self.W, self.dY, self.X, self.dX, self.dW, self.g, workspace=self.ws)
+
     def passes(self):
-        return (("fwd", self.fwd), ("dgrad", self.dgrad), ("wgrad", self.wgrad))
+        """(name, call, flops, part of the timed step): the step runs fwd and bwd; dgrad and wgrad alone are listed too."""
+        return (("fwd", self.fwd, self.flops, True), ("bwd", self.bwd, 2 * self.flops, True),
+                ("dgrad", self.dgrad, self.flops, False), ("wgrad", self.wgrad, self.flops, False))
 
 
 # HBM bytes one call moves (read + written, all kernels of the call), from the FETCH_SIZE and WRITE_SIZE hardware
@@ -223,8 +230,7 @@ def main():
                 L.fwd()
         for L in reversed(layers):
             for _ in range(L.mult):
-                L.dgrad()
-                L.wgrad()
+                L.bwd()  # data gradient and weight gradient of the layer in one call
 
     for _ in range(args.warmup):
         step()
@@ -241,11 +247,11 @@ def main():
     # instrumented pass: per-(layer, pass) launch duration with events on the launch stream
     per = {}
     for L in layers:
-        for pname, fn in L.passes():
+        for pname, fn, fl, in_step in L.passes():
             ms = event_time_ms(torch, fn, reps=50)
             per[f"{L.name}.{pname}"] = {
-                "ms": ms, "tflops": L.flops / ms / 1e9, "gbs": L.bytes[pname] / ms / 1e6, "mult": L.mult,
-                "flops": L.flops, "bytes": L.bytes[pname],
+                "ms": ms, "tflops": fl / ms / 1e9, "gbs": L.bytes[pname] / ms / 1e6, "mult": L.mult if in_step else 0,
+                "flops": fl, "bytes": L.bytes[pname],
             }
     dom = max(per, key=lambda k: per[k]["ms"] * per[k]["mult"])
     d = per[dom]
@@ -276,7 +282,8 @@ def main():
         "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32", "data": "synthetic",
         "config": {"workload": "ResNet-56 CIFAR conv shapes, fp32 NCHW, batch 128, 3x3 pad 1: 19x16->16@32, 17x32->32@16, "
-                               "18x64->64@8, 16->32 s2, 32->64 s2; forward + dgrad + wgrad per layer",
+                               "18x64->64@8, 16->32 s2, 32->64 s2; forward + dgrad + wgrad per layer (the two gradients of a layer "
+                               "issued as one crb_conv_bwd call)",
                    "batch": BATCH, "flops_per_step": step_flops},
         "roofline": roofline,
         "extra": {

@@ -51,6 +51,7 @@ SIGNATURES = {
     "crb_conv_dgrad": (ctypes.c_int, [_ptr, _ptr, _ptr, ctypes.POINTER(ConvGeom), _ptr]),
     "crb_conv_wgrad_workspace_bytes": (ctypes.c_size_t, [ctypes.POINTER(ConvGeom)]),
     "crb_conv_wgrad": (ctypes.c_int, [_ptr, _ptr, _ptr, ctypes.POINTER(ConvGeom), _ptr, ctypes.c_size_t, _ptr]),
+    "crb_conv_bwd": (ctypes.c_int, [_ptr, _ptr, _ptr, _ptr, _ptr, ctypes.POINTER(ConvGeom), _ptr, ctypes.c_size_t, _ptr]),
     "crb_conv_bias": (ctypes.c_int, [_ptr, _ptr, _u32, _u32, _u32, _ptr]),
     "crb_conv_bias_grad": (ctypes.c_int, [_ptr, _ptr, _u32, _u32, _u32, _ptr]),
     "crb_tensor_add_inplace": (ctypes.c_int, [_ptr, _ptr, _u32, _ptr]),
@@ -160,6 +161,12 @@ def conv_wgrad_workspace_bytes(geom):
 def conv_wgrad(dY, X, dW, geom, workspace=None, stream=None):
     nbytes = 0 if workspace is None else workspace.numel() * workspace.element_size()
     check(load().crb_conv_wgrad(_p(dY), _p(X), _p(dW), ctypes.byref(geom), _p(workspace), nbytes, _stream(stream)))
+
+
+def conv_bwd(W, dY, X, dX, dW, geom, workspace=None, stream=None):
+    """Data gradient and weight gradient of one layer in one call (one launch for the residual-network layer shapes)."""
+    nbytes = 0 if workspace is None else workspace.numel() * workspace.element_size()
+    check(load().crb_conv_bwd(_p(W), _p(dY), _p(X), _p(dX), _p(dW), ctypes.byref(geom), _p(workspace), nbytes, _stream(stream)))
 
 
 def conv_bias(Y, bias, N, C, HW, stream=None):

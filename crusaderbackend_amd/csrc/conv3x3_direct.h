@@ -75,6 +75,7 @@ struct DirectCfg {
     static constexpr int WSTR = WSTR_MIN + ((2 - WSTR_MIN % 4) + 4) % 4;
     static constexpr int X_SIZE = CI * XP;
     static constexpr int W_SIZE = OCT * WSTR;
+    static constexpr int SMEM_FLOATS = NBUF_ * (X_SIZE + W_SIZE);
     static_assert(W == 4 || W == 8 || W == 16 || W == 32, "grid width");
     static_assert(!MI || (S == 1 && FS == 3 && ROWS % 4 == 0), "stacked 4x4 images: 3x3 stride 1 only");
     static_assert(S == 1 || S == 2, "stride");
@@ -113,18 +114,20 @@ struct DirectArgs {
     u32 relu;
 };
 
+// The work of workgroup `bid` of the grid launch_direct sizes; `smem` = Cfg::SMEM_FLOATS floats of LDS, 16-byte aligned.
+// A device function so that a kernel can run it next to another kind of work in one launch.
 template <class Cfg>
-__global__ void __launch_bounds__(kThreads, Cfg::OCC) conv3x3_kernel(DirectArgs a) {
+__device__ __forceinline__ void conv3x3_body(const DirectArgs &a, const u32 bid, float *smem) {
     constexpr int W = Cfg::W, ROWS = Cfg::ROWS, CI = Cfg::CI, OCT = Cfg::OCT, PBW = Cfg::PBW, OBW = Cfg::OBW;
     constexpr int XS = Cfg::XS, XR = Cfg::XR, XP = Cfg::XP, NSTEP = Cfg::NSTEP, WSTR = Cfg::WSTR, SW = Cfg::SW;
     constexpr int NBUF = Cfg::NBUF, NPH = Cfg::NPH;
-    __shared__ __attribute__((aligned(16))) float sX[NBUF][Cfg::X_SIZE];
-    __shared__ __attribute__((aligned(16))) float sW[NBUF][Cfg::W_SIZE];
+    float(*sX)[Cfg::X_SIZE] = reinterpret_cast<float(*)[Cfg::X_SIZE]>(smem);
+    float(*sW)[Cfg::W_SIZE] = reinterpret_cast<float(*)[Cfg::W_SIZE]>(smem + NBUF * Cfg::X_SIZE);
 
     const u32 t = threadIdx.x;
     // Workgroups are dealt round-robin to the 8 XCDs. Decode the id so that the oc_tiles workgroups that read the same
     // input rows get ids 8 apart: they land on the same XCD, back to back, and share those rows through its L2.
-    const u32 xcd = blockIdx.x % kXcds, slot = blockIdx.x / kXcds;
+    const u32 xcd = bid % kXcds, slot = bid / kXcds;
     const u32 oct = slot % a.oc_tiles;
     const u32 rest = (slot / a.oc_tiles) * kXcds + xcd;
     if (rest >= a.tiles_total) return;
@@ -331,6 +334,12 @@ __global__ void __launch_bounds__(kThreads, Cfg::OCC) conv3x3_kernel(DirectArgs 
     store(0, PBW);
 }
 
+template <class Cfg>
+__global__ void __launch_bounds__(kThreads, Cfg::OCC) conv3x3_kernel(DirectArgs a) {
+    __shared__ __attribute__((aligned(16))) float smem[Cfg::SMEM_FLOATS];
+    conv3x3_body<Cfg>(a, blockIdx.x, smem);
+}
+
 // Shape gate of one configuration. Channel counts need not divide CI / OCT: ragged chunks and tiles are zero-filled.
 // (grid_H, grid_W) = extent of the pixel grid: the output image, or dY for the stride-2 data gradient.
 template <class Cfg>
@@ -339,10 +348,10 @@ inline bool direct_fits(u32 C_IN, u32 grid_H, u32 grid_W) {
     return grid_W == u32(Cfg::W) && grid_H % Cfg::ROWS == 0 && (Cfg::NBUF == 1 ? C_IN <= u32(Cfg::CI) : true);
 }
 
+// Kernel arguments and grid size of one configuration for one call.
 template <class Cfg>
-inline int launch_direct(const float *Wt, const float *X, float *Y, const float *bias, u32 N, u32 C_IN, u32 C_OUT, u32 grid_H,
-                         u32 in_H, u32 relu, hipStream_t s, const char *what) {
-    DirectArgs a;
+inline uint64_t direct_args(DirectArgs &a, const float *Wt, const float *X, float *Y, const float *bias, u32 N, u32 C_IN, u32 C_OUT,
+                            u32 grid_H, u32 in_H, u32 relu) {
     a.Wt = Wt, a.X = X, a.Y = Y, a.bias = bias;
     a.C_IN = C_IN, a.C_OUT = C_OUT, a.grid_H = grid_H, a.in_H = in_H;
     a.tiles_per_img = Cfg::MI ? 1 : grid_H / Cfg::ROWS;
@@ -350,7 +359,14 @@ inline int launch_direct(const float *Wt, const float *X, float *Y, const float 
     a.tiles_total = Cfg::MI ? ceil_div(N, u32(Cfg::IMGS)) : N * a.tiles_per_img;
     a.n_images = N;
     a.relu = relu;
-    const uint64_t wgs = uint64_t(ceil_div(a.tiles_total, kXcds)) * kXcds * a.oc_tiles;  // padded to whole XCD rounds
+    return uint64_t(ceil_div(a.tiles_total, kXcds)) * kXcds * a.oc_tiles;  // padded to whole XCD rounds
+}
+
+template <class Cfg>
+inline int launch_direct(const float *Wt, const float *X, float *Y, const float *bias, u32 N, u32 C_IN, u32 C_OUT, u32 grid_H,
+                         u32 in_H, u32 relu, hipStream_t s, const char *what) {
+    DirectArgs a;
+    const uint64_t wgs = direct_args<Cfg>(a, Wt, X, Y, bias, N, C_IN, C_OUT, grid_H, in_H, relu);
     if (wgs > 0x7fffffffull) return fail(CRB_EINVAL_SHAPE, "%s: launch grid too large", what);
     hipLaunchKernelGGL((conv3x3_kernel<Cfg>), dim3(u32(wgs)), dim3(kThreads), 0, s, a);
     return check_launch(what);

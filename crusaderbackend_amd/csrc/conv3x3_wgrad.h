@@ -72,11 +72,13 @@ struct WgradArgs {
     u32 accumulate;       // add to `out` instead of overwriting (splits == 1)
 };
 
+// The work of workgroup `bid` of the grid launch_wgrad_direct sizes; `smem` = Cfg::SMEM floats of LDS, 16-byte aligned
+// (buffer b: dY planes at b*BUF, X planes after them). A device function so that a kernel can run it next to another
+// kind of work in one launch.
 template <class Cfg>
-__global__ void __launch_bounds__(kThreads, Cfg::OCC) wgrad3x3_kernel(WgradArgs a) {
+__device__ __forceinline__ void wgrad3x3_body(const WgradArgs &a, const u32 bid, float *smem) {
     constexpr int W = Cfg::W, TR = Cfg::TR, TI = Cfg::TI, YP = Cfg::YP, XP = Cfg::XP, NSTEP = Cfg::NSTEP;
     constexpr int YIMG = Cfg::YIMG, XIMG = Cfg::XIMG;
-    __shared__ __attribute__((aligned(16))) float smem[Cfg::SMEM];  // buffer b: dY planes at b*BUF, X planes after them
 
     const u32 t = threadIdx.x;
     // The workgroups of one split z read the same tiles (different channel blocks). With ids 8 apart they run on the
@@ -84,11 +86,11 @@ __global__ void __launch_bounds__(kThreads, Cfg::OCC) wgrad3x3_kernel(WgradArgs 
     // Only done when there are at least 8 splits; with fewer, ids map plainly so every XCD still gets work.
     u32 pair, z;
     if (a.splits >= kXcds) {
-        const u32 xcd = blockIdx.x % kXcds, slot = blockIdx.x / kXcds;
+        const u32 xcd = bid % kXcds, slot = bid / kXcds;
         pair = slot % a.pairs, z = (slot / a.pairs) * kXcds + xcd;
         if (z >= a.splits) return;
     } else {
-        pair = blockIdx.x % a.pairs, z = blockIdx.x / a.pairs;
+        pair = bid % a.pairs, z = bid / a.pairs;
     }
     const u32 ob = pair / a.ic_blocks, ib = pair % a.ic_blocks;
     const u32 HW = a.H * W;                            // dY plane
@@ -277,6 +279,12 @@ __global__ void __launch_bounds__(kThreads, Cfg::OCC) wgrad3x3_kernel(WgradArgs 
     }
 }
 
+template <class Cfg>
+__global__ void __launch_bounds__(kThreads, Cfg::OCC) wgrad3x3_kernel(WgradArgs a) {
+    __shared__ __attribute__((aligned(16))) float smem[Cfg::SMEM];
+    wgrad3x3_body<Cfg>(a, blockIdx.x, smem);
+}
+
 struct WgradDirectPlan {
     u32 pairs, tiles, splits, tiles_per_z;
     size_t workspace_bytes;
@@ -302,11 +310,10 @@ inline WgradDirectPlan wgrad_direct_plan(u32 N, u32 IC, u32 OC, u32 H, u32 targe
     return p;
 }
 
+// Kernel arguments and grid size of one configuration for one call.
 template <class Cfg>
-inline int launch_wgrad_direct(const float *dY, const float *X, float *dW, float *ws, const WgradDirectPlan &p, u32 N, u32 IC,
-                               u32 OC, u32 H, hipStream_t s, const char *what) {
-    (void)N;
-    WgradArgs a;
+inline uint64_t wgrad_direct_args(WgradArgs &a, const float *dY, const float *X, float *dW, float *ws, const WgradDirectPlan &p, u32 IC,
+                                  u32 OC, u32 H) {
     a.dY = dY, a.X = X;
     a.out = p.splits > 1 ? ws : dW;
     a.OC = OC, a.IC = IC, a.H = H;
@@ -315,8 +322,16 @@ inline int launch_wgrad_direct(const float *dY, const float *X, float *dW, float
     a.tiles_per_img = H / Cfg::TR;
     a.accumulate = p.splits > 1 ? 0u : 1u;
     a.pairs = p.pairs, a.splits = p.splits;
-    const uint64_t wgs = p.splits >= kXcds ? uint64_t(ceil_div(p.splits, kXcds)) * kXcds * p.pairs  // whole XCD rounds
-                                           : uint64_t(p.splits) * p.pairs;
+    return p.splits >= kXcds ? uint64_t(ceil_div(p.splits, kXcds)) * kXcds * p.pairs  // whole XCD rounds
+                             : uint64_t(p.splits) * p.pairs;
+}
+
+template <class Cfg>
+inline int launch_wgrad_direct(const float *dY, const float *X, float *dW, float *ws, const WgradDirectPlan &p, u32 N, u32 IC,
+                               u32 OC, u32 H, hipStream_t s, const char *what) {
+    (void)N;
+    WgradArgs a;
+    const uint64_t wgs = wgrad_direct_args<Cfg>(a, dY, X, dW, ws, p, IC, OC, H);
     if (wgs > 0x7fffffffull) return fail(CRB_EINVAL_SHAPE, "%s: launch grid too large", what);
     hipLaunchKernelGGL((wgrad3x3_kernel<Cfg>), dim3(u32(wgs)), dim3(kThreads), 0, s, a);
     if (int st = check_launch(what)) return st;

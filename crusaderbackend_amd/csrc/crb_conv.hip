@@ -259,6 +259,72 @@ static bool wgrad_direct(const crb_conv_geom *g, bool run, const float *dY, cons
     return false;
 }
 
+// ---- data gradient and weight gradient of one layer in one launch ------------------------------------------------------
+// The two gradients of a layer are independent (dX = f(W, dY), dW += f(dY, X)), and each of their kernels alone leaves the
+// chip idle while it ramps up, loads its first tiles and drains. Launched as one grid — the weight-gradient workgroups
+// first, the data-gradient workgroups after them — they share every compute unit and those fixed phases are paid once.
+template <class DCfg, class WCfg>
+__global__ void __launch_bounds__(kThreads, 2) conv_bwd_kernel(DirectArgs d, WgradArgs w, u32 wgrad_wgs) {
+    constexpr int SM = DCfg::SMEM_FLOATS > WCfg::SMEM ? DCfg::SMEM_FLOATS : WCfg::SMEM;
+    __shared__ __attribute__((aligned(16))) float smem[SM];
+    if (blockIdx.x < wgrad_wgs)
+        wgrad3x3_body<WCfg>(w, blockIdx.x, smem);
+    else
+        conv3x3_body<DCfg>(d, blockIdx.x - wgrad_wgs, smem);
+}
+
+// One (data-gradient configuration, weight-gradient configuration) pair; `run` = false only computes the plan.
+template <class DCfg, class WCfg>
+static bool bwd_pair(const crb_conv_geom *g, bool run, const float *Wt, const float *dY, const float *X, float *dX, float *dW,
+                     float *ws, hipStream_t s, WgradDirectPlan &plan, int &status) {
+    if (!direct_fits<DCfg>(g->OC, g->OH, g->OW) || !wgrad_direct_fits<WCfg>(g->N, g->IC, g->OC, g->OH, g->OW)) return false;
+    plan = wgrad_direct_plan<WCfg>(g->N, g->IC, g->OC, g->OH, kWgradTargetWgs);
+    if (!run) return true;
+    DirectArgs d;
+    WgradArgs w;
+    const uint64_t dwgs = direct_args<DCfg>(d, Wt, dY, dX, nullptr, g->N, g->OC, g->IC, g->OH, g->OH, 0);
+    const uint64_t wwgs = wgrad_direct_args<WCfg>(w, dY, X, dW, ws, plan, g->IC, g->OC, g->OH);
+    if (dwgs + wwgs > 0x7fffffffull) {
+        status = fail(CRB_EINVAL_SHAPE, "crb_conv_bwd: launch grid too large");
+        return true;
+    }
+    hipLaunchKernelGGL((conv_bwd_kernel<DCfg, WCfg>), dim3(u32(dwgs + wwgs)), dim3(kThreads), 0, s, d, w, u32(wwgs));
+    status = check_launch("crb_conv_bwd");
+    if (status == CRB_OK && plan.splits > 1)
+        status = launch_splitk_reduce(ws, dW, g->OC * g->IC * 9, plan.splits, ReduceEpi{nullptr, 1, 1, EPI_ACCUM}, s, "crb_conv_bwd");
+    return true;
+}
+
+// Pairs for the layer shapes of CIFAR residual networks. The weight-gradient configuration is the one crb_conv_wgrad picks
+// for the shape (same split plan, same workspace); the data-gradient configuration has the chunking of the one
+// crb_conv_dgrad picks (only the output-channel tile may differ, which does not enter any element's summation order), so
+// results are identical to crb_conv_dgrad followed by crb_conv_wgrad.
+static bool bwd_fused(const crb_conv_geom *g, bool run, const float *Wt, const float *dY, const float *X, float *dX, float *dW,
+                      float *ws, hipStream_t s, WgradDirectPlan &plan, int &status) {
+#define CRB_PAIR(D, W) bwd_pair<D, W>(g, run, Wt, dY, X, dX, dW, ws, s, plan, status)
+    typedef DirectCfg<32, 8, 16, 16, 4, 1, true, 2, 1, 1, 3, 4> D32a;
+    typedef DirectCfg<16, 4, 16, 32, 1, 2, true, 2, 2, 1> D16a;
+    typedef DirectCfg<8, 8, 16, 32, 1, 2, true, 2, 2, 1> D8a;
+    typedef DirectCfg<16, 8, 8, 16, 2, 1, true, 2, 2, 2> D16s2;
+    typedef DirectCfg<8, 8, 8, 32, 1, 2, true, 2, 2, 2> D8s2;
+    typedef WgradCfg<32, 8, 1, 2, 1> W32a;
+    typedef WgradCfg<16, 16, 1, 2, 1> W16a;
+    typedef WgradCfg<8, 8, 4, 2, 1> W8a;
+    typedef WgradCfg<16, 8, 1, 1, 2> W16s2;
+    typedef WgradCfg<8, 8, 2, 1, 2> W8s2;
+    const u32 ci = g->OC, co = g->IC;  // channels the data gradient reads / writes
+    if (direct_shape(g, 1)) {
+        if (g->OW == 32 && ci <= 16 && ci > 8 && co <= 16) return CRB_PAIR(D32a, W32a);
+        if (g->OW == 16 && co > 16 && co <= 64 && ci > 8) return CRB_PAIR(D16a, W16a);
+        if (g->OW == 8 && co <= 64 && ci > 8) return CRB_PAIR(D8a, W8a);
+    } else if (direct_shape(g, 2)) {
+        if (g->OW == 16 && co <= 16) return CRB_PAIR(D16s2, W16s2);
+        if (g->OW == 8 && co > 16) return CRB_PAIR(D8s2, W8s2);
+    }
+#undef CRB_PAIR
+    return false;
+}
+
 __global__ void __launch_bounds__(256) conv_bias_kernel(float *__restrict__ Y, const float *__restrict__ bias,
                                                         u32 total, u32 C, FastDiv hw) {
     const u32 i = blockIdx.x * 256 + threadIdx.x;
@@ -486,6 +552,32 @@ int crb_conv_wgrad(const float *dY, const float *X, float *dW, const crb_conv_ge
     RowMajorEpi e{ws, nullptr, p.Ncols, p.M * p.Ncols, 0u};
     if (int st = run_by_m(a, b, e, p.M, p.Ncols, p.K, p.splits, 1, p.k_per_z, s, "crb_conv_wgrad")) return st;
     return launch_splitk_reduce(ws, dW, p.M * p.Ncols, p.splits, ReduceEpi{nullptr, 1, 1, EPI_ACCUM}, s, "crb_conv_wgrad(reduce)");
+}
+
+int crb_conv_bwd(const float *W, const float *dY, const float *X, float *dX, float *dW, const crb_conv_geom *g, void *workspace,
+                 size_t workspace_bytes, void *stream) {
+    if (!W || !dY || !X || !dX || !dW) return fail(CRB_ENULL, "crb_conv_bwd: null operand");
+    if (int st = check_geom("crb_conv_bwd", g)) return st;
+    if (aligned16(dY) && aligned16(X) && aligned16(dX)) {
+        WgradDirectPlan dp;
+        int st = CRB_OK;
+        if (bwd_fused(g, false, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, dp, st)) {
+            float *dws = static_cast<float *>(workspace);
+            if (dp.workspace_bytes) {
+                if (dws) {
+                    if (workspace_bytes < dp.workspace_bytes)
+                        return fail(CRB_EWORKSPACE, "crb_conv_bwd: workspace %zu bytes < required %zu", workspace_bytes, dp.workspace_bytes);
+                } else {
+                    dws = static_cast<float *>(arena_get(dp.workspace_bytes));
+                    if (!dws) return fail(CRB_EHIP, "crb_conv_bwd: cannot allocate %zu bytes of scratch", dp.workspace_bytes);
+                }
+            }
+            bwd_fused(g, true, W, dY, X, dX, dW, dws, hipStream_t(stream), dp, st);
+            return st;
+        }
+    }
+    if (int st = crb_conv_dgrad(W, dY, dX, g, stream)) return st;
+    return crb_conv_wgrad(dY, X, dW, g, workspace, workspace_bytes, stream);
 }
 
 int crb_conv_bias_grad(const float *dY, float *dB, uint32_t N, uint32_t C, uint32_t HW, void *stream) {

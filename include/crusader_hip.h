@@ -133,6 +133,15 @@ int crb_conv_wgrad(const float *dY, const float *X, float *dW, const crb_conv_ge
 /* Replaces seblas::convBias (cuConv.cu:808-818; kernel :709-729). Y[n,c,:,:] += bias[c], in place. */
 int crb_conv_bias(float *Y, const float *bias, uint32_t N, uint32_t C, uint32_t HW, void *stream);
 
+/* Both gradients of a convolution layer in one call: dX as crb_conv_dgrad writes it and dW as crb_conv_wgrad accumulates
+ * it (same workspace rule: crb_conv_wgrad_workspace_bytes(g) bytes, or NULL for the library arena). Replaces the pair of
+ * calls Conv2D::xGrads / Conv2D::paramGrads make back to back (seann/operands/seblas/Conv2D.cu:18-29: convDerive, then
+ * convError): the two are independent, and for the layer shapes of CIFAR residual networks they run as one launch that
+ * shares the chip; other shapes run the two calls one after the other. Results are identical to the separate calls.
+ * dX must not overlap X or dY. */
+int crb_conv_bwd(const float *W, const float *dY, const float *X, float *dX, float *dW, const crb_conv_geom *g, void *workspace,
+                 size_t workspace_bytes, void *stream);
+
 /* Bias gradient of a conv operand: dB[c] += sum_{n,h,w} dY[n,c,h,w], each element updated exactly once.
  * Stands in for the channelReduce call of Conv2D::paramGrads (seann/operands/seblas/Conv2D.cu:26-28), whose
  * size assertion (seblas/operations/cuReduce.cu:237) cannot hold for a C-element bias; this computes the

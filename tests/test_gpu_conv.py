@@ -292,3 +292,52 @@ POINTWISE = [(3, 24, 32, 32, 48), (2, 204, 32, 32, 48), (2, 108, 16, 16, 48), (4
 @pytest.mark.parametrize("N,IC,H,W,OC", POINTWISE)
 def test_conv1x1_paths(dev, N, IC, H, W, OC):
     run_layer(dev, N, IC, H, W, OC, 1, 1, 1, 1, 0, 0, bias=True, seed=31)
+
+
+# Both gradients in one call. Fused shapes (the five layer shapes of CIFAR residual networks, at a small and at the full
+# batch), neighbours that must take the two-call route (other channel counts, widths, filter, an odd batch for the 8x8
+# tile of 4 images, 1x1, 2x2 images), with and without a caller workspace.
+BWD_CASES = [(8, 16, 32, 16, 3, 1, 1), (128, 16, 32, 16, 3, 1, 1), (8, 32, 16, 32, 3, 1, 1), (128, 32, 16, 32, 3, 1, 1),
+             (8, 64, 8, 64, 3, 1, 1), (128, 64, 8, 64, 3, 1, 1), (8, 16, 32, 32, 3, 2, 1), (128, 16, 32, 32, 3, 2, 1),
+             (8, 32, 16, 64, 3, 2, 1), (128, 32, 16, 64, 3, 2, 1),
+             (6, 12, 32, 14, 3, 1, 1), (6, 24, 16, 40, 3, 1, 1), (6, 64, 8, 48, 3, 1, 1), (3, 64, 8, 64, 3, 1, 1),
+             (4, 3, 32, 16, 3, 1, 1), (4, 64, 32, 64, 3, 1, 1), (4, 128, 8, 128, 3, 1, 1), (4, 8, 12, 8, 3, 1, 1),
+             (4, 16, 16, 8, 5, 1, 2), (4, 24, 8, 12, 1, 1, 0), (4, 32, 2, 32, 3, 1, 1), (4, 32, 4, 32, 3, 1, 1)]
+
+
+@pytest.mark.parametrize("N,IC,H,OC,F,s,p", BWD_CASES)
+@pytest.mark.parametrize("own_ws", [False, True])
+def test_conv_bwd_equals_separate_calls(dev, N, IC, H, OC, F, s, p, own_ws):
+    import torch
+    capi, orc = _capi(), _oracle()
+    g = capi.ConvGeom.make(N, IC, H, H, OC, F, F, s, s, p, p)
+    X, W, dY = normal(1, N, IC, H, H), he_normal(2, OC, IC, F, F), normal(3, N, OC, g.OH, g.OW)
+    dW0 = normal(4, OC, IC, F, F)
+    Xd, Wd, dYd = to_dev(X, dev), to_dev(W, dev), to_dev(dY, dev)
+    ws = None
+    if own_ws:
+        nbytes = capi.conv_wgrad_workspace_bytes(g)
+        ws = torch.empty(max(nbytes // 4, 1), dtype=torch.float32, device=dev)
+    dX1, dW1 = _nan(dev, N, IC, H, H), to_dev(dW0, dev)
+    capi.conv_dgrad(Wd, dYd, dX1, g)
+    capi.conv_wgrad(dYd, Xd, dW1, g, workspace=ws)
+    dX2, dW2 = _nan(dev, N, IC, H, H), to_dev(dW0, dev)
+    capi.conv_bwd(Wd, dYd, Xd, dX2, dW2, g, workspace=ws)
+    assert np.array_equal(to_np(dX1), to_np(dX2)) and np.array_equal(to_np(dW1), to_np(dW2))
+    if N <= 8:  # and both are the layer's gradients
+        assert_close(to_np(dX2), orc.convDerive(W, dY, (H, H), s, s, p, p, threads=8), OC * F * F, "conv bwd dX")
+        assert_close(to_np(dW2), orc.convError(dY, X, dW0, s, s, p, p, threads=8), N * g.OH * g.OW, "conv bwd dW")
+
+
+def test_conv_bwd_errors(dev):
+    import ctypes
+    import torch
+    capi = _capi()
+    lib = capi.load()
+    t = torch.zeros(1 << 16, device=dev)
+    g = capi.ConvGeom.make(64, 16, 32, 32, 16, 3, 3, 1, 1, 1, 1)
+    p = t.data_ptr()
+    assert lib.crb_conv_bwd(p, p, p, p, p, ctypes.byref(g), p, 16, None) == capi.CRB_EWORKSPACE
+    assert lib.crb_conv_bwd(p, p, p, None, p, ctypes.byref(g), None, 0, None) == capi.CRB_ENULL
+    g = capi.ConvGeom.make(1, 2, 8, 8, 2, 3, 3, 1, 1, 1, 1, OH=7, OW=8)
+    assert lib.crb_conv_bwd(p, p, p, p, p, ctypes.byref(g), None, 0, None) == capi.CRB_EINVAL_SHAPE
