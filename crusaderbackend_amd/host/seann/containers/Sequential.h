@@ -47,7 +47,8 @@ public:
     // writes another operand's reserve must increment that operand's `reserveWriters` in its postWaiveInit.
     void pruneReserveFolds() const;
     // streamline: pruneReserveFolds plus letting every opening shortcut endpoint's output value alias its input (it only
-    // passes it on), which removes one device copy per residual block from the forward pass.
+    // passes it on), which removes one device copy per residual block from the forward pass, plus letting each convolution's
+    // xGrads compute the filter gradient in the same launch as the input gradient (backward() calls the two as a pair).
     void streamline() const;
     // learnFused: the momentum step of every parameter in one kernel launch instead of one launch per parameter.
     void learnFused();

@@ -48,6 +48,9 @@ public:
 
     virtual void collectNetParams(std::vector<NetParam *> &) {}  // every trainable parameter, for a fused update
     virtual void pruneReserveFolds() { foldReserveEnabled = reserveWriters > 0; }
+    // Lets xGrads also produce the parameter gradients where one launch can compute both; the paramGrads call that follows
+    // it in Sequential::backward then finds them done. Only for callers that always pair the two calls (Sequential does).
+    virtual void fuseGrads() {}
 
     // Y->dA += Y->dAReserve and the reserve is cleared, in one pass (the reference clears it after the gradient call, which
     // never reads it): the first thing every xGrads does

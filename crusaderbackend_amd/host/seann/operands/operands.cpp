@@ -26,16 +26,23 @@ void Conv2D::initNetParams(OptimizerInfo *info, shape4 inShape) {
 }
 
 void Conv2D::forward() {  // Conv2D.cu:8-16
+    filterGradDone = false;
     conv(filter->data(), X->A, Y->A, int(strideH), int(strideW), int(padH), int(padW), WITH_BIAS ? bias->data() : nullptr);
 }
 
 void Conv2D::xGrads() {  // Conv2D.cu:18-22
     foldReserve();
+    if (gradsFused) {  // both gradients in one call; paramGrads then only adds the bias gradient
+        convBackward(filter->data(), Y->dA, X->A, X->dA, filter->grad(), int(strideH), int(strideW), int(padH), int(padW));
+        filterGradDone = true;
+        return;
+    }
     convDerive(filter->data(), Y->dA, X->dA, int(strideH), int(strideW), int(padH), int(padW));
 }
 
 void Conv2D::paramGrads() {  // Conv2D.cu:24-29; the bias gradient is the per-channel sum of dY
-    convError(Y->dA, X->A, filter->grad(), int(strideH), int(strideW), int(padH), int(padW));
+    if (!filterGradDone) convError(Y->dA, X->A, filter->grad(), int(strideH), int(strideW), int(padH), int(padW));
+    filterGradDone = false;
     if (WITH_BIAS) {
         const shape4 &d = Y->dA->dims;
         throwOnStatus(crb_conv_bias_grad(Y->dA->elements, bias->grad()->elements, d.n, d.c, d.h * d.w, nullptr), __FILE__,
@@ -250,6 +257,7 @@ void Sequential::pruneReserveFolds() const {
 
 void Sequential::streamline() const {
     pruneReserveFolds();
+    for (OperandBase *op : operands) op->fuseGrads();  // backward() always calls xGrads and paramGrads as a pair
     if (hipDeviceSynchronize() != hipSuccess) assertHip(__FILE__, __LINE__);  // buffers are released below: nothing may be in flight
     for (uint32 i = 0; i + 1 < OPERAND_COUNT; i++) {
         OperandBase *op = operands[i];

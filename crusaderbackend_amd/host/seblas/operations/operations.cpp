@@ -126,6 +126,13 @@ Tensor *convError(Tensor *A, Tensor *B, Tensor *C, int strideH, int strideW, int
     return A;  // the reference returns its first argument (cuConv.cu:805)
 }
 
+void convBackward(Tensor *filter, Tensor *dY, Tensor *X, Tensor *dX, Tensor *dFilter, int strideH, int strideW, int padH, int padW) {
+    crb_conv_geom g = geom(filter, dX, dY, strideH, strideW, padH, padW);
+    require(X->dims == dX->dims && dFilter->dims == filter->dims, "convBackward: gradient shapes differ from their tensors");
+    finish(crb_conv_bwd(filter->elements, dY->elements, X->elements, dX->elements, dFilter->elements, &g, nullptr, 0, nullptr),
+           __FILE__, __LINE__);
+}
+
 Tensor *convBias(Tensor *Y, Tensor *biases) {
     require(biases->dims.size == Y->dims.c, "convBias: bias size != channels");  // cuConv.cu:809
     finish(crb_conv_bias(Y->elements, biases->elements, Y->dims.n, Y->dims.c, Y->dims.h * Y->dims.w, nullptr), __FILE__,

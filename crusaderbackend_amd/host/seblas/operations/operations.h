@@ -29,6 +29,10 @@ Tensor *convDerive(Tensor *A, Tensor *B, Tensor *C, int strideH, int strideW, in
 // A: errors N x OC x OH x OW, B: inputs N x IC x IH x IW, C: filter grads (accumulated). Returns A, as the
 // reference does (cuConv.cu:805).
 Tensor *convError(Tensor *A, Tensor *B, Tensor *C, int strideH, int strideW, int padH, int padW);
+// convDerive(filter, dY, dX, ...) and convError(dY, X, dFilter, ...) in one call: the two gradients of a layer are independent
+// and, for the layer shapes of CIFAR residual networks, run as one kernel launch. Same results as the two calls. No
+// counterpart in the reference.
+void convBackward(Tensor *filter, Tensor *dY, Tensor *X, Tensor *dX, Tensor *dFilter, int strideH, int strideW, int padH, int padW);
 Tensor *convBias(Tensor *Y, Tensor *biases);
 
 // ---- the elementwise / reduction operators a training step runs between those calls -------------------------------

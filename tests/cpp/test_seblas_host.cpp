@@ -517,6 +517,34 @@ static void gpu_sequential_tests() {
         for (float v : pull(fc->biases->grad())) CHECK(v == 0.f);
         CHECK(pull(c2->filter->data()) != before_w);
     }
+    // a convolution whose two gradients run as one launch (16 -> 16 channels on 32 x 32, with bias): same numbers as the
+    // two separate calls, gradient accumulation included
+    {
+        const uint32_t B = 8;
+        auto run = [&](bool fused, std::vector<float> &dx, std::vector<float> &dw, std::vector<float> &db) {
+            auto *cv = new Conv2D(shape4(16, 16, 3, 3), 1, 1, 1, 1, true);
+            cv->initNetParams(nullptr, shape4(B, 16, 32, 32));
+            cv->randFillNetParams();
+            cv->X->instantiate();  // stand-alone operand: it owns its input
+            if (fused) cv->fuseGrads();
+            auto xin = randn(B * 16 * 32 * 32, 61), dy = randn(B * 16 * 32 * 32, 62), g0 = randn(16 * 16 * 9, 63);
+            CHECK(hipMemcpy(cv->X->A->elements, xin.data(), xin.size() * 4, hipMemcpyHostToDevice) == hipSuccess);
+            CHECK(hipMemcpy(cv->filter->grad()->elements, g0.data(), g0.size() * 4, hipMemcpyHostToDevice) == hipSuccess);
+            cv->forward();
+            CHECK(hipMemcpy(cv->Y->dA->elements, dy.data(), dy.size() * 4, hipMemcpyHostToDevice) == hipSuccess);
+            cv->xGrads();
+            cv->paramGrads();
+            dx = pull(cv->X->dA), dw = pull(cv->filter->grad()), db = pull(cv->bias->grad());
+            if (fused) {  // paramGrads on its own still computes the filter gradient
+                cv->paramGrads();
+                CHECK(pull(cv->filter->grad()) != dw);
+            }
+        };
+        std::vector<float> dx1, dw1, db1, dx2, dw2, db2;
+        run(false, dx1, dw1, db1);
+        run(true, dx2, dw2, db2);
+        CHECK(dx1 == dx2 && dw1 == dw2 && db1 == db2);
+    }
     // the non-blocking mode gives the same numbers
     setBlocking(false);
     net.forward(X);
