@@ -261,20 +261,23 @@ static bool wgrad_direct(const crb_conv_geom *g, bool run, const float *dY, cons
 
 // ---- data gradient and weight gradient of one layer in one launch ------------------------------------------------------
 // The two gradients of a layer are independent (dX = f(W, dY), dW += f(dY, X)), and each of their kernels alone leaves the
-// chip idle while it ramps up, loads its first tiles and drains. Launched as one grid — the weight-gradient workgroups
-// first, the data-gradient workgroups after them — they share every compute unit and those fixed phases are paid once.
+// chip idle while it ramps up, loads its first tiles and drains. Launched as one grid — the longer-running kind of workgroup
+// first — they share every compute unit and those fixed phases are paid once.
 template <class DCfg, class WCfg>
-__global__ void __launch_bounds__(kThreads, 2) conv_bwd_kernel(DirectArgs d, WgradArgs w, u32 wgrad_wgs) {
+__global__ void __launch_bounds__(kThreads, 2) conv_bwd_kernel(DirectArgs d, WgradArgs w, u32 first_wgs, u32 dgrad_first) {
     constexpr int SM = DCfg::SMEM_FLOATS > WCfg::SMEM ? DCfg::SMEM_FLOATS : WCfg::SMEM;
     __shared__ __attribute__((aligned(16))) float smem[SM];
-    if (blockIdx.x < wgrad_wgs)
-        wgrad3x3_body<WCfg>(w, blockIdx.x, smem);
+    // the longer-running kind takes the low workgroup ids, which are dispatched first
+    const bool first = blockIdx.x < first_wgs;
+    const u32 bid = first ? blockIdx.x : blockIdx.x - first_wgs;
+    if (first == (dgrad_first != 0))
+        conv3x3_body<DCfg>(d, bid, smem);
     else
-        conv3x3_body<DCfg>(d, blockIdx.x - wgrad_wgs, smem);
+        wgrad3x3_body<WCfg>(w, bid, smem);
 }
 
 // One (data-gradient configuration, weight-gradient configuration) pair; `run` = false only computes the plan.
-template <class DCfg, class WCfg>
+template <class DCfg, class WCfg, bool DGRAD_FIRST = false>
 static bool bwd_pair(const crb_conv_geom *g, bool run, const float *Wt, const float *dY, const float *X, float *dX, float *dW,
                      float *ws, hipStream_t s, WgradDirectPlan &plan, int &status) {
     if (!direct_fits<DCfg>(g->OC, g->OH, g->OW) || !wgrad_direct_fits<WCfg>(g->N, g->IC, g->OC, g->OH, g->OW)) return false;
@@ -288,7 +291,8 @@ static bool bwd_pair(const crb_conv_geom *g, bool run, const float *Wt, const fl
         status = fail(CRB_EINVAL_SHAPE, "crb_conv_bwd: launch grid too large");
         return true;
     }
-    hipLaunchKernelGGL((conv_bwd_kernel<DCfg, WCfg>), dim3(u32(dwgs + wwgs)), dim3(kThreads), 0, s, d, w, u32(wwgs));
+    hipLaunchKernelGGL((conv_bwd_kernel<DCfg, WCfg>), dim3(u32(dwgs + wwgs)), dim3(kThreads), 0, s, d, w,
+                       u32(DGRAD_FIRST ? dwgs : wwgs), DGRAD_FIRST ? 1u : 0u);
     status = check_launch("crb_conv_bwd");
     if (status == CRB_OK && plan.splits > 1)
         status = launch_splitk_reduce(ws, dW, g->OC * g->IC * 9, plan.splits, ReduceEpi{nullptr, 1, 1, EPI_ACCUM}, s, "crb_conv_bwd");
@@ -301,7 +305,7 @@ static bool bwd_pair(const crb_conv_geom *g, bool run, const float *Wt, const fl
 // results are identical to crb_conv_dgrad followed by crb_conv_wgrad.
 static bool bwd_fused(const crb_conv_geom *g, bool run, const float *Wt, const float *dY, const float *X, float *dX, float *dW,
                       float *ws, hipStream_t s, WgradDirectPlan &plan, int &status) {
-#define CRB_PAIR(D, W) bwd_pair<D, W>(g, run, Wt, dY, X, dX, dW, ws, s, plan, status)
+#define CRB_PAIR(...) bwd_pair<__VA_ARGS__>(g, run, Wt, dY, X, dX, dW, ws, s, plan, status)
     typedef DirectCfg<32, 8, 16, 16, 4, 1, true, 2, 1, 1, 3, 4> D32a;
     typedef DirectCfg<16, 4, 16, 32, 1, 2, true, 2, 2, 1> D16a;
     typedef DirectCfg<8, 8, 16, 32, 1, 2, true, 2, 2, 1> D8a;
@@ -319,7 +323,7 @@ static bool bwd_fused(const crb_conv_geom *g, bool run, const float *Wt, const f
         if (g->OW == 8 && co <= 64 && ci > 8) return CRB_PAIR(D8a, W8a);
     } else if (direct_shape(g, 2)) {
         if (g->OW == 16 && co <= 16) return CRB_PAIR(D16s2, W16s2);
-        if (g->OW == 8 && co > 16) return CRB_PAIR(D8s2, W8s2);
+        if (g->OW == 8 && co > 16) return CRB_PAIR(D8s2, W8s2, true);  // here the data gradient is the longer half
     }
 #undef CRB_PAIR
     return false;
