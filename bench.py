@@ -105,6 +105,9 @@ MEASURED_HBM_BYTES = {
     "L3_64-64@8.fwd": 5.47e6, "L3_64-64@8.dgrad": 5.46e6, "L3_64-64@8.wgrad": 9.38e6,
     "T1_16-32s2.fwd": 13.12e6, "T1_16-32s2.dgrad": 13.35e6, "T1_16-32s2.wgrad": 17.57e6,
     "T2_32-64s2.fwd": 6.99e6, "T2_32-64s2.dgrad": 6.96e6, "T2_32-64s2.wgrad": 11.33e6,
+    # both gradients in one call: conv_bwd_kernel + the reduce kernel
+    "L1_16-16@32.bwd": 39.78e6, "L2_32-32@16.bwd": 24.36e6, "L3_64-64@8.bwd": 14.60e6,
+    "T1_16-32s2.bwd": 30.30e6, "T2_32-64s2.bwd": 18.0e6,
 }
 
 
