@@ -66,6 +66,11 @@ class Layer:
         self.dW = torch.zeros(OC, IC, F, F, device=dev)
         nbytes = capi.conv_wgrad_workspace_bytes(g)
         self.ws = torch.empty(max(nbytes // 4, 1), dtype=torch.float32, device=dev) if nbytes else None
+        # The timed step runs a layer shape `mult` times, as the network has `mult` such layers; with the slice summation
+        # postponed to the end of the backward pass every one of them owns its slices and its dW until then.
+        self.n_slices = capi.conv_bwd_slices(g)
+        self.ws_each = [torch.empty(max(nbytes // 4, 1), dtype=torch.float32, device=dev) for _ in range(mult)] if self.n_slices else []
+        self.dW_each = [torch.zeros(OC, IC, F, F, device=dev) for _ in range(mult)] if self.n_slices else []
         self.flops = 2.0 * batch * OC * g.OH * g.OW * IC * F * F
         nb = 0 if self.b is None else OC
         self.bytes = {
@@ -75,6 +80,7 @@ class Layer:
         }
         # both gradients in one call: dY is read by both halves but counted once
         self.bytes["bwd"] = 4.0 * (self.dY.numel() + self.W.numel() + self.dX.numel() + self.X.numel() + 2 * self.dW.numel())
+        self.bytes["bwd_sliced"] = self.bytes["bwd"]  # its share of the final summation included
         self.capi = capi
 
     def fwd(self):
@@ -89,10 +95,21 @@ class Layer:
     def bwd(self):
         self.capi.conv_bwd(self.W, self.dY, self.X, self.dX, self.dW, self.g, workspace=self.ws)
 
+    def bwd_sliced(self, k=0):
+        self.capi.conv_bwd_sliced(self.W, self.dY, self.X, self.dX, self.g, self.ws_each[k])
+
+    def slice_entries(self):
+        return [(ws, dW, self.n_slices) for ws, dW in zip(self.ws_each, self.dW_each)]
+
     def passes(self):
-        """(name, call, flops, part of the timed step): the step runs fwd and bwd; dgrad and wgrad alone are listed too."""
-        return (("fwd", self.fwd, self.flops, True), ("bwd", self.bwd, 2 * self.flops, True),
-                ("dgrad", self.dgrad, self.flops, False), ("wgrad", self.wgrad, self.flops, False))
+        """(name, call, flops, part of the timed step). The step runs fwd and bwd_sliced per layer and one summation of all
+        slices at its end; the self-contained backward call and the two gradients alone are listed too."""
+        out = [("fwd", self.fwd, self.flops, True)]
+        if self.n_slices:
+            out.append(("bwd_sliced", self.bwd_sliced, 2 * self.flops, True))
+        out += [("bwd", self.bwd, 2 * self.flops, not self.n_slices), ("dgrad", self.dgrad, self.flops, False),
+                ("wgrad", self.wgrad, self.flops, False)]
+        return out
 
 
 # HBM bytes one call moves (read + written, all kernels of the call), from the FETCH_SIZE and WRITE_SIZE hardware
@@ -108,6 +125,9 @@ MEASURED_HBM_BYTES = {
     # both gradients in one call: conv_bwd_kernel + the reduce kernel
     "L1_16-16@32.bwd": 39.78e6, "L2_32-32@16.bwd": 24.36e6, "L3_64-64@8.bwd": 14.60e6,
     "T1_16-32s2.bwd": 30.30e6, "T2_32-64s2.bwd": 18.0e6,
+    # conv_bwd_kernel alone (slices left for the end-of-step summation)
+    "L1_16-16@32.bwd_sliced": 37.34e6, "L2_32-32@16.bwd_sliced": 21.92e6, "L3_64-64@8.bwd_sliced": 11.93e6,
+    "T1_16-32s2.bwd_sliced": 27.86e6, "T2_32-64s2.bwd_sliced": 15.5e6,
 }
 
 
@@ -226,14 +246,21 @@ def main():
 
     layers = [Layer(torch, capi, dev, n, IC, H, OC, s, m, seed=10 + i) for i, (n, IC, H, OC, s, m) in enumerate(RESNET56)]
     step_flops = sum(3 * L.mult * L.flops for L in layers)
+    slice_entries = [e for L in layers for e in L.slice_entries()]
+    slice_table = capi.slice_sum_table(slice_entries) if slice_entries else None
 
     def step():
         for L in layers:
             for _ in range(L.mult):
                 L.fwd()
         for L in reversed(layers):
-            for _ in range(L.mult):
-                L.bwd()  # data gradient and weight gradient of the layer in one call
+            for k in range(L.mult):
+                if L.n_slices:
+                    L.bwd_sliced(k)  # data gradient + weight-gradient slices of the layer in one launch
+                else:
+                    L.bwd()
+        if slice_table is not None:
+            capi.sum_slices_multi(slice_table)  # every layer's dW += its slices, one launch
 
     for _ in range(args.warmup):
         step()
@@ -256,6 +283,7 @@ def main():
                 "ms": ms, "tflops": fl / ms / 1e9, "gbs": L.bytes[pname] / ms / 1e6, "mult": L.mult if in_step else 0,
                 "flops": fl, "bytes": L.bytes[pname],
             }
+    sum_ms = event_time_ms(torch, lambda: capi.sum_slices_multi(slice_table), reps=20) if slice_table is not None else 0.0
     dom = max(per, key=lambda k: per[k]["ms"] * per[k]["mult"])
     d = per[dom]
     roofline = {
@@ -266,7 +294,7 @@ def main():
         "flops_per_launch": d["flops"], "avg_launch_ms": d["ms"],
         "share_of_step": d["ms"] * d["mult"] / sum(v["ms"] * v["mult"] for v in per.values()),
     }
-    kern_sum_ms = sum(v["ms"] * v["mult"] for v in per.values())
+    kern_sum_ms = sum(v["ms"] * v["mult"] for v in per.values()) + sum_ms
 
     # headline GEMM target: 4096^3 sgemm
     n = 4096
@@ -286,7 +314,8 @@ def main():
         "dtype": "f32", "data": "synthetic",
         "config": {"workload": "ResNet-56 CIFAR conv shapes, fp32 NCHW, batch 128, 3x3 pad 1: 19x16->16@32, 17x32->32@16, "
                                "18x64->64@8, 16->32 s2, 32->64 s2; forward + dgrad + wgrad per layer (the two gradients of a layer "
-                               "issued as one crb_conv_bwd call)",
+                               "issued as one crb_conv_bwd_sliced call, the 55 layers' weight-gradient slices summed by one "
+                               "crb_sum_slices_multi call at the end of the step)",
                    "batch": BATCH, "flops_per_step": step_flops},
         "roofline": roofline,
         "extra": {
@@ -296,6 +325,7 @@ def main():
             "kernel_only_tflops": step_flops / kern_sum_ms / 1e9,
             "sgemm_4096_tflops": gemm_tflops, "sgemm_4096_ms": gemm_ms,
             "sgemm_4096_frac_peak": gemm_tflops / PEAK_FP32_MFMA_TFLOPS,
+            "slice_sum_all_layers_ms": sum_ms, "slice_sum_items": len(slice_entries),
             "per_kernel": {k: {"ms": round(v["ms"], 5), "tflops": round(v["tflops"], 2), "gbs": round(v["gbs"], 1)}
                            for k, v in per.items()},
             "full_network_steps_cpp_host": full_net,

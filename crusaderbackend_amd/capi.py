@@ -52,6 +52,9 @@ SIGNATURES = {
     "crb_conv_wgrad_workspace_bytes": (ctypes.c_size_t, [ctypes.POINTER(ConvGeom)]),
     "crb_conv_wgrad": (ctypes.c_int, [_ptr, _ptr, _ptr, ctypes.POINTER(ConvGeom), _ptr, ctypes.c_size_t, _ptr]),
     "crb_conv_bwd": (ctypes.c_int, [_ptr, _ptr, _ptr, _ptr, _ptr, ctypes.POINTER(ConvGeom), _ptr, ctypes.c_size_t, _ptr]),
+    "crb_conv_bwd_slices": (_u32, [ctypes.POINTER(ConvGeom)]),
+    "crb_conv_bwd_sliced": (ctypes.c_int, [_ptr, _ptr, _ptr, _ptr, ctypes.POINTER(ConvGeom), _ptr, ctypes.c_size_t, _ptr]),
+    "crb_sum_slices_multi": (ctypes.c_int, [_ptr, _u32, _ptr]),
     "crb_conv_bias": (ctypes.c_int, [_ptr, _ptr, _u32, _u32, _u32, _ptr]),
     "crb_conv_bias_grad": (ctypes.c_int, [_ptr, _ptr, _u32, _u32, _u32, _ptr]),
     "crb_tensor_add_inplace": (ctypes.c_int, [_ptr, _ptr, _u32, _ptr]),
@@ -167,6 +170,34 @@ def conv_bwd(W, dY, X, dX, dW, geom, workspace=None, stream=None):
     """Data gradient and weight gradient of one layer in one call (one launch for the residual-network layer shapes)."""
     nbytes = 0 if workspace is None else workspace.numel() * workspace.element_size()
     check(load().crb_conv_bwd(_p(W), _p(dY), _p(X), _p(dX), _p(dW), ctypes.byref(geom), _p(workspace), nbytes, _stream(stream)))
+
+
+def conv_bwd_slices(geom):
+    return load().crb_conv_bwd_slices(ctypes.byref(geom))
+
+
+def conv_bwd_sliced(W, dY, X, dX, geom, workspace, stream=None):
+    """dX now; the weight gradient stays as conv_bwd_slices(geom) partial sums in `workspace` until sum_slices_multi."""
+    nbytes = workspace.numel() * workspace.element_size()
+    check(load().crb_conv_bwd_sliced(_p(W), _p(dY), _p(X), _p(dX), ctypes.byref(geom), _p(workspace), nbytes, _stream(stream)))
+
+
+class SliceSumItem(ctypes.Structure):
+    """Mirror of ``crb_slice_sum_item``."""
+
+    _fields_ = [("slices", ctypes.c_void_p), ("dst", ctypes.c_void_p), ("count", _u32), ("n_slices", _u32)]
+
+
+def slice_sum_table(entries):
+    """entries: (workspace tensor, dW tensor, number of slices) -> host array for sum_slices_multi (keep the tensors alive)."""
+    arr = (SliceSumItem * len(entries))()
+    for i, (ws, dW, n) in enumerate(entries):
+        arr[i] = SliceSumItem(ws.data_ptr(), dW.data_ptr(), dW.numel(), n)
+    return arr
+
+
+def sum_slices_multi(table, stream=None):
+    check(load().crb_sum_slices_multi(ctypes.cast(table, ctypes.c_void_p), len(table), _stream(stream)))
 
 
 def conv_bias(Y, bias, N, C, HW, stream=None):

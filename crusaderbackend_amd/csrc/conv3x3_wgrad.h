@@ -335,7 +335,7 @@ inline int launch_wgrad_direct(const float *dY, const float *X, float *dW, float
     if (wgs > 0x7fffffffull) return fail(CRB_EINVAL_SHAPE, "%s: launch grid too large", what);
     hipLaunchKernelGGL((wgrad3x3_kernel<Cfg>), dim3(u32(wgs)), dim3(kThreads), 0, s, a);
     if (int st = check_launch(what)) return st;
-    if (p.splits > 1) {
+    if (p.splits > 1 && dW) {  // dW == nullptr: the caller sums the slices later
         return launch_splitk_reduce(ws, dW, OC * IC * 9, p.splits, ReduceEpi{nullptr, 1, 1, EPI_ACCUM}, s, what);
     }
     return CRB_OK;

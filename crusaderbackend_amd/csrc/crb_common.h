@@ -24,7 +24,7 @@ void arena_release();
 // q = (t + ((n - t) >> s1)) >> s2 with t = mulhi(m, n).
 struct FastDiv {
     u32 d, m, s1, s2;
-    FastDiv() : d(1), m(1), s1(0), s2(0) {}
+    __host__ __device__ FastDiv() : d(1), m(1), s1(0), s2(0) {}
     explicit FastDiv(u32 div) { init(div); }
     void init(u32 div) {
         d = div ? div : 1;

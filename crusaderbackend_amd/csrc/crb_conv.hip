@@ -226,6 +226,7 @@ static bool tiny2x2_shape(const crb_conv_geom *g) {
 // One entry per configuration <W, TR, TI, OCC>; `run` = false only computes the plan (workspace size).
 constexpr u32 kWgradTargetWgs = 256;  // one workgroup per CU: pairs x splits
 
+// dW == nullptr (with run): the slices are left in ws, unsummed.
 template <class Cfg>
 static bool wgrad_cfg(const crb_conv_geom *g, bool run, const float *dY, const float *X, float *dW, float *ws, hipStream_t s,
                       WgradDirectPlan &plan, int &status) {
@@ -294,7 +295,7 @@ static bool bwd_pair(const crb_conv_geom *g, bool run, const float *Wt, const fl
     hipLaunchKernelGGL((conv_bwd_kernel<DCfg, WCfg>), dim3(u32(dwgs + wwgs)), dim3(kThreads), 0, s, d, w,
                        u32(DGRAD_FIRST ? dwgs : wwgs), DGRAD_FIRST ? 1u : 0u);
     status = check_launch("crb_conv_bwd");
-    if (status == CRB_OK && plan.splits > 1)
+    if (status == CRB_OK && plan.splits > 1 && dW)  // dW == nullptr: the slices stay in ws, unsummed
         status = launch_splitk_reduce(ws, dW, g->OC * g->IC * 9, plan.splits, ReduceEpi{nullptr, 1, 1, EPI_ACCUM}, s, "crb_conv_bwd");
     return true;
 }
@@ -582,6 +583,51 @@ int crb_conv_bwd(const float *W, const float *dY, const float *X, float *dX, flo
     }
     if (int st = crb_conv_dgrad(W, dY, dX, g, stream)) return st;
     return crb_conv_wgrad(dY, X, dW, g, workspace, workspace_bytes, stream);
+}
+
+uint32_t crb_conv_bwd_slices(const crb_conv_geom *g) {
+    if (check_geom("crb_conv_bwd_slices", g)) return 0;
+    WgradDirectPlan dp;
+    int st = CRB_OK;
+    if (pointwise_shape(g) || tiny2x2_shape(g)) return 0;
+    if (!wgrad_direct(g, false, nullptr, nullptr, nullptr, nullptr, nullptr, dp, st)) return 0;
+    return dp.splits > 1 ? dp.splits : 0;
+}
+
+int crb_conv_bwd_sliced(const float *W, const float *dY, const float *X, float *dX, const crb_conv_geom *g, void *workspace,
+                        size_t workspace_bytes, void *stream) {
+    if (!W || !dY || !X || !dX || !workspace) return fail(CRB_ENULL, "crb_conv_bwd_sliced: null operand");
+    if (int st = check_geom("crb_conv_bwd_sliced", g)) return st;
+    if (!crb_conv_bwd_slices(g) || !aligned16(dY) || !aligned16(X) || !aligned16(dX) || !aligned16(workspace))
+        return fail(CRB_EINVAL_SHAPE, "crb_conv_bwd_sliced: this geometry (or operand alignment) has no sliced form; use crb_conv_bwd");
+    WgradDirectPlan dp;
+    int st = CRB_OK;
+    float *ws = static_cast<float *>(workspace);
+    hipStream_t s = hipStream_t(stream);
+    if (bwd_fused(g, false, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, dp, st)) {
+        if (workspace_bytes < dp.workspace_bytes)
+            return fail(CRB_EWORKSPACE, "crb_conv_bwd_sliced: workspace %zu bytes < required %zu", workspace_bytes, dp.workspace_bytes);
+        bwd_fused(g, true, W, dY, X, dX, nullptr, ws, s, dp, st);
+        return st;
+    }
+    wgrad_direct(g, false, nullptr, nullptr, nullptr, nullptr, nullptr, dp, st);
+    if (workspace_bytes < dp.workspace_bytes)
+        return fail(CRB_EWORKSPACE, "crb_conv_bwd_sliced: workspace %zu bytes < required %zu", workspace_bytes, dp.workspace_bytes);
+    if (int sd = crb_conv_dgrad(W, dY, dX, g, stream)) return sd;
+    wgrad_direct(g, true, dY, X, nullptr, ws, s, dp, st);
+    return st;
+}
+
+int crb_sum_slices_multi(const crb_slice_sum_item *items, uint32_t n_items, void *stream) {
+    if (!items && n_items) return fail(CRB_ENULL, "crb_sum_slices_multi: null item list");
+    static_assert(sizeof(crb_slice_sum_item) == sizeof(SliceSumItem), "item layout");
+    for (uint32_t i = 0; i < n_items; ++i) {
+        if (!items[i].slices || !items[i].dst) return fail(CRB_ENULL, "crb_sum_slices_multi: item %u has a null pointer", i);
+        if (!items[i].count || !items[i].n_slices) return fail(CRB_EINVAL_SHAPE, "crb_sum_slices_multi: item %u is empty", i);
+        if (uint64_t(items[i].count) * items[i].n_slices > 0x7fffffffull)
+            return fail(CRB_EINVAL_SHAPE, "crb_sum_slices_multi: item %u exceeds 2^31 elements", i);
+    }
+    return launch_slice_sum_multi(reinterpret_cast<const SliceSumItem *>(items), n_items, hipStream_t(stream), "crb_sum_slices_multi");
 }
 
 int crb_conv_bias_grad(const float *dY, float *dB, uint32_t N, uint32_t C, uint32_t HW, void *stream) {

@@ -336,13 +336,13 @@ static __global__ void __launch_bounds__(256) splitk_reduce_kernel(const float *
 
 // Same reduction with 16-byte loads: OL lanes cover 4 * OL consecutive results of one slice (a full 128-byte line
 // or more), 256 / OL lanes walk the slices.  Needs count % 4 == 0 and 16-byte aligned pointers.
+// `red` = 256 / OL rows of 4 * OL + 4 floats of LDS; `block` = which group of 4 * OL results this workgroup sums.
 template <int OL>
-static __global__ void __launch_bounds__(256) splitk_reduce_vec_kernel(const float *__restrict__ partial, float *__restrict__ C,
-                                                                       u32 count, u32 splits, ReduceEpi e, FastDiv bdiv) {
-    constexpr u32 ZL = 256 / OL, OUTS = 4 * OL;
-    __shared__ float red[ZL][OUTS + 4];
+__device__ __forceinline__ void reduce_vec_block(const float *__restrict__ partial, float *__restrict__ C, u32 count, u32 splits,
+                                                 const ReduceEpi &e, const FastDiv &bdiv, u32 block, float *red) {
+    constexpr u32 ZL = 256 / OL, OUTS = 4 * OL, RS = OUTS + 4;
     const u32 o = threadIdx.x % OL, g = threadIdx.x / OL;
-    const u32 i = blockIdx.x * OUTS + 4 * o;
+    const u32 i = block * OUTS + 4 * o;
     float4 s0 = make_float4(0.f, 0.f, 0.f, 0.f), s1 = s0;
     if (i < count) {
         const float *p = partial + i;
@@ -358,34 +358,46 @@ static __global__ void __launch_bounds__(256) splitk_reduce_vec_kernel(const flo
             s0.x += a.x, s0.y += a.y, s0.z += a.z, s0.w += a.w;
         }
     }
-    *reinterpret_cast<float4 *>(&red[g][4 * o]) = make_float4(s0.x + s1.x, s0.y + s1.y, s0.z + s1.z, s0.w + s1.w);
+    *reinterpret_cast<float4 *>(&red[g * RS + 4 * o]) = make_float4(s0.x + s1.x, s0.y + s1.y, s0.z + s1.z, s0.w + s1.w);
     __syncthreads();
-    const u32 j = blockIdx.x * OUTS + threadIdx.x;
+    const u32 j = block * OUTS + threadIdx.x;
     if (threadIdx.x < OUTS && j < count) {
-        float r = red[0][threadIdx.x];
+        float r = red[threadIdx.x];
 #pragma unroll
-        for (u32 k = 1; k < ZL; ++k) r += red[k][threadIdx.x];
+        for (u32 k = 1; k < ZL; ++k) r += red[k * RS + threadIdx.x];
         if (e.bias) r += e.bias[bdiv.div(j) % e.bias_mod];
         if (e.flags & EPI_ACCUM) r += C[j];
         if (e.flags & EPI_RELU) r = r > 0.f ? r : 0.f;
         C[j] = r;
     }
 }
+constexpr int kReduceVecLds = 1152;  // floats: the largest of (256 / OL) * (4 * OL + 4) over OL = 8, 16, 32, 64
+
+template <int OL>
+static __global__ void __launch_bounds__(256) splitk_reduce_vec_kernel(const float *__restrict__ partial, float *__restrict__ C,
+                                                                       u32 count, u32 splits, ReduceEpi e, FastDiv bdiv) {
+    __shared__ __attribute__((aligned(16))) float red[(256 / OL) * (4 * OL + 4)];
+    reduce_vec_block<OL>(partial, C, count, splits, e, bdiv, blockIdx.x, red);
+}
+
+// Lanes per result row of the 16-byte form for a given problem: slice lanes ~ splits / 2, so that every lane has at
+// least two independent loads in flight. The association of the sum depends on this choice, so every caller asks here.
+inline __host__ __device__ u32 reduce_vec_ol(u32 count, u32 splits) {
+    return splits >= 64 ? 8u : (splits >= 32 ? 16u : ((splits >= 16 || count < 256u * 512u) ? 32u : 64u));
+}
+inline bool reduce_vec_ok(const float *partial, u32 count) { return count % 4 == 0 && reinterpret_cast<uintptr_t>(partial) % 16 == 0; }
 
 inline int launch_splitk_reduce(const float *partial, float *C, u32 count, u32 splits, ReduceEpi e, hipStream_t s,
                                 const char *what) {
     FastDiv bdiv(e.bias_div ? e.bias_div : 1);
     if (!e.bias_mod) e.bias_mod = 1;
-    if (count % 4 == 0 && reinterpret_cast<uintptr_t>(partial) % 16 == 0) {
-        // slice lanes ~ splits / 2, so every lane has at least two independent loads in flight
-        if (splits >= 64)
-            hipLaunchKernelGGL(splitk_reduce_vec_kernel<8>, dim3(ceil_div(count, 32)), dim3(256), 0, s, partial, C, count, splits, e, bdiv);
-        else if (splits >= 32)
-            hipLaunchKernelGGL(splitk_reduce_vec_kernel<16>, dim3(ceil_div(count, 64)), dim3(256), 0, s, partial, C, count, splits, e, bdiv);
-        else if (splits >= 16 || count < 256u * 512u)
-            hipLaunchKernelGGL(splitk_reduce_vec_kernel<32>, dim3(ceil_div(count, 128)), dim3(256), 0, s, partial, C, count, splits, e, bdiv);
-        else
-            hipLaunchKernelGGL(splitk_reduce_vec_kernel<64>, dim3(ceil_div(count, 256)), dim3(256), 0, s, partial, C, count, splits, e, bdiv);
+    if (reduce_vec_ok(partial, count)) {
+        switch (reduce_vec_ol(count, splits)) {
+            case 8: hipLaunchKernelGGL(splitk_reduce_vec_kernel<8>, dim3(ceil_div(count, 32)), dim3(256), 0, s, partial, C, count, splits, e, bdiv); break;
+            case 16: hipLaunchKernelGGL(splitk_reduce_vec_kernel<16>, dim3(ceil_div(count, 64)), dim3(256), 0, s, partial, C, count, splits, e, bdiv); break;
+            case 32: hipLaunchKernelGGL(splitk_reduce_vec_kernel<32>, dim3(ceil_div(count, 128)), dim3(256), 0, s, partial, C, count, splits, e, bdiv); break;
+            default: hipLaunchKernelGGL(splitk_reduce_vec_kernel<64>, dim3(ceil_div(count, 256)), dim3(256), 0, s, partial, C, count, splits, e, bdiv); break;
+        }
         return check_launch(what);
     }
     // enough workgroups to cover the chip even when the result is small
@@ -396,6 +408,68 @@ inline int launch_splitk_reduce(const float *partial, float *C, u32 count, u32 s
     else
         hipLaunchKernelGGL(splitk_reduce_kernel<8>, dim3(ceil_div(count, 8)), dim3(256), 0, s, partial, C, count, splits, e, bdiv);
     return check_launch(what);
+}
+
+// The same accumulating reduction for many results in one launch: dst += sum over its slices, item by item, each with
+// the association launch_splitk_reduce would use for it (bit-identical results). The items travel in the kernel
+// arguments; a workgroup finds its item by its first-block table.
+struct SliceSumItem {
+    const float *slices;
+    float *dst;
+    u32 count, n_slices;
+};
+constexpr int kSliceSumItems = 96;
+struct SliceSumArgs {
+    SliceSumItem item[kSliceSumItems];
+    u32 first_block[kSliceSumItems + 1];
+    u32 n;
+};
+static __global__ void __launch_bounds__(256) slice_sum_multi_kernel(SliceSumArgs a) {
+    __shared__ __attribute__((aligned(16))) float red[kReduceVecLds];
+    u32 lo = 0, hi = a.n;  // last item whose first block is <= blockIdx.x
+    while (hi - lo > 1) {
+        const u32 mid = (lo + hi) / 2;
+        if (a.first_block[mid] <= blockIdx.x) lo = mid; else hi = mid;
+    }
+    const SliceSumItem it = a.item[lo];
+    const u32 block = blockIdx.x - a.first_block[lo];
+    const ReduceEpi e{nullptr, 1, 1, EPI_ACCUM};
+    const FastDiv bdiv;
+    switch (reduce_vec_ol(it.count, it.n_slices)) {
+        case 8: reduce_vec_block<8>(it.slices, it.dst, it.count, it.n_slices, e, bdiv, block, red); break;
+        case 16: reduce_vec_block<16>(it.slices, it.dst, it.count, it.n_slices, e, bdiv, block, red); break;
+        case 32: reduce_vec_block<32>(it.slices, it.dst, it.count, it.n_slices, e, bdiv, block, red); break;
+        default: reduce_vec_block<64>(it.slices, it.dst, it.count, it.n_slices, e, bdiv, block, red); break;
+    }
+}
+
+// items: host memory. Items the 16-byte form cannot take are reduced by launches of their own.
+inline int launch_slice_sum_multi(const SliceSumItem *items, u32 n_items, hipStream_t s, const char *what) {
+    SliceSumArgs a;
+    a.n = 0;
+    u32 blocks = 0;
+    auto flush = [&]() -> int {
+        if (!a.n) return CRB_OK;
+        a.first_block[a.n] = blocks;
+        hipLaunchKernelGGL(slice_sum_multi_kernel, dim3(blocks), dim3(256), 0, s, a);
+        a.n = 0, blocks = 0;
+        return check_launch(what);
+    };
+    for (u32 i = 0; i < n_items; ++i) {
+        const SliceSumItem &it = items[i];
+        if (!reduce_vec_ok(it.slices, it.count) || reinterpret_cast<uintptr_t>(it.dst) % 4 != 0) {
+            if (int st = launch_splitk_reduce(it.slices, it.dst, it.count, it.n_slices, ReduceEpi{nullptr, 1, 1, EPI_ACCUM}, s, what)) return st;
+            continue;
+        }
+        const u32 nb = ceil_div(it.count, 4 * reduce_vec_ol(it.count, it.n_slices));
+        if (a.n == u32(kSliceSumItems) || blocks + nb > 0x3fffffffu)
+            if (int st = flush()) return st;
+        a.item[a.n] = it;
+        a.first_block[a.n] = blocks;
+        blocks += nb;
+        ++a.n;
+    }
+    return flush();
 }
 
 // How to cut K when an M x N result gives too few macro-tiles to occupy 256 CUs.

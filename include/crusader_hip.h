@@ -142,6 +142,24 @@ int crb_conv_bias(float *Y, const float *bias, uint32_t N, uint32_t C, uint32_t 
 int crb_conv_bwd(const float *W, const float *dY, const float *X, float *dX, float *dW, const crb_conv_geom *g, void *workspace,
                  size_t workspace_bytes, void *stream);
 
+/* The backward call with the weight gradient's last step postponed, for callers that need dW only when the optimizer
+ * runs (no counterpart in the reference). crb_conv_bwd_sliced writes dX as crb_conv_bwd does and leaves the weight
+ * gradient of this call as crb_conv_bwd_slices(g) partial sums ("slices", each OC*IC*FH*FW floats, one after the other)
+ * in `workspace` (caller-owned, crb_conv_wgrad_workspace_bytes(g) bytes, 16-byte aligned, not shared with another pending
+ * call). crb_conv_bwd_slices returns 0 for geometries without a sliced form: use crb_conv_bwd for those.
+ * crb_sum_slices_multi then completes any number of such gradients in one launch: for every item,
+ * dst[i] += sum over z of slices[z*count + i]; `items` is host memory. The summation order per element is the one
+ * crb_conv_wgrad / crb_conv_bwd use internally, so the results are bit-identical to theirs. */
+typedef struct crb_slice_sum_item {
+    const float *slices;
+    float *dst;
+    uint32_t count, n_slices;
+} crb_slice_sum_item;
+uint32_t crb_conv_bwd_slices(const crb_conv_geom *g);
+int crb_conv_bwd_sliced(const float *W, const float *dY, const float *X, float *dX, const crb_conv_geom *g, void *workspace,
+                        size_t workspace_bytes, void *stream);
+int crb_sum_slices_multi(const crb_slice_sum_item *items, uint32_t n_items, void *stream);
+
 /* Bias gradient of a conv operand: dB[c] += sum_{n,h,w} dY[n,c,h,w], each element updated exactly once.
  * Stands in for the channelReduce call of Conv2D::paramGrads (seann/operands/seblas/Conv2D.cu:26-28), whose
  * size assertion (seblas/operations/cuReduce.cu:237) cannot hold for a C-element bias; this computes the

@@ -341,3 +341,69 @@ def test_conv_bwd_errors(dev):
     assert lib.crb_conv_bwd(p, p, p, None, p, ctypes.byref(g), None, 0, None) == capi.CRB_ENULL
     g = capi.ConvGeom.make(1, 2, 8, 8, 2, 3, 3, 1, 1, 1, 1, OH=7, OW=8)
     assert lib.crb_conv_bwd(p, p, p, p, p, ctypes.byref(g), None, 0, None) == capi.CRB_EINVAL_SHAPE
+
+
+def test_conv_bwd_sliced_then_one_sum_equals_bwd(dev):
+    """Several layers' backward calls with the slice summation postponed, completed by ONE crb_sum_slices_multi launch:
+    bit-identical to crb_conv_bwd layer by layer (fused shapes, a direct-kernel shape outside the fused pairs, both strides)."""
+    import torch
+    capi = _capi()
+    specs = [(128, 16, 32, 16, 1), (128, 32, 16, 32, 1), (128, 64, 8, 64, 1), (128, 16, 32, 32, 2), (128, 32, 16, 64, 2),
+             (16, 64, 32, 64, 1), (32, 128, 8, 128, 1), (8, 16, 32, 16, 1), (64, 48, 16, 12, 1)]
+    layers, entries = [], []
+    for i, (N, IC, H, OC, s) in enumerate(specs):
+        g = capi.ConvGeom.make(N, IC, H, H, OC, 3, 3, s, s, 1, 1)
+        n_slices = capi.conv_bwd_slices(g)
+        assert n_slices > 1, specs[i]
+        X, W = to_dev(normal(10 + i, N, IC, H, H), dev), to_dev(he_normal(30 + i, OC, IC, 3, 3), dev)
+        dY, dW0 = to_dev(normal(50 + i, N, OC, g.OH, g.OW), dev), normal(70 + i, OC, IC, 3, 3)
+        ws = torch.empty(capi.conv_wgrad_workspace_bytes(g) // 4, dtype=torch.float32, device=dev)
+        assert ws.numel() == n_slices * OC * IC * 9
+        dX1, dW1 = _nan(dev, N, IC, H, H), to_dev(dW0, dev)
+        capi.conv_bwd(W, dY, X, dX1, dW1, g)
+        dX2, dW2 = _nan(dev, N, IC, H, H), to_dev(dW0, dev)
+        capi.conv_bwd_sliced(W, dY, X, dX2, g, ws)
+        layers.append((dX1, dW1, dX2, dW2, dW0))
+        entries.append((ws, dW2, n_slices))
+    torch.cuda.synchronize()
+    for (dX1, dW1, dX2, dW2, dW0) in layers:  # before the sum: dX complete, dW untouched
+        assert np.array_equal(to_np(dX1), to_np(dX2)) and np.array_equal(to_np(dW2), dW0)
+    table = capi.slice_sum_table(entries)
+    capi.sum_slices_multi(table)
+    torch.cuda.synchronize()
+    for k, (dX1, dW1, dX2, dW2, dW0) in enumerate(layers):
+        assert np.array_equal(to_np(dW1), to_np(dW2)), specs[k]
+
+
+def test_conv_bwd_sliced_many_items_and_errors(dev):
+    import ctypes
+    import torch
+    capi = _capi()
+    lib = capi.load()
+    # more items than one launch carries (96), of mixed sizes, against a plain sum
+    rng = np.random.default_rng(3)
+    entries, refs = [], []
+    for i in range(130):
+        count, n = int(rng.choice([2304, 9216, 36864, 432, 100, 6])), int(rng.choice([2, 7, 16, 33, 64, 256]))
+        sl = rng.standard_normal((n, count)).astype(np.float32)
+        d0 = rng.standard_normal(count).astype(np.float32)
+        ws, dst = to_dev(sl, dev), to_dev(d0, dev)
+        entries.append((ws, dst, n))
+        refs.append(d0 + sl.astype(np.float64).sum(axis=0))
+    capi.sum_slices_multi(capi.slice_sum_table(entries))
+    torch.cuda.synchronize()
+    for (ws, dst, n), ref in zip(entries, refs):
+        assert_close(to_np(dst), ref, n, "slice sum")
+    # geometries without a sliced form
+    assert capi.conv_bwd_slices(capi.ConvGeom.make(4, 24, 8, 8, 12, 1, 1, 1, 1, 0, 0)) == 0
+    assert capi.conv_bwd_slices(capi.ConvGeom.make(4, 16, 12, 12, 8, 3, 3, 1, 1, 1, 1)) == 0
+    t = torch.zeros(1 << 16, device=dev)
+    p = t.data_ptr()
+    g = capi.ConvGeom.make(4, 16, 12, 12, 8, 3, 3, 1, 1, 1, 1)
+    assert lib.crb_conv_bwd_sliced(p, p, p, p, ctypes.byref(g), p, 1 << 18, None) == capi.CRB_EINVAL_SHAPE
+    g = capi.ConvGeom.make(64, 16, 32, 32, 16, 3, 3, 1, 1, 1, 1)
+    assert lib.crb_conv_bwd_sliced(p, p, p, p, ctypes.byref(g), p, 64, None) == capi.CRB_EWORKSPACE
+    assert lib.crb_conv_bwd_sliced(p, p, p, p, ctypes.byref(g), None, 0, None) == capi.CRB_ENULL
+    bad = (capi.SliceSumItem * 1)(capi.SliceSumItem(p, None, 16, 2))
+    assert lib.crb_sum_slices_multi(ctypes.cast(bad, ctypes.c_void_p), 1, None) == capi.CRB_ENULL
+    assert lib.crb_sum_slices_multi(None, 0, None) == 0
