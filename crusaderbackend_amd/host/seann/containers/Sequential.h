@@ -48,12 +48,14 @@ public:
     void pruneReserveFolds() const;
     // streamline: pruneReserveFolds plus letting every opening shortcut endpoint's output value alias its input (it only
     // passes it on), which removes one device copy per residual block from the forward pass, plus letting each convolution's
-    // xGrads compute the filter gradient in the same launch as the input gradient (backward() calls the two as a pair).
+    // xGrads compute the filter gradient in the same launch as the input gradient (backward() calls the two as a pair) and
+    // leave its last step, the sum of its partial results, to one launch for all convolutions at the end of backward().
     void streamline() const;
     // learnFused: the momentum step of every parameter in one kernel launch instead of one launch per parameter.
     void learnFused();
 
 private:
+    mutable std::vector<seblas::SliceSumItem> sliceItems;  // filter gradients left as partial sums by xGrads (streamline())
     void *fusedTable = nullptr;    // device copy of the parameter table used by learnFused
     std::vector<char> fusedHost;   // its host image, to detect changed rates
 };

@@ -16,6 +16,7 @@ public:
     bool WITH_BIAS = false;
     bool gradsFused = false;      // xGrads computes the filter gradient too (fuseGrads())
     bool filterGradDone = false;  // ... and has done so since the last forward / paramGrads
+    Tensor *gradSlices = nullptr;  // deferSliceSum(): xGrads leaves the filter gradient here as partial sums
 
     Conv2D(shape4 filterShape, uint32 strideH, uint32 strideW, uint32 padH, uint32 padW, bool WITH_BIAS)
         : filterShape(filterShape), strideH(strideH), strideW(strideW), padH(padH), padW(padW), WITH_BIAS(WITH_BIAS) {}
@@ -44,6 +45,7 @@ public:
         if (WITH_BIAS) out.push_back(bias);
     }
     void fuseGrads() override { gradsFused = true; }
+    void deferSliceSum(std::vector<seblas::SliceSumItem> &items) override;
     uint32 OPERAND_ID() override { return OPR_SEBLAS_CONV2D; }
     // info: filter dims, strides, paddings, has-bias flag (36 bytes); params: filter, then bias (Conv2D.cu:59-80)
     uint32 encodeInfo(std::fstream *fout, uint64 offset) override;

@@ -51,6 +51,10 @@ public:
     // Lets xGrads also produce the parameter gradients where one launch can compute both; the paramGrads call that follows
     // it in Sequential::backward then finds them done. Only for callers that always pair the two calls (Sequential does).
     virtual void fuseGrads() {}
+    // Lets xGrads leave the parameter gradient as partial sums and adds what completes them to `items`; the caller sums all
+    // items in one launch after the last xGrads of a backward pass (Sequential::backward does, once streamline() was
+    // called). An operand that has added an item must from then on be driven that way.
+    virtual void deferSliceSum(std::vector<seblas::SliceSumItem> &) {}
 
     // Y->dA += Y->dAReserve and the reserve is cleared, in one pass (the reference clears it after the gradient call, which
     // never reads it): the first thing every xGrads does

@@ -58,6 +58,9 @@ public:
     void fuseGrads() override {
         for (OperandBase *op : branchOperands) op->fuseGrads();
     }
+    void deferSliceSum(std::vector<seblas::SliceSumItem> &items) override {
+        for (OperandBase *op : branchOperands) op->deferSliceSum(items);
+    }
     std::string info() override { return "ShortcutEndpoint { " + std::to_string(operandCount) + " }"; }
     uint32 OPERAND_ID() override { return isContainer ? OPR_CTRL_SHORTCUTENDPOINT_END : OPR_CTRL_SHORTCUTENDPOINT_BEG; }
     // info: uuid, branch operand count, then for a closing endpoint the branch's type ids and infos; params: the branch's

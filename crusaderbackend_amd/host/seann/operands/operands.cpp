@@ -32,6 +32,11 @@ void Conv2D::forward() {  // Conv2D.cu:8-16
 
 void Conv2D::xGrads() {  // Conv2D.cu:18-22
     foldReserve();
+    if (gradSlices) {  // both gradients in one call, the filter gradient as partial sums that the caller completes
+        convBackwardSliced(filter->data(), Y->dA, X->A, X->dA, gradSlices, int(strideH), int(strideW), int(padH), int(padW));
+        filterGradDone = true;
+        return;
+    }
     if (gradsFused) {  // both gradients in one call; paramGrads then only adds the bias gradient
         convBackward(filter->data(), Y->dA, X->A, X->dA, filter->grad(), int(strideH), int(strideW), int(padH), int(padW));
         filterGradDone = true;
@@ -49,6 +54,14 @@ void Conv2D::paramGrads() {  // Conv2D.cu:24-29; the bias gradient is the per-ch
                       __LINE__);
         if (isBlocking() && hipStreamSynchronize(nullptr) != hipSuccess) assertHip(__FILE__, __LINE__);
     }
+}
+
+void Conv2D::deferSliceSum(std::vector<seblas::SliceSumItem> &items) {
+    if (gradSlices) return;
+    const uint32 n = convBackwardSlices(filter->data(), Y->dA, X->dA, int(strideH), int(strideW), int(padH), int(padW));
+    if (!n) return;  // no sliced form for this shape: xGrads keeps summing on its own
+    gradSlices = Tensor::create(shape4(1, convBackwardSliceFloats(filter->data(), Y->dA, X->dA, int(strideH), int(strideW), int(padH), int(padW))));
+    items.push_back(seblas::SliceSumItem{gradSlices->elements, filter->grad()->elements, filter->grad()->dims.size, n});
 }
 
 void Conv2D::randFillNetParams() {  // Conv2D.cu:45-50: N(0, sqrt(2/K)), K = IC*FH*FW; bias N(0, sqrt(2/OC))
@@ -236,6 +249,7 @@ Tensor *Sequential::backward(Tensor *label) const {
         operands[i]->xGrads();
         operands[i]->paramGrads();
     }
+    if (!sliceItems.empty()) sumSlicesMulti(sliceItems.data(), uint32(sliceItems.size()));
     return netX->dA;
 }
 
@@ -258,6 +272,8 @@ void Sequential::pruneReserveFolds() const {
 void Sequential::streamline() const {
     pruneReserveFolds();
     for (OperandBase *op : operands) op->fuseGrads();  // backward() always calls xGrads and paramGrads as a pair
+    sliceItems.clear();
+    for (OperandBase *op : operands) op->deferSliceSum(sliceItems);  // ... and sums all convolutions' slices at its end
     if (hipDeviceSynchronize() != hipSuccess) assertHip(__FILE__, __LINE__);  // buffers are released below: nothing may be in flight
     for (uint32 i = 0; i + 1 < OPERAND_COUNT; i++) {
         OperandBase *op = operands[i];

@@ -133,6 +133,29 @@ void convBackward(Tensor *filter, Tensor *dY, Tensor *X, Tensor *dX, Tensor *dFi
            __FILE__, __LINE__);
 }
 
+uint32 convBackwardSlices(Tensor *filter, Tensor *dY, Tensor *dX, int strideH, int strideW, int padH, int padW) {
+    crb_conv_geom g = geom(filter, dX, dY, strideH, strideW, padH, padW);
+    return crb_conv_bwd_slices(&g);
+}
+
+uint32 convBackwardSliceFloats(Tensor *filter, Tensor *dY, Tensor *dX, int strideH, int strideW, int padH, int padW) {
+    crb_conv_geom g = geom(filter, dX, dY, strideH, strideW, padH, padW);
+    return uint32(crb_conv_wgrad_workspace_bytes(&g) / sizeof(float));
+}
+
+void convBackwardSliced(Tensor *filter, Tensor *dY, Tensor *X, Tensor *dX, Tensor *slices, int strideH, int strideW, int padH, int padW) {
+    crb_conv_geom g = geom(filter, dX, dY, strideH, strideW, padH, padW);
+    require(X->dims == dX->dims, "convBackwardSliced: gradient shape differs from its tensor");
+    finish(crb_conv_bwd_sliced(filter->elements, dY->elements, X->elements, dX->elements, &g, slices->elements,
+                               size_t(slices->dims.size) * sizeof(float), nullptr),
+           __FILE__, __LINE__);
+}
+
+void sumSlicesMulti(const SliceSumItem *items, uint32 count) {
+    static_assert(sizeof(SliceSumItem) == sizeof(crb_slice_sum_item), "item layout");
+    finish(crb_sum_slices_multi(reinterpret_cast<const crb_slice_sum_item *>(items), count, nullptr), __FILE__, __LINE__);
+}
+
 Tensor *convBias(Tensor *Y, Tensor *biases) {
     require(biases->dims.size == Y->dims.c, "convBias: bias size != channels");  // cuConv.cu:809
     finish(crb_conv_bias(Y->elements, biases->elements, Y->dims.n, Y->dims.c, Y->dims.h * Y->dims.w, nullptr), __FILE__,

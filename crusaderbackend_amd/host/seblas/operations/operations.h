@@ -33,6 +33,19 @@ Tensor *convError(Tensor *A, Tensor *B, Tensor *C, int strideH, int strideW, int
 // and, for the layer shapes of CIFAR residual networks, run as one kernel launch. Same results as the two calls. No
 // counterpart in the reference.
 void convBackward(Tensor *filter, Tensor *dY, Tensor *X, Tensor *dX, Tensor *dFilter, int strideH, int strideW, int padH, int padW);
+// The same with the filter gradient's last step postponed: convBackwardSliced writes dX and leaves the filter gradient of
+// this call as convBackwardSlices(...) partial sums in `slices` (a device tensor of convBackwardSliceFloats(...) floats
+// that the caller keeps until the sum); sumSlicesMulti then completes any number of such gradients in one launch
+// (grad += sum of its slices; same bits as convBackward). convBackwardSlices returns 0 where there is no sliced form.
+struct SliceSumItem {  // layout of crb_slice_sum_item
+    const float *slices;
+    float *dst;
+    uint32 count, n_slices;
+};
+uint32 convBackwardSlices(Tensor *filter, Tensor *dY, Tensor *dX, int strideH, int strideW, int padH, int padW);
+uint32 convBackwardSliceFloats(Tensor *filter, Tensor *dY, Tensor *dX, int strideH, int strideW, int padH, int padW);
+void convBackwardSliced(Tensor *filter, Tensor *dY, Tensor *X, Tensor *dX, Tensor *slices, int strideH, int strideW, int padH, int padW);
+void sumSlicesMulti(const SliceSumItem *items, uint32 count);
 Tensor *convBias(Tensor *Y, Tensor *biases);
 
 // ---- the elementwise / reduction operators a training step runs between those calls -------------------------------

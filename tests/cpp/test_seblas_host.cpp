@@ -521,12 +521,18 @@ static void gpu_sequential_tests() {
     // two separate calls, gradient accumulation included
     {
         const uint32_t B = 8;
-        auto run = [&](bool fused, std::vector<float> &dx, std::vector<float> &dw, std::vector<float> &db) {
+        auto run = [&](int mode, std::vector<float> &dx, std::vector<float> &dw, std::vector<float> &db) {
+            const bool fused = mode >= 1, sliced = mode == 2;
+            std::vector<seblas::SliceSumItem> items;
             auto *cv = new Conv2D(shape4(16, 16, 3, 3), 1, 1, 1, 1, true);
             cv->initNetParams(nullptr, shape4(B, 16, 32, 32));
             cv->randFillNetParams();
             cv->X->instantiate();  // stand-alone operand: it owns its input
             if (fused) cv->fuseGrads();
+            if (sliced) {
+                cv->deferSliceSum(items);
+                CHECK(items.size() == 1 && items[0].n_slices > 1 && items[0].count == 16 * 16 * 9);
+            }
             auto xin = randn(B * 16 * 32 * 32, 61), dy = randn(B * 16 * 32 * 32, 62), g0 = randn(16 * 16 * 9, 63);
             CHECK(hipMemcpy(cv->X->A->elements, xin.data(), xin.size() * 4, hipMemcpyHostToDevice) == hipSuccess);
             CHECK(hipMemcpy(cv->filter->grad()->elements, g0.data(), g0.size() * 4, hipMemcpyHostToDevice) == hipSuccess);
@@ -534,16 +540,22 @@ static void gpu_sequential_tests() {
             CHECK(hipMemcpy(cv->Y->dA->elements, dy.data(), dy.size() * 4, hipMemcpyHostToDevice) == hipSuccess);
             cv->xGrads();
             cv->paramGrads();
+            if (sliced) {  // the filter gradient is still what it was until the slices are summed
+                CHECK(pull(cv->filter->grad()) == g0);
+                sumSlicesMulti(items.data(), uint32_t(items.size()));
+            }
             dx = pull(cv->X->dA), dw = pull(cv->filter->grad()), db = pull(cv->bias->grad());
             if (fused) {  // paramGrads on its own still computes the filter gradient
                 cv->paramGrads();
                 CHECK(pull(cv->filter->grad()) != dw);
             }
         };
-        std::vector<float> dx1, dw1, db1, dx2, dw2, db2;
-        run(false, dx1, dw1, db1);
-        run(true, dx2, dw2, db2);
+        std::vector<float> dx1, dw1, db1, dx2, dw2, db2, dx3, dw3, db3;
+        run(0, dx1, dw1, db1);
+        run(1, dx2, dw2, db2);
+        run(2, dx3, dw3, db3);
         CHECK(dx1 == dx2 && dw1 == dw2 && db1 == db2);
+        CHECK(dx1 == dx3 && dw1 == dw3 && db1 == db3);
     }
     // the non-blocking mode gives the same numbers
     setBlocking(false);
