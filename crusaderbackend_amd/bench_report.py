@@ -38,7 +38,7 @@ def run(torch, capi, dev, event_time_ms, Layer):
             L = Layer(torch, capi, dev, name, IC, H, OC, s, 1, seed=100 + i, batch=batch, F=F, pad=p, bias=bias)
             entries = {}
             for pname, fn, fl, _ in L.passes():
-                if pname == "bwd" and key != "resnet56":  # the one-call form of both gradients: residual-network shapes
+                if pname in ("bwd", "bwd_sliced") and key != "resnet56":  # the one-call forms of both gradients: residual-network shapes
                     continue
                 reps = 30 if L.flops < 2e9 else 10
                 entries[pname] = _entry(f"{name}.{pname}", event_time_ms(torch, fn, reps=reps), fl, L.bytes[pname])

@@ -312,7 +312,7 @@ template <int FL>
 __global__ void __launch_bounds__(256) batchnorm_fwd_kernel(const float *__restrict__ X, const float *__restrict__ beta,
                                                             const float *__restrict__ gamma, float *__restrict__ mean,
                                                             float *__restrict__ var, float *__restrict__ Y, float *__restrict__ xHat,
-                                                            u32 N, u32 F) {
+                                                            float *__restrict__ reluOut, u32 N, u32 F) {
     constexpr u32 G = 256 / FL;
     __shared__ float red[G][FL];
     const BnGeom<FL> t(F);
@@ -348,22 +348,21 @@ __global__ void __launch_bounds__(256) batchnorm_fwd_kernel(const float *__restr
     const float v = t.reduce(q, red) / float(N);
     if (!t.on) return;
     const float inv = 1.0f / sqrtf(v + 1e-8f), ga = gamma[t.f], be = beta[t.f];
+    // outputs a caller does not need are not written: Y and xHat may be null, reluOut = max(Y, 0) is optional
+    auto put = [&](u32 n, float xh) {
+        const float y = xh * ga + be;
+        if (xHat) xHat[size_t(n) * F + t.f] = xh;
+        if (Y) Y[size_t(n) * F + t.f] = y;
+        if (reluOut) reluOut[size_t(n) * F + t.f] = y > 0.f ? y : 0.f;
+    };
     if (cached) {
 #pragma unroll
         for (int i = 0; i < kBnCache; ++i) {
             const u32 n = t.g + G * i;
-            if (n < N) {
-                const float xh = (xv[i] - m) * inv;
-                xHat[size_t(n) * F + t.f] = xh;
-                Y[size_t(n) * F + t.f] = xh * ga + be;
-            }
+            if (n < N) put(n, (xv[i] - m) * inv);
         }
     } else {
-        for (u32 n = t.g; n < N; n += G) {
-            const float xh = (x[size_t(n) * F] - m) * inv;
-            xHat[size_t(n) * F + t.f] = xh;
-            Y[size_t(n) * F + t.f] = xh * ga + be;
-        }
+        for (u32 n = t.g; n < N; n += G) put(n, (x[size_t(n) * F] - m) * inv);
     }
     if (t.g == 0) mean[t.f] = m, var[t.f] = v;
 }
@@ -371,12 +370,20 @@ __global__ void __launch_bounds__(256) batchnorm_fwd_kernel(const float *__restr
 template <int FL>
 __global__ void __launch_bounds__(256) batchnorm_bwd_kernel(const float *__restrict__ dY, const float *__restrict__ gamma,
                                                             const float *__restrict__ X, float *__restrict__ dX,
-                                                            float *__restrict__ dGamma, float *__restrict__ dBeta, u32 N, u32 F) {
+                                                            float *__restrict__ dGamma, float *__restrict__ dBeta,
+                                                            const float *__restrict__ reluOut, u32 N, u32 F) {
     constexpr u32 G = 256 / FL;
     __shared__ float red[G][FL];
     const BnGeom<FL> t(F);
     const bool cached = N <= G * kBnCache;
     const float *x = X + (t.on ? t.f : 0), *dy = dY + (t.on ? t.f : 0);
+    // reluOut given: dY is the gradient behind a ReLU whose output is reluOut, so the gradient that reaches this
+    // normalisation is dY where reluOut > 0 and 0 elsewhere
+    const float *mk = reluOut ? reluOut + (t.on ? t.f : 0) : nullptr;
+    auto grad = [&](u32 n) -> float {
+        const float e = dy[size_t(n) * F];
+        return (mk && !(mk[size_t(n) * F] > 0.f)) ? 0.f : e;
+    };
     float xv[kBnCache], dv[kBnCache];
     float s = 0.f;
     if (cached) {
@@ -385,7 +392,7 @@ __global__ void __launch_bounds__(256) batchnorm_bwd_kernel(const float *__restr
             const u32 n = t.g + G * i;
             const bool ok = t.on && n < N;
             xv[i] = ok ? x[size_t(n) * F] : 0.f;
-            dv[i] = ok ? dy[size_t(n) * F] : 0.f;
+            dv[i] = ok ? grad(n) : 0.f;
         }
 #pragma unroll
         for (int i = 0; i < kBnCache; ++i) s += xv[i];
@@ -404,7 +411,7 @@ __global__ void __launch_bounds__(256) batchnorm_bwd_kernel(const float *__restr
         }
     } else if (t.on) {
         for (u32 n = t.g; n < N; n += G) {
-            const float d = x[size_t(n) * F] - m, e = dy[size_t(n) * F];
+            const float d = x[size_t(n) * F] - m, e = grad(n);
             q += d * d, sdd += e * d, sdy += e, sd += d;
         }
     }
@@ -424,7 +431,7 @@ __global__ void __launch_bounds__(256) batchnorm_bwd_kernel(const float *__restr
         }
     } else {
         for (u32 n = t.g; n < N; n += G)
-            dX[size_t(n) * F + t.f] = dy[size_t(n) * F] * ga * inv + dVar * (x[size_t(n) * F] - m) * 2.0f * invN + dMean * invN;
+            dX[size_t(n) * F + t.f] = grad(n) * ga * inv + dVar * (x[size_t(n) * F] - m) * 2.0f * invN + dMean * invN;
     }
 }
 
@@ -608,32 +615,54 @@ int crb_tensor_scale_inplace(float *a, float factor, uint32_t count, void *strea
     return launch_map2(a, nullptr, a, count, ScaleF{factor}, hipStream_t(stream), "crb_tensor_scale_inplace");
 }
 
+static int bn_fwd(const char *what, const float *X, const float *beta, const float *gamma, float *mean, float *var, float *Y,
+                  float *xHat, float *reluOut, uint32_t N, uint32_t F, void *stream) {
+    if (int st = check_bn(what, N, F)) return st;
+    hipStream_t s = hipStream_t(stream);
+    switch (bn_features_per_wg(F)) {
+        case 64: hipLaunchKernelGGL(batchnorm_fwd_kernel<64>, dim3(ceil_div(F, 64)), dim3(256), 0, s, X, beta, gamma, mean, var, Y, xHat, reluOut, N, F); break;
+        case 32: hipLaunchKernelGGL(batchnorm_fwd_kernel<32>, dim3(ceil_div(F, 32)), dim3(256), 0, s, X, beta, gamma, mean, var, Y, xHat, reluOut, N, F); break;
+        default: hipLaunchKernelGGL(batchnorm_fwd_kernel<16>, dim3(ceil_div(F, 16)), dim3(256), 0, s, X, beta, gamma, mean, var, Y, xHat, reluOut, N, F);
+    }
+    return check_launch(what);
+}
+
+static int bn_bwd(const char *what, const float *dY, const float *gamma, const float *X, float *dX, float *dGamma, float *dBeta,
+                  const float *reluOut, uint32_t N, uint32_t F, void *stream) {
+    if (int st = check_bn(what, N, F)) return st;
+    hipStream_t s = hipStream_t(stream);
+    switch (bn_features_per_wg(F)) {
+        case 64: hipLaunchKernelGGL(batchnorm_bwd_kernel<64>, dim3(ceil_div(F, 64)), dim3(256), 0, s, dY, gamma, X, dX, dGamma, dBeta, reluOut, N, F); break;
+        case 32: hipLaunchKernelGGL(batchnorm_bwd_kernel<32>, dim3(ceil_div(F, 32)), dim3(256), 0, s, dY, gamma, X, dX, dGamma, dBeta, reluOut, N, F); break;
+        default: hipLaunchKernelGGL(batchnorm_bwd_kernel<16>, dim3(ceil_div(F, 16)), dim3(256), 0, s, dY, gamma, X, dX, dGamma, dBeta, reluOut, N, F);
+    }
+    return check_launch(what);
+}
+
+int crb_batchnorm_relu_fwd(const float *X, const float *beta, const float *gamma, float *mean, float *var, float *Y_or_null,
+                           float *xHat_or_null, float *reluOut, uint32_t N, uint32_t F, void *stream) {
+    if (!X || !beta || !gamma || !mean || !var || !reluOut) return fail(CRB_ENULL, "crb_batchnorm_relu_fwd: null operand");
+    return bn_fwd("crb_batchnorm_relu_fwd", X, beta, gamma, mean, var, Y_or_null, xHat_or_null, reluOut, N, F, stream);
+}
+
+int crb_batchnorm_relu_bwd(const float *dY, const float *reluOut, const float *gamma, const float *X, float *dX, float *dGamma_or_null,
+                           float *dBeta_or_null, uint32_t N, uint32_t F, void *stream) {
+    if (!dY || !reluOut || !gamma || !X || !dX) return fail(CRB_ENULL, "crb_batchnorm_relu_bwd: null operand");
+    if (!dGamma_or_null != !dBeta_or_null) return fail(CRB_ENULL, "crb_batchnorm_relu_bwd: dGamma and dBeta go together");
+    return bn_bwd("crb_batchnorm_relu_bwd", dY, gamma, X, dX, dGamma_or_null, dBeta_or_null, reluOut, N, F, stream);
+}
+
 int crb_batchnorm_fwd(const float *X, const float *beta, const float *gamma, float *mean, float *var, float *Y, float *xHat,
                       uint32_t N, uint32_t F, void *stream) {
     if (!X || !beta || !gamma || !mean || !var || !Y || !xHat) return fail(CRB_ENULL, "crb_batchnorm_fwd: null operand");
-    if (int st = check_bn("crb_batchnorm_fwd", N, F)) return st;
-    hipStream_t s = hipStream_t(stream);
-    switch (bn_features_per_wg(F)) {
-        case 64: hipLaunchKernelGGL(batchnorm_fwd_kernel<64>, dim3(ceil_div(F, 64)), dim3(256), 0, s, X, beta, gamma, mean, var, Y, xHat, N, F); break;
-        case 32: hipLaunchKernelGGL(batchnorm_fwd_kernel<32>, dim3(ceil_div(F, 32)), dim3(256), 0, s, X, beta, gamma, mean, var, Y, xHat, N, F); break;
-        default: hipLaunchKernelGGL(batchnorm_fwd_kernel<16>, dim3(ceil_div(F, 16)), dim3(256), 0, s, X, beta, gamma, mean, var, Y, xHat, N, F);
-    }
-    return check_launch("crb_batchnorm_fwd");
+    return bn_fwd("crb_batchnorm_fwd", X, beta, gamma, mean, var, Y, xHat, nullptr, N, F, stream);
 }
 
 int crb_batchnorm_bwd(const float *dY, const float *gamma, const float *X, float *dX, float *dGamma_or_null, float *dBeta_or_null,
                       uint32_t N, uint32_t F, void *stream) {
     if (!dY || !gamma || !X || !dX) return fail(CRB_ENULL, "crb_batchnorm_bwd: null operand");
     if (!dGamma_or_null != !dBeta_or_null) return fail(CRB_ENULL, "crb_batchnorm_bwd: dGamma and dBeta go together");
-    float *dGamma = dGamma_or_null, *dBeta = dBeta_or_null;
-    if (int st = check_bn("crb_batchnorm_bwd", N, F)) return st;
-    hipStream_t s = hipStream_t(stream);
-    switch (bn_features_per_wg(F)) {
-        case 64: hipLaunchKernelGGL(batchnorm_bwd_kernel<64>, dim3(ceil_div(F, 64)), dim3(256), 0, s, dY, gamma, X, dX, dGamma, dBeta, N, F); break;
-        case 32: hipLaunchKernelGGL(batchnorm_bwd_kernel<32>, dim3(ceil_div(F, 32)), dim3(256), 0, s, dY, gamma, X, dX, dGamma, dBeta, N, F); break;
-        default: hipLaunchKernelGGL(batchnorm_bwd_kernel<16>, dim3(ceil_div(F, 16)), dim3(256), 0, s, dY, gamma, X, dX, dGamma, dBeta, N, F);
-    }
-    return check_launch("crb_batchnorm_bwd");
+    return bn_bwd("crb_batchnorm_bwd", dY, gamma, X, dX, dGamma_or_null, dBeta_or_null, nullptr, N, F, stream);
 }
 
 int crb_batchnorm_param_grads(const float *dY, const float *xHat, float *dGamma, float *dBeta, uint32_t N, uint32_t F,

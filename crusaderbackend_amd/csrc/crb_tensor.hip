@@ -64,7 +64,10 @@ __global__ void __launch_bounds__(256) copy_kernel(float *__restrict__ dst, cons
 }
 
 // Three-operand streaming forms used by the residual-connection operand. MODE 0: d = a + b. MODE 1: a += b; b = 0; d = a.
-// MODE 2: d = a; b = a (one source, two destinations).
+// MODE 2: d = a; b = a (one source, two destinations). MODE 3: d = max(a + b, 0).
+__device__ __forceinline__ float relu_of(float v) { return v > 0.f ? v : 0.f; }
+__device__ __forceinline__ v4f relu_of(v4f v) { return v4f{relu_of(v.x), relu_of(v.y), relu_of(v.z), relu_of(v.w)}; }
+
 template <int MODE>
 __global__ void __launch_bounds__(256) tri_kernel(float *d, float *a, float *b, u32 count, u32 vec) {
     const u32 stride = gridDim.x * 256;
@@ -75,9 +78,11 @@ __global__ void __launch_bounds__(256) tri_kernel(float *d, float *a, float *b, 
         } else if (MODE == 1) {
             const auto v = pa[k] + pb[k];
             pa[k] = v, pb[k] = zero, pd[k] = v;
-        } else {
+        } else if (MODE == 2) {
             const auto v = pa[k];
             pd[k] = v, pb[k] = v;
+        } else {
+            pd[k] = relu_of(pa[k] + pb[k]);
         }
     };
     if (vec) {
@@ -87,6 +92,24 @@ __global__ void __launch_bounds__(256) tri_kernel(float *d, float *a, float *b, 
         for (u32 r = nq * 4 + i; r < count; r += stride) one(d, a, b, r, 0.f);
     } else {
         for (; i < count; i += stride) one(d, a, b, i, 0.f);
+    }
+}
+
+// d1 = d2 = (mask > 0 ? src : 0): the gradient behind a ReLU whose output is `mask`, delivered to two consumers.
+__global__ void __launch_bounds__(256) relu_grad_copy2_kernel(float *d1, float *d2, const float *mask, const float *src, u32 count, u32 vec) {
+    const u32 stride = gridDim.x * 256;
+    u32 i = blockIdx.x * 256 + threadIdx.x;
+    auto pick = [](float m, float v) { return m > 0.f ? v : 0.f; };
+    if (vec) {
+        const u32 nq = count / 4;
+        for (u32 q = i; q < nq; q += stride) {
+            const v4f m = reinterpret_cast<const v4f *>(mask)[q], v = reinterpret_cast<const v4f *>(src)[q];
+            const v4f r = {pick(m.x, v.x), pick(m.y, v.y), pick(m.z, v.z), pick(m.w, v.w)};
+            reinterpret_cast<v4f *>(d1)[q] = r, reinterpret_cast<v4f *>(d2)[q] = r;
+        }
+        for (u32 k = nq * 4 + i; k < count; k += stride) d1[k] = d2[k] = pick(mask[k], src[k]);
+    } else {
+        for (; i < count; i += stride) d1[i] = d2[i] = pick(mask[i], src[i]);
     }
 }
 
@@ -138,6 +161,19 @@ int crb_tensor_copy(float *dst, const float *src, uint32_t count, void *stream) 
 
 int crb_tensor_add(float *dst, const float *a, const float *b, uint32_t count, void *stream) {
     return launch_tri<0>(dst, const_cast<float *>(a), const_cast<float *>(b), count, stream, "crb_tensor_add");
+}
+
+int crb_tensor_add_relu(float *dst, const float *a, const float *b, uint32_t count, void *stream) {
+    return launch_tri<3>(dst, const_cast<float *>(a), const_cast<float *>(b), count, stream, "crb_tensor_add_relu");
+}
+
+int crb_tensor_relu_grad_copy2(float *dst1, float *dst2, const float *relu_out, const float *dY, uint32_t count, void *stream) {
+    if (!dst1 || !dst2 || !relu_out || !dY) return fail(CRB_ENULL, "crb_tensor_relu_grad_copy2: null operand");
+    if (!count) return fail(CRB_EINVAL_SHAPE, "crb_tensor_relu_grad_copy2: zero size");
+    const u32 vec = ((reinterpret_cast<uintptr_t>(dst1) | reinterpret_cast<uintptr_t>(dst2) | reinterpret_cast<uintptr_t>(relu_out) |
+                      reinterpret_cast<uintptr_t>(dY)) & 15u) == 0;
+    hipLaunchKernelGGL(relu_grad_copy2_kernel, dim3(stream_grid(count)), dim3(256), 0, hipStream_t(stream), dst1, dst2, relu_out, dY, count, vec);
+    return check_launch("crb_tensor_relu_grad_copy2");
 }
 
 int crb_tensor_add_clear_copy(float *dst, float *a, float *b, uint32_t count, void *stream) {

@@ -49,7 +49,8 @@ public:
     // streamline: pruneReserveFolds plus letting every opening shortcut endpoint's output value alias its input (it only
     // passes it on), which removes one device copy per residual block from the forward pass, plus letting each convolution's
     // xGrads compute the filter gradient in the same launch as the input gradient (backward() calls the two as a pair) and
-    // leave its last step, the sum of its partial results, to one launch for all convolutions at the end of backward().
+    // leave its last step, the sum of its partial results, to one launch for all convolutions at the end of backward(), plus
+    // letting a batch normalisation or a closing shortcut endpoint compute the ReLU that follows it in its own passes.
     void streamline() const;
     // learnFused: the momentum step of every parameter in one kernel launch instead of one launch per parameter.
     void learnFused();

@@ -3,6 +3,8 @@
 // may have deposited in Y->dAReserve is folded into Y->dA first and cleared afterwards).
 // seann/operands/seblas/activate/ReLU.{cuh,cu}, pooling/MaxPool2D.{cuh,cu}, Softmax.{cuh,cu}.
 #pragma once
+#include <stdexcept>
+
 #include "OperandBase.h"
 
 #define OPR_SEBLAS_RELU 0xa002
@@ -31,10 +33,13 @@ public:
         X = Parameter::declare(inShape);
         Y = Parameter::create(inShape);
     }
-    void forward() override { relu(X->A, Y->A); }  // ReLU.cu:8-10
-    void xGrads() override {                         // ReLU.cu:13-17
+    OperandBase *absorbedBy = nullptr;  // set by Sequential::streamline(): the predecessor computes this operand's passes
+    void forward() override {             // ReLU.cu:8-10
+        if (!absorbedBy) relu(X->A, Y->A);
+    }
+    void xGrads() override {  // ReLU.cu:13-17
         foldReserve();
-        reluGradFast(X->A, Y->dA, X->dA);
+        if (!absorbedBy) reluGradFast(X->A, Y->dA, X->dA);
     }
     uint32 OPERAND_ID() override { return OPR_SEBLAS_RELU; }
 };
@@ -73,6 +78,11 @@ public:
     Tensor *variance{};
     Tensor *xHatP{};
     bool paramGradsDone = false;
+    OperandBase *fusedRelu = nullptr;  // the ReLU behind this operand whose passes it computes (absorbReLU)
+    bool absorbReLU(OperandBase *relu) override {
+        fusedRelu = relu;
+        return true;
+    }
     std::string info() override { return "BatchNorm"; }
     void initNetParams(OptimizerInfo *info, shape4 inShape) override {  // BatchNorm.cuh:27-37
         shape4 paramShape = {1, inShape.c, inShape.h, inShape.w};
@@ -90,16 +100,24 @@ public:
     }
     void forward() override {
         paramGradsDone = false;
+        if (fusedRelu) {  // Y and xHat are not needed: the ReLU's output is this operand's result, xGrads recomputes from X
+            batchNormRelu(X->A, beta->data(), gamma->data(), mean, variance, fusedRelu->Y->A);
+            return;
+        }
         batchNorm(X->A, beta->data(), gamma->data(), mean, variance, Y->A, xHatP);
     }
     // xGrads also produces the parameter gradients (they fall out of the same per-feature sums); the paramGrads call
     // that follows it in Sequential::backward then has nothing left to do. Called on its own, paramGrads computes them.
     void xGrads() override {  // BatchNorm.cu:17-21
         foldReserve();
-        batchNormGradAll(Y->dA, gamma->data(), X->A, X->dA, gamma->grad(), beta->grad());
+        if (fusedRelu)
+            batchNormReluGradAll(fusedRelu->Y->dA, fusedRelu->Y->A, gamma->data(), X->A, X->dA, gamma->grad(), beta->grad());
+        else
+            batchNormGradAll(Y->dA, gamma->data(), X->A, X->dA, gamma->grad(), beta->grad());
         paramGradsDone = true;
     }
     void paramGrads() override {
+        if (!paramGradsDone && fusedRelu) throw std::logic_error("BatchNorm: with an absorbed ReLU, paramGrads follows xGrads");
         if (!paramGradsDone) batchNormParamGrads(Y->dA, xHatP, gamma->grad(), beta->grad());
         paramGradsDone = false;
     }

@@ -55,6 +55,10 @@ public:
     // items in one launch after the last xGrads of a backward pass (Sequential::backward does, once streamline() was
     // called). An operand that has added an item must from then on be driven that way.
     virtual void deferSliceSum(std::vector<seblas::SliceSumItem> &) {}
+    // Asked of an operand whose successor in the chain is a ReLU: take over that ReLU's work (write its output in the same
+    // pass as your own, apply its gradient rule in your xGrads) and return true, or return false. The ReLU is then told
+    // to do nothing. Only Sequential::streamline() asks.
+    virtual bool absorbReLU(OperandBase *) { return false; }
 
     // Y->dA += Y->dAReserve and the reserve is cleared, in one pass (the reference clears it after the gradient call, which
     // never reads it): the first thing every xGrads does

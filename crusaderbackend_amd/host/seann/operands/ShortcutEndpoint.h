@@ -22,6 +22,12 @@ public:
     std::vector<OperandBase *> branchOperands;
     uint32 operandCount = 0;
     uint32 uuid;
+    OperandBase *fusedRelu = nullptr;  // closing endpoint: the ReLU behind it whose passes it computes (absorbReLU)
+    bool absorbReLU(OperandBase *relu) override {
+        if (!isContainer) return false;
+        fusedRelu = relu;
+        return true;
+    }
 
     ShortcutEndpoint(bool isContainer, uint32 uuid, std::initializer_list<OperandBase *> operands)
         : isContainer(isContainer), uuid(uuid) {

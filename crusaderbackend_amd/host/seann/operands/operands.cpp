@@ -159,11 +159,22 @@ void ShortcutEndpoint::forward() {  // :57-74: Y = X for the opening endpoint, Y
     }
     for (uint32 i = 0; i < operandCount; i++) branchOperands[i]->forward();
     Tensor *shortcut = operandCount > 0 ? branchOperands[operandCount - 1]->Y->A : other->Y->A;
+    if (fusedRelu) {  // the sum goes straight through the ReLU into that operand's output
+        addRelu(X->A, shortcut, fusedRelu->Y->A);
+        return;
+    }
     launched(crb_tensor_add(Y->A->elements, X->A->elements, shortcut->elements, n, nullptr), __FILE__, __LINE__);
 }
 
 void ShortcutEndpoint::xGrads() {  // :76-99
     const uint32 n = X->A->dims.size;
+    if (isContainer && fusedRelu) {
+        // the gradient behind the absorbed ReLU, masked by its output, goes to the main path and to the shortcut at once
+        Tensor *second = operandCount > 0 ? branchOperands[operandCount - 1]->Y->dA : other->Y->dAReserve;
+        reluGradTwice(fusedRelu->Y->A, fusedRelu->Y->dA, X->dA, second);
+        for (int i = int(operandCount) - 1; i >= 0; i--) branchOperands[i]->xGrads();
+        return;
+    }
     if (isContainer) {
         if (operandCount > 0) {
             // projection: the branch gets a copy of the gradient, as does the main path
@@ -274,6 +285,12 @@ void Sequential::streamline() const {
     for (OperandBase *op : operands) op->fuseGrads();  // backward() always calls xGrads and paramGrads as a pair
     sliceItems.clear();
     for (OperandBase *op : operands) op->deferSliceSum(sliceItems);  // ... and sums all convolutions' slices at its end
+    // a ReLU behind a batch normalisation or a closing shortcut endpoint is computed by that operand, in its passes
+    for (uint32 i = 0; i + 1 < OPERAND_COUNT; i++) {
+        if (operands[i + 1]->OPERAND_ID() != OPR_SEBLAS_RELU) continue;
+        auto *r = static_cast<ReLU *>(operands[i + 1]);
+        if (!r->absorbedBy && operands[i]->absorbReLU(r)) r->absorbedBy = operands[i];
+    }
     if (hipDeviceSynchronize() != hipSuccess) assertHip(__FILE__, __LINE__);  // buffers are released below: nothing may be in flight
     for (uint32 i = 0; i + 1 < OPERAND_COUNT; i++) {
         OperandBase *op = operands[i];

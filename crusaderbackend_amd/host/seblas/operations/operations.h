@@ -70,6 +70,15 @@ void batchNormParamGrads(Tensor *dY, Tensor *xHat, Tensor *dGamma, Tensor *dBeta
 // batchNormGrad and batchNormParamGrads in one pass over the data (no counterpart in the reference; same results up to
 // the rounding of xHat, which is recomputed instead of read back).
 Tensor *batchNormGradAll(Tensor *dY, Tensor *gamma, Tensor *X, Tensor *dX, Tensor *dGamma, Tensor *dBeta);
+// Normalisation and the ReLU behind it in one pass each way (same results as the two operators one after the other; no
+// counterpart in the reference). Forward writes reluOut = relu(batchNorm(X)), mean and var; backward takes the gradient
+// with respect to reluOut and yields dX, dGamma, dBeta.
+Tensor *batchNormRelu(Tensor *X, Tensor *beta, Tensor *gamma, Tensor *mean, Tensor *var, Tensor *reluOut);
+Tensor *batchNormReluGradAll(Tensor *dReluOut, Tensor *reluOut, Tensor *gamma, Tensor *X, Tensor *dX, Tensor *dGamma, Tensor *dBeta);
+// out = relu(A + B), and the ReLU's gradient (dOut where out > 0, else 0) written to two tensors at once: the closing
+// shortcut endpoint with the ReLU behind it.
+Tensor *addRelu(Tensor *A, Tensor *B, Tensor *out);
+void reluGradTwice(Tensor *out, Tensor *dOut, Tensor *d1, Tensor *d2);
 // cuOptim.cuh:16. V is the momentum buffer; Xgrad is cleared by the step.
 void momentumApply(Tensor *X, Tensor *Xgrad, Tensor *V, float LEARNING_RATE, float MOMENTUM);
 // Optimizers.cu:16-22 in one pass: X *= (1 - L2) then momentumApply. No separate counterpart in the reference.

@@ -653,6 +653,33 @@ static void codec_tests(const std::string &dir) {
     twin->forward(X), twin->backward(L), twin->learn();
     CHECK(all_params(*twin) == all_params(*net));
     CHECK(pull(net->forward(X)) == pull(twin->forward(X)));
+    // the streamlined form of the loaded network (one-launch convolution gradients, slices summed once, ReLUs absorbed by
+    // the batch normalisation / closing endpoint before them, one-launch update) computes the same bits as the plain one
+    {
+        auto all_grads = [](const Sequential &n) {
+            std::vector<NetParam *> ps;
+            for (auto *op : n.operands) op->collectNetParams(ps);
+            std::vector<float> out;
+            for (auto *p : ps) {
+                auto v = pull(p->grad());
+                out.insert(out.end(), v.begin(), v.end());
+            }
+            return out;
+        };
+        twin->streamline();
+        uint32_t absorbed = 0;
+        for (auto *op : twin->operands)
+            if (auto *r = dynamic_cast<ReLU *>(op)) absorbed += r->absorbedBy ? 1 : 0;
+        CHECK(absorbed == 3);
+        for (int step = 0; step < 2; step++) {
+            CHECK(pull(net->forward(X)) == pull(twin->forward(X)));
+            net->backward(L), twin->backward(L);
+            CHECK(all_grads(*net) == all_grads(*twin));
+            CHECK(pull(net->netX->dA) == pull(twin->netX->dA));
+            net->learn(), twin->learnFused();
+            CHECK(all_params(*net) == all_params(*twin));
+        }
+    }
     // a second save of an unchanged network replaces the file with the same bytes
     const std::string fa2 = dir + "/a2.crseq";
     seio::saveSequence(fa2.c_str(), twin, 18);

@@ -217,3 +217,53 @@ def test_momentum_multi_matches_single(dev):
     for i, ((x, g, m), (X, G, M)) in enumerate(zip(host, tens)):
         xr, gr, mr = orc.momentumApply(x, g, m, np.float32(0.01 * (i + 1)), 0.9, np.float32(1.0 - 5e-4 * (i % 2)))
         assert np.array_equal(to_np(X), xr) and np.array_equal(to_np(M), mr) and not to_np(G).any()
+
+
+@pytest.mark.parametrize("N,C,H,W", [(128, 16, 32, 32), (64, 32, 16, 16), (128, 64, 8, 8), (37, 3, 5, 7), (300, 2, 3, 3), (1, 4, 3, 3)])
+def test_batchnorm_relu_fused_equals_separate_calls(dev, N, C, H, W):
+    """Normalisation + the ReLU behind it in one pass each way: same bits as crb_batchnorm_* followed by / preceded by
+    crb_relu_*; optional outputs are left untouched when not asked for."""
+    capi = _capi()
+    F = C * H * W
+    x = normal(40, N, C, H, W) * 1.5 + 0.3
+    gamma, beta, dy = normal(41, F) + 1.0, normal(42, F), normal(43, N, C, H, W)
+    X, G, B, dY = to_dev(x, dev), to_dev(gamma, dev), to_dev(beta, dev), to_dev(dy, dev)
+    # separate
+    Y, xh, m, v, R = _nan(dev, N, F), _nan(dev, N, F), _nan(dev, F), _nan(dev, F), _nan(dev, N, F)
+    capi.batchnorm_fwd(X, B, G, m, v, Y, xh, N, F)
+    capi.relu_fwd(Y, R, N * F)
+    dZ, dX, dG, dB = _nan(dev, N, F), _nan(dev, N, F), _nan(dev, F), _nan(dev, F)
+    capi.relu_bwd(Y, dY, dZ, N * F)
+    capi.batchnorm_bwd(dZ, G, X, dX, N, F, dGamma=dG, dBeta=dB)
+    # fused, every optional output asked for
+    Y2, xh2, m2, v2, R2 = _nan(dev, N, F), _nan(dev, N, F), _nan(dev, F), _nan(dev, F), _nan(dev, N, F)
+    capi.batchnorm_relu_fwd(X, B, G, m2, v2, R2, N, F, Y=Y2, xHat=xh2)
+    for a, b in ((Y, Y2), (xh, xh2), (m, m2), (v, v2), (R, R2)):
+        assert np.array_equal(to_np(a), to_np(b), equal_nan=True)
+    dX2, dG2, dB2 = _nan(dev, N, F), _nan(dev, F), _nan(dev, F)
+    capi.batchnorm_relu_bwd(dY, R2, G, X, dX2, N, F, dGamma=dG2, dBeta=dB2)
+    for a, b in ((dX, dX2), (dG, dG2), (dB, dB2)):
+        assert np.array_equal(to_np(a), to_np(b), equal_nan=True)
+    # fused, only the ReLU output
+    m3, v3, R3 = _nan(dev, F), _nan(dev, F), _nan(dev, N, F)
+    capi.batchnorm_relu_fwd(X, B, G, m3, v3, R3, N, F)
+    assert np.array_equal(to_np(R3), to_np(R), equal_nan=True) and np.array_equal(to_np(m3), to_np(m))
+    dX3 = _nan(dev, N, F)
+    capi.batchnorm_relu_bwd(dY, R3, G, X, dX3, N, F)
+    assert np.array_equal(to_np(dX3), to_np(dX), equal_nan=True)
+
+
+@pytest.mark.parametrize("n", [1, 5, 4096, 128 * 16 * 32 * 32, 1000003])
+def test_add_relu_and_relu_grad_copy2(dev, n):
+    capi, orc = _capi(), _oracle()
+    a, b, dy = normal(50, n), normal(51, n), normal(52, n)
+    a[::7] = -b[::7]  # exact zeros in the sum: relu(0) = 0 and no gradient there
+    A, Bt, dY = to_dev(a, dev), to_dev(b, dev), to_dev(dy, dev)
+    R = _nan(dev, n)
+    capi.tensor_add_relu(R, A, Bt, n)
+    ref = orc.relu(orc.tensorAdd(a, b))
+    assert np.array_equal(to_np(R), ref)
+    d1, d2 = _nan(dev, n), _nan(dev, n)
+    capi.tensor_relu_grad_copy2(d1, d2, R, dY, n)
+    g = orc.reluGradFast(orc.tensorAdd(a, b), dy)
+    assert np.array_equal(to_np(d1), g) and np.array_equal(to_np(d2), g)
