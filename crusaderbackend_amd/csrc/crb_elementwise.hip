@@ -367,7 +367,7 @@ __global__ void __launch_bounds__(256) batchnorm_fwd_kernel(const float *__restr
     if (t.g == 0) mean[t.f] = m, var[t.f] = v;
 }
 
-template <int FL>
+template <int FL, bool MASK>
 __global__ void __launch_bounds__(256) batchnorm_bwd_kernel(const float *__restrict__ dY, const float *__restrict__ gamma,
                                                             const float *__restrict__ X, float *__restrict__ dX,
                                                             float *__restrict__ dGamma, float *__restrict__ dBeta,
@@ -379,10 +379,11 @@ __global__ void __launch_bounds__(256) batchnorm_bwd_kernel(const float *__restr
     const float *x = X + (t.on ? t.f : 0), *dy = dY + (t.on ? t.f : 0);
     // reluOut given: dY is the gradient behind a ReLU whose output is reluOut, so the gradient that reaches this
     // normalisation is dY where reluOut > 0 and 0 elsewhere
-    const float *mk = reluOut ? reluOut + (t.on ? t.f : 0) : nullptr;
+    const float *mk = MASK ? reluOut + (t.on ? t.f : 0) : nullptr;
     auto grad = [&](u32 n) -> float {
         const float e = dy[size_t(n) * F];
-        return (mk && !(mk[size_t(n) * F] > 0.f)) ? 0.f : e;
+        if (!MASK) return e;
+        return mk[size_t(n) * F] > 0.f ? e : 0.f;
     };
     float xv[kBnCache], dv[kBnCache];
     float s = 0.f;
@@ -392,7 +393,17 @@ __global__ void __launch_bounds__(256) batchnorm_bwd_kernel(const float *__restr
             const u32 n = t.g + G * i;
             const bool ok = t.on && n < N;
             xv[i] = ok ? x[size_t(n) * F] : 0.f;
-            dv[i] = ok ? grad(n) : 0.f;
+            dv[i] = ok ? dy[size_t(n) * F] : 0.f;
+        }
+        if (MASK) {  // all loads of the sweep are issued before any is used
+            float mv[kBnCache];
+#pragma unroll
+            for (int i = 0; i < kBnCache; ++i) {
+                const u32 n = t.g + G * i;
+                mv[i] = (t.on && n < N) ? mk[size_t(n) * F] : 0.f;
+            }
+#pragma unroll
+            for (int i = 0; i < kBnCache; ++i) dv[i] = mv[i] > 0.f ? dv[i] : 0.f;
         }
 #pragma unroll
         for (int i = 0; i < kBnCache; ++i) s += xv[i];
@@ -503,6 +514,16 @@ static int check_pool(const char *what, u32 planes, u32 IH, u32 IW, u32 sH, u32 
     if (IH < rH || IW < rW) return fail(CRB_EINVAL_SHAPE, "%s: window larger than the input", what);
     if (uint64_t(planes) * IH * IW > 0x7fffffffull) return fail(CRB_EINVAL_SHAPE, "%s: tensor exceeds 2^31 elements", what);
     return CRB_OK;
+}
+
+template <bool MASK>
+static void bn_bwd_launch(const float *dY, const float *gamma, const float *X, float *dX, float *dGamma, float *dBeta,
+                          const float *reluOut, uint32_t N, uint32_t F, hipStream_t s) {
+    switch (bn_features_per_wg(F)) {
+        case 64: hipLaunchKernelGGL((batchnorm_bwd_kernel<64, MASK>), dim3(ceil_div(F, 64)), dim3(256), 0, s, dY, gamma, X, dX, dGamma, dBeta, reluOut, N, F); break;
+        case 32: hipLaunchKernelGGL((batchnorm_bwd_kernel<32, MASK>), dim3(ceil_div(F, 32)), dim3(256), 0, s, dY, gamma, X, dX, dGamma, dBeta, reluOut, N, F); break;
+        default: hipLaunchKernelGGL((batchnorm_bwd_kernel<16, MASK>), dim3(ceil_div(F, 16)), dim3(256), 0, s, dY, gamma, X, dX, dGamma, dBeta, reluOut, N, F);
+    }
 }
 
 }  // namespace crb
@@ -630,12 +651,10 @@ static int bn_fwd(const char *what, const float *X, const float *beta, const flo
 static int bn_bwd(const char *what, const float *dY, const float *gamma, const float *X, float *dX, float *dGamma, float *dBeta,
                   const float *reluOut, uint32_t N, uint32_t F, void *stream) {
     if (int st = check_bn(what, N, F)) return st;
-    hipStream_t s = hipStream_t(stream);
-    switch (bn_features_per_wg(F)) {
-        case 64: hipLaunchKernelGGL(batchnorm_bwd_kernel<64>, dim3(ceil_div(F, 64)), dim3(256), 0, s, dY, gamma, X, dX, dGamma, dBeta, reluOut, N, F); break;
-        case 32: hipLaunchKernelGGL(batchnorm_bwd_kernel<32>, dim3(ceil_div(F, 32)), dim3(256), 0, s, dY, gamma, X, dX, dGamma, dBeta, reluOut, N, F); break;
-        default: hipLaunchKernelGGL(batchnorm_bwd_kernel<16>, dim3(ceil_div(F, 16)), dim3(256), 0, s, dY, gamma, X, dX, dGamma, dBeta, reluOut, N, F);
-    }
+    if (reluOut)
+        bn_bwd_launch<true>(dY, gamma, X, dX, dGamma, dBeta, reluOut, N, F, hipStream_t(stream));
+    else
+        bn_bwd_launch<false>(dY, gamma, X, dX, dGamma, dBeta, reluOut, N, F, hipStream_t(stream));
     return check_launch(what);
 }
 
