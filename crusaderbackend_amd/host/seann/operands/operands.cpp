@@ -331,10 +331,15 @@ void Sequential::learnFused() {
             learn();
             return;
         }
-        const uint32 count = p->data()->dims.size;
-        items.push_back({p->data()->elements, p->grad()->elements, m->m->elements, count, m->LEARNING_RATE, m->BETA,
-                         m->isWeight ? 1.0f - m->L2 : 1.0f});
-        maxCount = count > maxCount ? count : maxCount;
+        // a row of the launch grid covers one item with at most 64 workgroups: large tensors are entered in pieces so
+        // that they spread over the chip like the many small ones
+        const uint32 count = p->data()->dims.size, piece = 1u << 18;
+        for (uint32 at = 0; at < count; at += piece) {
+            const uint32 n = count - at < piece ? count - at : piece;
+            items.push_back({p->data()->elements + at, p->grad()->elements + at, m->m->elements + at, n, m->LEARNING_RATE, m->BETA,
+                             m->isWeight ? 1.0f - m->L2 : 1.0f});
+            maxCount = n > maxCount ? n : maxCount;
+        }
     }
     if (items.empty()) return;
     const size_t bytes = items.size() * sizeof(crb_momentum_item);
