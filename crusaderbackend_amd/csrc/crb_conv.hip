@@ -308,7 +308,7 @@ static bool bwd_fused(const crb_conv_geom *g, bool run, const float *Wt, const f
                       float *ws, hipStream_t s, WgradDirectPlan &plan, int &status) {
 #define CRB_PAIR(...) bwd_pair<__VA_ARGS__>(g, run, Wt, dY, X, dX, dW, ws, s, plan, status)
     typedef DirectCfg<32, 8, 16, 16, 4, 1, true, 2, 1, 1, 3, 4> D32a;
-    typedef DirectCfg<16, 4, 16, 32, 1, 2, true, 2, 2, 1> D16a;
+    typedef DirectCfg<16, 8, 16, 32, 2, 2, true, 2, 2, 1> D16a;
     typedef DirectCfg<8, 8, 16, 32, 1, 2, true, 2, 2, 1> D8a;
     typedef DirectCfg<16, 8, 8, 16, 2, 1, true, 2, 2, 2> D16s2;
     typedef DirectCfg<8, 8, 8, 32, 1, 2, true, 2, 2, 2> D8s2;
