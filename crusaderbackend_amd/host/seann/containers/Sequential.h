@@ -7,9 +7,15 @@
 
 #include "../operands/OperandBase.h"
 
+namespace seio {
+struct Dataset;
+}
+
 namespace seann {
 
 typedef void (*LossFunc)(Parameter *, Tensor *);
+// Called by train() after every batch: epoch, batch id, training loss per sample, test loss per sample (0 when not tested).
+typedef void (*TrainProgress)(uint32, uint32, float, float);
 typedef float (*LossFuncCalc)(Parameter *, Tensor *, Tensor *);
 
 class Sequential {
@@ -40,6 +46,12 @@ public:
     void learn() const;
     void learnBatch() const;
     void zeroGrads() const;
+    // The training loop (Sequential.cu:106-160): batches come from `data` (the next one is formed on another thread and
+    // stream while this one trains), every mini-batch runs forward, backward, loss and learn; after each batch learnBatch,
+    // and every TEST_FREQUENCY batches the test set's loss; when an epoch ends the gradients are cleared and, for epochs
+    // 0, 5, 10, ..., the model is saved. The reference writes <cache dir>cache.log and cache.crseq at a hard-coded Windows
+    // path and draws a console display; here the directory is an argument and progress goes to an optional callback.
+    void train(seio::Dataset *data, bool WITH_TEST, uint32 TEST_FREQUENCY, const char *cacheDir = ".", TrainProgress progress = nullptr);
 
     // Optional shortcuts with no counterpart in the reference; results are unchanged.
     // pruneReserveFolds: after construct(), stop folding Y->dAReserve into Y->dA in the xGrads of operands into whose

@@ -217,6 +217,48 @@ void Dataset::genBatch() {  // Dataset.cu:63-85
     epochID = uint32((uint64(batchID) * BATCH_SIZE) / EPOCH_SIZE);
 }
 
+void Dataset::allocTestSet() {
+    if (!fetcher) throw std::invalid_argument("Dataset::allocTestSet: no data fetcher");
+    const uint32 n = fetcher->TEST_SIZE;
+    if (!n || n % MINI_BATCH_SIZE) throw std::invalid_argument("Dataset::allocTestSet: test size must be a positive multiple of the mini-batch size");
+    TEST_SIZE = n;
+    const size_t xBytes = size_t(n) * dataShape.size, labFloats = size_t(n) * labelShape.size;
+    uint8_t *hostPix = nullptr, *devPix = nullptr;
+    float *hostLab = nullptr, *devXt = nullptr, *devLt = nullptr;
+    HIP_OK(hipHostMalloc(reinterpret_cast<void **>(&hostPix), xBytes, hipHostMallocDefault));
+    HIP_OK(hipHostMalloc(reinterpret_cast<void **>(&hostLab), labFloats * sizeof(float), hipHostMallocDefault));
+    HIP_OK(hipMalloc(reinterpret_cast<void **>(&devPix), xBytes));
+    HIP_OK(hipMalloc(reinterpret_cast<void **>(&devXt), xBytes * sizeof(float)));
+    HIP_OK(hipMalloc(reinterpret_cast<void **>(&devLt), labFloats * sizeof(float)));
+    Tensor *one = Tensor::createHost(dataShape), *lab = Tensor::createHost(labelShape);
+    std::vector<uint8_t> bytes(dataShape.size);
+    for (uint32 i = 0; i < n; i++) {  // fetchTest hands out floats of byte values: exact to turn back
+        fetcher->fetchTest(one, lab);
+        for (uint32 k = 0; k < dataShape.size; k++) hostPix[size_t(i) * dataShape.size + k] = uint8_t(one->elements[k]);
+        std::memcpy(hostLab + size_t(i) * labelShape.size, lab->elements, sizeof(float) * labelShape.size);
+    }
+    one->eliminateHost(), lab->eliminateHost();
+    hipStream_t s = hipStream_t(stream);
+    HIP_OK(hipMemcpyAsync(devPix, hostPix, xBytes, hipMemcpyHostToDevice, s));
+    HIP_OK(hipMemcpyAsync(devLt, hostLab, labFloats * sizeof(float), hipMemcpyHostToDevice, s));
+    throwOnStatus(crb_images_from_bytes(devPix, devXt, n, dataShape.c, dataShape.h, dataShape.w, preProc ? preProc->kind() : CRB_NORM_NONE,
+                                        preProc ? preProc->p0() : 0.0f, preProc ? preProc->p1() : 0.0f, nullptr, s),
+                  __FILE__, __LINE__);
+    HIP_OK(hipStreamSynchronize(s));
+    HIP_OK(hipHostFree(hostPix));
+    HIP_OK(hipHostFree(hostLab));
+    HIP_OK(hipFree(devPix));
+    const uint32 minis = n / MINI_BATCH_SIZE;
+    const shape4 procData(MINI_BATCH_SIZE, dataShape.c, dataShape.h, dataShape.w), procLabel(MINI_BATCH_SIZE, labelShape.c, labelShape.h, labelShape.w);
+    testset = new Data *[minis];
+    for (uint32 i = 0; i < minis; i++) {
+        Data *d = Data::declare(procData, procLabel);
+        d->X->attach(devXt + size_t(i) * procData.size, 0);
+        d->label->attach(devLt + size_t(i) * procLabel.size, 0);
+        testset[i] = d;
+    }
+}
+
 std::thread Dataset::genBatchAsync() {
     return std::thread([this] { genBatch(); });
 }

@@ -158,6 +158,8 @@ public:
 // (Dataset.cuh:17-83, Dataset.cu:20-92): genBatch() fills dataBatch[batchID % 2] and then advances batchID.
 struct Dataset {
     Data **dataBatch[2] = {nullptr, nullptr};  // device; views of one buffer per side
+    Data **testset = nullptr;                  // device mini-batches filled by allocTestSet()
+    uint32 TEST_SIZE = 0;
     DataFetcher *fetcher = nullptr;
     uint32 BATCH_SIZE = 0, EPOCH_SIZE = 0, MAX_EPOCH = 0, MINI_BATCH_SIZE = 0;
     uint32 batchID = 0, epochID = 0;
@@ -171,6 +173,9 @@ struct Dataset {
     void setProcSteps(std::initializer_list<DataTransformer *> steps);  // none or one
     void setAugmentSteps(std::initializer_list<DataAugmentor *> steps);
     void genBatch();
+    // TEST_SIZE (the fetcher's) samples drawn by fetchTest, transformed but not augmented, as TEST_SIZE / MINI_BATCH_SIZE
+    // device mini-batches in `testset` (Dataset.cu:94-134).
+    void allocTestSet();
     std::thread genBatchAsync();
     // What the last genBatch decided per image (for tests and logging).
     const std::vector<ImageAug> &lastAugmentations() const { return augHost; }

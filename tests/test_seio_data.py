@@ -75,3 +75,23 @@ def test_batches_formed_on_device_match_restatement(dev, tmp_path):
     for k, rec in enumerate((0, 5, 6, 11, 3)):
         x, lab = sio.cifar_bin_record(whole, rec)
         assert np.array_equal(cx[k], x) and np.array_equal(cl[k], lab), rec
+
+
+@pytest.mark.gpu
+def test_sequential_train_on_a_dataset_file(dev, tmp_path):
+    """Sequential::train end to end: batches formed from a .crdat file on a second thread and stream, per-mini-batch
+    forward / backward / update, test loss, log file and epoch model file."""
+    assert os.path.exists(BIN), f"{BIN} missing: run `make -C crusaderbackend_amd/host`"
+    d = str(tmp_path)
+    rng = np.random.default_rng(21)
+    n = 96 + 16
+    cls = rng.integers(0, 2, n)
+    images = rng.integers(0, 60, (n, 1, 8, 8), dtype=np.uint8)
+    for i in range(n):  # class 0: bright left half, class 1: bright right half
+        images[i, 0, :, (0 if cls[i] == 0 else 4):(4 if cls[i] == 0 else 8)] += 150
+    labels = np.eye(2, dtype=np.float32)[cls]
+    open(os.path.join(d, "toy.crdat"), "wb").write(sio.crdat_pack(images, labels))
+    r = subprocess.run([BIN, "train", d], capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0 and "train: OK" in r.stdout, r.stdout + r.stderr
+    log = open(os.path.join(d, "cache.log")).read()
+    assert len([v for v in log.replace(" ", "").split(",") if v]) == 16  # 8 batches trained on: training loss and test loss each
