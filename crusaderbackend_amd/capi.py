@@ -78,10 +78,10 @@ SIGNATURES = {
     "crb_batchnorm_fwd": (ctypes.c_int, [_ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _u32, _u32, _ptr]),
     "crb_batchnorm_bwd": (ctypes.c_int, [_ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _u32, _u32, _ptr]),
     "crb_batchnorm_param_grads": (ctypes.c_int, [_ptr, _ptr, _ptr, _ptr, _u32, _u32, _ptr]),
-    "crb_batchnorm_relu_fwd": (ctypes.c_int, [_ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _u32, _u32, _ptr]),
-    "crb_batchnorm_relu_bwd": (ctypes.c_int, [_ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _u32, _u32, _ptr]),
+    "crb_batchnorm_relu_fwd": (ctypes.c_int, [_ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _u32, _u32, _ptr]),
+    "crb_batchnorm_relu_bwd": (ctypes.c_int, [_ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _u32, _u32, _ptr]),
     "crb_tensor_add_relu": (ctypes.c_int, [_ptr, _ptr, _ptr, _u32, _ptr]),
-    "crb_tensor_relu_grad_copy2": (ctypes.c_int, [_ptr, _ptr, _ptr, _ptr, _u32, _ptr]),
+    "crb_tensor_relu_grad_copy2": (ctypes.c_int, [_ptr, _ptr, _ptr, _ptr, _ptr, _u32, _ptr]),
     "crb_momentum_apply": (ctypes.c_int, [_ptr, _ptr, _ptr, _u32, ctypes.c_float, ctypes.c_float, ctypes.c_float, _ptr]),
     "crb_images_from_bytes": (ctypes.c_int, [_ptr, _ptr, _u32, _u32, _u32, _u32, ctypes.c_int, ctypes.c_float, ctypes.c_float,
                                              _ptr, _ptr]),
@@ -341,17 +341,19 @@ def images_from_bytes(src, dst, images, channels, H, W, norm=NORM_NONE, p0=0.0, 
     check(load().crb_images_from_bytes(_p(src), _p(dst), images, channels, H, W, norm, p0, p1, _p(aug), _stream(stream)))
 
 
-def batchnorm_relu_fwd(X, beta, gamma, mean, var, reluOut, N, F, Y=None, xHat=None, stream=None):
-    check(load().crb_batchnorm_relu_fwd(_p(X), _p(beta), _p(gamma), _p(mean), _p(var), _p(Y), _p(xHat), _p(reluOut), N, F, _stream(stream)))
+def batchnorm_relu_fwd(X, beta, gamma, mean, var, reluOut, N, F, Y=None, xHat=None, addend=None, stream=None):
+    check(load().crb_batchnorm_relu_fwd(_p(X), _p(beta), _p(gamma), _p(mean), _p(var), _p(Y), _p(xHat), _p(addend), _p(reluOut), N, F,
+                                        _stream(stream)))
 
 
-def batchnorm_relu_bwd(dY, reluOut, gamma, X, dX, N, F, dGamma=None, dBeta=None, stream=None):
-    check(load().crb_batchnorm_relu_bwd(_p(dY), _p(reluOut), _p(gamma), _p(X), _p(dX), _p(dGamma), _p(dBeta), N, F, _stream(stream)))
+def batchnorm_relu_bwd(dY, reluOut, gamma, X, dX, N, F, dGamma=None, dBeta=None, dY2=None, dYmasked=None, stream=None):
+    check(load().crb_batchnorm_relu_bwd(_p(dY), _p(dY2), _p(reluOut), _p(gamma), _p(X), _p(dX), _p(dGamma), _p(dBeta), _p(dYmasked), N, F,
+                                        _stream(stream)))
 
 
 def tensor_add_relu(dst, a, b, count, stream=None):
     check(load().crb_tensor_add_relu(_p(dst), _p(a), _p(b), count, _stream(stream)))
 
 
-def tensor_relu_grad_copy2(dst1, dst2, relu_out, dY, count, stream=None):
-    check(load().crb_tensor_relu_grad_copy2(_p(dst1), _p(dst2), _p(relu_out), _p(dY), count, _stream(stream)))
+def tensor_relu_grad_copy2(dst1, dst2, relu_out, dY, count, dY2=None, stream=None):
+    check(load().crb_tensor_relu_grad_copy2(_p(dst1), _p(dst2), _p(relu_out), _p(dY), _p(dY2), count, _stream(stream)))

@@ -312,7 +312,7 @@ template <int FL>
 __global__ void __launch_bounds__(256) batchnorm_fwd_kernel(const float *__restrict__ X, const float *__restrict__ beta,
                                                             const float *__restrict__ gamma, float *__restrict__ mean,
                                                             float *__restrict__ var, float *__restrict__ Y, float *__restrict__ xHat,
-                                                            float *__restrict__ reluOut, u32 N, u32 F) {
+                                                            const float *__restrict__ addend, float *__restrict__ reluOut, u32 N, u32 F) {
     constexpr u32 G = 256 / FL;
     __shared__ float red[G][FL];
     const BnGeom<FL> t(F);
@@ -348,12 +348,16 @@ __global__ void __launch_bounds__(256) batchnorm_fwd_kernel(const float *__restr
     const float v = t.reduce(q, red) / float(N);
     if (!t.on) return;
     const float inv = 1.0f / sqrtf(v + 1e-8f), ga = gamma[t.f], be = beta[t.f];
-    // outputs a caller does not need are not written: Y and xHat may be null, reluOut = max(Y, 0) is optional
+    // outputs a caller does not need are not written: Y and xHat may be null; reluOut = max(Y + addend, 0) is optional
+    // (addend: the other summand of a residual connection that closes right behind this normalisation, or null)
     auto put = [&](u32 n, float xh) {
         const float y = xh * ga + be;
         if (xHat) xHat[size_t(n) * F + t.f] = xh;
         if (Y) Y[size_t(n) * F + t.f] = y;
-        if (reluOut) reluOut[size_t(n) * F + t.f] = y > 0.f ? y : 0.f;
+        if (reluOut) {
+            const float z = addend ? y + addend[size_t(n) * F + t.f] : y;
+            reluOut[size_t(n) * F + t.f] = z > 0.f ? z : 0.f;
+        }
     };
     if (cached) {
 #pragma unroll
@@ -367,8 +371,9 @@ __global__ void __launch_bounds__(256) batchnorm_fwd_kernel(const float *__restr
     if (t.g == 0) mean[t.f] = m, var[t.f] = v;
 }
 
-template <int FL, bool MASK>
-__global__ void __launch_bounds__(256) batchnorm_bwd_kernel(const float *__restrict__ dY, const float *__restrict__ gamma,
+template <int FL, bool MASK, bool SUM2>
+__global__ void __launch_bounds__(256) batchnorm_bwd_kernel(const float *__restrict__ dY, const float *__restrict__ dY2,
+                                                            float *__restrict__ dyOut, const float *__restrict__ gamma,
                                                             const float *__restrict__ X, float *__restrict__ dX,
                                                             float *__restrict__ dGamma, float *__restrict__ dBeta,
                                                             const float *__restrict__ reluOut, u32 N, u32 F) {
@@ -379,9 +384,14 @@ __global__ void __launch_bounds__(256) batchnorm_bwd_kernel(const float *__restr
     const float *x = X + (t.on ? t.f : 0), *dy = dY + (t.on ? t.f : 0);
     // reluOut given: dY is the gradient behind a ReLU whose output is reluOut, so the gradient that reaches this
     // normalisation is dY where reluOut > 0 and 0 elsewhere
+    // SUM2: the gradient arrives in two parts that are added first (a residual connection opens right behind the ReLU).
+    // dyOut, when given, receives the gradient as it reaches this normalisation (the copy the residual connection that
+    // closes in front of the ReLU hands to its shortcut).
     const float *mk = MASK ? reluOut + (t.on ? t.f : 0) : nullptr;
+    const float *dy2 = SUM2 ? dY2 + (t.on ? t.f : 0) : nullptr;
     auto grad = [&](u32 n) -> float {
-        const float e = dy[size_t(n) * F];
+        float e = dy[size_t(n) * F];
+        if (SUM2) e = e + dy2[size_t(n) * F];
         if (!MASK) return e;
         return mk[size_t(n) * F] > 0.f ? e : 0.f;
     };
@@ -395,7 +405,17 @@ __global__ void __launch_bounds__(256) batchnorm_bwd_kernel(const float *__restr
             xv[i] = ok ? x[size_t(n) * F] : 0.f;
             dv[i] = ok ? dy[size_t(n) * F] : 0.f;
         }
-        if (MASK) {  // all loads of the sweep are issued before any is used
+        if (SUM2) {  // all loads of the sweep are issued before any is used
+            float ev[kBnCache];
+#pragma unroll
+            for (int i = 0; i < kBnCache; ++i) {
+                const u32 n = t.g + G * i;
+                ev[i] = (t.on && n < N) ? dy2[size_t(n) * F] : 0.f;
+            }
+#pragma unroll
+            for (int i = 0; i < kBnCache; ++i) dv[i] = dv[i] + ev[i];
+        }
+        if (MASK) {
             float mv[kBnCache];
 #pragma unroll
             for (int i = 0; i < kBnCache; ++i) {
@@ -438,11 +458,17 @@ __global__ void __launch_bounds__(256) batchnorm_bwd_kernel(const float *__restr
 #pragma unroll
         for (int i = 0; i < kBnCache; ++i) {
             const u32 n = t.g + G * i;
-            if (n < N) dX[size_t(n) * F + t.f] = dv[i] * ga * inv + dVar * (xv[i] - m) * 2.0f * invN + dMean * invN;
+            if (n < N) {
+                dX[size_t(n) * F + t.f] = dv[i] * ga * inv + dVar * (xv[i] - m) * 2.0f * invN + dMean * invN;
+                if (dyOut) dyOut[size_t(n) * F + t.f] = dv[i];
+            }
         }
     } else {
-        for (u32 n = t.g; n < N; n += G)
-            dX[size_t(n) * F + t.f] = grad(n) * ga * inv + dVar * (x[size_t(n) * F] - m) * 2.0f * invN + dMean * invN;
+        for (u32 n = t.g; n < N; n += G) {
+            const float e = grad(n);
+            dX[size_t(n) * F + t.f] = e * ga * inv + dVar * (x[size_t(n) * F] - m) * 2.0f * invN + dMean * invN;
+            if (dyOut) dyOut[size_t(n) * F + t.f] = e;
+        }
     }
 }
 
@@ -516,13 +542,13 @@ static int check_pool(const char *what, u32 planes, u32 IH, u32 IW, u32 sH, u32 
     return CRB_OK;
 }
 
-template <bool MASK>
-static void bn_bwd_launch(const float *dY, const float *gamma, const float *X, float *dX, float *dGamma, float *dBeta,
-                          const float *reluOut, uint32_t N, uint32_t F, hipStream_t s) {
+template <bool MASK, bool SUM2>
+static void bn_bwd_launch(const float *dY, const float *dY2, float *dyOut, const float *gamma, const float *X, float *dX, float *dGamma,
+                          float *dBeta, const float *reluOut, uint32_t N, uint32_t F, hipStream_t s) {
     switch (bn_features_per_wg(F)) {
-        case 64: hipLaunchKernelGGL((batchnorm_bwd_kernel<64, MASK>), dim3(ceil_div(F, 64)), dim3(256), 0, s, dY, gamma, X, dX, dGamma, dBeta, reluOut, N, F); break;
-        case 32: hipLaunchKernelGGL((batchnorm_bwd_kernel<32, MASK>), dim3(ceil_div(F, 32)), dim3(256), 0, s, dY, gamma, X, dX, dGamma, dBeta, reluOut, N, F); break;
-        default: hipLaunchKernelGGL((batchnorm_bwd_kernel<16, MASK>), dim3(ceil_div(F, 16)), dim3(256), 0, s, dY, gamma, X, dX, dGamma, dBeta, reluOut, N, F);
+        case 64: hipLaunchKernelGGL((batchnorm_bwd_kernel<64, MASK, SUM2>), dim3(ceil_div(F, 64)), dim3(256), 0, s, dY, dY2, dyOut, gamma, X, dX, dGamma, dBeta, reluOut, N, F); break;
+        case 32: hipLaunchKernelGGL((batchnorm_bwd_kernel<32, MASK, SUM2>), dim3(ceil_div(F, 32)), dim3(256), 0, s, dY, dY2, dyOut, gamma, X, dX, dGamma, dBeta, reluOut, N, F); break;
+        default: hipLaunchKernelGGL((batchnorm_bwd_kernel<16, MASK, SUM2>), dim3(ceil_div(F, 16)), dim3(256), 0, s, dY, dY2, dyOut, gamma, X, dX, dGamma, dBeta, reluOut, N, F);
     }
 }
 
@@ -637,51 +663,56 @@ int crb_tensor_scale_inplace(float *a, float factor, uint32_t count, void *strea
 }
 
 static int bn_fwd(const char *what, const float *X, const float *beta, const float *gamma, float *mean, float *var, float *Y,
-                  float *xHat, float *reluOut, uint32_t N, uint32_t F, void *stream) {
+                  float *xHat, const float *addend, float *reluOut, uint32_t N, uint32_t F, void *stream) {
     if (int st = check_bn(what, N, F)) return st;
     hipStream_t s = hipStream_t(stream);
     switch (bn_features_per_wg(F)) {
-        case 64: hipLaunchKernelGGL(batchnorm_fwd_kernel<64>, dim3(ceil_div(F, 64)), dim3(256), 0, s, X, beta, gamma, mean, var, Y, xHat, reluOut, N, F); break;
-        case 32: hipLaunchKernelGGL(batchnorm_fwd_kernel<32>, dim3(ceil_div(F, 32)), dim3(256), 0, s, X, beta, gamma, mean, var, Y, xHat, reluOut, N, F); break;
-        default: hipLaunchKernelGGL(batchnorm_fwd_kernel<16>, dim3(ceil_div(F, 16)), dim3(256), 0, s, X, beta, gamma, mean, var, Y, xHat, reluOut, N, F);
+        case 64: hipLaunchKernelGGL(batchnorm_fwd_kernel<64>, dim3(ceil_div(F, 64)), dim3(256), 0, s, X, beta, gamma, mean, var, Y, xHat, addend, reluOut, N, F); break;
+        case 32: hipLaunchKernelGGL(batchnorm_fwd_kernel<32>, dim3(ceil_div(F, 32)), dim3(256), 0, s, X, beta, gamma, mean, var, Y, xHat, addend, reluOut, N, F); break;
+        default: hipLaunchKernelGGL(batchnorm_fwd_kernel<16>, dim3(ceil_div(F, 16)), dim3(256), 0, s, X, beta, gamma, mean, var, Y, xHat, addend, reluOut, N, F);
     }
     return check_launch(what);
 }
 
-static int bn_bwd(const char *what, const float *dY, const float *gamma, const float *X, float *dX, float *dGamma, float *dBeta,
-                  const float *reluOut, uint32_t N, uint32_t F, void *stream) {
+static int bn_bwd(const char *what, const float *dY, const float *dY2, float *dyOut, const float *gamma, const float *X, float *dX,
+                  float *dGamma, float *dBeta, const float *reluOut, uint32_t N, uint32_t F, void *stream) {
     if (int st = check_bn(what, N, F)) return st;
-    if (reluOut)
-        bn_bwd_launch<true>(dY, gamma, X, dX, dGamma, dBeta, reluOut, N, F, hipStream_t(stream));
+    hipStream_t s = hipStream_t(stream);
+    if (reluOut && dY2)
+        bn_bwd_launch<true, true>(dY, dY2, dyOut, gamma, X, dX, dGamma, dBeta, reluOut, N, F, s);
+    else if (reluOut)
+        bn_bwd_launch<true, false>(dY, dY2, dyOut, gamma, X, dX, dGamma, dBeta, reluOut, N, F, s);
+    else if (dY2)
+        bn_bwd_launch<false, true>(dY, dY2, dyOut, gamma, X, dX, dGamma, dBeta, reluOut, N, F, s);
     else
-        bn_bwd_launch<false>(dY, gamma, X, dX, dGamma, dBeta, reluOut, N, F, hipStream_t(stream));
+        bn_bwd_launch<false, false>(dY, dY2, dyOut, gamma, X, dX, dGamma, dBeta, reluOut, N, F, s);
     return check_launch(what);
 }
 
 int crb_batchnorm_relu_fwd(const float *X, const float *beta, const float *gamma, float *mean, float *var, float *Y_or_null,
-                           float *xHat_or_null, float *reluOut, uint32_t N, uint32_t F, void *stream) {
+                           float *xHat_or_null, const float *addend_or_null, float *reluOut, uint32_t N, uint32_t F, void *stream) {
     if (!X || !beta || !gamma || !mean || !var || !reluOut) return fail(CRB_ENULL, "crb_batchnorm_relu_fwd: null operand");
-    return bn_fwd("crb_batchnorm_relu_fwd", X, beta, gamma, mean, var, Y_or_null, xHat_or_null, reluOut, N, F, stream);
+    return bn_fwd("crb_batchnorm_relu_fwd", X, beta, gamma, mean, var, Y_or_null, xHat_or_null, addend_or_null, reluOut, N, F, stream);
 }
 
-int crb_batchnorm_relu_bwd(const float *dY, const float *reluOut, const float *gamma, const float *X, float *dX, float *dGamma_or_null,
-                           float *dBeta_or_null, uint32_t N, uint32_t F, void *stream) {
+int crb_batchnorm_relu_bwd(const float *dY, const float *dY2_or_null, const float *reluOut, const float *gamma, const float *X, float *dX,
+                           float *dGamma_or_null, float *dBeta_or_null, float *dYmasked_or_null, uint32_t N, uint32_t F, void *stream) {
     if (!dY || !reluOut || !gamma || !X || !dX) return fail(CRB_ENULL, "crb_batchnorm_relu_bwd: null operand");
     if (!dGamma_or_null != !dBeta_or_null) return fail(CRB_ENULL, "crb_batchnorm_relu_bwd: dGamma and dBeta go together");
-    return bn_bwd("crb_batchnorm_relu_bwd", dY, gamma, X, dX, dGamma_or_null, dBeta_or_null, reluOut, N, F, stream);
+    return bn_bwd("crb_batchnorm_relu_bwd", dY, dY2_or_null, dYmasked_or_null, gamma, X, dX, dGamma_or_null, dBeta_or_null, reluOut, N, F, stream);
 }
 
 int crb_batchnorm_fwd(const float *X, const float *beta, const float *gamma, float *mean, float *var, float *Y, float *xHat,
                       uint32_t N, uint32_t F, void *stream) {
     if (!X || !beta || !gamma || !mean || !var || !Y || !xHat) return fail(CRB_ENULL, "crb_batchnorm_fwd: null operand");
-    return bn_fwd("crb_batchnorm_fwd", X, beta, gamma, mean, var, Y, xHat, nullptr, N, F, stream);
+    return bn_fwd("crb_batchnorm_fwd", X, beta, gamma, mean, var, Y, xHat, nullptr, nullptr, N, F, stream);
 }
 
 int crb_batchnorm_bwd(const float *dY, const float *gamma, const float *X, float *dX, float *dGamma_or_null, float *dBeta_or_null,
                       uint32_t N, uint32_t F, void *stream) {
     if (!dY || !gamma || !X || !dX) return fail(CRB_ENULL, "crb_batchnorm_bwd: null operand");
     if (!dGamma_or_null != !dBeta_or_null) return fail(CRB_ENULL, "crb_batchnorm_bwd: dGamma and dBeta go together");
-    return bn_bwd("crb_batchnorm_bwd", dY, gamma, X, dX, dGamma_or_null, dBeta_or_null, nullptr, N, F, stream);
+    return bn_bwd("crb_batchnorm_bwd", dY, nullptr, nullptr, gamma, X, dX, dGamma_or_null, dBeta_or_null, nullptr, N, F, stream);
 }
 
 int crb_batchnorm_param_grads(const float *dY, const float *xHat, float *dGamma, float *dBeta, uint32_t N, uint32_t F,

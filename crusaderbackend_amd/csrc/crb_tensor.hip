@@ -95,21 +95,26 @@ __global__ void __launch_bounds__(256) tri_kernel(float *d, float *a, float *b, 
     }
 }
 
-// d1 = d2 = (mask > 0 ? src : 0): the gradient behind a ReLU whose output is `mask`, delivered to two consumers.
-__global__ void __launch_bounds__(256) relu_grad_copy2_kernel(float *d1, float *d2, const float *mask, const float *src, u32 count, u32 vec) {
+// d1 = d2 = (mask > 0 ? src (+ src2) : 0): the gradient behind a ReLU whose output is `mask`, delivered to two consumers;
+// with src2 the gradient arrives in two parts that are added first.
+template <bool SUM2>
+__global__ void __launch_bounds__(256) relu_grad_copy2_kernel(float *d1, float *d2, const float *mask, const float *src, const float *src2,
+                                                              u32 count, u32 vec) {
     const u32 stride = gridDim.x * 256;
     u32 i = blockIdx.x * 256 + threadIdx.x;
     auto pick = [](float m, float v) { return m > 0.f ? v : 0.f; };
     if (vec) {
         const u32 nq = count / 4;
         for (u32 q = i; q < nq; q += stride) {
-            const v4f m = reinterpret_cast<const v4f *>(mask)[q], v = reinterpret_cast<const v4f *>(src)[q];
+            const v4f m = reinterpret_cast<const v4f *>(mask)[q];
+            v4f v = reinterpret_cast<const v4f *>(src)[q];
+            if (SUM2) v = v + reinterpret_cast<const v4f *>(src2)[q];
             const v4f r = {pick(m.x, v.x), pick(m.y, v.y), pick(m.z, v.z), pick(m.w, v.w)};
             reinterpret_cast<v4f *>(d1)[q] = r, reinterpret_cast<v4f *>(d2)[q] = r;
         }
-        for (u32 k = nq * 4 + i; k < count; k += stride) d1[k] = d2[k] = pick(mask[k], src[k]);
+        for (u32 k = nq * 4 + i; k < count; k += stride) d1[k] = d2[k] = pick(mask[k], SUM2 ? src[k] + src2[k] : src[k]);
     } else {
-        for (; i < count; i += stride) d1[i] = d2[i] = pick(mask[i], src[i]);
+        for (; i < count; i += stride) d1[i] = d2[i] = pick(mask[i], SUM2 ? src[i] + src2[i] : src[i]);
     }
 }
 
@@ -167,12 +172,18 @@ int crb_tensor_add_relu(float *dst, const float *a, const float *b, uint32_t cou
     return launch_tri<3>(dst, const_cast<float *>(a), const_cast<float *>(b), count, stream, "crb_tensor_add_relu");
 }
 
-int crb_tensor_relu_grad_copy2(float *dst1, float *dst2, const float *relu_out, const float *dY, uint32_t count, void *stream) {
+int crb_tensor_relu_grad_copy2(float *dst1, float *dst2, const float *relu_out, const float *dY, const float *dY2_or_null, uint32_t count,
+                               void *stream) {
     if (!dst1 || !dst2 || !relu_out || !dY) return fail(CRB_ENULL, "crb_tensor_relu_grad_copy2: null operand");
     if (!count) return fail(CRB_EINVAL_SHAPE, "crb_tensor_relu_grad_copy2: zero size");
     const u32 vec = ((reinterpret_cast<uintptr_t>(dst1) | reinterpret_cast<uintptr_t>(dst2) | reinterpret_cast<uintptr_t>(relu_out) |
-                      reinterpret_cast<uintptr_t>(dY)) & 15u) == 0;
-    hipLaunchKernelGGL(relu_grad_copy2_kernel, dim3(stream_grid(count)), dim3(256), 0, hipStream_t(stream), dst1, dst2, relu_out, dY, count, vec);
+                      reinterpret_cast<uintptr_t>(dY) | reinterpret_cast<uintptr_t>(dY2_or_null)) & 15u) == 0;
+    if (dY2_or_null)
+        hipLaunchKernelGGL(relu_grad_copy2_kernel<true>, dim3(stream_grid(count)), dim3(256), 0, hipStream_t(stream), dst1, dst2, relu_out, dY,
+                           dY2_or_null, count, vec);
+    else
+        hipLaunchKernelGGL(relu_grad_copy2_kernel<false>, dim3(stream_grid(count)), dim3(256), 0, hipStream_t(stream), dst1, dst2, relu_out, dY,
+                           dY2_or_null, count, vec);
     return check_launch("crb_tensor_relu_grad_copy2");
 }
 

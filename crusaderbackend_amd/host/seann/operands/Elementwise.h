@@ -79,8 +79,17 @@ public:
     Tensor *xHatP{};
     bool paramGradsDone = false;
     OperandBase *fusedRelu = nullptr;  // the ReLU behind this operand whose passes it computes (absorbReLU)
+    // Set by Sequential::streamline() when an identity shortcut closes between this operand and the absorbed ReLU: the
+    // shortcut's value is added before the ReLU, and the masked gradient is copied to the shortcut's reserve gradient.
+    Tensor *shortcutValue = nullptr, *shortcutGrad = nullptr;
+    Tensor *gradPartA = nullptr, *gradPartB = nullptr;  // takeGradientInParts
     bool absorbReLU(OperandBase *relu) override {
         fusedRelu = relu;
+        return true;
+    }
+    bool takeGradientInParts(Tensor *a, Tensor *b) override {
+        if (!fusedRelu) return false;
+        gradPartA = a, gradPartB = b;
         return true;
     }
     std::string info() override { return "BatchNorm"; }
@@ -101,7 +110,7 @@ public:
     void forward() override {
         paramGradsDone = false;
         if (fusedRelu) {  // Y and xHat are not needed: the ReLU's output is this operand's result, xGrads recomputes from X
-            batchNormRelu(X->A, beta->data(), gamma->data(), mean, variance, fusedRelu->Y->A);
+            batchNormRelu(X->A, beta->data(), gamma->data(), mean, variance, fusedRelu->Y->A, shortcutValue);
             return;
         }
         batchNorm(X->A, beta->data(), gamma->data(), mean, variance, Y->A, xHatP);
@@ -111,7 +120,8 @@ public:
     void xGrads() override {  // BatchNorm.cu:17-21
         foldReserve();
         if (fusedRelu)
-            batchNormReluGradAll(fusedRelu->Y->dA, fusedRelu->Y->A, gamma->data(), X->A, X->dA, gamma->grad(), beta->grad());
+            batchNormReluGradAll(gradPartA ? gradPartA : fusedRelu->Y->dA, fusedRelu->Y->A, gamma->data(), X->A, X->dA, gamma->grad(),
+                                 beta->grad(), gradPartB, shortcutGrad);
         else
             batchNormGradAll(Y->dA, gamma->data(), X->A, X->dA, gamma->grad(), beta->grad());
         paramGradsDone = true;

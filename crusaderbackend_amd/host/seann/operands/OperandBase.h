@@ -59,6 +59,10 @@ public:
     // pass as your own, apply its gradient rule in your xGrads) and return true, or return false. The ReLU is then told
     // to do nothing. Only Sequential::streamline() asks.
     virtual bool absorbReLU(OperandBase *) { return false; }
+    // Asked of an operand that has absorbed a ReLU behind which a residual connection opens: from now on the gradient with
+    // respect to that ReLU's output arrives in two parts (the opening endpoint's main-path and shortcut gradients), which
+    // the operand adds on the fly; the opening endpoint then has nothing left to do in xGrads. False = not supported.
+    virtual bool takeGradientInParts(Tensor *, Tensor *) { return false; }
 
     // Y->dA += Y->dAReserve and the reserve is cleared, in one pass (the reference clears it after the gradient call, which
     // never reads it): the first thing every xGrads does

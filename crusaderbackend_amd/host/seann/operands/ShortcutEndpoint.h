@@ -23,9 +23,19 @@ public:
     uint32 operandCount = 0;
     uint32 uuid;
     OperandBase *fusedRelu = nullptr;  // closing endpoint: the ReLU behind it whose passes it computes (absorbReLU)
+    Tensor *gradPartA = nullptr, *gradPartB = nullptr;  // takeGradientInParts
+    // Set by Sequential::streamline(): this endpoint's passes are computed by a neighbour — a closing identity endpoint's by
+    // the batch normalisation in front of it, an opening endpoint's gradient sum by the operand that absorbed the ReLU in
+    // front of it — and forward / xGrads do nothing.
+    bool idleForward = false, idleGrad = false;
     bool absorbReLU(OperandBase *relu) override {
         if (!isContainer) return false;
         fusedRelu = relu;
+        return true;
+    }
+    bool takeGradientInParts(Tensor *a, Tensor *b) override {
+        if (!isContainer || !fusedRelu) return false;
+        gradPartA = a, gradPartB = b;
         return true;
     }
 

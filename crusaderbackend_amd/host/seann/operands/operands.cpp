@@ -153,6 +153,7 @@ static void launched(int status, const char *file, int line) {
 
 void ShortcutEndpoint::forward() {  // :57-74: Y = X for the opening endpoint, Y = X + shortcut for the closing one
     const uint32 n = X->A->dims.size;
+    if (idleForward) return;
     if (!isContainer) {
         if (Y->A->elements != X->A->elements) X->A->copyToD2D(Y->A);  // aliased by Sequential::streamline()
         return;
@@ -168,10 +169,11 @@ void ShortcutEndpoint::forward() {  // :57-74: Y = X for the opening endpoint, Y
 
 void ShortcutEndpoint::xGrads() {  // :76-99
     const uint32 n = X->A->dims.size;
+    if (idleGrad) return;
     if (isContainer && fusedRelu) {
         // the gradient behind the absorbed ReLU, masked by its output, goes to the main path and to the shortcut at once
         Tensor *second = operandCount > 0 ? branchOperands[operandCount - 1]->Y->dA : other->Y->dAReserve;
-        reluGradTwice(fusedRelu->Y->A, fusedRelu->Y->dA, X->dA, second);
+        reluGradTwice(fusedRelu->Y->A, gradPartA ? gradPartA : fusedRelu->Y->dA, X->dA, second, gradPartB);
         for (int i = int(operandCount) - 1; i >= 0; i--) branchOperands[i]->xGrads();
         return;
     }
@@ -290,6 +292,26 @@ void Sequential::streamline() const {
         if (operands[i + 1]->OPERAND_ID() != OPR_SEBLAS_RELU) continue;
         auto *r = static_cast<ReLU *>(operands[i + 1]);
         if (!r->absorbedBy && operands[i]->absorbReLU(r)) r->absorbedBy = operands[i];
+    }
+    // batch normalisation, closing identity endpoint, ReLU: the normalisation also adds the shortcut's value and hands the
+    // shortcut its gradient, and the endpoint is idle
+    for (uint32 i = 0; i + 2 < OPERAND_COUNT; i++) {
+        auto *bn = dynamic_cast<BatchNorm *>(operands[i]);
+        if (!bn || bn->fusedRelu || operands[i + 1]->OPERAND_ID() != OPR_CTRL_SHORTCUTENDPOINT_END) continue;
+        auto *end = static_cast<ShortcutEndpoint *>(operands[i + 1]);
+        if (end->operandCount > 0 || !end->fusedRelu || end->fusedRelu != operands[i + 2] || end->idleForward) continue;
+        auto *r = static_cast<ReLU *>(operands[i + 2]);
+        bn->fusedRelu = r, bn->shortcutValue = end->other->Y->A, bn->shortcutGrad = end->other->Y->dAReserve;
+        r->absorbedBy = bn;
+        end->fusedRelu = nullptr, end->idleForward = end->idleGrad = true;
+    }
+    // absorbed ReLU, opening endpoint: the operand that absorbed the ReLU adds the endpoint's two gradients itself
+    for (uint32 i = 0; i + 1 < OPERAND_COUNT; i++) {
+        if (operands[i]->OPERAND_ID() != OPR_SEBLAS_RELU || operands[i + 1]->OPERAND_ID() != OPR_CTRL_SHORTCUTENDPOINT_BEG) continue;
+        auto *r = static_cast<ReLU *>(operands[i]);
+        auto *beg = static_cast<ShortcutEndpoint *>(operands[i + 1]);
+        if (!r->absorbedBy || beg->idleGrad || !beg->foldReserveEnabled) continue;
+        if (r->absorbedBy->takeGradientInParts(beg->Y->dA, beg->Y->dAReserve)) beg->idleGrad = true;
     }
     if (hipDeviceSynchronize() != hipSuccess) assertHip(__FILE__, __LINE__);  // buffers are released below: nothing may be in flight
     for (uint32 i = 0; i + 1 < OPERAND_COUNT; i++) {

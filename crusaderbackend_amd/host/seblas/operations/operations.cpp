@@ -260,24 +260,29 @@ Tensor *batchNormGradAll(Tensor *dY, Tensor *gamma, Tensor *X, Tensor *dX, Tenso
     return dX;
 }
 
-Tensor *batchNormRelu(Tensor *X, Tensor *beta, Tensor *gamma, Tensor *mean, Tensor *var, Tensor *reluOut) {
+Tensor *batchNormRelu(Tensor *X, Tensor *beta, Tensor *gamma, Tensor *mean, Tensor *var, Tensor *reluOut, Tensor *addend) {
     require(X->dims.n == reluOut->dims.n && X->dims.size == reluOut->dims.size, "batchNormRelu: X and the output differ");
     const uint32 F = X->dims.size / X->dims.n;
     require(beta->dims.size == F && gamma->dims.size == F && mean->dims.size == F && var->dims.size == F,
             "batchNormRelu: beta / gamma / mean / var must hold one value per feature");
+    require(!addend || addend->dims.size == X->dims.size, "batchNormRelu: addend size");
     finish(crb_batchnorm_relu_fwd(X->elements, beta->elements, gamma->elements, mean->elements, var->elements, nullptr, nullptr,
-                                  reluOut->elements, X->dims.n, F, nullptr),
+                                  addend ? addend->elements : nullptr, reluOut->elements, X->dims.n, F, nullptr),
            __FILE__, __LINE__);
     return reluOut;
 }
 
-Tensor *batchNormReluGradAll(Tensor *dReluOut, Tensor *reluOut, Tensor *gamma, Tensor *X, Tensor *dX, Tensor *dGamma, Tensor *dBeta) {
+Tensor *batchNormReluGradAll(Tensor *dReluOut, Tensor *reluOut, Tensor *gamma, Tensor *X, Tensor *dX, Tensor *dGamma, Tensor *dBeta,
+                             Tensor *dReluOut2, Tensor *maskedCopy) {
     require(dReluOut->dims.size == X->dims.size && reluOut->dims.size == X->dims.size && dX->dims.size == X->dims.size,
             "batchNormReluGradAll: tensor sizes differ");
     const uint32 F = X->dims.size / X->dims.n;
     require(gamma->dims.size == F && dGamma->dims.size == F && dBeta->dims.size == F, "batchNormReluGradAll: one value per feature");
-    finish(crb_batchnorm_relu_bwd(dReluOut->elements, reluOut->elements, gamma->elements, X->elements, dX->elements, dGamma->elements,
-                                  dBeta->elements, X->dims.n, F, nullptr),
+    require((!dReluOut2 || dReluOut2->dims.size == X->dims.size) && (!maskedCopy || maskedCopy->dims.size == X->dims.size),
+            "batchNormReluGradAll: optional tensor sizes differ");
+    finish(crb_batchnorm_relu_bwd(dReluOut->elements, dReluOut2 ? dReluOut2->elements : nullptr, reluOut->elements, gamma->elements,
+                                  X->elements, dX->elements, dGamma->elements, dBeta->elements, maskedCopy ? maskedCopy->elements : nullptr,
+                                  X->dims.n, F, nullptr),
            __FILE__, __LINE__);
     return dX;
 }
@@ -288,10 +293,13 @@ Tensor *addRelu(Tensor *A, Tensor *B, Tensor *out) {
     return out;
 }
 
-void reluGradTwice(Tensor *out, Tensor *dOut, Tensor *d1, Tensor *d2) {
+void reluGradTwice(Tensor *out, Tensor *dOut, Tensor *d1, Tensor *d2, Tensor *dOut2) {
     require(out->dims.size == dOut->dims.size && out->dims.size == d1->dims.size && out->dims.size == d2->dims.size,
             "reluGradTwice: element counts differ");
-    finish(crb_tensor_relu_grad_copy2(d1->elements, d2->elements, out->elements, dOut->elements, out->dims.size, nullptr), __FILE__, __LINE__);
+    require(!dOut2 || dOut2->dims.size == out->dims.size, "reluGradTwice: second gradient part size");
+    finish(crb_tensor_relu_grad_copy2(d1->elements, d2->elements, out->elements, dOut->elements, dOut2 ? dOut2->elements : nullptr,
+                                      out->dims.size, nullptr),
+           __FILE__, __LINE__);
 }
 
 void batchNormParamGrads(Tensor *dY, Tensor *xHat, Tensor *dGamma, Tensor *dBeta) {

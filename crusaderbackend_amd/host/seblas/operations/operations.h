@@ -73,12 +73,17 @@ Tensor *batchNormGradAll(Tensor *dY, Tensor *gamma, Tensor *X, Tensor *dX, Tenso
 // Normalisation and the ReLU behind it in one pass each way (same results as the two operators one after the other; no
 // counterpart in the reference). Forward writes reluOut = relu(batchNorm(X)), mean and var; backward takes the gradient
 // with respect to reluOut and yields dX, dGamma, dBeta.
-Tensor *batchNormRelu(Tensor *X, Tensor *beta, Tensor *gamma, Tensor *mean, Tensor *var, Tensor *reluOut);
-Tensor *batchNormReluGradAll(Tensor *dReluOut, Tensor *reluOut, Tensor *gamma, Tensor *X, Tensor *dX, Tensor *dGamma, Tensor *dBeta);
+// addend (or null): the other summand of a residual connection that closes between the normalisation and the ReLU.
+// dReluOut2 (or null): second part of the gradient (a residual connection opens right behind the ReLU: its main-path
+// and shortcut gradients are added here instead of in a pass of their own). maskedCopy (or null) receives the gradient as
+// it reaches the normalisation, for the shortcut of the connection that closes in front of the ReLU.
+Tensor *batchNormRelu(Tensor *X, Tensor *beta, Tensor *gamma, Tensor *mean, Tensor *var, Tensor *reluOut, Tensor *addend = nullptr);
+Tensor *batchNormReluGradAll(Tensor *dReluOut, Tensor *reluOut, Tensor *gamma, Tensor *X, Tensor *dX, Tensor *dGamma, Tensor *dBeta,
+                             Tensor *dReluOut2 = nullptr, Tensor *maskedCopy = nullptr);
 // out = relu(A + B), and the ReLU's gradient (dOut where out > 0, else 0) written to two tensors at once: the closing
 // shortcut endpoint with the ReLU behind it.
 Tensor *addRelu(Tensor *A, Tensor *B, Tensor *out);
-void reluGradTwice(Tensor *out, Tensor *dOut, Tensor *d1, Tensor *d2);
+void reluGradTwice(Tensor *out, Tensor *dOut, Tensor *d1, Tensor *d2, Tensor *dOut2 = nullptr);  // dOut2: second part of the gradient
 // cuOptim.cuh:16. V is the momentum buffer; Xgrad is cleared by the step.
 void momentumApply(Tensor *X, Tensor *Xgrad, Tensor *V, float LEARNING_RATE, float MOMENTUM);
 // Optimizers.cu:16-22 in one pass: X *= (1 - L2) then momentumApply. No separate counterpart in the reference.

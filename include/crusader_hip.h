@@ -187,9 +187,11 @@ int crb_tensor_add_clear(float *a, float *b, uint32_t count, void *stream);
 
 /* The closing shortcut endpoint with the ReLU that follows it (no counterpart in the reference: ShortcutEndpoint.cu:57-99
  * and ReLU.cu:8-17 are separate operands). crb_tensor_add_relu: dst = max(a + b, 0). crb_tensor_relu_grad_copy2:
- * dst1 = dst2 = (relu_out > 0 ? dY : 0), the ReLU's gradient delivered to the main path and to the shortcut at once. */
+ * dst1 = dst2 = (relu_out > 0 ? dY (+ dY2 when given) : 0), the ReLU's gradient delivered to the main path and to the
+ * shortcut at once. */
 int crb_tensor_add_relu(float *dst, const float *a, const float *b, uint32_t count, void *stream);
-int crb_tensor_relu_grad_copy2(float *dst1, float *dst2, const float *relu_out, const float *dY, uint32_t count, void *stream);
+int crb_tensor_relu_grad_copy2(float *dst1, float *dst2, const float *relu_out, const float *dY, const float *dY2_or_null, uint32_t count,
+                               void *stream);
 
 /* Fused forms of the copies and adds the shortcut operand performs (seann/operands/controlling/ShortcutEndpoint.cu):
  *   crb_tensor_add:             dst = a + b           (forward of the closing endpoint, :59-73: copy then add; dst may be a)
@@ -273,15 +275,19 @@ int crb_batchnorm_bwd(const float *dY, const float *gamma, const float *X, float
                       uint32_t N, uint32_t F, void *stream);
 
 /* Batch normalisation with the ReLU that follows it, in one pass each way (no counterpart in the reference, where
- * BatchNorm and ReLU are separate operands: seann/operands/seblas/BatchNorm.cu:13-21, activate/ReLU.cu:8-17).
- * Forward: what crb_batchnorm_fwd computes, plus reluOut = max(Y, 0); Y and xHat are written only when given.
- * Backward: dY is the gradient with respect to reluOut; the gradient reaching the normalisation is dY where reluOut > 0
- * and 0 elsewhere (reluGradFast's rule, since reluOut > 0 exactly where the ReLU's input is), then crb_batchnorm_bwd.
- * Results are bit-identical to the two separate calls. */
+ * BatchNorm, ShortcutEndpoint and ReLU are separate operands: seann/operands/seblas/BatchNorm.cu:13-21,
+ * controlling/ShortcutEndpoint.cu:57-99, activate/ReLU.cu:8-17).
+ * Forward: what crb_batchnorm_fwd computes, plus reluOut = max(Y + addend, 0); addend (or NULL) is the other summand of a
+ * residual connection that closes between the normalisation and the ReLU; Y and xHat are written only when given.
+ * Backward: dY (+ dY2 when given: the gradient arrives in two parts, as it does when a residual connection opens right
+ * behind the ReLU) is the gradient with respect to reluOut; the gradient reaching the normalisation is that sum where
+ * reluOut > 0 and 0 elsewhere (reluGradFast's rule, since reluOut > 0 exactly where the ReLU's input is), then
+ * crb_batchnorm_bwd. dYmasked, when given, receives that masked gradient (what the closing residual connection hands to
+ * its shortcut). Results are bit-identical to the separate calls. */
 int crb_batchnorm_relu_fwd(const float *X, const float *beta, const float *gamma, float *mean, float *var, float *Y_or_null,
-                           float *xHat_or_null, float *reluOut, uint32_t N, uint32_t F, void *stream);
-int crb_batchnorm_relu_bwd(const float *dY, const float *reluOut, const float *gamma, const float *X, float *dX, float *dGamma_or_null,
-                           float *dBeta_or_null, uint32_t N, uint32_t F, void *stream);
+                           float *xHat_or_null, const float *addend_or_null, float *reluOut, uint32_t N, uint32_t F, void *stream);
+int crb_batchnorm_relu_bwd(const float *dY, const float *dY2_or_null, const float *reluOut, const float *gamma, const float *X, float *dX,
+                           float *dGamma_or_null, float *dBeta_or_null, float *dYmasked_or_null, uint32_t N, uint32_t F, void *stream);
 
 /* Replaces seblas::batchNormParamGrads (cuBatchNorm.cu:190-202; kernel :127-148): dBeta = sum_n dY, dGamma = sum_n dY*xHat.
  * Both are overwritten, not accumulated. */

@@ -267,3 +267,33 @@ def test_add_relu_and_relu_grad_copy2(dev, n):
     capi.tensor_relu_grad_copy2(d1, d2, R, dY, n)
     g = orc.reluGradFast(orc.tensorAdd(a, b), dy)
     assert np.array_equal(to_np(d1), g) and np.array_equal(to_np(d2), g)
+
+
+@pytest.mark.parametrize("N,C,H,W", [(128, 16, 32, 32), (128, 64, 8, 8), (37, 3, 5, 7), (300, 2, 3, 3)])
+def test_batchnorm_relu_with_residual_parts_equals_separate_calls(dev, N, C, H, W):
+    """The forms used when a residual connection closes between the normalisation and the ReLU (forward: + addend) and
+    another one opens right behind the ReLU (backward: gradient in two parts, masked copy for the shortcut)."""
+    capi = _capi()
+    F = C * H * W
+    x, add = normal(60, N, C, H, W) * 1.5 + 0.3, normal(61, N, C, H, W)
+    gamma, beta, dy, dy2 = normal(62, F) + 1.0, normal(63, F), normal(64, N, C, H, W), normal(65, N, C, H, W)
+    X, A, G, B, dY, dY2 = (to_dev(v, dev) for v in (x, add, gamma, beta, dy, dy2))
+    Y, xh, m, v, Z, R = _nan(dev, N, F), _nan(dev, N, F), _nan(dev, F), _nan(dev, F), _nan(dev, N, F), _nan(dev, N, F)
+    capi.batchnorm_fwd(X, B, G, m, v, Y, xh, N, F)
+    capi.tensor_add(Z, Y, A, N * F)
+    capi.relu_fwd(Z, R, N * F)
+    g, dZ, dX, dG, dB = _nan(dev, N, F), _nan(dev, N, F), _nan(dev, N, F), _nan(dev, F), _nan(dev, F)
+    capi.tensor_add(g, dY, dY2, N * F)
+    capi.relu_bwd(Z, g, dZ, N * F)
+    capi.batchnorm_bwd(dZ, G, X, dX, N, F, dGamma=dG, dBeta=dB)
+    m2, v2, R2 = _nan(dev, F), _nan(dev, F), _nan(dev, N, F)
+    capi.batchnorm_relu_fwd(X, B, G, m2, v2, R2, N, F, addend=A)
+    assert np.array_equal(to_np(R), to_np(R2)) and np.array_equal(to_np(m), to_np(m2)) and np.array_equal(to_np(v), to_np(v2))
+    dX2, dG2, dB2, dM = _nan(dev, N, F), _nan(dev, F), _nan(dev, F), _nan(dev, N, F)
+    capi.batchnorm_relu_bwd(dY, R2, G, X, dX2, N, F, dGamma=dG2, dBeta=dB2, dY2=dY2, dYmasked=dM)
+    for a, b in ((dX, dX2), (dG, dG2), (dB, dB2), (dZ, dM)):
+        assert np.array_equal(to_np(a), to_np(b), equal_nan=True)
+    # two-part gradient without a mask copy, and through the shortcut form
+    d1, d2 = _nan(dev, N * F), _nan(dev, N * F)
+    capi.tensor_relu_grad_copy2(d1, d2, R, dY, N * F, dY2=dY2)
+    assert np.array_equal(to_np(d1).ravel(), to_np(dZ).ravel()) and np.array_equal(to_np(d2).ravel(), to_np(dZ).ravel())
