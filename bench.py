@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the seblas conv/GEMM hot path on one MI355X.
 
-Default workload (BASELINE config 2): the convolution layers of ResNet-56 on CIFAR-shaped tensors, fp32 NCHW,
+Default workload (benchmark configuration 2): the convolution layers of ResNet-56 on CIFAR-shaped tensors, fp32 NCHW,
 batch 128. One *step* = forward + data-gradient + weight-gradient of every 3x3 conv layer of the network's three
 stages and two stride-2 transitions, with the layer multiplicities of the reference's archived model
 (archive/Resnet56: 19x 16->16@32, 17x 32->32@16, 18x 64->64@8, 1x 16->32 s2, 1x 32->64 s2), on synthetic
@@ -12,7 +12,7 @@ Prints ONE JSON line. `value` is TFLOP/s over the timed steps; `extra` carries i
 `roofline` describes the kernel that takes the most time in the step, timed per launch with HIP events on the
 launch stream in a separate instrumented pass. `cpu_baseline` is the CPU oracle on a bounded sample.
 
-  python bench.py [--gpus 1] [--steps K] [--warmup W] [--report FILE]   (--report adds every BASELINE config)
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--report FILE]   (--report adds every benchmark configuration)
 """
 import argparse
 import json
@@ -43,7 +43,7 @@ def parse():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--report", type=str, default=None, help="also time every BASELINE config and write a JSON report")
+    ap.add_argument("--report", type=str, default=None, help="also time every benchmark configuration and write a JSON report")
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     ap.add_argument("--calibrate", action="store_true",
                     help="only run a plain streaming kernel of known size (a += b on 64 Mi floats: reads 512 MiB, writes "

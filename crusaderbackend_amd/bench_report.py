@@ -1,4 +1,4 @@
-"""Extended timing report over every BASELINE configuration (used by ``bench.py --report FILE``).
+"""Extended timing report over every benchmark configuration (used by ``bench.py --report FILE``).
 
 Each entry: launch duration from HIP events on the launch stream (average of back-to-back launches), nominal
 flops, algorithmic bytes (each operand read once, output written once), TFLOP/s, GB/s and the fraction of the

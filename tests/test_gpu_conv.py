@@ -1,7 +1,7 @@
 """GPU parity of the convolution entry points (through the C ABI) against the CPU oracle.
 
 The reference only ever tested dgrad with stride 1 / pad 0 (validation/UnitTestTools.cu:172-300);
-this grid keeps that family and adds strides, padding, forward, wgrad, bias and the BASELINE layer shapes.
+this grid keeps that family and adds strides, padding, forward, wgrad, bias and the benchmark configurations' layer shapes.
 """
 import numpy as np
 import pytest
@@ -95,14 +95,14 @@ RESNET = [
 
 @pytest.mark.parametrize("IC,H,OC,s", RESNET)
 def test_conv_resnet56_layers(dev, IC, H, OC, s):
-    """BASELINE config 2 layer shapes (3x3, pad 1) at batch 16; the full batch-128 shapes are covered by the
+    """ResNet-56 layer shapes (benchmark configuration 2) (3x3, pad 1) at batch 16; the full batch-128 shapes are covered by the
     adjoint property test below."""
     run_layer(dev, 16, IC, H, H, OC, 3, 3, s, s, 1, 1, seed=4)
 
 
 @pytest.mark.parametrize("IC,H", [(24, 32), (108, 16), (330, 8)])
 def test_conv_densenet_layers(dev, IC, H):
-    """BASELINE config 4: 1x1 IC->48 bottleneck then 3x3 48->12, with bias, batch 8."""
+    """benchmark configuration 4 (DenseNet-BC bottleneck): 1x1 IC->48 bottleneck then 3x3 48->12, with bias, batch 8."""
     run_layer(dev, 8, IC, H, H, 48, 1, 1, 1, 1, 0, 0, bias=True, seed=5)
     run_layer(dev, 8, 48, H, H, 12, 3, 3, 1, 1, 1, 1, bias=True, seed=6)
 
@@ -114,7 +114,7 @@ def test_conv_vgg_stem_and_wide(dev):
 
 @pytest.mark.parametrize("IC,H,OC,s", RESNET)
 def test_conv_full_batch_adjoint(dev, IC, H, OC, s):
-    """Size-independent property at the full BASELINE batch (128): <conv(W,X), dY> = <X, dgrad(W,dY)> =
+    """Size-independent property at the full benchmark batch (128): <conv(W,X), dY> = <X, dgrad(W,dY)> =
     <W, wgrad(dY,X)>, inner products accumulated in float64 on the device results."""
     import torch
     capi = _capi()

@@ -63,7 +63,7 @@ def run_nta(dev, M, N, K, batch, seed):
 
 
 def test_sgemm_config1_1024(dev):
-    """BASELINE config 1: M=N=K=1024, uniform[-1,1], fixed seeds."""
+    """benchmark configuration 1: M=N=K=1024, uniform[-1,1], fixed seeds."""
     run_nn(dev, 1024, 1024, 1024, 1, seed=1)
 
 
