@@ -8,6 +8,7 @@ namespace crb {
 // problems that would not fill 256 CUs with large tiles.
 typedef TileCfg<128, 128, 16, 2, 2, 2> CfgLarge;
 typedef TileCfg<64, 64, 16, 2, 2, 2> CfgSmall;
+typedef TileCfg<64, 64, 64, 2, 2, 2> CfgSmallDeep;  // 64-wide K slabs: one workgroup per CU has nobody to hide its loads behind
 
 static inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
@@ -39,6 +40,9 @@ static int run_tiles(const AOp &a, const BOp &b, const RowMajorEpi &e, u32 M, u3
     const uint64_t tiles_s = uint64_t(ceil_div(M, 64)) * ceil_div(N, 64) * zdim;
     if (M > 64 && N > 64) {
         if (tiles_l >= 160) return run_cfg<CfgLarge>(a, b, e, M, N, K, zdim, s, what);
+        // at most one small tile per CU and a long contraction: longer slabs, so that a slab's loads have a whole slab of
+        // MFMAs (2048 clocks) to arrive in
+        if (tiles_s >= 160 && tiles_s <= 256 && K >= 512 && K < 2048) return run_cfg<CfgSmallDeep>(a, b, e, M, N, K, zdim, s, what);
         if (tiles_s >= 160 && K < 2048) return run_cfg<CfgSmall>(a, b, e, M, N, K, zdim, s, what);
         const SplitPlan sp = plan_split(M, N, K, 128, 128, 16, zdim);
         if (sp.splits > 1 && sp.k_per_z >= 512) return run_cfg<CfgLarge>(a, b, e, M, N, K, zdim, s, what);
