@@ -9,6 +9,7 @@ namespace crb {
 typedef TileCfg<128, 128, 16, 2, 2, 2> CfgLarge;
 typedef TileCfg<64, 64, 16, 2, 2, 2> CfgSmall;
 typedef TileCfg<64, 64, 64, 2, 2, 2> CfgSmallDeep;  // 64-wide K slabs: one workgroup per CU has nobody to hide its loads behind
+typedef TileCfg<64, 64, 32, 2, 2, 2, 2> CfgSmallAhead;  // loads run two slabs ahead: small tiles finish a slab faster than a load takes
 
 static inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
@@ -34,16 +35,20 @@ static int run_cfg(const AOp &a, const BOp &b, const RowMajorEpi &e, u32 M, u32 
 template <class AOp, class BOp>
 static int run_tiles(const AOp &a, const BOp &b, const RowMajorEpi &e, u32 M, u32 N, u32 K, u32 zdim, hipStream_t s,
                      const char *what) {
-    // Large tiles when their grid alone occupies the chip; otherwise small tiles if those do; otherwise split K —
-    // with large tiles only when each slice keeps a long contraction (the split costs a second pass over the result).
+    // Tile choice by how many workgroups the grid gives a CU; when neither tile size fills the chip, K is split — with
+    // large tiles only when each slice keeps a long contraction (the split costs a second pass over the result).
     const uint64_t tiles_l = uint64_t(ceil_div(M, 128)) * ceil_div(N, 128) * zdim;
     const uint64_t tiles_s = uint64_t(ceil_div(M, 64)) * ceil_div(N, 64) * zdim;
     if (M > 64 && N > 64) {
-        if (tiles_l >= 160) return run_cfg<CfgLarge>(a, b, e, M, N, K, zdim, s, what);
+        // measured on square and skinny-K problems: large tiles win once they give a CU three or more workgroups; below
+        // that, small tiles with loads two slabs ahead win as soon as there are two of them per CU
+        if (tiles_l >= 800) return run_cfg<CfgLarge>(a, b, e, M, N, K, zdim, s, what);
+        if (tiles_s >= 512) return run_cfg<CfgSmallAhead>(a, b, e, M, N, K, zdim, s, what);
         // at most one small tile per CU and a long contraction: longer slabs, so that a slab's loads have a whole slab of
         // MFMAs (2048 clocks) to arrive in
-        if (tiles_s >= 160 && tiles_s <= 256 && K >= 512 && K < 2048) return run_cfg<CfgSmallDeep>(a, b, e, M, N, K, zdim, s, what);
-        if (tiles_s >= 160 && K < 2048) return run_cfg<CfgSmall>(a, b, e, M, N, K, zdim, s, what);
+        if (tiles_s >= 160 && K >= 512 && K < 2048) return run_cfg<CfgSmallDeep>(a, b, e, M, N, K, zdim, s, what);
+        if (tiles_s >= 160 && K < 2048) return run_cfg<CfgSmallAhead>(a, b, e, M, N, K, zdim, s, what);
+        if (tiles_l >= 160) return run_cfg<CfgLarge>(a, b, e, M, N, K, zdim, s, what);
         const SplitPlan sp = plan_split(M, N, K, 128, 128, 16, zdim);
         if (sp.splits > 1 && sp.k_per_z >= 512) return run_cfg<CfgLarge>(a, b, e, M, N, K, zdim, s, what);
     }

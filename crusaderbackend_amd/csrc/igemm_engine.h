@@ -37,9 +37,12 @@ struct IgemmDims {
     u32 split_k;  // 0: blockIdx.z is a batch index; 1: blockIdx.z is a K-split index
 };
 
-template <int BM_, int BN_, int BK_, int WM_, int WN_, int OCC_>
+// PF_: how many K slabs ahead of the MFMAs the global loads run (1: the next slab's loads have one slab of MFMAs to
+// arrive in; 2: two register sets, two slabs in flight — for grids that leave a CU a single workgroup).
+template <int BM_, int BN_, int BK_, int WM_, int WN_, int OCC_, int PF_ = 1>
 struct TileCfg {
-    static constexpr int BM = BM_, BN = BN_, BK = BK_, WM = WM_, WN = WN_, OCC = OCC_;
+    static constexpr int BM = BM_, BN = BN_, BK = BK_, WM = WM_, WN = WN_, OCC = OCC_, PF = PF_;
+    static_assert(PF == 1 || PF == 2, "prefetch distance");
     static constexpr int WTM = BM / WM, WTN = BN / WN;  // wave tile
     static constexpr int TM = WTM / 32, TN = WTN / 32;  // 32x32 MFMA blocks per wave tile
     static_assert(WM * WN == 4, "4 waves per workgroup");
@@ -237,21 +240,8 @@ __global__ void __launch_bounds__(kThreads, Cfg::OCC) igemm_kernel(AOp a, BOp b,
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[mi][ni][r] = 0.0f;
 
-    if (kbeg < kend) {
-        la.fetch(a, kbeg, kend);
-        lb.fetch(b, kbeg, kend);
-        la.commit(sA[0]);
-        lb.commit(sB[0]);
-    }
-    __syncthreads();
-
-    int buf = 0;
-    for (u32 k0 = kbeg; k0 < kend; k0 += BK, buf ^= 1) {
-        const bool more = k0 + BK < kend;
-        if (more) {
-            la.fetch(a, k0 + BK, kend);
-            lb.fetch(b, k0 + BK, kend);
-        }
+    // the MFMAs of the slab held by LDS buffer `buf`
+    auto multiply = [&](int buf) {
         const float *pa = sA[buf], *pb = sB[buf];
 #pragma unroll
         for (int g = 0; g < BK / 8; ++g) {
@@ -266,11 +256,67 @@ __global__ void __launch_bounds__(kThreads, Cfg::OCC) igemm_kernel(AOp a, BOp b,
                     for (int ni = 0; ni < TN; ++ni)
                         acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[s][mi], fb[s][ni], acc[mi][ni], 0, 0, 0);
         }
-        if (more) {
-            la.commit(sA[buf ^ 1]);
-            lb.commit(sB[buf ^ 1]);
+    };
+
+    if constexpr (Cfg::PF == 2) {
+        // Two register sets: slab t travels in set t % 2. While slab s is multiplied, slab s + 1 is already on its way
+        // (issued one iteration earlier) and slab s + 2 is issued; slab s + 1 is committed to LDS after the MFMAs.
+        LA la2;
+        LB lb2;
+        la2.init(a, row0);
+        lb2.init(b, col0);
+        if (kbeg < kend) {
+            la.fetch(a, kbeg, kend);
+            lb.fetch(b, kbeg, kend);
+            if (kbeg + BK < kend) {
+                la2.fetch(a, kbeg + BK, kend);
+                lb2.fetch(b, kbeg + BK, kend);
+            }
+            la.commit(sA[0]);
+            lb.commit(sB[0]);
         }
         __syncthreads();
+        // one step: multiply slab k0 (buffer `buf`), issue slab k0 + 2 BK into `far` (the set slab k0 arrived in),
+        // commit slab k0 + BK from `near`
+        auto step = [&](u32 k0, int buf, LA &far_a, LB &far_b, LA &near_a, LB &near_b) {
+            if (k0 + 2 * BK < kend) {
+                far_a.fetch(a, k0 + 2 * BK, kend);
+                far_b.fetch(b, k0 + 2 * BK, kend);
+            }
+            multiply(buf);
+            if (k0 + BK < kend) {
+                near_a.commit(sA[buf ^ 1]);
+                near_b.commit(sB[buf ^ 1]);
+            }
+            __syncthreads();
+        };
+        for (u32 k0 = kbeg; k0 < kend; k0 += 2 * BK) {
+            step(k0, 0, la, lb, la2, lb2);
+            if (k0 + BK < kend) step(k0 + BK, 1, la2, lb2, la, lb);
+        }
+    } else {
+        if (kbeg < kend) {
+            la.fetch(a, kbeg, kend);
+            lb.fetch(b, kbeg, kend);
+            la.commit(sA[0]);
+            lb.commit(sB[0]);
+        }
+        __syncthreads();
+
+        int buf = 0;
+        for (u32 k0 = kbeg; k0 < kend; k0 += BK, buf ^= 1) {
+            const bool more = k0 + BK < kend;
+            if (more) {
+                la.fetch(a, k0 + BK, kend);
+                lb.fetch(b, k0 + BK, kend);
+            }
+            multiply(buf);
+            if (more) {
+                la.commit(sA[buf ^ 1]);
+                lb.commit(sB[buf ^ 1]);
+            }
+            __syncthreads();
+        }
     }
 
     // epilogue: accumulator register r of lane l is D[8*(r/4) + 4*(l/32) + r%4][l%32] of its block
