@@ -181,8 +181,11 @@ int conv2x2_wgrad(const float *dY, const float *X, float *dW, float *G, u32 N, u
     MatR<true> b{X, Nc, Nc, 0};
     // G may be the library's scratch arena, so the contraction is never split here
     const uint64_t tiles_l = uint64_t(ceil_div(M, 128)) * ceil_div(Nc, 128);
-    int st = tiles_l >= 128 ? launch_igemm<CfgLarge>(a, b, e, M, Nc, N, 1, 0, N, s, what)
-                            : launch_igemm<CfgSmall>(a, b, e, M, Nc, N, 1, 0, N, s, what);
+    const uint64_t tiles_s = uint64_t(ceil_div(M, 64)) * ceil_div(Nc, 64);
+    int st = tiles_l >= 800   ? launch_igemm<CfgLarge>(a, b, e, M, Nc, N, 1, 0, N, s, what)
+             : tiles_s >= 512 ? launch_igemm<CfgSmallAhead>(a, b, e, M, Nc, N, 1, 0, N, s, what)
+             : tiles_l >= 128 ? launch_igemm<CfgLarge>(a, b, e, M, Nc, N, 1, 0, N, s, what)
+                              : launch_igemm<CfgSmall>(a, b, e, M, Nc, N, 1, 0, N, s, what);
     if (st) return st;
     hipLaunchKernelGGL(conv2x2_fold_kernel, dim3(ceil_div(OC * IC, 256)), dim3(256), 0, s, G, dW, OC, IC);
     return check_launch(what);
