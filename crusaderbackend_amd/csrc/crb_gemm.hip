@@ -52,6 +52,7 @@ static int run_tiles(const AOp &a, const BOp &b, const RowMajorEpi &e, u32 M, u3
         const SplitPlan sp = plan_split(M, N, K, 128, 128, 16, zdim);
         if (sp.splits > 1 && sp.k_per_z >= 512) return run_cfg<CfgLarge>(a, b, e, M, N, K, zdim, s, what);
     }
+    if (K >= 32768) return run_cfg<CfgSmallAhead>(a, b, e, M, N, K, zdim, s, what);  // very long contraction: slices stay long after the split
     return run_cfg<CfgSmall>(a, b, e, M, N, K, zdim, s, what);
 }
 
