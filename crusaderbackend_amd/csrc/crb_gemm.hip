@@ -18,8 +18,12 @@ static inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t
 // them in fixed order and applies the epilogue (bias / accumulate / ReLU).
 template <class Cfg, class AOp, class BOp>
 static int run_cfg(const AOp &a, const BOp &b, const RowMajorEpi &e, u32 M, u32 N, u32 K, u32 zdim, hipStream_t s,
-                   const char *what) {
-    const SplitPlan sp = plan_split(M, N, K, Cfg::BM, Cfg::BN, Cfg::BK, zdim);
+                   const char *what, u32 want_splits = 0) {
+    SplitPlan sp = plan_split(M, N, K, Cfg::BM, Cfg::BN, Cfg::BK, zdim);
+    if (want_splits > 1 && zdim == 1 && sp.splits == 1) {  // the caller wants K cut although the tile grid covers the chip
+        sp.k_per_z = ceil_div(ceil_div(K, want_splits), u32(Cfg::BK)) * Cfg::BK;
+        sp.splits = ceil_div(K, sp.k_per_z);
+    }
     if (sp.splits == 1) return launch_igemm<Cfg>(a, b, e, M, N, K, zdim, 0, K, s, what);
     if (e.ld != N) return launch_igemm<Cfg>(a, b, e, M, N, K, zdim, 0, K, s, what);  // partials assume a dense result
     const size_t need = size_t(sp.splits) * M * N * sizeof(float);
@@ -48,6 +52,8 @@ static int run_tiles(const AOp &a, const BOp &b, const RowMajorEpi &e, u32 M, u3
         // MFMAs (2048 clocks) to arrive in
         if (tiles_s >= 160 && K >= 512 && K < 2048) return run_cfg<CfgSmallDeep>(a, b, e, M, N, K, zdim, s, what);
         if (tiles_s >= 160 && K < 2048) return run_cfg<CfgSmallAhead>(a, b, e, M, N, K, zdim, s, what);
+        // one small tile per CU at most but a long contraction: two K slices per tile put two workgroups on every CU
+        if (tiles_s >= 160 && K >= 2048 && zdim == 1 && e.ld == N) return run_cfg<CfgSmallAhead>(a, b, e, M, N, K, zdim, s, what, 2);
         if (tiles_l >= 160) return run_cfg<CfgLarge>(a, b, e, M, N, K, zdim, s, what);
         const SplitPlan sp = plan_split(M, N, K, 128, 128, 16, zdim);
         if (sp.splits > 1 && sp.k_per_z >= 512) return run_cfg<CfgLarge>(a, b, e, M, N, K, zdim, s, what);
