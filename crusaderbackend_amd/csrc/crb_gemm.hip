@@ -46,6 +46,8 @@ static int run_tiles(const AOp &a, const BOp &b, const RowMajorEpi &e, u32 M, u3
     if (M > 64 && N > 64) {
         // measured on square and skinny-K problems: large tiles win once they give a CU three or more workgroups; below
         // that, small tiles with loads two slabs ahead win as soon as there are two of them per CU
+        // a short contraction (16 large slabs or fewer) is mostly prologue and epilogue for a large tile
+        if (tiles_l >= 800 && K <= 256) return run_cfg<CfgSmallAhead>(a, b, e, M, N, K, zdim, s, what);
         if (tiles_l >= 800) return run_cfg<CfgLarge>(a, b, e, M, N, K, zdim, s, what);
         if (tiles_s >= 512) return run_cfg<CfgSmallAhead>(a, b, e, M, N, K, zdim, s, what);
         // at most one small tile per CU and a long contraction: longer slabs, so that a slab's loads have a whole slab of
