@@ -57,6 +57,8 @@ static int run_tiles(const AOp &a, const BOp &b, const RowMajorEpi &e, u32 M, u3
         // one small tile per CU at most but a long contraction: two K slices per tile put two workgroups on every CU
         if (tiles_s >= 160 && K >= 2048 && zdim == 1 && e.ld == N) return run_cfg<CfgSmallAhead>(a, b, e, M, N, K, zdim, s, what, 2);
         if (tiles_l >= 160) return run_cfg<CfgLarge>(a, b, e, M, N, K, zdim, s, what);
+        // A grid of small tiles somewhat short of the chip, cut over K by plan_split, beats large tiles cut deeper.
+        if (tiles_s >= 100 && K >= 512 && K < 2048) return run_cfg<CfgSmallAhead>(a, b, e, M, N, K, zdim, s, what);
         const SplitPlan sp = plan_split(M, N, K, 128, 128, 16, zdim);
         if (sp.splits > 1 && sp.k_per_z >= 512) return run_cfg<CfgLarge>(a, b, e, M, N, K, zdim, s, what);
     }
