@@ -16,8 +16,9 @@ int fail(int st, const char *fmt, ...);
 int check_hip(hipError_t e, const char *what);
 int check_launch(const char *what);
 
-// Lazily grown device scratch (split-K partial sums). Returns nullptr on allocation failure.
-void *arena_get(size_t bytes);
+// Lazily grown device scratch (split-K partial sums) of the current device and `stream`; the block stays valid for work
+// queued on that stream until a later arena_get on the same stream asks for more. Returns nullptr on allocation failure.
+void *arena_get(size_t bytes, hipStream_t stream);
 void arena_release();
 
 // Exact floor(n / d) for any n, d in [1, 2^32): round-up magic multiply (Granlund-Montgomery).

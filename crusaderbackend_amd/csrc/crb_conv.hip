@@ -67,7 +67,7 @@ static int run_nchw(const AOp &a, const BOp &b, NchwEpi e, u32 M, u32 N, u32 K, 
     if (sp.splits == 1) return run_by_m(a, b, e, M, N, K, 1, 0, K, s, what);
     const u32 count = M * N;  // N = batch * H * W, so M*N is the whole NCHW tensor
     const size_t need = size_t(sp.splits) * count * sizeof(float);
-    float *ws = static_cast<float *>(arena_get(need));
+    float *ws = static_cast<float *>(arena_get(need, s));
     if (!ws) return fail(CRB_EHIP, "%s: cannot allocate %zu bytes of split-K scratch", what, need);
     NchwEpi pe = e;
     pe.T = ws, pe.row_bias = nullptr, pe.flags = 0u, pe.zstride = count;
@@ -513,7 +513,7 @@ int crb_conv_wgrad(const float *dY, const float *X, float *dW, const crb_conv_ge
             if (workspace_bytes < need || !aligned16(G))
                 return fail(CRB_EWORKSPACE, "crb_conv_wgrad: workspace %zu bytes < required %zu (or not 16-byte aligned)", workspace_bytes, need);
         } else {
-            G = static_cast<float *>(arena_get(need));
+            G = static_cast<float *>(arena_get(need, s));
             if (!G) return fail(CRB_EHIP, "crb_conv_wgrad: cannot allocate %zu bytes of scratch", need);
         }
         return conv2x2_wgrad(dY, X, dW, G, g->N, g->IC, g->OC, s, "crb_conv_wgrad");
@@ -529,7 +529,7 @@ int crb_conv_wgrad(const float *dY, const float *X, float *dW, const crb_conv_ge
                         return fail(CRB_EWORKSPACE, "crb_conv_wgrad: workspace %zu bytes < required %zu", workspace_bytes,
                                     dp.workspace_bytes);
                 } else {
-                    dws = static_cast<float *>(arena_get(dp.workspace_bytes));
+                    dws = static_cast<float *>(arena_get(dp.workspace_bytes, s));
                     if (!dws) return fail(CRB_EHIP, "crb_conv_wgrad: cannot allocate %zu bytes of scratch", dp.workspace_bytes);
                 }
             }
@@ -551,7 +551,7 @@ int crb_conv_wgrad(const float *dY, const float *X, float *dW, const crb_conv_ge
         if (workspace_bytes < need)
             return fail(CRB_EWORKSPACE, "crb_conv_wgrad: workspace %zu bytes < required %zu", workspace_bytes, need);
     } else {
-        ws = static_cast<float *>(arena_get(need));
+        ws = static_cast<float *>(arena_get(need, s));
         if (!ws) return fail(CRB_EHIP, "crb_conv_wgrad: cannot allocate %zu bytes of scratch", need);
     }
     RowMajorEpi e{ws, nullptr, p.Ncols, p.M * p.Ncols, 0u};
@@ -573,7 +573,7 @@ int crb_conv_bwd(const float *W, const float *dY, const float *X, float *dX, flo
                     if (workspace_bytes < dp.workspace_bytes)
                         return fail(CRB_EWORKSPACE, "crb_conv_bwd: workspace %zu bytes < required %zu", workspace_bytes, dp.workspace_bytes);
                 } else {
-                    dws = static_cast<float *>(arena_get(dp.workspace_bytes));
+                    dws = static_cast<float *>(arena_get(dp.workspace_bytes, hipStream_t(stream)));
                     if (!dws) return fail(CRB_EHIP, "crb_conv_bwd: cannot allocate %zu bytes of scratch", dp.workspace_bytes);
                 }
             }
@@ -645,7 +645,7 @@ int crb_conv_bias_grad(const float *dY, float *dB, uint32_t N, uint32_t C, uint3
     const u32 rows_per_slice = ceil_div(N, slices);
     slices = ceil_div(N, rows_per_slice);
     const size_t need = size_t(slices) * cols * sizeof(float);
-    float *part = static_cast<float *>(arena_get(need));
+    float *part = static_cast<float *>(arena_get(need, s));
     if (!part) return fail(CRB_EHIP, "crb_conv_bias_grad: cannot allocate %zu bytes of scratch", need);
     if (vec)
         hipLaunchKernelGGL(bias_grad_colsum_kernel<true>, dim3(col_wgs, slices), dim3(256), 0, s, dY, part, N, cols, rows_per_slice);

@@ -27,7 +27,7 @@ static int run_cfg(const AOp &a, const BOp &b, const RowMajorEpi &e, u32 M, u32 
     if (sp.splits == 1) return launch_igemm<Cfg>(a, b, e, M, N, K, zdim, 0, K, s, what);
     if (e.ld != N) return launch_igemm<Cfg>(a, b, e, M, N, K, zdim, 0, K, s, what);  // partials assume a dense result
     const size_t need = size_t(sp.splits) * M * N * sizeof(float);
-    float *ws = static_cast<float *>(arena_get(need));
+    float *ws = static_cast<float *>(arena_get(need, s));
     if (!ws) return fail(CRB_EHIP, "%s: cannot allocate %zu bytes of split-K scratch", what, need);
     RowMajorEpi pe{ws, nullptr, N, M * N, 0u};
     if (int st = launch_igemm<Cfg>(a, b, pe, M, N, K, sp.splits, 1, sp.k_per_z, s, what)) return st;

@@ -48,8 +48,12 @@ int crb_abi_version(void);
 /* Message for the most recent non-OK status returned to the calling thread ("" if none). */
 const char *crb_last_error_string(void);
 
-/* Releases the library's lazily grown split-K scratch arena (safe to call at any time when no
- * library kernel is in flight). */
+/* Releases the library's lazily grown split-K scratch arenas (safe to call at any time when no
+ * library kernel is in flight). The library keeps one arena per (device, stream), so calls queued on
+ * different streams never share scratch and may overlap; calls on one stream run in order and reuse
+ * that stream's arena. An arena grows with hipMalloc on first use or when a call needs more (after
+ * waiting for that stream), so callers that must not allocate pass their own workspace where an
+ * entry point takes one. */
 void crb_release_workspace(void);
 
 /* GEMM family ------------------------------------------------------------------------------ */

@@ -185,3 +185,31 @@ def test_split_k_nta_small_output_and_bias_epilogue(dev):
     Y2 = _empty(dev, batch, OUT)
     capi.linear_fwd(to_dev(X, dev), to_dev(W, dev), to_dev(b, dev), Y2, batch, IN, OUT, flags=capi.CRB_FLAG_RELU)
     assert np.array_equal(to_np(Y), to_np(Y2))
+
+
+def test_split_k_on_two_streams_keeps_scratch_apart(dev):
+    """Split-K calls queued on two streams at once use separate scratch: each result equals the one the same call gives alone."""
+    import torch
+    capi = _capi()
+    shapes = [(256, 256, 4096), (192, 320, 6144)]
+    ops = []
+    for i, (M, N, K) in enumerate(shapes):
+        A, B = to_dev(uniform(60 + i, M, K), dev), to_dev(uniform(70 + i, K, N), dev)
+        alone = _empty(dev, M, N)
+        capi.sgemm_nn(A, B, alone, M, N, K)
+        ops.append((A, B, alone, M, N, K))
+    torch.cuda.synchronize()
+    streams = [torch.cuda.Stream(device=dev) for _ in shapes]
+    outs = [[_empty(dev, M, N) for _ in range(8)] for (_, _, _, M, N, K) in ops]
+    for rep in range(8):  # interleaved, so the two streams' kernels overlap on the device
+        for (A, B, _, M, N, K), st, out in zip(ops, streams, outs):
+            capi.sgemm_nn(A, B, out[rep], M, N, K, stream=st)
+    torch.cuda.synchronize()
+    for (_, _, alone, M, N, K), out in zip(ops, outs):
+        for rep in range(8):
+            assert torch.equal(out[rep], alone), f"{M}x{N}x{K} repeat {rep}"
+    capi.load().crb_release_workspace()
+    again = _empty(dev, *shapes[0][:2])
+    capi.sgemm_nn(ops[0][0], ops[0][1], again, *shapes[0])  # the arena comes back after a release
+    torch.cuda.synchronize()
+    assert torch.equal(again, ops[0][2])
