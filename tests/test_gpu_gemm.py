@@ -213,3 +213,55 @@ def test_split_k_on_two_streams_keeps_scratch_apart(dev):
     capi.sgemm_nn(ops[0][0], ops[0][1], again, *shapes[0])  # the arena comes back after a release
     torch.cuda.synchronize()
     assert torch.equal(again, ops[0][2])
+
+
+def test_sgemm_4096_cubed_full_size(dev):
+    """The headline GEMM shape at full size: against the oracle on seeded uniform[-1,1] inputs, and exactly against a product
+    whose value is known in closed form (B a signed permutation: every output element is one input element, sign flipped or not)."""
+    import torch
+    n = 4096
+    capi = _capi()
+    A = uniform(5, n, n)
+    B = uniform(6, n, n)
+    C = _empty(dev, n, n)
+    Ad = to_dev(A, dev)
+    capi.sgemm_nn(Ad, to_dev(B, dev), C, n, n, n)
+    assert_close(to_np(C), _oracle().sgemm(A, B[None], threads=16)[0], n, "sgemm_nn 4096^3")
+    perm = rng_perm(7, n)
+    sign = np.where(np.arange(n) % 3 == 0, -1.0, 1.0).astype(np.float32)
+    P = np.zeros((n, n), dtype=np.float32)
+    P[perm, np.arange(n)] = sign  # column j of A*P is sign[j] * column perm[j] of A
+    capi.sgemm_nn(Ad, to_dev(P, dev), C, n, n, n)
+    assert np.array_equal(to_np(C), A[:, perm] * sign[None, :])
+    # and the transposed-operand forms on the same inputs give the same matrix as the NN form, to rounding
+    Ct = _empty(dev, n, n)
+    capi.sgemm_tn(to_dev(np.ascontiguousarray(A.T), dev), to_dev(P, dev), Ct, n, n, n)
+    assert np.array_equal(to_np(Ct), to_np(C))
+    capi.sgemm_nt(Ad, to_dev(np.ascontiguousarray(P.T), dev), Ct, n, n, n)
+    assert np.array_equal(to_np(Ct), to_np(C))
+
+
+def rng_perm(seed, n):
+    return np.random.default_rng(seed).permutation(n)
+
+
+def test_dense_sweep_configuration_full_size(dev):
+    """benchmark configuration 5: batch 256 through FC 4096 -> 4096 in the forward (NT), data-gradient (NN) and
+    weight-gradient (TN) forms, plus the tall-skinny im2col product 32768 x 64 x 576; uniform[-1,1], fixed seeds."""
+    capi, orc = _capi(), _oracle()
+    batch, IN, OUT = 256, 4096, 4096
+    X, W, b, dY = uniform(1, batch, IN), uniform(2, OUT, IN), uniform(3, OUT), uniform(4, batch, OUT)
+    Xd, Wd, dYd = to_dev(X, dev), to_dev(W, dev), to_dev(dY, dev)
+    Y = _empty(dev, batch, OUT)
+    capi.linear_fwd(Xd, Wd, to_dev(b, dev), Y, batch, IN, OUT)
+    assert_close(to_np(Y), orc.linear(X, W, b, threads=16), IN, "linear 256x4096x4096")
+    dX = _empty(dev, batch, IN)
+    capi.linear_dgrad(dYd, Wd, dX, batch, IN, OUT)
+    assert_close(to_np(dX), orc.linearXGrad(dY, W, threads=16), OUT, "linearXGrad 256x4096x4096")
+    dW0, dB0 = uniform(5, OUT, IN), uniform(6, OUT)
+    dW, dB = to_dev(dW0, dev), to_dev(dB0, dev)
+    capi.linear_wgrad(dYd, Xd, dW, dB, batch, IN, OUT)
+    rW, rB = orc.linearParamGrad(dY, X, dW0, dB0, threads=16)
+    assert_close(to_np(dW), rW, batch, "linearParamGrad dW 4096x4096x256")
+    assert_close(to_np(dB), rB, batch, "linearParamGrad dB")
+    run_nn(dev, 32768, 64, 576, 1, seed=9)
