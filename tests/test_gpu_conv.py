@@ -107,6 +107,19 @@ def test_conv_densenet_layers(dev, IC, H):
     run_layer(dev, 8, 48, H, H, 12, 3, 3, 1, 1, 1, 1, bias=True, seed=6)
 
 
+@pytest.mark.parametrize("IC,H,OC,s", RESNET)
+def test_conv_resnet56_layers_full_batch(dev, IC, H, OC, s):
+    """benchmark configuration 2 at its own batch (128): forward and both gradients against the oracle, workspace from the caller."""
+    run_layer(dev, 128, IC, H, H, OC, 3, 3, s, s, 1, 1, seed=14, ws=True)
+
+
+@pytest.mark.parametrize("IC,H", [(24, 32), (168, 32), (108, 16), (228, 16), (150, 8), (342, 8)])
+def test_conv_densenet_layers_full_batch(dev, IC, H):
+    """benchmark configuration 4 at its own batch (64): first and last bottleneck of each stage, then the 3x3 48 -> 12 layer."""
+    run_layer(dev, 64, IC, H, H, 48, 1, 1, 1, 1, 0, 0, seed=15)
+    run_layer(dev, 64, 48, H, H, 12, 3, 3, 1, 1, 1, 1, seed=16)
+
+
 def test_conv_vgg_stem_and_wide(dev):
     run_layer(dev, 4, 3, 32, 32, 64, 3, 3, 1, 1, 1, 1, bias=True, seed=7)
     run_layer(dev, 2, 256, 4, 4, 512, 3, 3, 1, 1, 1, 1, bias=True, seed=8)
