@@ -220,6 +220,15 @@ __device__ __forceinline__ void conv3x3_body(const DirectArgs &a, const u32 bid,
     const int xbase = kq * XP + Cfg::pix_off(q0) + 3;
     const int wbase = (wo * OBW * 16 + li) * WSTR + kq;
 
+    // The bias values of this lane's output channels, requested before the main loop: a load in the epilogue would wait,
+    // through the in-order memory counter, for every store issued before it.
+    float bias_v[OBW];
+#pragma unroll
+    for (int o = 0; o < OBW; ++o) {
+        const u32 oc = oc0 + (wo * OBW + o) * 16 + li;
+        bias_v[o] = (a.bias && oc < a.C_OUT) ? a.bias[oc] : 0.f;
+    }
+
     v4f acc[NPH][PBW][OBW];
 #pragma unroll
     for (int ph = 0; ph < NPH; ++ph)
@@ -268,7 +277,7 @@ __device__ __forceinline__ void conv3x3_body(const DirectArgs &a, const u32 bid,
         for (int o = 0; o < OBW; ++o) {
             const u32 oc = oc0 + (wo * OBW + o) * 16 + li;
             if (oc >= a.C_OUT) continue;
-            const float b = a.bias ? a.bias[oc] : 0.f;
+            const float b = bias_v[o];
 #pragma unroll
             for (int p = 0; p < PBW; ++p) {
                 if (p < p_lo || p >= p_lo + p_cnt) continue;
