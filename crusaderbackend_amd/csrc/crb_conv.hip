@@ -126,7 +126,9 @@ static int try_direct(const float *Wt, const float *X, float *Y, const float *bi
             CRB_TRY(16, 8, 8, 16, 2, 1, DG, 2, 2, 1)
             CRB_TRY(16, 4, 8, 16, 1, 1, DG, 2, 2, 1)
         } else if (gW == 8) {
-            if (C_OUT > 128 && C_IN > 8) { CRB_TRY(8, 8, 16, 64, 1, 4, DG, 2, 2, 1) }
+            // 64 output channels with chunks of 8: chunks of 16 would need more LDS than lets two workgroups share a CU, and a
+            // SIMD with a single wave issues its MFMAs a third slower
+            if (C_OUT > 128 && C_IN > 8) { CRB_TRY(8, 8, 8, 64, 1, 4, DG, 2, 2, 1) }
             if (C_OUT > 64 && C_IN > 8) { CRB_TRY(8, 8, 16, 32, 1, 2, DG, 2, 2, 1) }
             if (C_IN > 8) { CRB_TRY(8, 8, 16, 16, 1, 1, DG, 2, 2, 1) }
             CRB_TRY(8, 8, 8, 16, 1, 1, DG, 2, 2, 1)
