@@ -266,12 +266,12 @@ int crb_momentum_apply_multi(const crb_momentum_item *items_on_device, uint32_t 
 
 /* Batch normalisation with per-feature statistics: X is N x F, F = c*h*w, and each of the F positions is normalised
  * over the N samples (biased variance, eps 1e-8); beta, gamma, mean, var hold F floats.
- * Replaces seblas::batchNorm (seblas/operations/cuBatchNorm.cu:158-173; kernel :13-60): Y = xHat*gamma + beta, and
+ * Replaces seblas::batchNorm (seblas/operations/cuBatchNorm.cu:150-164; kernel :13-61): Y = xHat*gamma + beta, and
  * mean, var, xHat are stored. The reference's N <= 96 limit (:9,164) does not apply. */
 int crb_batchnorm_fwd(const float *X, const float *beta, const float *gamma, float *mean, float *var, float *Y, float *xHat,
                       uint32_t N, uint32_t F, void *stream);
 
-/* Replaces seblas::batchNormGrad (cuBatchNorm.cu:176-188; kernel :62-125): dX from dY, gamma and X (statistics are
+/* Replaces seblas::batchNormGrad (cuBatchNorm.cu:167-178; kernel :63-125): dX from dY, gamma and X (statistics are
  * recomputed from X, as in the reference). When dGamma / dBeta are given (both or neither) the parameter gradients are
  * written too — they are by-products of the same sums (dBeta = sum dY, dGamma = sum dY*xHat) — which saves the separate
  * crb_batchnorm_param_grads pass. */
@@ -293,7 +293,7 @@ int crb_batchnorm_relu_fwd(const float *X, const float *beta, const float *gamma
 int crb_batchnorm_relu_bwd(const float *dY, const float *dY2_or_null, const float *reluOut, const float *gamma, const float *X, float *dX,
                            float *dGamma_or_null, float *dBeta_or_null, float *dYmasked_or_null, uint32_t N, uint32_t F, void *stream);
 
-/* Replaces seblas::batchNormParamGrads (cuBatchNorm.cu:190-202; kernel :127-148): dBeta = sum_n dY, dGamma = sum_n dY*xHat.
+/* Replaces seblas::batchNormParamGrads (cuBatchNorm.cu:180-191; kernel :127-147): dBeta = sum_n dY, dGamma = sum_n dY*xHat.
  * Both are overwritten, not accumulated. */
 int crb_batchnorm_param_grads(const float *dY, const float *xHat, float *dGamma, float *dBeta, uint32_t N, uint32_t F,
                               void *stream);

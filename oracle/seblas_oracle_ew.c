@@ -158,12 +158,12 @@ void oracle_momentumApply(float *X, float *G, float *M, u32 n, float lr, float b
 
 /* ---- batch normalisation over the batch dimension, per feature -----------------------------------------------------
  * A "feature" is one (c, h, w) position: X is viewed as N x F with F = C*H*W, and every column is normalised with its
- * own statistics over the N samples (seblas/operations/cuBatchNorm.cu:13-60: one thread per feature index, loop over
+ * own statistics over the N samples (seblas/operations/cuBatchNorm.cu:13-61: one thread per feature index, loop over
  * depth = sample). beta, gamma, mean, var hold F values. Pinned in tests/test_oracle_elementwise.py by torch-CPU
  * batch_norm (training mode, eps 1e-8) on the N x F view in float64, its autograd for all three gradients, the
  * zero-mean / unit-variance property of xHat, and finite differences. */
 
-/* batchNorm (cuBatchNorm.cu:13-60, host :158-173): mean = sum/N, var = sum (x-mean)^2 / N (biased),
+/* batchNorm (cuBatchNorm.cu:13-61, host :150-164): mean = sum/N, var = sum (x-mean)^2 / N (biased),
  * xHat = (x - mean) / sqrt(var + 1e-8), Y = xHat*gamma + beta; mean, var and xHat are stored. The reference asserts
  * N <= 96 (its shared-memory staging, :9,164); that limit does not exist here. */
 void oracle_batchNorm(const float *X, const float *beta, const float *gamma, float *mean, float *var, float *Y,
@@ -188,7 +188,7 @@ void oracle_batchNorm(const float *X, const float *beta, const float *gamma, flo
     }
 }
 
-/* batchNormGrad (cuBatchNorm.cu:62-125, host :176-188): statistics are recomputed from X, then with dxHat = dY*gamma
+/* batchNormGrad (cuBatchNorm.cu:63-125, host :167-178): statistics are recomputed from X, then with dxHat = dY*gamma
  *   dVar  = sum dxHat*(x-mean) * -0.5*(var+1e-8)^(-3/2)
  *   dMean = sum dxHat * -1/sqrt(var+1e-8)  +  dVar * sum(-2(x-mean)) / N
  *   dX    = dxHat/sqrt(var+1e-8) + dVar*2(x-mean)/N + dMean/N. */
@@ -221,9 +221,9 @@ void oracle_batchNormGrad(const float *dY, const float *gamma, const float *X, f
     }
 }
 
-/* batchNormParamGrads (cuBatchNorm.cu:127-148, host :190-202): dBeta = sum dY, dGamma = sum dY*xHat; both OVERWRITE.
+/* batchNormParamGrads (cuBatchNorm.cu:127-147, host :180-191): dBeta = sum dY, dGamma = sum dY*xHat; both OVERWRITE.
  * (The BatchNorm operand of the reference passes the two output tensors in swapped order,
- * seann/operands/seblas/BatchNorm.cu:24 against cuBatchNorm.cu:190, so its beta receives dGamma and its gamma dBeta;
+ * seann/operands/seblas/BatchNorm.cu:24 against cuBatchNorm.cu:180, so its beta receives dGamma and its gamma dBeta;
  * that slip is not reproduced: here dGamma is the gradient of gamma.) */
 void oracle_batchNormParamGrads(const float *dY, const float *xHat, float *dGamma, float *dBeta, u32 N, u32 F) {
     for (u32 f = 0; f < F; ++f) {
