@@ -16,7 +16,8 @@ import pytest
 from oracle import crseq_oracle as crseq
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-BIN = os.path.join(ROOT, "tests", "cpp", "bin", "test_seblas_host")
+# CRB_HOST_TEST_BIN: another build of the same program (e.g. one with host sanitizers)
+BIN = os.environ.get("CRB_HOST_TEST_BIN") or os.path.join(ROOT, "tests", "cpp", "bin", "test_seblas_host")
 HOST_LIB = os.path.join(ROOT, "crusaderbackend_amd", "lib", "libseblas_host.so")
 
 

@@ -5,7 +5,8 @@ import subprocess
 import pytest
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-BIN = os.path.join(ROOT, "tests", "cpp", "bin", "test_seblas_host")
+# CRB_HOST_TEST_BIN: another build of the same program (e.g. one with host sanitizers)
+BIN = os.environ.get("CRB_HOST_TEST_BIN") or os.path.join(ROOT, "tests", "cpp", "bin", "test_seblas_host")
 
 
 def _run(mode):

@@ -10,7 +10,8 @@ import pytest
 from oracle import seio_oracle as sio
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-BIN = os.path.join(ROOT, "tests", "cpp", "bin", "test_seblas_host")
+# CRB_HOST_TEST_BIN: another build of the same program (e.g. one with host sanitizers)
+BIN = os.environ.get("CRB_HOST_TEST_BIN") or os.path.join(ROOT, "tests", "cpp", "bin", "test_seblas_host")
 
 
 @pytest.mark.gpu
