@@ -112,6 +112,7 @@ struct DirectArgs {
     u32 tiles_per_img, oc_tiles, tiles_total;  // tiles_total = N * tiles_per_img (stacked 4x4 images: ceil(N / IMGS))
     u32 n_images;
     u32 relu;
+    u32 xcd_shift;      // log2 of the run of consecutive tiles that shares an XCD (0: tiles are dealt to XCDs one by one)
 };
 
 // The work of workgroup `bid` of the grid launch_direct sizes; `smem` = Cfg::SMEM_FLOATS floats of LDS, 16-byte aligned.
@@ -129,7 +130,9 @@ __device__ __forceinline__ void conv3x3_body(const DirectArgs &a, const u32 bid,
     // input rows get ids 8 apart: they land on the same XCD, back to back, and share those rows through its L2.
     const u32 xcd = bid % kXcds, slot = bid / kXcds;
     const u32 oct = slot % a.oc_tiles;
-    const u32 rest = (slot / a.oc_tiles) * kXcds + xcd;
+    // runs of 2^xcd_shift consecutive tiles stay on one XCD (the XCD that a companion kernel body reads the same rows on)
+    const u32 sp = slot / a.oc_tiles;
+    const u32 rest = ((((sp >> a.xcd_shift) * kXcds) + xcd) << a.xcd_shift) + (sp & ((1u << a.xcd_shift) - 1u));
     if (rest >= a.tiles_total) return;
     const u32 tile = Cfg::MI ? 0 : rest % a.tiles_per_img;
     const u32 n = Cfg::MI ? rest * Cfg::IMGS : rest / a.tiles_per_img;  // (first) image of this tile
@@ -368,6 +371,7 @@ inline uint64_t direct_args(DirectArgs &a, const float *Wt, const float *X, floa
     a.tiles_total = Cfg::MI ? ceil_div(N, u32(Cfg::IMGS)) : N * a.tiles_per_img;
     a.n_images = N;
     a.relu = relu;
+    a.xcd_shift = 0;
     return uint64_t(ceil_div(a.tiles_total, kXcds)) * kXcds * a.oc_tiles;  // padded to whole XCD rounds
 }
 

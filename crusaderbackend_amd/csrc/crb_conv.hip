@@ -288,8 +288,20 @@ static bool bwd_pair(const crb_conv_geom *g, bool run, const float *Wt, const fl
     if (!run) return true;
     DirectArgs d;
     WgradArgs w;
-    const uint64_t dwgs = direct_args<DCfg>(d, Wt, dY, dX, nullptr, g->N, g->OC, g->IC, g->OH, g->OH, 0);
+    uint64_t dwgs = direct_args<DCfg>(d, Wt, dY, dX, nullptr, g->N, g->OC, g->IC, g->OH, g->OH, 0);
     const uint64_t wwgs = wgrad_direct_args<WCfg>(w, dY, X, dW, ws, plan, g->IC, g->OC, g->OH);
+    // Both bodies read dY. A weight-gradient slice z runs on XCD z % 8 and covers tiles_per_z consecutive tiles; the data
+    // gradient's tiles over the same rows are dealt to that XCD too, so that its L2 serves the second reader.
+    if (!DCfg::MI && plan.splits >= kXcds) {
+        const u32 run = plan.tiles_per_z * u32(WCfg::TR * WCfg::TI) / u32(DCfg::ROWS);  // data-gradient tiles per slice
+        if (run >= 2 && (run & (run - 1)) == 0 && u32(WCfg::TR * WCfg::TI) % u32(DCfg::ROWS) == 0) {
+            u32 sh = 0;
+            while ((1u << sh) < run) ++sh;
+            d.xcd_shift = sh;
+            const u32 round = kXcds << sh;
+            dwgs = uint64_t(ceil_div(d.tiles_total, round)) * round * d.oc_tiles;
+        }
+    }
     if (dwgs + wwgs > 0x7fffffffull) {
         status = fail(CRB_EINVAL_SHAPE, "crb_conv_bwd: launch grid too large");
         return true;
