@@ -123,11 +123,11 @@ MEASURED_HBM_BYTES = {
     "T1_16-32s2.fwd": 13.12e6, "T1_16-32s2.dgrad": 13.35e6, "T1_16-32s2.wgrad": 17.57e6,
     "T2_32-64s2.fwd": 6.99e6, "T2_32-64s2.dgrad": 6.96e6, "T2_32-64s2.wgrad": 11.33e6,
     # both gradients in one call: conv_bwd_kernel + the reduce kernel
-    "L1_16-16@32.bwd": 39.78e6, "L2_32-32@16.bwd": 24.36e6, "L3_64-64@8.bwd": 14.60e6,
-    "T1_16-32s2.bwd": 30.30e6, "T2_32-64s2.bwd": 18.0e6,
+    "L1_16-16@32.bwd": 33.57e6, "L2_32-32@16.bwd": 17.97e6, "L3_64-64@8.bwd": 12.76e6,
+    "T1_16-32s2.bwd": 26.16e6, "T2_32-64s2.bwd": 16.17e6,
     # conv_bwd_kernel alone (slices left for the end-of-step summation)
-    "L1_16-16@32.bwd_sliced": 37.34e6, "L2_32-32@16.bwd_sliced": 21.92e6, "L3_64-64@8.bwd_sliced": 11.93e6,
-    "T1_16-32s2.bwd_sliced": 27.86e6, "T2_32-64s2.bwd_sliced": 15.5e6,
+    "L1_16-16@32.bwd_sliced": 31.13e6, "L2_32-32@16.bwd_sliced": 15.53e6, "L3_64-64@8.bwd_sliced": 10.09e6,
+    "T1_16-32s2.bwd_sliced": 23.72e6, "T2_32-64s2.bwd_sliced": 13.67e6,
 }
 
 
