@@ -115,6 +115,8 @@ static int try_direct(const float *Wt, const float *X, float *Y, const float *bi
     if constexpr (S == 1) {
         if (gW == 32) {
             if (C_IN <= 16 && C_IN > 8 && C_OUT <= 16) { CRB_TRY(32, 8, 16, 16, 4, 1, DG, 2, 1, 1, 3, 4) }  // one LDS-resident chunk
+            // too few 8-row tiles for two workgroups per CU: 4-row tiles
+            if (C_OUT <= 16 && C_IN > 16 && N * (gH / 8) < 512) { CRB_TRY(32, 4, 16, 16, 2, 1, DG, 2, 2, 1) }
             if (C_OUT > 32) { CRB_TRY(32, 8, 8, 64, 4, 4, DG, 2, 2, 1) }
             if (C_OUT > 16) { CRB_TRY(32, 8, 8, 32, 4, 2, DG, 2, 2, 1) }
             CRB_TRY(32, 8, 8, 16, 4, 1, DG, 2, 2, 1)
