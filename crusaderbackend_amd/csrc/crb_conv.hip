@@ -117,6 +117,9 @@ static int try_direct(const float *Wt, const float *X, float *Y, const float *bi
             if (C_IN <= 16 && C_IN > 8 && C_OUT <= 16) { CRB_TRY(32, 8, 16, 16, 4, 1, DG, 2, 1, 1, 3, 4) }  // one LDS-resident chunk
             // too few 8-row tiles for two workgroups per CU: 4-row tiles
             if (C_OUT <= 16 && C_IN > 16 && N * (gH / 8) < 512) { CRB_TRY(32, 4, 16, 16, 2, 1, DG, 2, 2, 1) }
+            // 33..48 output channels: a 48-wide tile instead of a quarter-empty 64-wide one
+            if (C_OUT > 32 && C_OUT <= 48 && N * (gH / 8) < 512) { CRB_TRY(32, 4, 8, 48, 2, 3, DG, 2, 2, 1) }
+            if (C_OUT > 32 && C_OUT <= 48) { CRB_TRY(32, 8, 8, 48, 4, 3, DG, 2, 2, 1) }
             if (C_OUT > 32) { CRB_TRY(32, 8, 8, 64, 4, 4, DG, 2, 2, 1) }
             if (C_OUT > 16) { CRB_TRY(32, 8, 8, 32, 4, 2, DG, 2, 2, 1) }
             CRB_TRY(32, 8, 8, 16, 4, 1, DG, 2, 2, 1)

@@ -250,6 +250,8 @@ DIRECT = [
     # channel counts that divide neither the channel chunk nor the channel tile (zero-filled tails)
     (2, 3, 32, 32, 16), (2, 48, 32, 32, 12), (2, 5, 16, 16, 7), (4, 13, 8, 8, 19), (2, 3, 32, 32, 64), (2, 17, 16, 16, 33),
     (4, 1, 8, 8, 1), (2, 9, 32, 32, 70),
+    # 33..48 output channels at width 32: 48-wide tiles, 8 rows with enough tiles for the chip, else 4 rows
+    (128, 8, 32, 32, 40), (6, 20, 32, 32, 48),
     # 4x4 images (four stacked per tile; batch sizes that leave a partial stack)
     (8, 64, 4, 4, 64), (5, 20, 4, 4, 70), (3, 7, 4, 4, 5), (6, 40, 4, 4, 33), (1, 16, 4, 4, 16), (13, 96, 4, 4, 128),
     (16, 48, 4, 4, 40), (24, 17, 4, 4, 16), (12, 16, 4, 4, 20), (128, 256, 4, 4, 80),
