@@ -302,6 +302,9 @@ inline WgradDirectPlan wgrad_direct_plan(u32 N, u32 IC, u32 OC, u32 H, u32 targe
     WgradDirectPlan p;
     p.pairs = ceil_div(OC, 16u) * ceil_div(IC, 16u);
     p.tiles = (N / Cfg::TI) * (H / Cfg::TR);
+    // Wide layers (16 or more channel-block pairs) with at least four tiles per slice left: twice the workgroups, so that
+    // every SIMD holds two waves (a lone wave issues its MFMAs a third slower and has nobody to hide its loads behind).
+    if (p.pairs >= 16 && uint64_t(p.tiles) * p.pairs >= uint64_t(8) * target_wgs) target_wgs *= 2;
     u32 splits = p.pairs >= target_wgs ? 1 : target_wgs / p.pairs;
     if (splits > p.tiles) splits = p.tiles;
     p.tiles_per_z = ceil_div(p.tiles, splits);

@@ -231,7 +231,7 @@ static bool tiny2x2_shape(const crb_conv_geom *g) {
 
 // ---- direct 3x3 / pad 1 weight gradient (stride 1 and 2) ---------------------------------------------------------
 // One entry per configuration <W, TR, TI, OCC>; `run` = false only computes the plan (workspace size).
-constexpr u32 kWgradTargetWgs = 256;  // one workgroup per CU: pairs x splits
+constexpr u32 kWgradTargetWgs = 256;  // one workgroup per CU: pairs x splits (two per CU for wide layers, see wgrad_direct_plan)
 
 // dW == nullptr (with run): the slices are left in ws, unsummed.
 template <class Cfg>
