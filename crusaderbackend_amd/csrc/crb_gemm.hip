@@ -50,8 +50,11 @@ static int run_tiles(const AOp &a, const BOp &b, const RowMajorEpi &e, u32 M, u3
         if (tiles_l >= 800 && K <= 256) return run_cfg<CfgSmallAhead>(a, b, e, M, N, K, zdim, s, what);
         if (tiles_l >= 800) return run_cfg<CfgLarge>(a, b, e, M, N, K, zdim, s, what);
         if (tiles_s >= 512) return run_cfg<CfgSmallAhead>(a, b, e, M, N, K, zdim, s, what);
-        // at most one small tile per CU and a long contraction: longer slabs, so that a slab's loads have a whole slab of
-        // MFMAs (2048 clocks) to arrive in
+        // at most one small tile per CU: a contraction long enough is cut in two, so that two workgroups per CU hide each
+        // other's loads (measured: pays from K = 1280, from 1024 when the tiles do not cover the CUs evenly) ...
+        if (tiles_s >= 160 && K < 2048 && (K >= 1280 || (K >= 1024 && tiles_s > 256)) && zdim == 1 && e.ld == N)
+            return run_cfg<CfgSmallAhead>(a, b, e, M, N, K, zdim, s, what, 2);
+        // ... a shorter one gets longer slabs, so that a slab's loads have a whole slab of MFMAs (2048 clocks) to arrive in
         if (tiles_s >= 160 && K >= 512 && K < 2048) return run_cfg<CfgSmallDeep>(a, b, e, M, N, K, zdim, s, what);
         if (tiles_s >= 160 && K < 2048) return run_cfg<CfgSmallAhead>(a, b, e, M, N, K, zdim, s, what);
         // one small tile per CU at most but a long contraction: two K slices per tile put two workgroups on every CU
