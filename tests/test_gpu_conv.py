@@ -422,3 +422,37 @@ def test_conv_bwd_sliced_many_items_and_errors(dev):
     bad = (capi.SliceSumItem * 1)(capi.SliceSumItem(p, None, 16, 2))
     assert lib.crb_sum_slices_multi(ctypes.cast(bad, ctypes.c_void_p), 1, None) == capi.CRB_ENULL
     assert lib.crb_sum_slices_multi(None, 0, None) == 0
+
+
+@pytest.mark.parametrize("shape", [(4, 16, 32, 32, 16, 3, 3, 1, 1, 1, 1), (4, 32, 16, 16, 64, 3, 3, 2, 2, 1, 1),
+                                   (4, 24, 16, 16, 48, 1, 1, 1, 1, 0, 0), (3, 8, 2, 2, 8, 3, 3, 1, 1, 1, 1),
+                                   (2, 5, 9, 7, 6, 3, 2, 2, 1, 1, 0)])
+def test_conv_operands_aligned_to_4_bytes_only(dev, shape):
+    """Every operand one float past a 16-byte boundary: the 16-byte-load kernels must not be chosen (or must cope), results as usual."""
+    import torch
+    capi, orc = _capi(), _oracle()
+    N, IC, IH, IW, OC, FH, FW, sH, sW, pH, pW = shape
+    g = capi.ConvGeom.make(*shape)
+
+    def shifted(a):  # device copy whose first element sits 4 bytes past an allocation (allocations are 256-byte aligned)
+        buf = torch.empty(a.size + 1, dtype=torch.float32, device=dev)
+        v = buf[1:].view(*a.shape)
+        v.copy_(to_dev(a, dev))
+        assert v.data_ptr() % 16 == 4
+        return v
+
+    X, W, dY = normal(1, N, IC, IH, IW), he_normal(2, OC, IC, FH, FW), normal(3, N, OC, g.OH, g.OW)
+    b, dW0 = normal(4, OC), normal(5, OC, IC, FH, FW)
+    Xd, Wd, dYd, bd = shifted(X), shifted(W), shifted(dY), shifted(b)
+    Y = shifted(np.full((N, OC, g.OH, g.OW), np.nan, np.float32))
+    capi.conv_fwd(Wd, Xd, Y, bd, g)
+    assert_close(to_np(Y), orc.conv(W, X, b, sH, sW, pH, pW, threads=8), IC * FH * FW, "fwd, 4-byte aligned")
+    dX = shifted(np.full((N, IC, IH, IW), np.nan, np.float32))
+    capi.conv_dgrad(Wd, dYd, dX, g)
+    assert_close(to_np(dX), orc.convDerive(W, dY, (IH, IW), sH, sW, pH, pW, threads=8), OC * FH * FW, "dgrad, 4-byte aligned")
+    dW = shifted(dW0)
+    capi.conv_wgrad(dYd, Xd, dW, g)
+    assert_close(to_np(dW), orc.convError(dY, X, dW0, sH, sW, pH, pW, threads=8), N * g.OH * g.OW, "wgrad, 4-byte aligned")
+    dX2, dW2 = shifted(np.full((N, IC, IH, IW), np.nan, np.float32)), shifted(dW0)
+    capi.conv_bwd(Wd, dYd, Xd, dX2, dW2, g)
+    assert np.array_equal(to_np(dX2), to_np(dX)) and np.array_equal(to_np(dW2), to_np(dW))

@@ -265,3 +265,34 @@ def test_dense_sweep_configuration_full_size(dev):
     assert_close(to_np(dW), rW, batch, "linearParamGrad dW 4096x4096x256")
     assert_close(to_np(dB), rB, batch, "linearParamGrad dB")
     run_nn(dev, 32768, 64, 576, 1, seed=9)
+
+
+@pytest.mark.parametrize("M,N,K", [(128, 128, 64), (260, 132, 516), (64, 1024, 2048)])
+def test_gemm_operands_aligned_to_4_bytes_only(dev, M, N, K):
+    """Every operand one float past a 16-byte boundary, sizes that would otherwise take the 16-byte-load paths."""
+    import torch
+    capi, orc = _capi(), _oracle()
+
+    def shifted(a):
+        buf = torch.empty(a.size + 1, dtype=torch.float32, device=dev)
+        v = buf[1:].view(*a.shape)
+        v.copy_(to_dev(a, dev))
+        assert v.data_ptr() % 16 == 4
+        return v
+
+    A, B, Bt, At = uniform(1, M, K), uniform(2, K, N), uniform(3, N, K), uniform(4, K, M)
+    C = shifted(np.full((M, N), np.nan, np.float32))
+    capi.sgemm_nn(shifted(A), shifted(B), C, M, N, K)
+    assert_close(to_np(C), orc.sgemm(A, B, threads=8), K, "nn, 4-byte aligned")
+    capi.sgemm_nt(shifted(A), shifted(Bt), C, M, N, K)
+    assert_close(to_np(C), orc.sgemmNT(A, Bt, threads=8), K, "nt, 4-byte aligned")
+    capi.sgemm_tn(shifted(At), shifted(B), C, M, N, K)
+    assert_close(to_np(C), orc.sgemmTN(At, B, threads=8), K, "tn, 4-byte aligned")
+    C0 = uniform(5, M, N)
+    Cacc = shifted(C0)
+    capi.sgemm_nta(shifted(A[None]), shifted(Bt[None]), Cacc, M, N, K, 1)
+    assert_close(to_np(Cacc), orc.sgemmNTA(A[None], Bt[None], C0, threads=8), K, "nta, 4-byte aligned")
+    bias = uniform(6, N)
+    Y = shifted(np.full((M, N), np.nan, np.float32))
+    capi.linear_fwd(shifted(A), shifted(Bt), shifted(bias), Y, M, K, N)
+    assert_close(to_np(Y), orc.linear(A, Bt, bias, threads=8), K, "linear, 4-byte aligned")
