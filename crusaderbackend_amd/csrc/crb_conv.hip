@@ -523,6 +523,7 @@ int crb_conv_wgrad(const float *dY, const float *X, float *dW, const crb_conv_ge
                    size_t workspace_bytes, void *stream) {
     if (!dY || !X || !dW) return fail(CRB_ENULL, "crb_conv_wgrad: null operand");
     if (int st = check_geom("crb_conv_wgrad", g)) return st;
+    if (workspace && !aligned16(workspace)) return fail(CRB_EWORKSPACE, "crb_conv_wgrad: workspace is not 16-byte aligned");
     hipStream_t s = hipStream_t(stream);
     if (pointwise_shape(g)) return crb_sgemm_nta(dY, X, dW, g->OC, g->IC, g->IH * g->IW, g->N, stream);
     if (tiny2x2_shape(g) && aligned16(dY) && aligned16(X)) {
@@ -582,6 +583,7 @@ int crb_conv_bwd(const float *W, const float *dY, const float *X, float *dX, flo
                  size_t workspace_bytes, void *stream) {
     if (!W || !dY || !X || !dX || !dW) return fail(CRB_ENULL, "crb_conv_bwd: null operand");
     if (int st = check_geom("crb_conv_bwd", g)) return st;
+    if (workspace && !aligned16(workspace)) return fail(CRB_EWORKSPACE, "crb_conv_bwd: workspace is not 16-byte aligned");
     if (aligned16(dY) && aligned16(X) && aligned16(dX)) {
         WgradDirectPlan dp;
         int st = CRB_OK;

@@ -129,8 +129,8 @@ size_t crb_conv_wgrad_workspace_bytes(const crb_conv_geom *g);
  * dW[oc,ic,fh,fw] += sum_{n,oh,ow} dY[n,oc,oh,ow] * X[n,ic,oh*sH-pH+fh,ow*sW-pW+fw]. Accumulate.
  * The reduction over n*OH*OW is split across workgroups and combined in a fixed order (no atomics),
  * so results are bit-reproducible. `workspace` may be NULL: the library then uses its own lazily
- * grown arena (which may call hipMalloc on first use / growth); otherwise it must hold at least
- * crb_conv_wgrad_workspace_bytes(g) bytes. */
+ * grown arena (which may call hipMalloc on first use / growth); otherwise it must be 16-byte aligned
+ * and hold at least crb_conv_wgrad_workspace_bytes(g) bytes (CRB_EWORKSPACE if not). */
 int crb_conv_wgrad(const float *dY, const float *X, float *dW, const crb_conv_geom *g, void *workspace,
                    size_t workspace_bytes, void *stream);
 

@@ -354,6 +354,9 @@ def test_conv_bwd_errors(dev):
     p = t.data_ptr()
     assert lib.crb_conv_bwd(p, p, p, p, p, ctypes.byref(g), p, 16, None) == capi.CRB_EWORKSPACE
     assert lib.crb_conv_bwd(p, p, p, None, p, ctypes.byref(g), None, 0, None) == capi.CRB_ENULL
+    assert lib.crb_conv_bwd(p, p, p, p, p, ctypes.byref(g), p + 4, 1 << 17, None) == capi.CRB_EWORKSPACE  # 4-byte aligned workspace
+    assert lib.crb_conv_wgrad(p, p, p, ctypes.byref(g), p + 4, 1 << 17, None) == capi.CRB_EWORKSPACE
+    assert b"16-byte aligned" in lib.crb_last_error_string()
     g = capi.ConvGeom.make(1, 2, 8, 8, 2, 3, 3, 1, 1, 1, 1, OH=7, OW=8)
     assert lib.crb_conv_bwd(p, p, p, p, p, ctypes.byref(g), None, 0, None) == capi.CRB_EINVAL_SHAPE
 
