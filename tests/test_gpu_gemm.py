@@ -296,3 +296,51 @@ def test_gemm_operands_aligned_to_4_bytes_only(dev, M, N, K):
     Y = shifted(np.full((M, N), np.nan, np.float32))
     capi.linear_fwd(shifted(A), shifted(Bt), shifted(bias), Y, M, K, N)
     assert_close(to_np(Y), orc.linear(A, Bt, bias, threads=8), K, "linear, 4-byte aligned")
+
+
+def test_two_host_threads_on_their_own_streams(dev):
+    """Two host threads issue split-K GEMMs and weight gradients at once, each on its own stream (ctypes releases the
+    interpreter lock during a call): every result equals the one the same call gives alone, and an error raised in one
+    thread leaves the other thread's error text alone."""
+    import threading
+    import torch
+    capi = _capi()
+    lib = capi.load()
+    M, N, K = 192, 256, 4096
+    g = capi.ConvGeom.make(16, 16, 32, 32, 16, 3, 3, 1, 1, 1, 1)
+    A, B = to_dev(uniform(80, M, K), dev), to_dev(uniform(81, K, N), dev)
+    dY, X = to_dev(uniform(82, 16, 16, 32, 32), dev), to_dev(uniform(83, 16, 16, 32, 32), dev)
+    C_alone, dW_alone = _empty(dev, M, N), torch.zeros(16, 16, 3, 3, device=dev)
+    capi.sgemm_nn(A, B, C_alone, M, N, K)
+    capi.conv_wgrad(dY, X, dW_alone, g)
+    torch.cuda.synchronize()
+    failures = []
+
+    def worker(tag):
+        try:
+            st = torch.cuda.Stream(device=dev)
+            outs = []
+            for rep in range(25):
+                C, dW = _empty(dev, M, N), torch.zeros(16, 16, 3, 3, device=dev)
+                with torch.cuda.stream(st):  # allocations above are on the default stream and complete; work goes to st
+                    capi.sgemm_nn(A, B, C, M, N, K, stream=st)
+                    capi.conv_wgrad(dY, X, dW, g, stream=st)
+                outs.append((C, dW))
+                if rep == 10:  # a failing call in this thread: its text must be this thread's
+                    assert lib.crb_sgemm_nn(None, B.data_ptr(), C.data_ptr(), M, N, K, 1, None) == capi.CRB_ENULL
+                    assert b"crb_sgemm_nn" in lib.crb_last_error_string()
+            st.synchronize()
+            for C, dW in outs:
+                if not (torch.equal(C, C_alone) and torch.equal(dW, dW_alone)):
+                    failures.append(tag)
+                    break
+        except Exception as e:  # surfaced in the main thread below
+            failures.append(f"{tag}: {e!r}")
+
+    threads = [threading.Thread(target=worker, args=(i,)) for i in range(2)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    torch.cuda.synchronize()
+    assert not failures, failures
