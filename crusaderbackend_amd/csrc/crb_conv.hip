@@ -2,6 +2,7 @@
 // standalone bias add, all as implicit GEMMs on the MFMA engine (no im2col buffer is materialised).
 #include "conv3x3_direct.h"
 #include "conv3x3_wgrad.h"
+#include "conv1x1_s2.h"
 #include "gemm_internal.h"
 #include "operands.h"
 
@@ -222,6 +223,12 @@ static bool pointwise_shape(const crb_conv_geom *g) {
 static bool direct_shape(const crb_conv_geom *g, u32 stride) {
     return g->FH == 3 && g->FW == 3 && g->sH == stride && g->sW == stride && g->pH == 1 && g->pW == 1 &&
            g->IH == stride * g->OH && g->IW == stride * g->OW;
+}
+
+// 1x1, stride 2, no padding, even input extents, at most 64 channels on either side (conv1x1_s2.h)
+static bool shortcut_shape(const crb_conv_geom *g) {
+    return g->FH == 1 && g->FW == 1 && g->sH == 2 && g->sW == 2 && g->pH == 0 && g->pW == 0 && g->IH == 2 * g->OH &&
+           g->IW == 2 * g->OW && g->IC % 4 == 0 && g->IC <= kScMaxC && g->OC <= kScMaxC;
 }
 
 // 3x3 / pad 1 / stride 1 on 2x2 images: dense products over (channel, pixel) pairs (gemm_internal.h)
@@ -490,6 +497,8 @@ int crb_conv_dgrad(const float *W, const float *dY, float *dX, const crb_conv_ge
                                                   hipStream_t(stream), "crb_conv_dgrad", done);
         if (done) return st;
     }
+    if (shortcut_shape(g) && aligned16(dX))
+        return launch_sc_dgrad(W, dY, dX, g->N, g->IC, g->OC, g->OH, g->OW, hipStream_t(stream), "crb_conv_dgrad");
     const u32 FHW = g->FH * g->FW;
     const u32 M = g->IC, N = g->N * g->IH * g->IW, K = g->OC * FHW;
     SepK a{W, g->IC, FHW, g->IC * FHW, 1, FastDiv(FHW)};
@@ -510,6 +519,7 @@ size_t crb_conv_wgrad_workspace_bytes(const crb_conv_geom *g) {
     if (check_geom("crb_conv_wgrad_workspace_bytes", g)) return 0;
     if (pointwise_shape(g)) return 0;  // accumulate-NT GEMM form; its split scratch comes from the library arena
     if (tiny2x2_shape(g)) return size_t(g->OC) * g->IC * 16 * sizeof(float);  // (oc, p) x (ic, p') product before the tap fold
+    if (shortcut_shape(g)) return sc_wgrad_plan(g->N, g->IC, g->OC, g->OH, g->OW).workspace_bytes;
     {
         WgradDirectPlan dp;
         int st = 0;
@@ -537,6 +547,18 @@ int crb_conv_wgrad(const float *dY, const float *X, float *dW, const crb_conv_ge
             if (!G) return fail(CRB_EHIP, "crb_conv_wgrad: cannot allocate %zu bytes of scratch", need);
         }
         return conv2x2_wgrad(dY, X, dW, G, g->N, g->IC, g->OC, s, "crb_conv_wgrad");
+    }
+    if (shortcut_shape(g)) {
+        const ScWgradPlan sp = sc_wgrad_plan(g->N, g->IC, g->OC, g->OH, g->OW);
+        float *part = static_cast<float *>(workspace);
+        if (part) {
+            if (workspace_bytes < sp.workspace_bytes)
+                return fail(CRB_EWORKSPACE, "crb_conv_wgrad: workspace %zu bytes < required %zu", workspace_bytes, sp.workspace_bytes);
+        } else {
+            part = static_cast<float *>(arena_get(sp.workspace_bytes, s));
+            if (!part) return fail(CRB_EHIP, "crb_conv_wgrad: cannot allocate %zu bytes of scratch", sp.workspace_bytes);
+        }
+        return launch_sc_wgrad(dY, X, dW, part, sp, g->N, g->IC, g->OC, g->OH, g->OW, s, "crb_conv_wgrad");
     }
     if (aligned16(dY) && aligned16(X)) {
         WgradDirectPlan dp;

@@ -459,3 +459,15 @@ def test_conv_operands_aligned_to_4_bytes_only(dev, shape):
     dX2, dW2 = shifted(np.full((N, IC, IH, IW), np.nan, np.float32)), shifted(dW0)
     capi.conv_bwd(Wd, dYd, Xd, dX2, dW2, g)
     assert np.array_equal(to_np(dX2), to_np(dX)) and np.array_equal(to_np(dW2), to_np(dW))
+
+
+SHORTCUTS = [(128, 16, 32, 32, 32), (128, 32, 16, 16, 64), (3, 4, 8, 8, 4), (2, 12, 6, 10, 7), (5, 64, 4, 4, 64), (2, 8, 16, 12, 40),
+             (4, 36, 8, 8, 9), (7, 40, 2, 2, 5), (1, 4, 2, 2, 1), (33, 16, 32, 32, 32),
+             (2, 8, 7, 9, 4), (2, 6, 8, 8, 4), (2, 68, 8, 8, 4)]  # the last three: odd image / channel counts outside the streaming kernels
+
+
+@pytest.mark.parametrize("N,IC,H,W,OC", SHORTCUTS)
+def test_conv1x1_stride2_shortcuts(dev, N, IC, H, W, OC):
+    """Projection shortcuts of residual networks (1x1, stride 2, no padding), with the caller's workspace and the library's."""
+    run_layer(dev, N, IC, H, W, OC, 1, 1, 2, 2, 0, 0, bias=False, seed=21)
+    run_layer(dev, N, IC, H, W, OC, 1, 1, 2, 2, 0, 0, bias=True, seed=22, ws=True)
