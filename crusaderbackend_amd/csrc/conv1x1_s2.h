@@ -144,11 +144,13 @@ inline int launch_sc_dgrad(const float *W, const float *dY, float *dX, u32 N, u3
 }
 
 // part: plan.workspace_bytes of scratch, 16-byte aligned; dW accumulated by the split reduction in fixed order
+// (dW == nullptr: the slices are left in part, unsummed)
 inline int launch_sc_wgrad(const float *dY, const float *X, float *dW, float *part, const ScWgradPlan &plan, u32 N, u32 IC, u32 OC,
                            u32 OH, u32 OW, hipStream_t s, const char *what) {
     hipLaunchKernelGGL(sc_wgrad_kernel, dim3(plan.splits), dim3(256), 0, s, dY, X, part, IC, OC, OH, OW, N * OH * OW, plan.tiles_per_z,
                        FastDiv(OW), FastDiv(OH * OW));
     if (int st = check_launch(what)) return st;
+    if (!dW) return CRB_OK;
     return launch_splitk_reduce(part, dW, OC * IC, plan.splits, ReduceEpi{nullptr, 1, 1, EPI_ACCUM}, s, what);
 }
 

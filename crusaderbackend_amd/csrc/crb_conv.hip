@@ -633,6 +633,10 @@ uint32_t crb_conv_bwd_slices(const crb_conv_geom *g) {
     WgradDirectPlan dp;
     int st = CRB_OK;
     if (pointwise_shape(g) || tiny2x2_shape(g)) return 0;
+    if (shortcut_shape(g)) {
+        const u32 n = sc_wgrad_plan(g->N, g->IC, g->OC, g->OH, g->OW).splits;
+        return n > 1 ? n : 0;
+    }
     if (!wgrad_direct(g, false, nullptr, nullptr, nullptr, nullptr, nullptr, dp, st)) return 0;
     return dp.splits > 1 ? dp.splits : 0;
 }
@@ -647,6 +651,13 @@ int crb_conv_bwd_sliced(const float *W, const float *dY, const float *X, float *
     int st = CRB_OK;
     float *ws = static_cast<float *>(workspace);
     hipStream_t s = hipStream_t(stream);
+    if (shortcut_shape(g)) {
+        const ScWgradPlan sp = sc_wgrad_plan(g->N, g->IC, g->OC, g->OH, g->OW);
+        if (workspace_bytes < sp.workspace_bytes)
+            return fail(CRB_EWORKSPACE, "crb_conv_bwd_sliced: workspace %zu bytes < required %zu", workspace_bytes, sp.workspace_bytes);
+        if (int sd = crb_conv_dgrad(W, dY, dX, g, stream)) return sd;
+        return launch_sc_wgrad(dY, X, nullptr, ws, sp, g->N, g->IC, g->OC, g->OH, g->OW, s, "crb_conv_bwd_sliced");
+    }
     if (bwd_fused(g, false, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, dp, st)) {
         if (workspace_bytes < dp.workspace_bytes)
             return fail(CRB_EWORKSPACE, "crb_conv_bwd_sliced: workspace %zu bytes < required %zu", workspace_bytes, dp.workspace_bytes);

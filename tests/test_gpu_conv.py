@@ -471,3 +471,28 @@ def test_conv1x1_stride2_shortcuts(dev, N, IC, H, W, OC):
     """Projection shortcuts of residual networks (1x1, stride 2, no padding), with the caller's workspace and the library's."""
     run_layer(dev, N, IC, H, W, OC, 1, 1, 2, 2, 0, 0, bias=False, seed=21)
     run_layer(dev, N, IC, H, W, OC, 1, 1, 2, 2, 0, 0, bias=True, seed=22, ws=True)
+
+
+def test_shortcut_weight_gradients_join_the_postponed_sum(dev):
+    """1x1 stride-2 shortcuts have a sliced form too: dX at once, dW after crb_sum_slices_multi, both as crb_conv_bwd gives them."""
+    import torch
+    capi = _capi()
+    layers, entries = [], []
+    for i, (N, IC, H, OC) in enumerate([(128, 16, 32, 32), (128, 32, 16, 64), (6, 12, 8, 20)]):
+        g = capi.ConvGeom.make(N, IC, H, H, OC, 1, 1, 2, 2, 0, 0)
+        n_slices = capi.conv_bwd_slices(g)
+        assert n_slices > 1
+        X, W = to_dev(normal(10 + i, N, IC, H, H), dev), to_dev(he_normal(30 + i, OC, IC, 1, 1), dev)
+        dY, dW0 = to_dev(normal(50 + i, N, OC, g.OH, g.OW), dev), normal(70 + i, OC, IC, 1, 1)
+        ws = torch.empty(capi.conv_wgrad_workspace_bytes(g) // 4, dtype=torch.float32, device=dev)
+        assert ws.numel() == n_slices * OC * IC
+        dX1, dW1 = _nan(dev, N, IC, H, H), to_dev(dW0, dev)
+        capi.conv_bwd(W, dY, X, dX1, dW1, g)
+        dX2, dW2 = _nan(dev, N, IC, H, H), to_dev(dW0, dev)
+        capi.conv_bwd_sliced(W, dY, X, dX2, g, ws)
+        layers.append((dX1, dW1, dX2, dW2))
+        entries.append((ws, dW2, n_slices))
+    capi.sum_slices_multi(capi.slice_sum_table(entries))
+    torch.cuda.synchronize()
+    for dX1, dW1, dX2, dW2 in layers:
+        assert np.array_equal(to_np(dX1), to_np(dX2)) and np.array_equal(to_np(dW1), to_np(dW2))
