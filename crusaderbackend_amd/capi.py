@@ -40,6 +40,11 @@ SIGNATURES = {
     "crb_abi_version": (ctypes.c_int, []),
     "crb_last_error_string": (ctypes.c_char_p, []),
     "crb_release_workspace": (None, []),
+    "crb_bind_workspace": (ctypes.c_int, [_ptr, ctypes.c_size_t, _ptr]),
+    "crb_gemm_workspace_bytes": (ctypes.c_size_t, [_u32, _u32, _u32, _u32]),
+    "crb_conv_fwd_workspace_bytes": (ctypes.c_size_t, [ctypes.POINTER(ConvGeom), ctypes.c_int]),
+    "crb_conv_dgrad_workspace_bytes": (ctypes.c_size_t, [ctypes.POINTER(ConvGeom), ctypes.c_int]),
+    "crb_conv_bias_grad_workspace_bytes": (ctypes.c_size_t, [_u32, _u32, _u32]),
     "crb_sgemm_nn": (ctypes.c_int, [_ptr, _ptr, _ptr, _u32, _u32, _u32, _u32, _ptr]),
     "crb_sgemm_tn": (ctypes.c_int, [_ptr, _ptr, _ptr, _u32, _u32, _u32, _u32, _ptr]),
     "crb_sgemm_nt": (ctypes.c_int, [_ptr, _ptr, _ptr, _u32, _u32, _u32, _ptr]),
@@ -168,6 +173,28 @@ def conv_wgrad_workspace_bytes(geom):
 def conv_wgrad(dY, X, dW, geom, workspace=None, stream=None):
     nbytes = 0 if workspace is None else workspace.numel() * workspace.element_size()
     check(load().crb_conv_wgrad(_p(dY), _p(X), _p(dW), ctypes.byref(geom), _p(workspace), nbytes, _stream(stream)))
+
+
+def bind_workspace(workspace, stream=None):
+    """Bind `workspace` (a torch tensor, or None to unbind) as the split scratch of calls on `stream`."""
+    nbytes = 0 if workspace is None else workspace.numel() * workspace.element_size()
+    check(load().crb_bind_workspace(_p(workspace), nbytes, _stream(stream)))
+
+
+def gemm_workspace_bytes(M, N, K, batch=1):
+    return load().crb_gemm_workspace_bytes(M, N, K, batch)
+
+
+def conv_fwd_workspace_bytes(geom, aligned16=True):
+    return load().crb_conv_fwd_workspace_bytes(ctypes.byref(geom), int(aligned16))
+
+
+def conv_dgrad_workspace_bytes(geom, aligned16=True):
+    return load().crb_conv_dgrad_workspace_bytes(ctypes.byref(geom), int(aligned16))
+
+
+def conv_bias_grad_workspace_bytes(N, C, HW):
+    return load().crb_conv_bias_grad_workspace_bytes(N, C, HW)
 
 
 def conv_bwd(W, dY, X, dX, dW, geom, workspace=None, stream=None):

@@ -16,10 +16,31 @@ int fail(int st, const char *fmt, ...);
 int check_hip(hipError_t e, const char *what);
 int check_launch(const char *what);
 
-// Lazily grown device scratch (split-K partial sums) of the current device and `stream`; the block stays valid for work
-// queued on that stream until a later arena_get on the same stream asks for more. Returns nullptr on allocation failure.
-void *arena_get(size_t bytes, hipStream_t stream);
+// Device scratch for partial sums (`bytes` > 0) of a call queued on `stream` of the current device: the calling thread's
+// open ScratchScope, else the workspace bound to the stream, else the library's lazily grown arena of that stream. A block
+// stays valid for work queued on that stream until crb_release_workspace. Returns CRB_OK and the block, or an error
+// (CRB_EWORKSPACE: the scope / bound workspace is too small, or growth was needed during a stream capture; CRB_EHIP:
+// allocation failed).
+int scratch_get(size_t bytes, hipStream_t stream, const char *what, void **out);
+template <class T>
+inline int scratch_get(size_t bytes, hipStream_t stream, const char *what, T **out) {
+    void *p = nullptr;
+    const int st = scratch_get(bytes, stream, what, &p);
+    *out = static_cast<T *>(p);
+    return st;
+}
+int scratch_bind(void *ptr, size_t bytes, hipStream_t stream);
 void arena_release();
+// While alive, every scratch_get of this thread is served from [ptr, ptr + bytes) or refused; nothing is allocated.
+struct ScratchScope {
+    ScratchScope(void *ptr, size_t bytes);
+    ~ScratchScope();
+    ScratchScope(const ScratchScope &) = delete;
+    ScratchScope &operator=(const ScratchScope &) = delete;
+  private:
+    void *prev_ptr;
+    size_t prev_bytes;
+};
 
 // Exact floor(n / d) for any n, d in [1, 2^32): round-up magic multiply (Granlund-Montgomery).
 // q = (t + ((n - t) >> s1)) >> s2 with t = mulhi(m, n).

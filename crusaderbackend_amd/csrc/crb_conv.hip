@@ -68,12 +68,19 @@ static int run_nchw(const AOp &a, const BOp &b, NchwEpi e, u32 M, u32 N, u32 K, 
     if (sp.splits == 1) return run_by_m(a, b, e, M, N, K, 1, 0, K, s, what);
     const u32 count = M * N;  // N = batch * H * W, so M*N is the whole NCHW tensor
     const size_t need = size_t(sp.splits) * count * sizeof(float);
-    float *ws = static_cast<float *>(arena_get(need, s));
-    if (!ws) return fail(CRB_EHIP, "%s: cannot allocate %zu bytes of split-K scratch", what, need);
+    float *ws = nullptr;
+    if (int st = scratch_get(need, s, what, &ws)) return st;
     NchwEpi pe = e;
     pe.T = ws, pe.row_bias = nullptr, pe.flags = 0u, pe.zstride = count;
     if (int st = run_by_m(a, b, pe, M, N, K, sp.splits, 1, sp.k_per_z, s, what)) return st;
     return launch_splitk_reduce(ws, e.T, count, sp.splits, ReduceEpi{e.row_bias, e.HW, e.C, e.flags}, s, what);
+}
+
+// Scratch bytes run_nchw asks for (0: the contraction is not cut).
+static size_t nchw_scratch_bytes(u32 M, u32 N, u32 K) {
+    const u32 bm = M <= 32 ? 32 : (M <= 64 ? 64 : 128);
+    const SplitPlan sp = plan_split(M, N, K, bm, 128, 16, 1);
+    return sp.splits > 1 ? size_t(sp.splits) * M * N * sizeof(float) : 0;
 }
 
 static u32 tile_m_for(u32 M) { return M <= 32 ? 32 : (M <= 64 ? 64 : 128); }
@@ -106,11 +113,12 @@ static WgradPlan wgrad_plan(const crb_conv_geom *g) {
 // (gH, gW) is the pixel grid: the output image, or dY for the stride-2 data gradient; in_H the rows of the staged tensor.
 template <bool DG, int S>
 static int try_direct(const float *Wt, const float *X, float *Y, const float *bias, u32 N, u32 C_IN, u32 C_OUT, u32 gH,
-                      u32 gW, u32 in_H, u32 relu, hipStream_t s, const char *what, bool &done) {
+                      u32 gW, u32 in_H, u32 relu, hipStream_t s, const char *what, bool &done, bool probe = false) {
     done = true;
+    // probe: only report (through `done`) whether a configuration takes the shape, launch nothing
 #define CRB_TRY(...)                                                                                          \
     if (direct_fits<DirectCfg<__VA_ARGS__>>(C_IN, gH, gW))                                                     \
-        return launch_direct<DirectCfg<__VA_ARGS__>>(Wt, X, Y, bias, N, C_IN, C_OUT, gH, in_H, relu, s, what);
+        return probe ? int(CRB_OK) : launch_direct<DirectCfg<__VA_ARGS__>>(Wt, X, Y, bias, N, C_IN, C_OUT, gH, in_H, relu, s, what);
     // output-channel tile: the smallest of 16 / 32 / 64 that covers C_OUT, 64 beyond; chunks of 16 input channels at
     // stride 1 when C_IN > 8, chunks of 8 otherwise (stride 2 stages wider / more rows per chunk)
     if constexpr (S == 1) {
@@ -172,7 +180,7 @@ static int try_direct(const float *Wt, const float *X, float *Y, const float *bi
 // yields enough workgroups for the chip; if none does, the batched GEMM forms run instead.
 template <bool DG>
 static int try_pointwise(const float *Wt, const float *X, float *Y, const float *bias, u32 N, u32 C_IN, u32 C_OUT, u32 gH, u32 gW,
-                         u32 relu, hipStream_t s, const char *what, bool &done) {
+                         u32 relu, hipStream_t s, const char *what, bool &done, bool probe = false) {
     done = true;
     if ((gW != 32 && gW != 16 && gW != 8) || gH % 8 != 0) {  // every configuration below tiles rows by 8 or 4
         done = false;
@@ -185,7 +193,7 @@ static int try_pointwise(const float *Wt, const float *X, float *Y, const float 
     };
 #define CRB_TRY(...)                                                                                          \
     if (direct_fits<DirectCfg<__VA_ARGS__>>(C_IN, gH, gW))                                                     \
-        return launch_direct<DirectCfg<__VA_ARGS__>>(Wt, X, Y, bias, N, C_IN, C_OUT, gH, gH, relu, s, what);
+        return probe ? int(CRB_OK) : launch_direct<DirectCfg<__VA_ARGS__>>(Wt, X, Y, bias, N, C_IN, C_OUT, gH, gH, relu, s, what);
     // long contractions with few workgroups: half-height tiles, so two workgroups share a CU and one multiplies while
     // the other waits for its next channel chunk
     const bool half = C_IN > 64 && tiles * ceil_div(C_OUT, 48u) < 512;
@@ -433,6 +441,21 @@ __global__ void __launch_bounds__(256) bias_grad_fold_kernel(const float *__rest
     if (threadIdx.x == 0) dB[c] += red[0];
 }
 
+// Row slicing of the bias gradient's first pass: rows are cut into slices until the grid covers the chip (at least 16
+// rows per slice).
+struct BiasGradPlan {
+    u32 col_wgs, slices, rows_per_slice;
+};
+static BiasGradPlan bias_grad_plan(u32 N, u32 cols, bool vec) {
+    BiasGradPlan p;
+    p.col_wgs = ceil_div(cols, vec ? 64u : 32u);
+    u32 slices = p.col_wgs >= 512 ? 1 : ceil_div(512u, p.col_wgs);
+    if (slices > ceil_div(N, 16u)) slices = ceil_div(N, 16u);
+    p.rows_per_slice = ceil_div(N, slices);
+    p.slices = ceil_div(N, p.rows_per_slice);
+    return p;
+}
+
 }  // namespace crb
 
 using namespace crb;
@@ -517,7 +540,8 @@ int crb_conv_dgrad(const float *W, const float *dY, float *dX, const crb_conv_ge
 
 size_t crb_conv_wgrad_workspace_bytes(const crb_conv_geom *g) {
     if (check_geom("crb_conv_wgrad_workspace_bytes", g)) return 0;
-    if (pointwise_shape(g)) return 0;  // accumulate-NT GEMM form; its split scratch comes from the library arena
+    if (pointwise_shape(g))  // accumulate-NT GEMM form over the batch-concatenated contraction
+        return uint64_t(g->IH) * g->IW * g->N > 0x7fffffffull ? 0 : gemm_scratch_bytes(g->OC, g->IC, g->IH * g->IW * g->N, 1);
     if (tiny2x2_shape(g)) return size_t(g->OC) * g->IC * 16 * sizeof(float);  // (oc, p) x (ic, p') product before the tap fold
     if (shortcut_shape(g)) return sc_wgrad_plan(g->N, g->IC, g->OC, g->OH, g->OW).workspace_bytes;
     {
@@ -535,16 +559,19 @@ int crb_conv_wgrad(const float *dY, const float *X, float *dW, const crb_conv_ge
     if (int st = check_geom("crb_conv_wgrad", g)) return st;
     if (workspace && !aligned16(workspace)) return fail(CRB_EWORKSPACE, "crb_conv_wgrad: workspace is not 16-byte aligned");
     hipStream_t s = hipStream_t(stream);
-    if (pointwise_shape(g)) return crb_sgemm_nta(dY, X, dW, g->OC, g->IC, g->IH * g->IW, g->N, stream);
+    if (pointwise_shape(g)) {
+        if (!workspace) return crb_sgemm_nta(dY, X, dW, g->OC, g->IC, g->IH * g->IW, g->N, stream);
+        ScratchScope scope(workspace, workspace_bytes);  // the GEMM's split scratch comes from the caller's block
+        return crb_sgemm_nta(dY, X, dW, g->OC, g->IC, g->IH * g->IW, g->N, stream);
+    }
     if (tiny2x2_shape(g) && aligned16(dY) && aligned16(X)) {
         const size_t need = size_t(g->OC) * g->IC * 16 * sizeof(float);
         float *G = static_cast<float *>(workspace);
         if (G) {
             if (workspace_bytes < need || !aligned16(G))
                 return fail(CRB_EWORKSPACE, "crb_conv_wgrad: workspace %zu bytes < required %zu (or not 16-byte aligned)", workspace_bytes, need);
-        } else {
-            G = static_cast<float *>(arena_get(need, s));
-            if (!G) return fail(CRB_EHIP, "crb_conv_wgrad: cannot allocate %zu bytes of scratch", need);
+        } else if (int st = scratch_get(need, s, "crb_conv_wgrad", &G)) {
+            return st;
         }
         return conv2x2_wgrad(dY, X, dW, G, g->N, g->IC, g->OC, s, "crb_conv_wgrad");
     }
@@ -554,9 +581,8 @@ int crb_conv_wgrad(const float *dY, const float *X, float *dW, const crb_conv_ge
         if (part) {
             if (workspace_bytes < sp.workspace_bytes)
                 return fail(CRB_EWORKSPACE, "crb_conv_wgrad: workspace %zu bytes < required %zu", workspace_bytes, sp.workspace_bytes);
-        } else {
-            part = static_cast<float *>(arena_get(sp.workspace_bytes, s));
-            if (!part) return fail(CRB_EHIP, "crb_conv_wgrad: cannot allocate %zu bytes of scratch", sp.workspace_bytes);
+        } else if (int st = scratch_get(sp.workspace_bytes, s, "crb_conv_wgrad", &part)) {
+            return st;
         }
         return launch_sc_wgrad(dY, X, dW, part, sp, g->N, g->IC, g->OC, g->OH, g->OW, s, "crb_conv_wgrad");
     }
@@ -570,9 +596,8 @@ int crb_conv_wgrad(const float *dY, const float *X, float *dW, const crb_conv_ge
                     if (workspace_bytes < dp.workspace_bytes)
                         return fail(CRB_EWORKSPACE, "crb_conv_wgrad: workspace %zu bytes < required %zu", workspace_bytes,
                                     dp.workspace_bytes);
-                } else {
-                    dws = static_cast<float *>(arena_get(dp.workspace_bytes, s));
-                    if (!dws) return fail(CRB_EHIP, "crb_conv_wgrad: cannot allocate %zu bytes of scratch", dp.workspace_bytes);
+                } else if (int sg = scratch_get(dp.workspace_bytes, s, "crb_conv_wgrad", &dws)) {
+                    return sg;
                 }
             }
             wgrad_direct(g, true, dY, X, dW, dws, s, dp, st);
@@ -592,13 +617,51 @@ int crb_conv_wgrad(const float *dY, const float *X, float *dW, const crb_conv_ge
     if (ws) {
         if (workspace_bytes < need)
             return fail(CRB_EWORKSPACE, "crb_conv_wgrad: workspace %zu bytes < required %zu", workspace_bytes, need);
-    } else {
-        ws = static_cast<float *>(arena_get(need, s));
-        if (!ws) return fail(CRB_EHIP, "crb_conv_wgrad: cannot allocate %zu bytes of scratch", need);
+    } else if (int st = scratch_get(need, s, "crb_conv_wgrad", &ws)) {
+        return st;
     }
     RowMajorEpi e{ws, nullptr, p.Ncols, p.M * p.Ncols, 0u};
     if (int st = run_by_m(a, b, e, p.M, p.Ncols, p.K, p.splits, 1, p.k_per_z, s, "crb_conv_wgrad")) return st;
     return launch_splitk_reduce(ws, dW, p.M * p.Ncols, p.splits, ReduceEpi{nullptr, 1, 1, EPI_ACCUM}, s, "crb_conv_wgrad(reduce)");
+}
+
+size_t crb_conv_fwd_workspace_bytes(const crb_conv_geom *g, int operands_aligned16) {
+    if (check_geom("crb_conv_fwd_workspace_bytes", g)) return 0;
+    bool done = false;
+    if (pointwise_shape(g) && operands_aligned16) {
+        try_pointwise<false>(nullptr, nullptr, nullptr, nullptr, g->N, g->IC, g->OC, g->OH, g->OW, 0, nullptr, "", done, true);
+        if (done) return 0;
+    }
+    if (pointwise_shape(g)) return gemm_scratch_bytes(g->OC, g->IH * g->IW, g->IC, g->N);
+    if (tiny2x2_shape(g) && operands_aligned16) return gemm_scratch_bytes(g->N, g->OC * 4, g->IC * 4, 1);
+    if (operands_aligned16 && (direct_shape(g, 1) || direct_shape(g, 2))) {
+        if (g->sH == 1)
+            try_direct<false, 1>(nullptr, nullptr, nullptr, nullptr, g->N, g->IC, g->OC, g->OH, g->OW, g->IH, 0, nullptr, "", done, true);
+        else
+            try_direct<false, 2>(nullptr, nullptr, nullptr, nullptr, g->N, g->IC, g->OC, g->OH, g->OW, g->IH, 0, nullptr, "", done, true);
+        if (done) return 0;
+    }
+    return nchw_scratch_bytes(g->OC, g->N * g->OH * g->OW, g->IC * g->FH * g->FW);
+}
+
+size_t crb_conv_dgrad_workspace_bytes(const crb_conv_geom *g, int operands_aligned16) {
+    if (check_geom("crb_conv_dgrad_workspace_bytes", g)) return 0;
+    bool done = false;
+    if (pointwise_shape(g) && operands_aligned16) {
+        try_pointwise<true>(nullptr, nullptr, nullptr, nullptr, g->N, g->OC, g->IC, g->OH, g->OW, 0, nullptr, "", done, true);
+        if (done) return 0;
+    }
+    if (pointwise_shape(g)) return gemm_scratch_bytes(g->IC, g->IH * g->IW, g->OC, g->N);
+    if (tiny2x2_shape(g) && operands_aligned16) return gemm_scratch_bytes(g->N, g->IC * 4, g->OC * 4, 1);
+    if (operands_aligned16 && (direct_shape(g, 1) || direct_shape(g, 2))) {
+        if (g->sH == 1)
+            try_direct<true, 1>(nullptr, nullptr, nullptr, nullptr, g->N, g->OC, g->IC, g->OH, g->OW, g->OH, 0, nullptr, "", done, true);
+        else
+            try_direct<true, 2>(nullptr, nullptr, nullptr, nullptr, g->N, g->OC, g->IC, g->OH, g->OW, g->OH, 0, nullptr, "", done, true);
+        if (done) return 0;
+    }
+    if (shortcut_shape(g) && operands_aligned16) return 0;
+    return nchw_scratch_bytes(g->IC, g->N * g->IH * g->IW, g->OC * g->FH * g->FW);
 }
 
 int crb_conv_bwd(const float *W, const float *dY, const float *X, float *dX, float *dW, const crb_conv_geom *g, void *workspace,
@@ -615,9 +678,8 @@ int crb_conv_bwd(const float *W, const float *dY, const float *X, float *dX, flo
                 if (dws) {
                     if (workspace_bytes < dp.workspace_bytes)
                         return fail(CRB_EWORKSPACE, "crb_conv_bwd: workspace %zu bytes < required %zu", workspace_bytes, dp.workspace_bytes);
-                } else {
-                    dws = static_cast<float *>(arena_get(dp.workspace_bytes, hipStream_t(stream)));
-                    if (!dws) return fail(CRB_EHIP, "crb_conv_bwd: cannot allocate %zu bytes of scratch", dp.workspace_bytes);
+                } else if (int sg = scratch_get(dp.workspace_bytes, hipStream_t(stream), "crb_conv_bwd", &dws)) {
+                    return sg;
                 }
             }
             bwd_fused(g, true, W, dY, X, dX, dW, dws, hipStream_t(stream), dp, st);
@@ -684,6 +746,13 @@ int crb_sum_slices_multi(const crb_slice_sum_item *items, uint32_t n_items, void
     return launch_slice_sum_multi(reinterpret_cast<const SliceSumItem *>(items), n_items, hipStream_t(stream), "crb_sum_slices_multi");
 }
 
+size_t crb_conv_bias_grad_workspace_bytes(uint32_t N, uint32_t C, uint32_t HW) {
+    if (!N || !C || !HW || uint64_t(N) * C * HW > 0x7fffffffull) return 0;
+    // the scalar form (operands not 16-byte friendly) has the narrower column blocks, hence the most slices
+    const BiasGradPlan v = bias_grad_plan(N, C * HW, true), sc = bias_grad_plan(N, C * HW, false);
+    return size_t(v.slices > sc.slices ? v.slices : sc.slices) * C * HW * sizeof(float);
+}
+
 int crb_conv_bias_grad(const float *dY, float *dB, uint32_t N, uint32_t C, uint32_t HW, void *stream) {
     if (!dY || !dB) return fail(CRB_ENULL, "crb_conv_bias_grad: null operand");
     if (!N || !C || !HW) return fail(CRB_EINVAL_SHAPE, "crb_conv_bias_grad: zero dimension");
@@ -692,15 +761,11 @@ int crb_conv_bias_grad(const float *dY, float *dB, uint32_t N, uint32_t C, uint3
     hipStream_t s = hipStream_t(stream);
     const u32 cols = C * HW;
     const bool vec = cols % 4 == 0 && aligned16(dY);
-    const u32 col_wgs = ceil_div(cols, vec ? 64u : 32u);
-    // rows are cut into slices until the grid covers the chip (at least 16 rows per slice)
-    u32 slices = col_wgs >= 512 ? 1 : ceil_div(512u, col_wgs);
-    if (slices > ceil_div(N, 16u)) slices = ceil_div(N, 16u);
-    const u32 rows_per_slice = ceil_div(N, slices);
-    slices = ceil_div(N, rows_per_slice);
+    const BiasGradPlan bp = bias_grad_plan(N, cols, vec);
+    const u32 col_wgs = bp.col_wgs, slices = bp.slices, rows_per_slice = bp.rows_per_slice;
     const size_t need = size_t(slices) * cols * sizeof(float);
-    float *part = static_cast<float *>(arena_get(need, s));
-    if (!part) return fail(CRB_EHIP, "crb_conv_bias_grad: cannot allocate %zu bytes of scratch", need);
+    float *part = nullptr;
+    if (int st = scratch_get(need, s, "crb_conv_bias_grad", &part)) return st;
     if (vec)
         hipLaunchKernelGGL(bias_grad_colsum_kernel<true>, dim3(col_wgs, slices), dim3(256), 0, s, dY, part, N, cols, rows_per_slice);
     else

@@ -13,22 +13,65 @@ typedef TileCfg<64, 64, 32, 2, 2, 2, 2> CfgSmallAhead;  // loads run two slabs a
 
 static inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
+// Tile choice by how many workgroups the grid gives a CU; when neither tile size fills the chip, K is split — with
+// large tiles only when each slice keeps a long contraction (the split costs a second pass over the result).
+// `dense` = the result rows are contiguous (ld == N), which the partial results of a split assume.
+enum GemmTile { TILE_LARGE, TILE_SMALL, TILE_SMALL_DEEP, TILE_SMALL_AHEAD };
+struct GemmChoice {
+    GemmTile tile;
+    u32 want_splits;  // > 1: cut K this many times although the tile grid covers the chip
+};
+static GemmChoice choose_tiles(u32 M, u32 N, u32 K, u32 zdim, bool dense) {
+    const uint64_t tiles_l = uint64_t(ceil_div(M, 128)) * ceil_div(N, 128) * zdim;
+    const uint64_t tiles_s = uint64_t(ceil_div(M, 64)) * ceil_div(N, 64) * zdim;
+    if (M > 64 && N > 64) {
+        // measured on square and skinny-K problems: large tiles win once they give a CU three or more workgroups; below
+        // that, small tiles with loads two slabs ahead win as soon as there are two of them per CU
+        // a short contraction (16 large slabs or fewer) is mostly prologue and epilogue for a large tile
+        if (tiles_l >= 800 && K <= 256) return {TILE_SMALL_AHEAD, 0};
+        if (tiles_l >= 800) return {TILE_LARGE, 0};
+        if (tiles_s >= 512) return {TILE_SMALL_AHEAD, 0};
+        // at most one small tile per CU: a contraction long enough is cut in two, so that two workgroups per CU hide each
+        // other's loads (measured: pays from K = 1280, from 1024 when the tiles do not cover the CUs evenly) ...
+        if (tiles_s >= 160 && K < 2048 && (K >= 1280 || (K >= 1024 && tiles_s > 256)) && zdim == 1 && dense) return {TILE_SMALL_AHEAD, 2};
+        // ... a shorter one gets longer slabs, so that a slab's loads have a whole slab of MFMAs (2048 clocks) to arrive in
+        if (tiles_s >= 160 && K >= 512 && K < 2048) return {TILE_SMALL_DEEP, 0};
+        if (tiles_s >= 160 && K < 2048) return {TILE_SMALL_AHEAD, 0};
+        // one small tile per CU at most but a long contraction: two K slices per tile put two workgroups on every CU
+        if (tiles_s >= 160 && K >= 2048 && zdim == 1 && dense) return {TILE_SMALL_AHEAD, 2};
+        if (tiles_l >= 160) return {TILE_LARGE, 0};
+        // A grid of small tiles somewhat short of the chip, cut over K by plan_split, beats large tiles cut deeper.
+        if (tiles_s >= 100 && K >= 512 && K < 2048) return {TILE_SMALL_AHEAD, 0};
+        const SplitPlan sp = plan_split(M, N, K, 128, 128, 16, zdim);
+        if (sp.splits > 1 && sp.k_per_z >= 512) return {TILE_LARGE, 0};
+    }
+    if (K >= 32768) return {TILE_SMALL_AHEAD, 0};  // very long contraction: slices stay long after the split
+    return {TILE_SMALL, 0};
+}
+
+// The K split of a tile configuration for a problem (splits == 1: none).
+template <class Cfg>
+static SplitPlan split_for(u32 M, u32 N, u32 K, u32 zdim, u32 want_splits, bool dense) {
+    SplitPlan sp = plan_split(M, N, K, Cfg::BM, Cfg::BN, Cfg::BK, zdim);
+    if (want_splits > 1 && zdim == 1 && sp.splits == 1) {  // the caller wants K cut although the tile grid covers the chip
+        sp.k_per_z = ceil_div(ceil_div(K, want_splits), u32(Cfg::BK)) * Cfg::BK;
+        sp.splits = ceil_div(K, sp.k_per_z);
+    }
+    if (!dense) sp = SplitPlan{1, K};  // partials assume a dense result
+    return sp;
+}
+
 // Runs C = A*B through the engine. `e` describes the final result; when the M x N tile grid is too small to occupy the
 // chip (and there is no batch), K is cut into slices whose partial results go to scratch and a second kernel combines
 // them in fixed order and applies the epilogue (bias / accumulate / ReLU).
 template <class Cfg, class AOp, class BOp>
 static int run_cfg(const AOp &a, const BOp &b, const RowMajorEpi &e, u32 M, u32 N, u32 K, u32 zdim, hipStream_t s,
                    const char *what, u32 want_splits = 0) {
-    SplitPlan sp = plan_split(M, N, K, Cfg::BM, Cfg::BN, Cfg::BK, zdim);
-    if (want_splits > 1 && zdim == 1 && sp.splits == 1) {  // the caller wants K cut although the tile grid covers the chip
-        sp.k_per_z = ceil_div(ceil_div(K, want_splits), u32(Cfg::BK)) * Cfg::BK;
-        sp.splits = ceil_div(K, sp.k_per_z);
-    }
+    const SplitPlan sp = split_for<Cfg>(M, N, K, zdim, want_splits, e.ld == N);
     if (sp.splits == 1) return launch_igemm<Cfg>(a, b, e, M, N, K, zdim, 0, K, s, what);
-    if (e.ld != N) return launch_igemm<Cfg>(a, b, e, M, N, K, zdim, 0, K, s, what);  // partials assume a dense result
     const size_t need = size_t(sp.splits) * M * N * sizeof(float);
-    float *ws = static_cast<float *>(arena_get(need, s));
-    if (!ws) return fail(CRB_EHIP, "%s: cannot allocate %zu bytes of split-K scratch", what, need);
+    float *ws = nullptr;
+    if (int st = scratch_get(need, s, what, &ws)) return st;
     RowMajorEpi pe{ws, nullptr, N, M * N, 0u};
     if (int st = launch_igemm<Cfg>(a, b, pe, M, N, K, sp.splits, 1, sp.k_per_z, s, what)) return st;
     if (e.row_bias) return launch_splitk_reduce(ws, e.C, M * N, sp.splits, ReduceEpi{e.row_bias, N, M, e.flags}, s, what);
@@ -39,34 +82,26 @@ static int run_cfg(const AOp &a, const BOp &b, const RowMajorEpi &e, u32 M, u32 
 template <class AOp, class BOp>
 static int run_tiles(const AOp &a, const BOp &b, const RowMajorEpi &e, u32 M, u32 N, u32 K, u32 zdim, hipStream_t s,
                      const char *what) {
-    // Tile choice by how many workgroups the grid gives a CU; when neither tile size fills the chip, K is split — with
-    // large tiles only when each slice keeps a long contraction (the split costs a second pass over the result).
-    const uint64_t tiles_l = uint64_t(ceil_div(M, 128)) * ceil_div(N, 128) * zdim;
-    const uint64_t tiles_s = uint64_t(ceil_div(M, 64)) * ceil_div(N, 64) * zdim;
-    if (M > 64 && N > 64) {
-        // measured on square and skinny-K problems: large tiles win once they give a CU three or more workgroups; below
-        // that, small tiles with loads two slabs ahead win as soon as there are two of them per CU
-        // a short contraction (16 large slabs or fewer) is mostly prologue and epilogue for a large tile
-        if (tiles_l >= 800 && K <= 256) return run_cfg<CfgSmallAhead>(a, b, e, M, N, K, zdim, s, what);
-        if (tiles_l >= 800) return run_cfg<CfgLarge>(a, b, e, M, N, K, zdim, s, what);
-        if (tiles_s >= 512) return run_cfg<CfgSmallAhead>(a, b, e, M, N, K, zdim, s, what);
-        // at most one small tile per CU: a contraction long enough is cut in two, so that two workgroups per CU hide each
-        // other's loads (measured: pays from K = 1280, from 1024 when the tiles do not cover the CUs evenly) ...
-        if (tiles_s >= 160 && K < 2048 && (K >= 1280 || (K >= 1024 && tiles_s > 256)) && zdim == 1 && e.ld == N)
-            return run_cfg<CfgSmallAhead>(a, b, e, M, N, K, zdim, s, what, 2);
-        // ... a shorter one gets longer slabs, so that a slab's loads have a whole slab of MFMAs (2048 clocks) to arrive in
-        if (tiles_s >= 160 && K >= 512 && K < 2048) return run_cfg<CfgSmallDeep>(a, b, e, M, N, K, zdim, s, what);
-        if (tiles_s >= 160 && K < 2048) return run_cfg<CfgSmallAhead>(a, b, e, M, N, K, zdim, s, what);
-        // one small tile per CU at most but a long contraction: two K slices per tile put two workgroups on every CU
-        if (tiles_s >= 160 && K >= 2048 && zdim == 1 && e.ld == N) return run_cfg<CfgSmallAhead>(a, b, e, M, N, K, zdim, s, what, 2);
-        if (tiles_l >= 160) return run_cfg<CfgLarge>(a, b, e, M, N, K, zdim, s, what);
-        // A grid of small tiles somewhat short of the chip, cut over K by plan_split, beats large tiles cut deeper.
-        if (tiles_s >= 100 && K >= 512 && K < 2048) return run_cfg<CfgSmallAhead>(a, b, e, M, N, K, zdim, s, what);
-        const SplitPlan sp = plan_split(M, N, K, 128, 128, 16, zdim);
-        if (sp.splits > 1 && sp.k_per_z >= 512) return run_cfg<CfgLarge>(a, b, e, M, N, K, zdim, s, what);
+    const GemmChoice c = choose_tiles(M, N, K, zdim, e.ld == N);
+    switch (c.tile) {
+        case TILE_LARGE: return run_cfg<CfgLarge>(a, b, e, M, N, K, zdim, s, what, c.want_splits);
+        case TILE_SMALL_DEEP: return run_cfg<CfgSmallDeep>(a, b, e, M, N, K, zdim, s, what, c.want_splits);
+        case TILE_SMALL_AHEAD: return run_cfg<CfgSmallAhead>(a, b, e, M, N, K, zdim, s, what, c.want_splits);
+        default: return run_cfg<CfgSmall>(a, b, e, M, N, K, zdim, s, what, c.want_splits);
     }
-    if (K >= 32768) return run_cfg<CfgSmallAhead>(a, b, e, M, N, K, zdim, s, what);  // very long contraction: slices stay long after the split
-    return run_cfg<CfgSmall>(a, b, e, M, N, K, zdim, s, what);
+}
+
+// Scratch bytes run_tiles asks for on a dense M x N result with contraction length K (0: the contraction is not cut).
+size_t gemm_scratch_bytes(u32 M, u32 N, u32 K, u32 zdim) {
+    const GemmChoice c = choose_tiles(M, N, K, zdim, true);
+    SplitPlan sp;
+    switch (c.tile) {
+        case TILE_LARGE: sp = split_for<CfgLarge>(M, N, K, zdim, c.want_splits, true); break;
+        case TILE_SMALL_DEEP: sp = split_for<CfgSmallDeep>(M, N, K, zdim, c.want_splits, true); break;
+        case TILE_SMALL_AHEAD: sp = split_for<CfgSmallAhead>(M, N, K, zdim, c.want_splits, true); break;
+        default: sp = split_for<CfgSmall>(M, N, K, zdim, c.want_splits, true); break;
+    }
+    return sp.splits > 1 ? size_t(sp.splits) * M * N * sizeof(float) : 0;
 }
 
 static int check_dims(const char *what, u32 M, u32 N, u32 K, u32 batch) {
@@ -219,6 +254,11 @@ int gemm_tn_batched(const float *A, const float *B, float *C, u32 M, u32 N, u32 
 using namespace crb;
 
 extern "C" {
+
+size_t crb_gemm_workspace_bytes(uint32_t M, uint32_t N, uint32_t K, uint32_t batch) {
+    if (check_dims("crb_gemm_workspace_bytes", M, N, K, batch)) return 0;
+    return gemm_scratch_bytes(M, N, K, batch);
+}
 
 int crb_sgemm_nn(const float *A, const float *B, float *C, uint32_t M, uint32_t N, uint32_t K, uint32_t batch,
                  void *stream) {

@@ -48,15 +48,35 @@ int crb_abi_version(void);
 /* Message for the most recent non-OK status returned to the calling thread ("" if none). */
 const char *crb_last_error_string(void);
 
-/* Releases the library's lazily grown split-K scratch arenas (safe to call at any time when no
- * library kernel is in flight). The library keeps one arena per (device, stream), so calls queued on
- * different streams never share scratch and may overlap; calls on one stream run in order and reuse
- * that stream's arena. An arena grows with hipMalloc on first use or when a call needs more (after
- * waiting for that stream), so callers that must not allocate pass their own workspace where an
- * entry point takes one. */
+/* Releases the library's lazily grown split-K scratch arenas (call it only when no library kernel is in
+ * flight and no recorded graph that used the arenas will be replayed). The library keeps one arena per
+ * (device, stream), so calls queued on different streams never share scratch and may overlap; calls on
+ * one stream run in order and reuse that stream's arena. An arena grows with hipMalloc on first use or
+ * when a call needs more; a block it has outgrown stays allocated until this call, because work in
+ * flight or a recorded graph may still name it. Growth is refused (CRB_EWORKSPACE) while the stream is
+ * being captured. Callers that must not allocate bind their own block (crb_bind_workspace) or pass a
+ * workspace where an entry point takes one. */
 void crb_release_workspace(void);
 
+/* Binds a caller-owned block of device memory (256-byte aligned) to `stream` of the current device as the split scratch
+ * of every entry point that takes no workspace argument of its own (the GEMM and dense-layer families, the general
+ * convolution forward / data-gradient path, crb_conv_bias_grad, and the convolution entry points when their workspace
+ * argument is NULL). While a block is bound, calls on that stream never allocate: a call that needs more than the block
+ * holds returns CRB_EWORKSPACE. The *_workspace_bytes queries below tell what a call needs. workspace == NULL unbinds
+ * (the library arena serves the stream again). The block must stay valid until the work queued on the stream that uses
+ * it has finished; the library never frees it. No counterpart in the reference, whose operators never need scratch
+ * (seblas/operations/cuGEMM.cu:1649-1714 launches one kernel per call). For callers that record the calls into a HIP
+ * graph or must not allocate on their hot path. One stream must not be driven by several host threads at once. */
+int crb_bind_workspace(void *workspace, size_t workspace_bytes, void *stream);
+
 /* GEMM family ------------------------------------------------------------------------------ */
+
+/* Bytes of split scratch a call of the GEMM or dense-layer family needs (0: none) when its result is M x N per batch
+ * entry and its contraction has length K: crb_sgemm_nn / crb_sgemm_tn (M, N, K, batch); crb_sgemm_nt (M, N, K, 1);
+ * crb_sgemm_nta (M, N, K * batch, 1); crb_linear_fwd (batch, OUT, IN, 1); crb_linear_dgrad (batch, IN, OUT, 1);
+ * crb_linear_wgrad (OUT, IN, batch, 1). The scratch comes from the block bound with crb_bind_workspace, else from the
+ * library arena. */
+size_t crb_gemm_workspace_bytes(uint32_t M, uint32_t N, uint32_t K, uint32_t batch);
 
 /* Replaces seblas::sgemm (seblas/operations/cuGEMM.cu:1649-1664; kernels :34-210, :791-999).
  * For nd in [0,batch): C[nd] (MxN) = A (MxK) * B[nd] (KxN). A is shared across the batch
@@ -122,14 +142,22 @@ int crb_conv_fwd(const float *W, const float *X, float *Y, const float *bias_or_
  * W[oc,ic,fh,fw] * dY[n,oc,oh,ow]. Overwrite. */
 int crb_conv_dgrad(const float *W, const float *dY, float *dX, const crb_conv_geom *g, void *stream);
 
-/* Bytes of scratch crb_conv_wgrad needs for this geometry (0 if none). */
+/* Bytes of split scratch crb_conv_fwd / crb_conv_dgrad need for this geometry (0 for every shape with a kernel of its
+ * own; the general implicit-GEMM path cuts short-and-wide contractions). operands_aligned16: whether the activation
+ * tensors are 16-byte aligned (hipMalloc'd ones are); other alignments take the general path. Served from the block
+ * bound with crb_bind_workspace, else from the library arena. */
+size_t crb_conv_fwd_workspace_bytes(const crb_conv_geom *g, int operands_aligned16);
+size_t crb_conv_dgrad_workspace_bytes(const crb_conv_geom *g, int operands_aligned16);
+
+/* Bytes of scratch crb_conv_wgrad needs for this geometry with 16-byte aligned tensors (0 if none). */
 size_t crb_conv_wgrad_workspace_bytes(const crb_conv_geom *g);
 
 /* Replaces seblas::convError (cuConv.cu:793-806; kernel :488-707).
  * dW[oc,ic,fh,fw] += sum_{n,oh,ow} dY[n,oc,oh,ow] * X[n,ic,oh*sH-pH+fh,ow*sW-pW+fw]. Accumulate.
  * The reduction over n*OH*OW is split across workgroups and combined in a fixed order (no atomics),
- * so results are bit-reproducible. `workspace` may be NULL: the library then uses its own lazily
- * grown arena (which may call hipMalloc on first use / growth); otherwise it must be 16-byte aligned
+ * so results are bit-reproducible. `workspace` may be NULL: the library then uses the block bound to
+ * the stream (crb_bind_workspace) or its own lazily grown arena (which may call hipMalloc on first
+ * use / growth, and refuses to during a stream capture); otherwise it must be 16-byte aligned
  * and hold at least crb_conv_wgrad_workspace_bytes(g) bytes (CRB_EWORKSPACE if not). */
 int crb_conv_wgrad(const float *dY, const float *X, float *dW, const crb_conv_geom *g, void *workspace,
                    size_t workspace_bytes, void *stream);
@@ -169,6 +197,8 @@ int crb_sum_slices_multi(const crb_slice_sum_item *items, uint32_t n_items, void
  * size assertion (seblas/operations/cuReduce.cu:237) cannot hold for a C-element bias; this computes the
  * per-channel sum that call is meant to produce. Accumulate. */
 int crb_conv_bias_grad(const float *dY, float *dB, uint32_t N, uint32_t C, uint32_t HW, void *stream);
+/* Bytes of scratch crb_conv_bias_grad needs (partial column sums; from the bound workspace or the library arena). */
+size_t crb_conv_bias_grad_workspace_bytes(uint32_t N, uint32_t C, uint32_t HW);
 
 /* Tensor helpers the conv / linear operands use around the hot path ---------------------------- */
 
