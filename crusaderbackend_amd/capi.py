@@ -45,6 +45,7 @@ SIGNATURES = {
     "crb_conv_fwd_workspace_bytes": (ctypes.c_size_t, [ctypes.POINTER(ConvGeom), ctypes.c_int]),
     "crb_conv_dgrad_workspace_bytes": (ctypes.c_size_t, [ctypes.POINTER(ConvGeom), ctypes.c_int]),
     "crb_conv_bias_grad_workspace_bytes": (ctypes.c_size_t, [_u32, _u32, _u32]),
+    "crb_conv_wgrad_noalloc": (ctypes.c_int, [_ptr, _ptr, _ptr, ctypes.POINTER(ConvGeom), _ptr]),
     "crb_sgemm_nn": (ctypes.c_int, [_ptr, _ptr, _ptr, _u32, _u32, _u32, _u32, _ptr]),
     "crb_sgemm_tn": (ctypes.c_int, [_ptr, _ptr, _ptr, _u32, _u32, _u32, _u32, _ptr]),
     "crb_sgemm_nt": (ctypes.c_int, [_ptr, _ptr, _ptr, _u32, _u32, _u32, _ptr]),
@@ -173,6 +174,14 @@ def conv_wgrad_workspace_bytes(geom):
 def conv_wgrad(dY, X, dW, geom, workspace=None, stream=None):
     nbytes = 0 if workspace is None else workspace.numel() * workspace.element_size()
     check(load().crb_conv_wgrad(_p(dY), _p(X), _p(dW), ctypes.byref(geom), _p(workspace), nbytes, _stream(stream)))
+
+
+def conv_wgrad_noalloc(dY, X, dW, geom, stream=None):
+    """conv_wgrad on the library's built-in scratch buffer: the call allocates nothing."""
+    check(load().crb_conv_wgrad_noalloc(_p(dY), _p(X), _p(dW), ctypes.byref(geom), _stream(stream)))
+
+
+NOALLOC_SCRATCH_BYTES = 8 << 20  # CRB_NOALLOC_SCRATCH_BYTES
 
 
 def bind_workspace(workspace, stream=None):

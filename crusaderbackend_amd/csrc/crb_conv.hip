@@ -6,6 +6,8 @@
 #include "gemm_internal.h"
 #include "operands.h"
 
+#include <mutex>
+
 namespace crb {
 
 // Macro-tiles chosen by the channel extent on the GEMM-M side; the pixel (or tap) side is 128 wide.
@@ -456,6 +458,32 @@ static BiasGradPlan bias_grad_plan(u32 N, u32 cols, bool vec) {
     return p;
 }
 
+// ---- built-in scratch of the entry point that allocates nothing -----------------------------------------------------------
+// Device memory that exists as long as the code object is loaded: one copy per GPU, at an address of its own on each. In
+// host code the array's name is only a handle for hipGetSymbolAddress; kernels and copies get the address that call
+// returns for the current device.
+constexpr size_t kStaticScratchBytes = CRB_NOALLOC_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+constexpr int kMaxDevices = 64;
+static std::mutex g_static_mu;
+static void *g_static_ptr[kMaxDevices];
+
+// The current device's copy of `scratch` (looked up once per device, with that device current).
+static int static_scratch_ptr(const char *what, void **out) {
+    int dev = 0;
+    if (hipError_t e = hipGetDevice(&dev)) return check_hip(e, what);
+    if (dev < 0 || dev >= kMaxDevices) return fail(CRB_EHIP, "%s: device ordinal %d out of range", what, dev);
+    std::lock_guard<std::mutex> lk(g_static_mu);
+    if (!g_static_ptr[dev]) {
+        void *p = nullptr;
+        if (hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch))) return check_hip(e, what);
+        if (!p) return fail(CRB_EHIP, "%s: the built-in scratch buffer has no device address", what);
+        g_static_ptr[dev] = p;
+    }
+    *out = g_static_ptr[dev];
+    return CRB_OK;
+}
+
 }  // namespace crb
 
 using namespace crb;
@@ -623,6 +651,21 @@ int crb_conv_wgrad(const float *dY, const float *X, float *dW, const crb_conv_ge
     RowMajorEpi e{ws, nullptr, p.Ncols, p.M * p.Ncols, 0u};
     if (int st = run_by_m(a, b, e, p.M, p.Ncols, p.K, p.splits, 1, p.k_per_z, s, "crb_conv_wgrad")) return st;
     return launch_splitk_reduce(ws, dW, p.M * p.Ncols, p.splits, ReduceEpi{nullptr, 1, 1, EPI_ACCUM}, s, "crb_conv_wgrad(reduce)");
+}
+
+int crb_conv_wgrad_noalloc(const float *dY, const float *X, float *dW, const crb_conv_geom *g, void *stream) {
+    if (!dY || !X || !dW) return fail(CRB_ENULL, "crb_conv_wgrad_noalloc: null operand");
+    if (int st = check_geom("crb_conv_wgrad_noalloc", g)) return st;
+    const size_t need = crb_conv_wgrad_workspace_bytes(g);
+    if (need > kStaticScratchBytes)
+        return fail(CRB_EWORKSPACE,
+                    "crb_conv_wgrad_noalloc: this geometry needs %zu bytes of scratch, the built-in buffer holds %zu; use "
+                    "crb_conv_wgrad with a caller workspace", need, kStaticScratchBytes);
+    void *ptr = nullptr;
+    if (int st = static_scratch_ptr("crb_conv_wgrad_noalloc", &ptr)) return st;
+    // every scratch request below this call is served from the built-in buffer or refused: nothing allocates
+    ScratchScope scope(ptr, kStaticScratchBytes);
+    return crb_conv_wgrad(dY, X, dW, g, ptr, kStaticScratchBytes, stream);
 }
 
 size_t crb_conv_fwd_workspace_bytes(const crb_conv_geom *g, int operands_aligned16) {

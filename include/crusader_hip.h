@@ -162,6 +162,15 @@ size_t crb_conv_wgrad_workspace_bytes(const crb_conv_geom *g);
 int crb_conv_wgrad(const float *dY, const float *X, float *dW, const crb_conv_geom *g, void *workspace,
                    size_t workspace_bytes, void *stream);
 
+/* crb_conv_wgrad for callers that cannot allocate and have no workspace to pass: code under HIP graph capture, tight
+ * serving or training loops, harnesses that forbid hipMalloc. No counterpart in the reference. Same result as
+ * crb_conv_wgrad (bit for bit); the split scratch is a buffer of CRB_NOALLOC_SCRATCH_BYTES built into the library (device
+ * memory each GPU the library runs on holds until the process ends), so the call allocates nothing. Geometries whose
+ * crb_conv_wgrad_workspace_bytes exceed that size return CRB_EWORKSPACE. Every call on a GPU uses that GPU's one buffer:
+ * calls on one stream run in order and are safe; calls that overlap on different streams of one GPU race. */
+#define CRB_NOALLOC_SCRATCH_BYTES (8u << 20)
+int crb_conv_wgrad_noalloc(const float *dY, const float *X, float *dW, const crb_conv_geom *g, void *stream);
+
 /* Replaces seblas::convBias (cuConv.cu:808-818; kernel :709-729). Y[n,c,:,:] += bias[c], in place. */
 int crb_conv_bias(float *Y, const float *bias, uint32_t N, uint32_t C, uint32_t HW, void *stream);
 
