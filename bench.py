@@ -8,6 +8,16 @@ stages and two stride-2 transitions, with the layer multiplicities of the refere
 N(0,1) activations/gradients and He-normal filters already resident in HBM. Flops are nominal
 (2*N*OC*OH*OW*IC*FH*FW per pass; zeros from stride/padding are not discounted).
 
+The timed step issues, per layer, crb_conv_fwd and crb_conv_bwd_sliced (both gradients in one launch) and sums all
+weight-gradient slices with one crb_sum_slices_multi at its end. `three_call_step` times the same work through the
+reference's own call sequence (conv, convDerive, convError as three separate calls per layer: crb_conv_fwd,
+crb_conv_dgrad, crb_conv_wgrad; seann/operands/seblas/Conv2D.cu:8-29), also over exactly K steps.
+
+Cache state: a layer shape is run `mult` times on ONE set of X / W / dY buffers, so a launch finds its inputs in L2 or
+the memory-side cache (in a whole network, where inputs arrive from the previous operator, the same kernels measure 4-8 %
+longer). `extra.cold_ms_per_step` repeats both step forms with every layer instance on buffers of its own (about 1 GB of
+distinct operands per step, beyond L2 and the 256 MB memory-side cache).
+
 Prints ONE JSON line. `value` is TFLOP/s over the timed steps; `extra` carries images/s and the 4096^3 sgemm rate.
 `roofline` describes the kernel that takes the most time in the step, timed per launch with HIP events on the
 launch stream in a separate instrumented pass. `cpu_baseline` is the CPU oracle on a bounded sample.
@@ -82,6 +92,29 @@ class Layer:
         self.bytes["bwd"] = 4.0 * (self.dY.numel() + self.W.numel() + self.dX.numel() + self.X.numel() + 2 * self.dW.numel())
         self.bytes["bwd_sliced"] = self.bytes["bwd"]  # its share of the final summation included
         self.capi = capi
+        self.sets = None
+
+    def make_cold_sets(self, torch, dev):
+        """One X / dY / Y / dX set per layer instance (the filters and their gradients are per instance already)."""
+        self.sets = [(torch.randn_like(self.X), torch.randn_like(self.dY), torch.empty_like(self.Y), torch.empty_like(self.dX),
+                      self.W.clone(), torch.zeros_like(self.dW)) for _ in range(self.mult)]
+
+    def fwd_cold(self, k):
+        X, dY, Y, dX, W, dW = self.sets[k]
+        self.capi.conv_fwd(W, X, Y, self.b, self.g)
+
+    def bwd_sliced_cold(self, k):
+        X, dY, Y, dX, W, dW = self.sets[k]
+        self.capi.conv_bwd_sliced(W, dY, X, dX, self.g, self.ws_each[k])
+
+    def bwd_cold(self, k):
+        X, dY, Y, dX, W, dW = self.sets[k]
+        self.capi.conv_bwd(W, dY, X, dX, dW, self.g, workspace=self.ws)
+
+    def dgrad_wgrad_cold(self, k):
+        X, dY, Y, dX, W, dW = self.sets[k]
+        self.capi.conv_dgrad(W, dY, dX, self.g)
+        self.capi.conv_wgrad(dY, X, dW, self.g, workspace=self.ws)
 
     def fwd(self):
         self.capi.conv_fwd(self.W, self.X, self.Y, self.b, self.g)
@@ -262,14 +295,65 @@ def main():
         if slice_table is not None:
             capi.sum_slices_multi(slice_table)  # every layer's dW += its slices, one launch
 
-    for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        step()
-    torch.cuda.synchronize()
-    dt = time.perf_counter() - t0
+    def step_three_call():
+        """The reference's call sequence: conv per layer on the way forward, convDerive then convError per layer on the way back."""
+        for L in layers:
+            for _ in range(L.mult):
+                L.fwd()
+        for L in reversed(layers):
+            for _ in range(L.mult):
+                L.dgrad()
+                L.wgrad()
+
+    def timed(fn):
+        for _ in range(args.warmup):
+            fn()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            fn()
+        torch.cuda.synchronize()
+        return time.perf_counter() - t0
+
+    dt = timed(step)
+    dt3 = timed(step_three_call)
+    three_call = {
+        "value": step_flops * args.steps / dt3 / 1e12, "unit": "TFLOP/s", "ms_per_step": dt3 / args.steps * 1e3,
+        "frac_fp32_mfma_peak": step_flops * args.steps / dt3 / 1e12 / PEAK_FP32_MFMA_TFLOPS,
+        "images_per_s": BATCH * args.steps / dt3, "steps": args.steps,
+        "calls": "crb_conv_fwd, crb_conv_dgrad, crb_conv_wgrad per layer (the reference's conv / convDerive / convError sequence)",
+    }
+
+    # cold variants: every layer instance on buffers of its own
+    for L in layers:
+        L.make_cold_sets(torch, dev)
+
+    def step_cold():
+        for L in layers:
+            for k in range(L.mult):
+                L.fwd_cold(k)
+        for L in reversed(layers):
+            for k in range(L.mult):
+                if L.n_slices:
+                    L.bwd_sliced_cold(k)
+                else:
+                    L.bwd_cold(k)
+        if slice_table is not None:
+            capi.sum_slices_multi(slice_table)
+
+    def step_three_call_cold():
+        for L in layers:
+            for k in range(L.mult):
+                L.fwd_cold(k)
+        for L in reversed(layers):
+            for k in range(L.mult):
+                L.dgrad_wgrad_cold(k)
+
+    dt_cold, dt3_cold = timed(step_cold), timed(step_three_call_cold)
+    cold_bytes = sum(sum(t.numel() * 4 for t in st) for L in layers for st in L.sets)
+    for L in layers:
+        L.sets = None
+    torch.cuda.empty_cache()
     ms_per_step = dt / args.steps * 1e3
     tflops = step_flops * args.steps / dt / 1e12
     images_per_s = BATCH * args.steps / dt
@@ -318,7 +402,12 @@ def main():
                                "crb_sum_slices_multi call at the end of the step)",
                    "batch": BATCH, "flops_per_step": step_flops},
         "roofline": roofline,
+        "three_call_step": three_call,
         "extra": {
+            "cold_ms_per_step": dt_cold / args.steps * 1e3, "cold_tflops": step_flops * args.steps / dt_cold / 1e12,
+            "cold_three_call_ms_per_step": dt3_cold / args.steps * 1e3,
+            "cold_three_call_tflops": step_flops * args.steps / dt3_cold / 1e12,
+            "cold_distinct_operand_bytes": cold_bytes,
             "frac_fp32_mfma_peak": tflops / PEAK_FP32_MFMA_TFLOPS,
             "resnet56_conv_images_per_s": images_per_s,
             "resnet56_conv_images_per_s_kernel_only": BATCH / (kern_sum_ms / 1e3),

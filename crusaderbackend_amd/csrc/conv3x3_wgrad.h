@@ -18,16 +18,26 @@
 // accumulator register r = dW[oc = 4*(l/16) + r][ic = l%16]; 9 accumulator tiles (one per tap) per wave.
 // The 4 waves take different rows (or images) of the tile; their accumulators are summed through LDS in fixed
 // wave order at the end and written either as this split's partial result or, without splitting, added to dW.
+//
+// Eight-wave form (WAVES = 8): waves w and w + 4 take the SAME pixels and split the taps (0..4 and 5..8), so every SIMD
+// holds two waves that fill each other's issue gaps (a lone wave keeps the matrix pipe about two thirds busy) while each
+// accumulator still sees exactly the MFMA sequence of the four-wave form: results are bit-identical.
 #pragma once
+#include <type_traits>
+
 #include "igemm_engine.h"
 
 namespace crb {
 
 // W_: dY width; TR_: dY rows per image per tile; TI_: images per tile (more than 4: whole small images, TI/4 per wave);
-// S_: stride.
-template <int W_, int TR_, int TI_, int OCC_, int S_ = 1>
+// S_: stride; WAVES_: 4, or 8 (two waves per pixel group, each with half of the taps).
+template <int W_, int TR_, int TI_, int OCC_, int S_ = 1, int WAVES_ = 4>
 struct WgradCfg {
     static constexpr int W = W_, TR = TR_, TI = TI_, OCC = OCC_, S = S_;
+    static constexpr int WAVES = WAVES_, NT = 64 * WAVES_;  // threads per workgroup
+    static_assert(WAVES == 4 || WAVES == 8, "waves per workgroup");
+    static constexpr bool SPLIT = WAVES == 8;  // a wave multiplies half of the taps
+    static constexpr int TAP_SPLIT = 5;  // eight-wave form: waves 0..3 take taps 0..4, waves 4..7 taps 5..8
     static constexpr int WPI = TI >= 4 ? 1 : 4 / TI;  // waves per image of the tile
     static constexpr int IPW = TI >= 4 ? TI / 4 : 1;  // images per wave (small images: TR is the whole image height)
     static constexpr int RW = TR / WPI;        // rows per wave (per image)
@@ -80,6 +90,7 @@ __device__ __forceinline__ void wgrad3x3_body(const WgradArgs &a, const u32 bid,
     constexpr int W = Cfg::W, TR = Cfg::TR, TI = Cfg::TI, YP = Cfg::YP, XP = Cfg::XP, NSTEP = Cfg::NSTEP;
     constexpr int YIMG = Cfg::YIMG, XIMG = Cfg::XIMG;
 
+    constexpr int NT = Cfg::NT;
     const u32 t = threadIdx.x;
     // The workgroups of one split z read the same tiles (different channel blocks). With ids 8 apart they run on the
     // same XCD and share the tiles through its L2 (workgroups are dealt round-robin to the 8 XCDs).
@@ -103,8 +114,8 @@ __device__ __forceinline__ void wgrad3x3_body(const WgradArgs &a, const u32 bid,
     // so per tile and item the address arithmetic is one add of a compile-time multiple of the row pitch.
     constexpr int YRQ = W / 4, XRQ = Cfg::XRW / 4;      // quads per dY row / per input row
     constexpr int YC = TI * 16 * YRQ, XC = TI * 16 * XRQ;  // columns
-    static_assert(kThreads % YC == 0 && kThreads % XC == 0, "columns must divide the workgroup");
-    constexpr int YRPP = kThreads / YC, XRPP = kThreads / XC;  // rows covered per pass
+    static_assert(NT % YC == 0 && NT % XC == 0, "columns must divide the workgroup");
+    constexpr int YRPP = NT / YC, XRPP = NT / XC;  // rows covered per pass
     constexpr int YNP = (TR + YRPP - 1) / YRPP, XNP = (Cfg::XROWS + XRPP - 1) / XRPP;
     v4f yreg[YNP], xreg[XNP];
 
@@ -120,7 +131,7 @@ __device__ __forceinline__ void wgrad3x3_body(const WgradArgs &a, const u32 bid,
     const float *xsrc = a.X + (size_t(ximg) * a.IC + ib * 16 + xc) * in_HW + 4 * xq;
     const u32 xlds = xc * XP + 4 + ximg * XIMG + (Cfg::S == 1 ? 4 * xq : 2 * xq);
 
-    auto fetch = [&](u32 tile) {
+    auto fetch = [&](u32 tile, v4f *yr, v4f *xr) {
         const u32 n0 = (tile / a.tiles_per_img) * TI;
         const int r0 = int(tile % a.tiles_per_img) * TR;
         const float *yp = ysrc + size_t(n0) * a.OC * HW + u32(r0) * W;
@@ -128,7 +139,7 @@ __device__ __forceinline__ void wgrad3x3_body(const WgradArgs &a, const u32 bid,
         for (int i = 0; i < YNP; ++i) {
             v4f v = {0.f, 0.f, 0.f, 0.f};
             if (ychan_ok && (TR % YRPP == 0 || i * YRPP + int(yrp) < TR)) v = *reinterpret_cast<const v4f *>(yp + i * YRPP * W);
-            yreg[i] = v;
+            yr[i] = v;
         }
         // first staged input row: r0 - 1 (stride 1), 2*(r0 - 1) (stride 2: both parities of the halo row pair)
         const int row0 = (Cfg::S == 1 ? r0 - 1 : 2 * (r0 - 1)) + int(xrp);
@@ -139,32 +150,32 @@ __device__ __forceinline__ void wgrad3x3_body(const WgradArgs &a, const u32 bid,
             const int row = row0 + i * XRPP;
             if (xchan_ok && (Cfg::XROWS % XRPP == 0 || i * XRPP + int(xrp) < Cfg::XROWS) && row >= 0 && row < int(in_H))
                 v = *reinterpret_cast<const v4f *>(xp + row * Cfg::XRW);
-            xreg[i] = v;
+            xr[i] = v;
         }
     };
 
     // LDS store of staged item i (dY items first, then X items)
-    auto commit_item = [&](int i, float *dYs, float *dXs) {
+    auto commit_item = [&](int i, const v4f *yr, const v4f *xr, float *dYs, float *dXs) {
         if (i < YNP) {
             if (TR % YRPP == 0 || i * YRPP + int(yrp) < TR) {
                 float *p = dYs + ylds + i * YRPP * W;
-                *reinterpret_cast<v2f *>(p) = v2f{yreg[i].x, yreg[i].y};
-                *reinterpret_cast<v2f *>(p + 2) = v2f{yreg[i].z, yreg[i].w};
+                *reinterpret_cast<v2f *>(p) = v2f{yr[i].x, yr[i].y};
+                *reinterpret_cast<v2f *>(p + 2) = v2f{yr[i].z, yr[i].w};
             }
         } else {
             const int ix = i - YNP;
             if (Cfg::XROWS % XRPP == 0 || ix * XRPP + int(xrp) < Cfg::XROWS) {
                 if constexpr (Cfg::S == 1) {
                     float *p = dXs + xlds + (ix * XRPP + xrp) * W;
-                    *reinterpret_cast<v2f *>(p) = v2f{xreg[ix].x, xreg[ix].y};
-                    *reinterpret_cast<v2f *>(p + 2) = v2f{xreg[ix].z, xreg[ix].w};
+                    *reinterpret_cast<v2f *>(p) = v2f{xr[ix].x, xr[ix].y};
+                    *reinterpret_cast<v2f *>(p + 2) = v2f{xr[ix].z, xr[ix].w};
                 } else {
                     // de-interleave: staged row j has row parity j % 2 and plane row j / 2; the quad's even columns go
                     // to the column-parity-0 plane, its odd columns to the column-parity-1 plane
                     const u32 j = ix * XRPP + xrp;
                     float *p = dXs + xlds + (j & 1) * 2 * Cfg::PL + (j >> 1) * W;
-                    *reinterpret_cast<v2f *>(p) = v2f{xreg[ix].x, xreg[ix].z};
-                    *reinterpret_cast<v2f *>(p + Cfg::PL) = v2f{xreg[ix].y, xreg[ix].w};
+                    *reinterpret_cast<v2f *>(p) = v2f{xr[ix].x, xr[ix].z};
+                    *reinterpret_cast<v2f *>(p + Cfg::PL) = v2f{xr[ix].y, xr[ix].w};
                 }
             }
         }
@@ -172,14 +183,15 @@ __device__ __forceinline__ void wgrad3x3_body(const WgradArgs &a, const u32 bid,
     constexpr int NITEM = YNP + XNP;
 
     // leading / trailing pad floats of every X plane stay zero (they are read, multiplied by a zeroed dY value)
-    for (u32 e = t; e < 2u * 16 * 8; e += kThreads) {
+    for (u32 e = t; e < 2u * 16 * 8; e += NT) {
         float *plane = smem + (e / 128) * Cfg::BUF + Cfg::Y_SIZE + ((e % 128) / 8) * XP;
         const u32 k = e % 8;
         plane[k < 4 ? k : 4 + TI * XIMG + (k - 4)] = 0.f;
     }
 
     // ---- per-lane fragment addressing ---------------------------------------------------------------------
-    const int lane = t & 63, wave = t >> 6;
+    const int lane = t & 63, wave = (t >> 6) & 3;  // wave: the pixel group (eight-wave form: shared by waves w and w + 4)
+    const int tap_half = t >> 8;                   // eight-wave form: which part of the taps this wave multiplies
     const int li = lane & 15, kq = lane >> 4;
     const int img_w = (wave / Cfg::WPI) * Cfg::IPW, row_w = (wave % Cfg::WPI) * Cfg::RW;
     const int ybase = li * YP + kq + img_w * YIMG + row_w * W;
@@ -193,13 +205,15 @@ __device__ __forceinline__ void wgrad3x3_body(const WgradArgs &a, const u32 bid,
     // this call) are spread over the last steps, one item per step, so they issue in the shadow of the MFMAs instead
     // of forming a store burst between tiles.
     constexpr int FIRST_STORE_STEP = NSTEP > NITEM ? NSTEP - NITEM : 0;
-    auto compute = [&](const float *cy, const float *cx, float *ny, float *nx) {
+    // T0, T1 (integral constants): the taps [T0, T1) this wave multiplies.
+    auto compute = [&](auto T0c, auto T1c, const float *cy, const float *cx, float *ny, float *nx) {
+        constexpr int T0 = decltype(T0c)::value, T1 = decltype(T1c)::value;
         const float *py = cy + ybase, *px = cx + xbase;
         float av[2], bv[2][9];
         auto read_step = [&](int s, int slot) {
             av[slot] = py[4 * s];
 #pragma unroll
-            for (int k = 0; k < 9; ++k) bv[slot][k] = px[Cfg::x_off(s) + Cfg::tap_off(k)];
+            for (int k = T0; k < T1; ++k) bv[slot][k] = px[Cfg::x_off(s) + Cfg::tap_off(k)];
         };
         read_step(0, 0);
 #pragma unroll
@@ -210,39 +224,50 @@ __device__ __forceinline__ void wgrad3x3_body(const WgradArgs &a, const u32 bid,
             const float a0 = ((4 * s) % W == 0) ? (kq == 0 ? 0.f : am) : am;
             const float a2 = (Cfg::S == 1 && (4 * s + 4) % W == 0) ? (kq == 3 ? 0.f : am) : am;
 #pragma unroll
-            for (int k = 0; k < 9; ++k)
+            for (int k = T0; k < T1; ++k)
                 acc[k] = __builtin_amdgcn_mfma_f32_16x16x4f32(k % 3 == 0 ? a0 : (k % 3 == 2 ? a2 : am), bv[s & 1][k], acc[k], 0, 0, 0);
             if (s >= FIRST_STORE_STEP) {
                 // items per step: all remaining ones on the last step if there are more items than steps
                 const int first = s - FIRST_STORE_STEP, last = (s == NSTEP - 1) ? NITEM : first + 1;
 #pragma unroll
-                for (int i = first; i < last; ++i) commit_item(i, ny, nx);
+                for (int i = first; i < last; ++i) commit_item(i, yreg, xreg, ny, nx);
             }
             // issue order inside the step: one MFMA, then one of the next step's LDS reads, and so on, so the matrix
             // pipe never waits for the read burst; the fence keeps the steps themselves in order
 #pragma unroll
-            for (int k = 0; k < 9; ++k) {
+            for (int k = T0; k < T1; ++k) {
                 __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // MFMA
                 __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // DS read
             }
             __builtin_amdgcn_sched_barrier(0);
         }
     };
+    // the tap range of this wave
+    auto compute_taps = [&](const float *cy, const float *cx, float *ny, float *nx) {
+        typedef std::integral_constant<int, 0> I0;
+        typedef std::integral_constant<int, 9> I9;
+        typedef std::integral_constant<int, Cfg::TAP_SPLIT> IS;
+        if constexpr (!Cfg::SPLIT) {
+            compute(I0(), I9(), cy, cx, ny, nx);
+        } else if (tap_half == 0) {
+            compute(I0(), IS(), cy, cx, ny, nx);
+        } else {
+            compute(IS(), I9(), cy, cx, ny, nx);
+        }
+    };
 
     // ---- main loop over this split's tiles (double-buffered) ------------------------------------------------
-    if (t_begin < t_end) {
-        fetch(t_begin);
+    fetch(t_begin, yreg, xreg);
 #pragma unroll
-        for (int i = 0; i < NITEM; ++i) commit_item(i, smem, smem + Cfg::Y_SIZE);
-    }
+    for (int i = 0; i < NITEM; ++i) commit_item(i, yreg, xreg, smem, smem + Cfg::Y_SIZE);
     __syncthreads();
     for (u32 tile = t_begin; tile < t_end; ++tile) {
         const u32 b = (tile - t_begin) & 1;
-        // After the last tile nothing new was fetched: the stores inside compute() then rewrite stale registers into the
-        // idle buffer, which nothing reads before the reduction scratch overwrites it.
-        if (tile + 1 < t_end) fetch(tile + 1);
+        // After the last tile nothing new was fetched: the stores inside compute() then rewrite stale registers into
+        // the idle buffer, which nothing reads before the reduction scratch overwrites it.
+        if (tile + 1 < t_end) fetch(tile + 1, yreg, xreg);
         float *cur = smem + b * Cfg::BUF, *nxt = smem + (b ^ 1) * Cfg::BUF;
-        compute(cur, cur + Cfg::Y_SIZE, nxt, nxt + Cfg::Y_SIZE);
+        compute_taps(cur, cur + Cfg::Y_SIZE, nxt, nxt + Cfg::Y_SIZE);
         __syncthreads();
     }
 
@@ -252,17 +277,22 @@ __device__ __forceinline__ void wgrad3x3_body(const WgradArgs &a, const u32 bid,
     // writes the sums back transposed to [oc][ic][tap], the order dW has in memory. Pass 3: coalesced store.
     float *red = smem;                 // [wave][tap][lane][4]  (4*9*256 floats)
     float *tr = smem + 4 * 9 * 256;    // [oc 16][ic 16][tap 9] (2304 floats)
+    // (eight-wave form: every wave parks the taps it holds; the threads of the upper half sum the upper taps)
 #pragma unroll
-    for (int k = 0; k < 9; ++k) *reinterpret_cast<v4f *>(red + ((wave * 9 + k) * 64 + lane) * 4) = acc[k];
+    for (int k = 0; k < 9; ++k)
+        if (!Cfg::SPLIT || (k < Cfg::TAP_SPLIT) == (tap_half == 0))
+            *reinterpret_cast<v4f *>(red + ((wave * 9 + k) * 64 + lane) * 4) = acc[k];
     __syncthreads();
     {
-        const u32 l2 = t >> 2, r = t & 3;
+        const u32 tq = t & 255;
+        const u32 l2 = tq >> 2, r = tq & 3;
         const u32 oc = 4 * (l2 >> 4) + r, ic = l2 & 15;
 #pragma unroll
         for (int k = 0; k < 9; ++k) {
-            float sum = red[k * 256 + t];
+            if (Cfg::SPLIT && (k < Cfg::TAP_SPLIT) != (tap_half == 0)) continue;
+            float sum = red[k * 256 + tq];
 #pragma unroll
-            for (int w = 1; w < 4; ++w) sum += red[(w * 9 + k) * 256 + t];
+            for (int w = 1; w < 4; ++w) sum += red[(w * 9 + k) * 256 + tq];
             tr[(oc * 16 + ic) * 9 + k] = sum;
         }
     }
@@ -270,8 +300,9 @@ __device__ __forceinline__ void wgrad3x3_body(const WgradArgs &a, const u32 bid,
     const size_t count = size_t(a.OC) * a.IC * 9;
     float *out = a.out + size_t(z) * count * (a.accumulate ? 0 : 1);
 #pragma unroll
-    for (int i = 0; i < 9; ++i) {
-        const u32 e = t + i * kThreads;       // e = oc*144 + ic*9 + tap
+    for (int i = 0; i < (2304 + NT - 1) / NT; ++i) {
+        const u32 e = t + i * NT;             // e = oc*144 + ic*9 + tap
+        if (2304 % NT != 0 && e >= 2304u) continue;
         const u32 oc = e / 144, rest = e % 144;  // rest = ic*9 + tap: contiguous in dW for one oc
         if (ob * 16 + oc >= a.OC || ib * 16 + rest / 9 >= a.IC) continue;
         float *dst = out + (size_t(ob * 16 + oc) * a.IC + ib * 16) * 9 + rest;
@@ -280,7 +311,7 @@ __device__ __forceinline__ void wgrad3x3_body(const WgradArgs &a, const u32 bid,
 }
 
 template <class Cfg>
-__global__ void __launch_bounds__(kThreads, Cfg::OCC) wgrad3x3_kernel(WgradArgs a) {
+__global__ void __launch_bounds__(Cfg::NT, Cfg::OCC) wgrad3x3_kernel(WgradArgs a) {
     __shared__ __attribute__((aligned(16))) float smem[Cfg::SMEM];
     wgrad3x3_body<Cfg>(a, blockIdx.x, smem);
 }
@@ -336,7 +367,7 @@ inline int launch_wgrad_direct(const float *dY, const float *X, float *dW, float
     WgradArgs a;
     const uint64_t wgs = wgrad_direct_args<Cfg>(a, dY, X, dW, ws, p, IC, OC, H);
     if (wgs > 0x7fffffffull) return fail(CRB_EINVAL_SHAPE, "%s: launch grid too large", what);
-    hipLaunchKernelGGL((wgrad3x3_kernel<Cfg>), dim3(u32(wgs)), dim3(kThreads), 0, s, a);
+    hipLaunchKernelGGL((wgrad3x3_kernel<Cfg>), dim3(u32(wgs)), dim3(Cfg::NT), 0, s, a);
     if (int st = check_launch(what)) return st;
     if (p.splits > 1 && dW) {  // dW == nullptr: the caller sums the slices later
         return launch_splitk_reduce(ws, dW, OC * IC * 9, p.splits, ReduceEpi{nullptr, 1, 1, EPI_ACCUM}, s, what);

@@ -260,26 +260,39 @@ static bool wgrad_cfg(const crb_conv_geom *g, bool run, const float *dY, const f
     return true;
 }
 
-// Configurations <W (dY width), TR, TI, OCC, S>.
+// Configurations <W (dY width), TR, TI, OCC, S, WAVES>.
+// One workgroup per CU (the usual plan: pairs x splits = 256) runs the eight-wave form, so that every SIMD holds two waves;
+// wide layers, whose plan puts two four-wave workgroups on a CU anyway, keep the four-wave form (measured: 1-5 % faster
+// there). Both forms produce identical bits, and the plan (splits, workspace) does not depend on the form.
+template <int W, int TR, int TI, int OCC, int S>
+static bool wgrad_cfg2(const crb_conv_geom *g, bool run, const float *dY, const float *X, float *dW, float *ws, hipStream_t s,
+                       WgradDirectPlan &plan, int &status) {
+    typedef WgradCfg<W, TR, TI, OCC, S, 4> Four;
+    typedef WgradCfg<W, TR, TI, 1, S, 8> Eight;
+    if (!wgrad_direct_fits<Four>(g->N, g->IC, g->OC, g->OH, g->OW)) return false;
+    const WgradDirectPlan p = wgrad_direct_plan<Four>(g->N, g->IC, g->OC, g->OH, kWgradTargetWgs);
+    if (uint64_t(p.pairs) * p.splits > kWgradTargetWgs) return wgrad_cfg<Four>(g, run, dY, X, dW, ws, s, plan, status);
+    return wgrad_cfg<Eight>(g, run, dY, X, dW, ws, s, plan, status);
+}
 static bool wgrad_direct(const crb_conv_geom *g, bool run, const float *dY, const float *X, float *dW, float *ws,
                          hipStream_t s, WgradDirectPlan &plan, int &status) {
     if (direct_shape(g, 1)) {
-        if (g->OW == 32) return wgrad_cfg<WgradCfg<32, 8, 1, 2, 1>>(g, run, dY, X, dW, ws, s, plan, status);
+        if (g->OW == 32) return wgrad_cfg2<32, 8, 1, 2, 1>(g, run, dY, X, dW, ws, s, plan, status);
         if (g->OW == 16)
-            return wgrad_cfg<WgradCfg<16, 16, 1, 2, 1>>(g, run, dY, X, dW, ws, s, plan, status) ||
-                   wgrad_cfg<WgradCfg<16, 8, 1, 2, 1>>(g, run, dY, X, dW, ws, s, plan, status);
+            return wgrad_cfg2<16, 16, 1, 2, 1>(g, run, dY, X, dW, ws, s, plan, status) ||
+                   wgrad_cfg2<16, 8, 1, 2, 1>(g, run, dY, X, dW, ws, s, plan, status);
         if (g->OW == 8)
-            return wgrad_cfg<WgradCfg<8, 8, 4, 2, 1>>(g, run, dY, X, dW, ws, s, plan, status) ||
-                   wgrad_cfg<WgradCfg<8, 8, 2, 2, 1>>(g, run, dY, X, dW, ws, s, plan, status);
+            return wgrad_cfg2<8, 8, 4, 2, 1>(g, run, dY, X, dW, ws, s, plan, status) ||
+                   wgrad_cfg2<8, 8, 2, 2, 1>(g, run, dY, X, dW, ws, s, plan, status);
         if (g->OW == 4)  // 4x4 images: 8 (or 4) whole images per tile
-            return wgrad_cfg<WgradCfg<4, 4, 8, 2, 1>>(g, run, dY, X, dW, ws, s, plan, status) ||
-                   wgrad_cfg<WgradCfg<4, 4, 4, 2, 1>>(g, run, dY, X, dW, ws, s, plan, status);
+            return wgrad_cfg2<4, 4, 8, 2, 1>(g, run, dY, X, dW, ws, s, plan, status) ||
+                   wgrad_cfg2<4, 4, 4, 2, 1>(g, run, dY, X, dW, ws, s, plan, status);
     } else if (direct_shape(g, 2)) {
-        if (g->OW == 32) return wgrad_cfg<WgradCfg<32, 4, 1, 1, 2>>(g, run, dY, X, dW, ws, s, plan, status);
-        if (g->OW == 16) return wgrad_cfg<WgradCfg<16, 8, 1, 1, 2>>(g, run, dY, X, dW, ws, s, plan, status);
+        if (g->OW == 32) return wgrad_cfg2<32, 4, 1, 1, 2>(g, run, dY, X, dW, ws, s, plan, status);
+        if (g->OW == 16) return wgrad_cfg2<16, 8, 1, 1, 2>(g, run, dY, X, dW, ws, s, plan, status);
         if (g->OW == 8)
-            return wgrad_cfg<WgradCfg<8, 8, 2, 1, 2>>(g, run, dY, X, dW, ws, s, plan, status) ||
-                   wgrad_cfg<WgradCfg<8, 4, 2, 1, 2>>(g, run, dY, X, dW, ws, s, plan, status);
+            return wgrad_cfg2<8, 8, 2, 1, 2>(g, run, dY, X, dW, ws, s, plan, status) ||
+                   wgrad_cfg2<8, 4, 2, 1, 2>(g, run, dY, X, dW, ws, s, plan, status);
     }
     return false;
 }

@@ -389,30 +389,50 @@ __device__ __forceinline__ void reduce_vec_block(const float *__restrict__ parti
     constexpr u32 ZL = 256 / OL, OUTS = 4 * OL, RS = OUTS + 4;
     const u32 o = threadIdx.x % OL, g = threadIdx.x / OL;
     const u32 i = block * OUTS + 4 * o;
+    // the result's previous value (accumulating forms) is requested before the slices, not after their sum, so that it
+    // does not cost a memory round trip of its own at the end
+    const u32 j = block * OUTS + threadIdx.x;
+    float prev = 0.f;
+    if ((e.flags & EPI_ACCUM) && threadIdx.x < OUTS && j < count) prev = C[j];
     float4 s0 = make_float4(0.f, 0.f, 0.f, 0.f), s1 = s0;
+    auto add = [](float4 &s, const float4 &v) { s.x += v.x, s.y += v.y, s.z += v.z, s.w += v.w; };
     if (i < count) {
         const float *p = partial + i;
         u32 zz = g;
-        for (; zz + ZL < splits; zz += 2 * ZL) {
+        // A lane's slices are requested eight, then four, then two at a time (all loads of a batch in flight together);
+        // the two running sums take them alternately in slice order whatever the batch size, so the association — and
+        // with it every bit of the result — depends on (splits, OL) alone.
+        for (; zz + 7 * ZL < splits; zz += 8 * ZL) {
+            float4 v[8];
+#pragma unroll
+            for (u32 q = 0; q < 8; ++q) v[q] = *reinterpret_cast<const float4 *>(p + size_t(zz + q * ZL) * count);
+#pragma unroll
+            for (u32 q = 0; q < 8; q += 2) add(s0, v[q]), add(s1, v[q + 1]);
+        }
+        if (zz + 3 * ZL < splits) {
+            float4 v[4];
+#pragma unroll
+            for (u32 q = 0; q < 4; ++q) v[q] = *reinterpret_cast<const float4 *>(p + size_t(zz + q * ZL) * count);
+#pragma unroll
+            for (u32 q = 0; q < 4; q += 2) add(s0, v[q]), add(s1, v[q + 1]);
+            zz += 4 * ZL;
+        }
+        if (zz + ZL < splits) {
             const float4 a = *reinterpret_cast<const float4 *>(p + size_t(zz) * count);
             const float4 b = *reinterpret_cast<const float4 *>(p + size_t(zz + ZL) * count);
-            s0.x += a.x, s0.y += a.y, s0.z += a.z, s0.w += a.w;
-            s1.x += b.x, s1.y += b.y, s1.z += b.z, s1.w += b.w;
+            add(s0, a), add(s1, b);
+            zz += 2 * ZL;
         }
-        if (zz < splits) {
-            const float4 a = *reinterpret_cast<const float4 *>(p + size_t(zz) * count);
-            s0.x += a.x, s0.y += a.y, s0.z += a.z, s0.w += a.w;
-        }
+        if (zz < splits) add(s0, *reinterpret_cast<const float4 *>(p + size_t(zz) * count));
     }
     *reinterpret_cast<float4 *>(&red[g * RS + 4 * o]) = make_float4(s0.x + s1.x, s0.y + s1.y, s0.z + s1.z, s0.w + s1.w);
     __syncthreads();
-    const u32 j = block * OUTS + threadIdx.x;
     if (threadIdx.x < OUTS && j < count) {
         float r = red[threadIdx.x];
 #pragma unroll
         for (u32 k = 1; k < ZL; ++k) r += red[k * RS + threadIdx.x];
         if (e.bias) r += e.bias[bdiv.div(j) % e.bias_mod];
-        if (e.flags & EPI_ACCUM) r += C[j];
+        if (e.flags & EPI_ACCUM) r += prev;
         if (e.flags & EPI_RELU) r = r > 0.f ? r : 0.f;
         C[j] = r;
     }
