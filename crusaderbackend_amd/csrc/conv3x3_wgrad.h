@@ -283,6 +283,8 @@ __device__ __forceinline__ void wgrad3x3_body(const WgradArgs &a, const u32 bid,
         if (!Cfg::SPLIT || (k < Cfg::TAP_SPLIT) == (tap_half == 0))
             *reinterpret_cast<v4f *>(red + ((wave * 9 + k) * 64 + lane) * 4) = acc[k];
     __syncthreads();
+    const size_t count = size_t(a.OC) * a.IC * 9;
+    float *out = a.out + size_t(z) * count * (a.accumulate ? 0 : 1);
     {
         const u32 tq = t & 255;
         const u32 l2 = tq >> 2, r = tq & 3;
@@ -297,8 +299,17 @@ __device__ __forceinline__ void wgrad3x3_body(const WgradArgs &a, const u32 bid,
         }
     }
     __syncthreads();
-    const size_t count = size_t(a.OC) * a.IC * 9;
-    float *out = a.out + size_t(z) * count * (a.accumulate ? 0 : 1);
+    // whole channel blocks: an output channel's 144 floats are contiguous and 16-byte aligned in dW, so lanes store quads
+    if (!a.accumulate && a.OC % 16 == 0 && a.IC % 16 == 0 && (reinterpret_cast<uintptr_t>(out) & 15u) == 0) {
+#pragma unroll
+        for (int i = 0; i < (576 + NT - 1) / NT; ++i) {
+            const u32 q = t + i * NT;  // quad q = oc*36 + j
+            if (576 % NT != 0 && q >= 576u) continue;
+            const u32 oc = q / 36, j = q % 36;
+            *reinterpret_cast<v4f *>(out + (size_t(ob * 16 + oc) * a.IC + ib * 16) * 9 + 4 * j) = *reinterpret_cast<const v4f *>(tr + 4 * q);
+        }
+        return;
+    }
 #pragma unroll
     for (int i = 0; i < (2304 + NT - 1) / NT; ++i) {
         const u32 e = t + i * NT;             // e = oc*144 + ic*9 + tap
