@@ -113,6 +113,17 @@ static WgradPlan wgrad_plan(const crb_conv_geom *g) {
 // Configurations <W, ROWS, CI, OCT, PBW, OBW, DGRAD, OCC, NBUF, S>, picked by grid width and channel counts.
 // Tried in order; the first whose constraints hold is used, otherwise the implicit-GEMM engine runs.
 // (gH, gW) is the pixel grid: the output image, or dY for the stride-2 data gradient; in_H the rows of the staged tensor.
+// Shape rules shared by try_direct and bwd_fused (which must chunk the contraction exactly as the separate data-gradient
+// call does, so that both produce the same bits). C_IN / C_OUT: channels the pass reads / writes; gH: rows of its pixel grid.
+static bool one_chunk_w16(u32 N, u32 C_IN, u32 C_OUT, u32 gH) {  // stride 1, width 16: all 17..32 input channels LDS-resident
+    return C_IN > 16 && C_IN <= 32 && N * (gH / 8) * ceil_div(C_OUT, 16u) >= 512;
+}
+static bool one_chunk_w8(u32 N, u32 C_IN, u32 C_OUT, u32 gH) {  // stride 1, width 8: all 33..64 input channels LDS-resident
+    return C_IN > 32 && C_IN <= 64 && C_OUT <= 64 && N * (gH / 8) * ceil_div(C_OUT, 16u) >= 512;
+}
+static bool s2_dgrad_w16_c16(u32 N, u32 C_IN, u32 C_OUT, u32 gH) { return C_IN > 8 && C_OUT <= 16 && N * (gH / 4) >= 512; }
+static bool s2_dgrad_w8_c16(u32 N, u32 C_IN, u32 C_OUT) { return C_IN > 8 && N * ceil_div(C_OUT, 16u) >= 256; }
+
 template <bool DG, int S>
 static int try_direct(const float *Wt, const float *X, float *Y, const float *bias, u32 N, u32 C_IN, u32 C_OUT, u32 gH,
                       u32 gW, u32 in_H, u32 relu, hipStream_t s, const char *what, bool &done, bool probe = false) {
@@ -136,12 +147,19 @@ static int try_direct(const float *Wt, const float *X, float *Y, const float *bi
             CRB_TRY(32, 8, 8, 16, 4, 1, DG, 2, 2, 1)
             CRB_TRY(32, 4, 8, 16, 2, 1, DG, 2, 2, 1)
         } else if (gW == 16) {
+            // 17..32 input channels and enough tiles for two workgroups per CU: the whole contraction as one LDS-resident
+            // chunk, stores in two pixel groups (32 -> 32, batch 128: 9.2 -> 8.3 us forward, 9.0 -> 8.3 us data gradient)
+            if (one_chunk_w16(N, C_IN, C_OUT, gH)) { CRB_TRY(16, 8, 32, 16, 2, 1, DG, 2, 1, 1, 3, 2) }
             if (C_OUT > 64) { CRB_TRY(16, 8, 8, 64, 2, 4, DG, 2, 2, 1) }
             if (C_OUT > 16 && C_IN > 8) { CRB_TRY(16, 4, 16, 32, 1, 2, DG, 2, 2, 1) }
             if (C_OUT > 16) { CRB_TRY(16, 4, 8, 32, 1, 2, DG, 2, 2, 1) }
             CRB_TRY(16, 8, 8, 16, 2, 1, DG, 2, 2, 1)
             CRB_TRY(16, 4, 8, 16, 1, 1, DG, 2, 2, 1)
         } else if (gW == 8) {
+            // 33..64 input channels, at most 64 output channels: one LDS-resident chunk (64 -> 64, batch 128: 9.0 -> 8.65 us).
+            // Forward only: the data gradient keeps the chunking of the one-launch backward kernel, which has no room in
+            // LDS for a resident 64-channel chunk next to the weight-gradient workgroup and is slower with 16-wide tiles.
+            if (!DG && one_chunk_w8(N, C_IN, C_OUT, gH)) { CRB_TRY(8, 8, 64, 16, 1, 1, DG, 2, 1, 1) }
             // 64 output channels with chunks of 8: chunks of 16 would need more LDS than lets two workgroups share a CU, and a
             // SIMD with a single wave issues its MFMAs a third slower
             if (C_OUT > 128 && C_IN > 8) { CRB_TRY(8, 8, 8, 64, 1, 4, DG, 2, 2, 1) }
@@ -163,10 +181,16 @@ static int try_direct(const float *Wt, const float *X, float *Y, const float *bi
             CRB_TRY(32, 8, 8, 16, 4, 1, DG, 2, 2, 2)
             CRB_TRY(32, 4, 8, 16, 2, 1, DG, 2, 2, 2)
         } else if (gW == 16) {
+            // measured on the residual-network transitions at batch 128 (16 -> 32: forward 7.2 -> 6.2 us, data gradient 8.5 -> 7.2 us)
+            if (!DG && C_IN > 8 && C_IN <= 16 && C_OUT > 16 && N * (gH / 4) >= 512) { CRB_TRY(16, 4, 16, 32, 1, 2, DG, 2, 1, 2) }
+            if (DG && s2_dgrad_w16_c16(N, C_IN, C_OUT, gH)) { CRB_TRY(16, 4, 16, 16, 1, 1, DG, 2, 2, 2) }
             if (C_OUT > 16) { CRB_TRY(16, 8, 8, 32, 2, 2, DG, 2, 2, 2) }
             CRB_TRY(16, 8, 8, 16, 2, 1, DG, 2, 2, 2)
             CRB_TRY(16, 4, 8, 16, 1, 1, DG, 2, 2, 2)
         } else if (gW == 8) {
+            // (32 -> 64: forward 7.2 -> 6.65 us, data gradient 10.9 -> 7.1 us: 16-channel tiles give every CU a workgroup)
+            if (!DG && C_IN > 8 && C_OUT > 16 && N * (gH / 4) >= 256) { CRB_TRY(8, 4, 16, 32, 1, 1, DG, 2, 2, 2) }
+            if (DG && s2_dgrad_w8_c16(N, C_IN, C_OUT)) { CRB_TRY(8, 8, 16, 16, 1, 1, DG, 2, 2, 2) }
             if (C_OUT > 16) { CRB_TRY(8, 8, 8, 32, 1, 2, DG, 2, 2, 2) }
             CRB_TRY(8, 8, 8, 16, 1, 1, DG, 2, 2, 2)
             CRB_TRY(8, 4, 8, 32, 1, 1, DG, 2, 2, 2)
@@ -357,10 +381,13 @@ static bool bwd_fused(const crb_conv_geom *g, bool run, const float *Wt, const f
                       float *ws, hipStream_t s, WgradDirectPlan &plan, int &status) {
 #define CRB_PAIR(...) bwd_pair<__VA_ARGS__>(g, run, Wt, dY, X, dX, dW, ws, s, plan, status)
     typedef DirectCfg<32, 8, 16, 16, 4, 1, true, 2, 1, 1, 3, 4> D32a;
-    typedef DirectCfg<16, 8, 16, 32, 2, 2, true, 2, 2, 1> D16a;
+    typedef DirectCfg<16, 8, 16, 32, 2, 2, true, 2, 2, 1> D16a;             // chunks of 16 channels
+    typedef DirectCfg<16, 8, 32, 32, 2, 2, true, 2, 1, 1, 3, 2> D16r;       // one resident chunk of up to 32
     typedef DirectCfg<8, 8, 16, 32, 1, 2, true, 2, 2, 1> D8a;
-    typedef DirectCfg<16, 8, 8, 16, 2, 1, true, 2, 2, 2> D16s2;
+    typedef DirectCfg<16, 8, 8, 16, 2, 1, true, 2, 2, 2> D16s2;             // chunks of 8
+    typedef DirectCfg<16, 8, 16, 16, 2, 1, true, 2, 2, 2> D16s2c;           // chunks of 16
     typedef DirectCfg<8, 8, 8, 32, 1, 2, true, 2, 2, 2> D8s2;
+    typedef DirectCfg<8, 8, 16, 32, 1, 2, true, 2, 2, 2> D8s2c;
     typedef WgradCfg<32, 8, 1, 2, 1> W32a;
     typedef WgradCfg<16, 16, 1, 2, 1> W16a;
     typedef WgradCfg<8, 8, 4, 2, 1> W8a;
@@ -369,11 +396,13 @@ static bool bwd_fused(const crb_conv_geom *g, bool run, const float *Wt, const f
     const u32 ci = g->OC, co = g->IC;  // channels the data gradient reads / writes
     if (direct_shape(g, 1)) {
         if (g->OW == 32 && ci <= 16 && ci > 8 && co <= 16) return CRB_PAIR(D32a, W32a);
-        if (g->OW == 16 && co > 16 && co <= 64 && ci > 8) return CRB_PAIR(D16a, W16a);
+        if (g->OW == 16 && co > 16 && co <= 64 && ci > 8)
+            return one_chunk_w16(g->N, ci, co, g->OH) ? CRB_PAIR(D16r, W16a) : CRB_PAIR(D16a, W16a);
         if (g->OW == 8 && co <= 64 && ci > 8) return CRB_PAIR(D8a, W8a);
     } else if (direct_shape(g, 2)) {
-        if (g->OW == 16 && co <= 16) return CRB_PAIR(D16s2, W16s2);
-        if (g->OW == 8 && co > 16) return CRB_PAIR(D8s2, W8s2, true);  // here the data gradient is the longer half
+        if (g->OW == 16 && co <= 16) return s2_dgrad_w16_c16(g->N, ci, co, g->OH) ? CRB_PAIR(D16s2c, W16s2) : CRB_PAIR(D16s2, W16s2);
+        if (g->OW == 8 && co > 16)  // here the data gradient is the longer half
+            return s2_dgrad_w8_c16(g->N, ci, co) ? CRB_PAIR(D8s2c, W8s2, true) : CRB_PAIR(D8s2, W8s2, true);
     }
 #undef CRB_PAIR
     return false;
