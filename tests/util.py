@@ -29,6 +29,10 @@ def tolerance(ref, K):
     return 1e-5 * math.sqrt(max(K, 1)) * np.maximum(np.abs(ref), rms)
 
 
+# worst err / tol seen per checked quantity in this process (written out by conftest at the end of a GPU session)
+MARGINS = {}
+
+
 def assert_close(got, ref, K, what=""):
     got = np.asarray(got, dtype=np.float64)
     ref64 = np.asarray(ref, dtype=np.float64)
@@ -36,6 +40,15 @@ def assert_close(got, ref, K, what=""):
     assert np.all(np.isfinite(got)), f"{what}: non-finite values"
     err = np.abs(got - ref64)
     tol = tolerance(ref64, K)
+    if err.size:
+        with np.errstate(divide="ignore", invalid="ignore"):
+            ratio = float(np.nanmax(np.where(tol > 0, err / tol, 0.0)))
+            # the same error against the plain relative bound 1e-5*sqrt(K)*|ref| (no RMS floor), on elements that are not tiny
+            big = np.abs(ref64) >= 1e-3 * (np.sqrt(np.mean(ref64 * ref64)) + 1e-300)
+            rel = float(np.max(err[big] / (1e-5 * math.sqrt(max(K, 1)) * np.abs(ref64[big])))) if big.any() else 0.0
+        old = MARGINS.get(what)
+        if old is None or ratio > old["err_over_tol"]:
+            MARGINS[what] = {"err_over_tol": ratio, "err_over_plain_relative_bound": rel, "K": int(K), "elements": int(err.size)}
     bad = err > tol
     if bad.any():
         idx = np.unravel_index(np.argmax(err - tol), err.shape)
