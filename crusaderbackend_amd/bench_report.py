@@ -95,6 +95,50 @@ def run(torch, capi, dev, event_time_ms, Layer):
         dn.append((f"3x3_48-12@{H}", 48, H, 12, 3, 1, 1))
     conv_entries("densenet", dn, 64, True)
 
+    # config 4 as a whole: the convolution work of one DenseNet-BC-100 training step at batch 64 — 48 bottleneck pairs
+    # (seann/operands/prefabs/DenseBlock.cuh:42-61: 1x1 IC -> 48 then 3x3 48 -> 12, IC = 24 + 12 i @32x32, 108 + 12 i @16x16,
+    # 150 + 12 i @8x8, i = 0..15; archive/Densenet100:2-34), every layer on tensors of its own, forward in network order,
+    # then conv / convDerive / convError as separate calls per layer in reverse order.
+    pairs = []
+    for (H, base) in ((32, 24), (16, 108), (8, 150)):
+        for i in range(16):
+            IC = base + 12 * i
+            pairs.append((Layer(torch, capi, dev, f"1x1_{IC}-48@{H}", IC, H, 48, 1, 1, seed=300 + i, batch=64, F=1, pad=0, bias=True),
+                          Layer(torch, capi, dev, f"3x3_48-12@{H}", 48, H, 12, 1, 1, seed=400 + i, batch=64, F=3, pad=1, bias=True)))
+
+    def dn_step(kinds):
+        def run():
+            for pw, c3 in pairs:
+                if "1x1" in kinds:
+                    pw.fwd()
+                if "3x3" in kinds:
+                    c3.fwd()
+            for pw, c3 in reversed(pairs):
+                if "3x3" in kinds:
+                    c3.dgrad(), c3.wgrad()
+                if "1x1" in kinds:
+                    pw.dgrad(), pw.wgrad()
+        return run
+
+    def work(idx):
+        return (sum(3 * p[idx].flops for p in pairs), sum(p[idx].bytes["fwd"] + p[idx].bytes["dgrad"] + p[idx].bytes["wgrad"] for p in pairs))
+
+    all_ms = event_time_ms(torch, dn_step(("1x1", "3x3")), reps=5, warm=2)
+    pw_ms = event_time_ms(torch, dn_step(("1x1",)), reps=5, warm=2)
+    c3_ms = event_time_ms(torch, dn_step(("3x3",)), reps=5, warm=2)
+    (pw_fl, pw_by), (c3_fl, c3_by) = work(0), work(1)
+    out["densenet_full_step"] = {
+        "workload": "DenseNet-BC-100 (k = 12) convolution layers, batch 64: 48 x (1x1 IC->48, 3x3 48->12), fwd + dgrad + wgrad as separate calls",
+        "us": round(all_ms * 1e3, 1), "gflop": round((pw_fl + c3_fl) / 1e9, 2), "mbytes": round((pw_by + c3_by) / 1e6, 1),
+        "tflops": round((pw_fl + c3_fl) / all_ms / 1e9, 2), "images_per_s": round(64 / all_ms * 1e3, 1),
+        "pointwise_us": round(pw_ms * 1e3, 1), "pointwise_mbytes": round(pw_by / 1e6, 1), "pointwise_gbs": round(pw_by / pw_ms / 1e6, 1),
+        "pointwise_frac_hbm": round(pw_by / pw_ms / 1e6 / PEAK_GBS, 4), "pointwise_tflops": round(pw_fl / pw_ms / 1e9, 2),
+        "conv3x3_us": round(c3_ms * 1e3, 1), "conv3x3_gflop": round(c3_fl / 1e9, 2), "conv3x3_tflops": round(c3_fl / c3_ms / 1e9, 2),
+        "conv3x3_frac_mfma": round(c3_fl / c3_ms / 1e9 / PEAK_TF, 4),
+    }
+    del pairs
+    torch.cuda.empty_cache()
+
     # config 5: dense sweep (batch 256, 4096 <-> 4096) through linear* and the raw GEMM forms, plus tall-skinny
     b, n = 256, 4096
     X, W, bias = rnd(b, n), rnd(n, n), rnd(n)
@@ -172,7 +216,7 @@ def run(torch, capi, dev, event_time_ms, Layer):
                 "tflops": round(sum(e["gflop"] for e in es) / max(sum(e["us"] for e in es), 1e-9) * 1e3, 2)}
 
     out["summary"] = {"vgg16_conv_fc_train_step": total("vgg16"), "vgg16_fwd": total("vgg16", ".fwd"),
-                      "vgg16_full_train_step": out["vgg16_full_step"],
+                      "vgg16_full_train_step": out["vgg16_full_step"], "densenet_bc100_conv_step": out["densenet_full_step"],
                       "peak_fp32_mfma_tflops": PEAK_TF, "peak_hbm_gbs": PEAK_GBS, "ridge_flop_per_byte": round(RIDGE, 2)}
     return out
 
