@@ -1,5 +1,6 @@
 // C-ABI entry points of the GEMM and dense-layer families (fp32, row-major) on the MFMA engine.
 #include "gemm_internal.h"
+#include "gemm_tiny.h"
 #include "operands.h"
 
 namespace crb {
@@ -93,6 +94,7 @@ static int run_tiles(const AOp &a, const BOp &b, const RowMajorEpi &e, u32 M, u3
 
 // Scratch bytes run_tiles asks for on a dense M x N result with contraction length K (0: the contraction is not cut).
 size_t gemm_scratch_bytes(u32 M, u32 N, u32 K, u32 zdim) {
+    if (tiny_gemm_fits(M, N, K, zdim)) return 0;  // one launch, no partial results
     const GemmChoice c = choose_tiles(M, N, K, zdim, true);
     SplitPlan sp;
     switch (c.tile) {
@@ -144,6 +146,8 @@ __global__ void __launch_bounds__(256) colsum_accum_kernel(const float *__restri
 
 static int gemm_nn(const float *A, const float *B, float *C, u32 M, u32 N, u32 K, u32 batch, const float *col_bias,
                    u32 flags, hipStream_t s, const char *what, const float *row_bias = nullptr) {
+    if (tiny_gemm_fits(M, N, K, batch))  // A (M x K) row-major, B (K x N) row-major
+        return launch_tiny_gemm(TinyGemmArgs{A, B, C, col_bias, row_bias, M, N, K, K, 1, N, 1, N, flags}, K, 0, 0, s, what);
     RowMajorEpi e{C, col_bias, N, M * N, flags};
     e.row_bias = row_bias;
     if (K % 4 == 0 && N % 4 == 0 && aligned16(A) && aligned16(B)) {
@@ -158,6 +162,8 @@ static int gemm_nn(const float *A, const float *B, float *C, u32 M, u32 N, u32 K
 
 static int gemm_tn(const float *A, const float *B, float *C, u32 M, u32 N, u32 K, u32 batch, u32 flags,
                    hipStream_t s, const char *what) {
+    if (tiny_gemm_fits(M, N, K, batch))  // A stored K x M, B (K x N) row-major
+        return launch_tiny_gemm(TinyGemmArgs{A, B, C, nullptr, nullptr, M, N, K, 1, M, N, 1, N, flags}, K, 0, 0, s, what);
     RowMajorEpi e{C, nullptr, N, M * N, flags};
     if (M % 4 == 0 && N % 4 == 0 && aligned16(A) && aligned16(B)) {
         MatR<true> a{A, M, M, 0};
@@ -171,6 +177,8 @@ static int gemm_tn(const float *A, const float *B, float *C, u32 M, u32 N, u32 K
 
 static int gemm_nt(const float *A, const float *B, float *C, u32 M, u32 N, u32 K, const float *col_bias, u32 flags,
                    hipStream_t s, const char *what) {
+    if (tiny_gemm_fits(M, N, K, 1))  // A (M x K) row-major, B stored N x K
+        return launch_tiny_gemm(TinyGemmArgs{A, B, C, col_bias, nullptr, M, N, K, K, 1, 1, K, N, flags}, K, 0, 0, s, what);
     RowMajorEpi e{C, col_bias, N, 0, flags};
     if (K % 4 == 0 && aligned16(A) && aligned16(B)) {
         MatK<true> a{A, M, K, 0};
@@ -288,6 +296,8 @@ int crb_sgemm_nta(const float *A, const float *B, float *C, uint32_t M, uint32_t
     const u32 KK = K * batch;
     RowMajorEpi e{C, nullptr, N, 0, EPI_ACCUM};
     hipStream_t s = hipStream_t(stream);
+    if (tiny_gemm_fits(M, N, KK, 1))  // the batch concatenated along the contraction
+        return launch_tiny_gemm(TinyGemmArgs{A, B, C, nullptr, nullptr, M, N, KK, K, 1, 1, K, N, EPI_ACCUM}, K, M * K, N * K, s, "crb_sgemm_nta");
     if (K % 4 == 0 && aligned16(A) && aligned16(B)) {
         MatKCat<true> a{A, M, K, M * K, FastDiv(K)};
         MatKCat<true> b{B, N, K, N * K, FastDiv(K)};

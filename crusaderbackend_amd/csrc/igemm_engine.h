@@ -321,18 +321,33 @@ __global__ void __launch_bounds__(kThreads, Cfg::OCC) igemm_kernel(AOp a, BOp b,
 
     // epilogue: accumulator register r of lane l is D[8*(r/4) + 4*(l/32) + r%4][l%32] of its block
     const int j = lane & 31, h = lane >> 5;
-#pragma unroll
-    for (int ni = 0; ni < TN; ++ni) {
-        const u32 col = col0 + wave_n * Cfg::WTN + (BOp::kKFast ? ni * 32 + j : j * TN + ni);
-        const typename Epi::ColS cs = epi.prep_col(col, d.N);
+    if constexpr (!BOp::kKFast && TN == 2 && Epi::kPairStore) {
+        // row-fast B: a lane's two blocks are neighbouring columns, stored (and, accumulating, loaded) as one 8-byte access,
+        // so that a store instruction writes whole 256-byte runs instead of every other float of them
+        const u32 col = col0 + wave_n * Cfg::WTN + j * 2;
+        const typename Epi::ColS c0 = epi.prep_col(col, d.N), c1 = epi.prep_col(col + 1, d.N);
 #pragma unroll
         for (int mi = 0; mi < TM; ++mi)
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
                 const int id = 8 * (r / 4) + 4 * h + (r % 4);
                 const u32 row = row0 + wave_m * Cfg::WTM + (AOp::kKFast ? mi * 32 + id : id * TM + mi);
-                if (row < d.M) epi.store(row, cs, acc[mi][ni][r]);
+                if (row < d.M && c0.ok) epi.store2(row, c0, c1, acc[mi][0][r], acc[mi][1][r]);
             }
+    } else {
+#pragma unroll
+        for (int ni = 0; ni < TN; ++ni) {
+            const u32 col = col0 + wave_n * Cfg::WTN + (BOp::kKFast ? ni * 32 + j : j * TN + ni);
+            const typename Epi::ColS cs = epi.prep_col(col, d.N);
+#pragma unroll
+            for (int mi = 0; mi < TM; ++mi)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int id = 8 * (r / 4) + 4 * h + (r % 4);
+                    const u32 row = row0 + wave_m * Cfg::WTM + (AOp::kKFast ? mi * 32 + id : id * TM + mi);
+                    if (row < d.M) epi.store(row, cs, acc[mi][ni][r]);
+                }
+        }
     }
 }
 

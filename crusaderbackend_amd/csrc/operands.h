@@ -286,6 +286,27 @@ struct RowMajorEpi {
         if (flags & EPI_RELU) v = v > 0.0f ? v : 0.0f;
         *p = v;
     }
+    // Two neighbouring columns of one row (c1.col == c0.col + 1) as one 8-byte access where the address allows it.
+    static constexpr bool kPairStore = true;
+    __device__ __forceinline__ void store2(u32 row, const ColS &c0, const ColS &c1, float v0, float v1) const {
+        float *p = C + size_t(row) * ld + c0.col;
+        if (!c1.ok || (reinterpret_cast<uintptr_t>(p) & 7u)) {
+            store(row, c0, v0);
+            store(row, c1, v1);
+            return;
+        }
+        v0 += c0.bias, v1 += c1.bias;
+        if (row_bias) {
+            const float rb = row_bias[row];
+            v0 += rb, v1 += rb;
+        }
+        if (flags & EPI_ACCUM) {
+            const v2f old = *reinterpret_cast<const v2f *>(p);
+            v0 += old.x, v1 += old.y;
+        }
+        if (flags & EPI_RELU) v0 = v0 > 0.0f ? v0 : 0.0f, v1 = v1 > 0.0f ? v1 : 0.0f;
+        *reinterpret_cast<v2f *>(p) = v2f{v0, v1};
+    }
 };
 
 // NCHW scatter: row = channel, col = n*HW + p  ->  T[(n*C + row)*HW + p], optional per-row bias, ReLU.
@@ -299,6 +320,8 @@ struct NchwEpi {
         u32 off;
         bool ok;
     };
+    static constexpr bool kPairStore = false;
+    __device__ __forceinline__ void store2(u32, const ColS &, const ColS &, float, float) const {}
     __device__ __forceinline__ void bind(u32 z) { T += size_t(z) * zstride; }
     __device__ __forceinline__ ColS prep_col(u32 col, u32 ncols) const {
         u32 n, p;

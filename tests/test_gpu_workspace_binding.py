@@ -136,7 +136,7 @@ def test_pointwise_wgrad_honours_the_workspace_argument(dev):
     import torch
     from crusaderbackend_amd import capi
 
-    N, IC, H, OC = 8, 24, 8, 48  # 1x1: the accumulate-NT GEMM form, one tile, long contraction: cut
+    N, IC, H, OC = 64, 24, 16, 48  # 1x1: the accumulate-NT GEMM form, one tile, contraction of 16384: cut
     g = capi.ConvGeom.make(N, IC, H, H, OC, 1, 1)
     need = capi.conv_wgrad_workspace_bytes(g)
     assert need > 0

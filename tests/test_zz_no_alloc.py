@@ -29,7 +29,7 @@ def _pair(dev, N, IC, H, OC, F, s, p, seed):
 # (N, IC, H, OC, F, stride, pad): direct 3x3 at three widths, stride 2, 1x1 (GEMM form, cut contraction), 1x1 stride-2
 # shortcut, 2x2 images, a 5x5 filter on the general path
 SHAPES = [(128, 16, 32, 16, 3, 1, 1), (64, 32, 16, 32, 3, 1, 1), (32, 64, 8, 64, 3, 1, 1), (32, 16, 32, 32, 3, 2, 1),
-          (8, 24, 8, 48, 1, 1, 0), (16, 16, 32, 32, 1, 2, 0), (64, 32, 2, 32, 3, 1, 1), (4, 12, 12, 20, 5, 1, 2)]
+          (64, 24, 16, 48, 1, 1, 0), (16, 16, 32, 32, 1, 2, 0), (64, 32, 2, 32, 3, 1, 1), (4, 12, 12, 20, 5, 1, 2)]
 
 
 def test_noalloc_two_calls_in_a_row_match_conv_wgrad(dev):
