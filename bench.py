@@ -55,6 +55,10 @@ def parse():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--report", type=str, default=None, help="also time every benchmark configuration and write a JSON report")
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
+    ap.add_argument("--traffic", action="store_true",
+                    help="only run every (layer, pass) call of the workload three times, each group behind a one-float fill "
+                         "launch as a separator, and print the order: under rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE the "
+                         "dispatch list then splits into calls (profiles/resnet56_conv_step_b128.md is built from it)")
     ap.add_argument("--calibrate", action="store_true",
                     help="only run a plain streaming kernel of known size (a += b on 64 Mi floats: reads 512 MiB, writes "
                          "256 MiB per launch) so hardware byte counters can be scaled against it, then exit")
@@ -145,23 +149,37 @@ class Layer:
         return out
 
 
-# HBM bytes one call moves (read + written, all kernels of the call), from the FETCH_SIZE and WRITE_SIZE hardware
-# counters of this workload under rocprofv3 --pmc, scaled by what the same counters read for a copy kernel of known
-# size (`--calibrate`): FETCH_SIZE x2.00, WRITE_SIZE x1.00. A property of the kernels' access pattern, not of a run;
-# the counter summaries are kept under profiles/.
-MEASURED_HBM_BYTES = {
-    "L1_16-16@32.fwd": 18.51e6, "L1_16-16@32.dgrad": 18.51e6, "L1_16-16@32.wgrad": 22.25e6,
-    "L2_32-32@16.fwd": 11.95e6, "L2_32-32@16.dgrad": 11.95e6, "L2_32-32@16.wgrad": 13.34e6,
-    "L3_64-64@8.fwd": 5.47e6, "L3_64-64@8.dgrad": 5.46e6, "L3_64-64@8.wgrad": 9.38e6,
-    "T1_16-32s2.fwd": 13.12e6, "T1_16-32s2.dgrad": 13.35e6, "T1_16-32s2.wgrad": 17.57e6,
-    "T2_32-64s2.fwd": 6.99e6, "T2_32-64s2.dgrad": 6.96e6, "T2_32-64s2.wgrad": 11.33e6,
-    # both gradients in one call: conv_bwd_kernel + the reduce kernel
-    "L1_16-16@32.bwd": 33.57e6, "L2_32-32@16.bwd": 17.97e6, "L3_64-64@8.bwd": 12.76e6,
-    "T1_16-32s2.bwd": 26.16e6, "T2_32-64s2.bwd": 16.17e6,
-    # conv_bwd_kernel alone (slices left for the end-of-step summation)
-    "L1_16-16@32.bwd_sliced": 31.13e6, "L2_32-32@16.bwd_sliced": 15.53e6, "L3_64-64@8.bwd_sliced": 10.09e6,
-    "T1_16-32s2.bwd_sliced": 23.72e6, "T2_32-64s2.bwd_sliced": 13.67e6,
-}
+# HBM bytes one call moves (read + written, all kernels of the call) come from the hardware counters FETCH_SIZE and
+# WRITE_SIZE of `bench.py --traffic` under rocprofv3 --pmc, scaled by what the same counters read for a copy kernel of
+# known size (`--calibrate`). They are a property of the kernels' access pattern, not of a run, so they are not measured
+# here: the table "HBM bytes per call" of the tracked profile summary below is the one source, together with the commit
+# and kernel names it was taken at.
+TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "resnet56_conv_step_b128.md")
+
+
+def measured_hbm_bytes():
+    """{call key: bytes per call} and the commit the counters were taken at, from the tracked profile summary ({} if absent)."""
+    table, commit = {}, None
+    try:
+        lines = open(TRAFFIC_PROFILE).read().splitlines()
+    except OSError:
+        return table, commit
+    on = False
+    for ln in lines:
+        if ln.startswith("Counters taken at commit"):
+            commit = ln.split("`")[1] if "`" in ln else None
+        if ln.startswith("## HBM bytes per call"):
+            on = True
+            continue
+        if on and ln.startswith("## "):
+            break
+        if on and ln.startswith("| ") and not ln.startswith("| call") and not ln.startswith("|---"):
+            cells = [c.strip() for c in ln.strip("|").split("|")]
+            try:
+                table[cells[0].strip("`")] = float(cells[-1]) * 1e6  # last column: total MB per call
+            except (ValueError, IndexError):
+                pass
+    return table, commit
 
 
 def device_clock_khz():
@@ -278,6 +296,23 @@ def main():
         return
 
     layers = [Layer(torch, capi, dev, n, IC, H, OC, s, m, seed=10 + i) for i, (n, IC, H, OC, s, m) in enumerate(RESNET56)]
+    if args.traffic:
+        sep = torch.zeros(1, device=dev)
+        order = []
+        for L in layers:
+            for pname, fn, _, _ in L.passes():
+                for _ in range(2):  # untimed: lets every kernel of the call load its code and grow nothing later
+                    fn()
+                torch.cuda.synchronize()
+                capi.tensor_fill(sep, 0.0, 1)  # opening separator: one fill launch of one float
+                for _ in range(3):
+                    fn()
+                capi.tensor_fill(sep, 0.0, 1)  # closing separator
+                torch.cuda.synchronize()
+                order.append(f"{L.name}.{pname}")
+        print(json.dumps({"traffic_order": order, "calls_per_group": 3,
+                          "separator": "a fill of 1 float before and after each group of three calls"}))
+        return
     step_flops = sum(3 * L.mult * L.flops for L in layers)
     slice_entries = [e for L in layers for e in L.slice_entries()]
     slice_table = capi.slice_sum_table(slice_entries) if slice_entries else None
@@ -370,10 +405,12 @@ def main():
     sum_ms = event_time_ms(torch, lambda: capi.sum_slices_multi(slice_table), reps=20) if slice_table is not None else 0.0
     dom = max(per, key=lambda k: per[k]["ms"] * per[k]["mult"])
     d = per[dom]
+    hbm_bytes, hbm_commit = measured_hbm_bytes()
     roofline = {
         "bound": "mfma", "kernel": dom, "achieved": d["tflops"], "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s",
-        "frac": d["tflops"] / PEAK_FP32_MFMA_TFLOPS, "traffic": MEASURED_HBM_BYTES.get(dom),
-        "traffic_unit": "bytes per launch (FETCH_SIZE x2.00 + WRITE_SIZE x1.00, rocprofv3 --pmc)",
+        "frac": d["tflops"] / PEAK_FP32_MFMA_TFLOPS, "traffic": hbm_bytes.get(dom),
+        "traffic_unit": "bytes per call (FETCH_SIZE and WRITE_SIZE of rocprofv3 --pmc, scaled against a copy kernel)",
+        "traffic_source": "profiles/resnet56_conv_step_b128.md, table 'HBM bytes per call', counters taken at commit %s (not measured by this run)" % hbm_commit,
         "algorithmic_bytes": d["bytes"],
         "flops_per_launch": d["flops"], "avg_launch_ms": d["ms"],
         "share_of_step": d["ms"] * d["mult"] / sum(v["ms"] * v["mult"] for v in per.values()),
