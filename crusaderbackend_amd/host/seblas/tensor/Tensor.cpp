@@ -138,6 +138,18 @@ Tensor *Tensor::attach(float *element, int deviceID) {
     return this;
 }
 
+static bool g_blocking = true;
+void setBlocking(bool blocking) { g_blocking = blocking; }
+bool isBlocking() { return g_blocking; }
+
+// Every device operator ends like the reference's (cudaDeviceSynchronize(); assertCuda(...), e.g. Tensor.cu:482-483): status
+// check, then — in blocking mode — a wait for the stream, so that an asynchronous fault surfaces at the operator that caused it.
+static void launched(int status, const char *file, int line) {
+    throwOnStatus(status, file, line);
+    if (isBlocking() && hipStreamSynchronize(nullptr) != hipSuccess) assertHip(file, line);
+    assertHip(file, line);
+}
+
 Tensor *Tensor::operator+(Tensor *other) {
     require(dims.size == other->dims.size, "Tensor::operator+: element counts differ");
     require(deviceId == other->deviceId, "Tensor::operator+: tensors live on different devices");
@@ -145,14 +157,9 @@ Tensor *Tensor::operator+(Tensor *other) {
         for (uint32 i = 0; i < dims.size; ++i) elements[i] += other->elements[i];
         return this;
     }
-    throwOnStatus(crb_tensor_add_inplace(elements, other->elements, dims.size, nullptr), __FILE__, __LINE__);
-    assertHip(__FILE__, __LINE__);
+    launched(crb_tensor_add_inplace(elements, other->elements, dims.size, nullptr), __FILE__, __LINE__);
     return this;
 }
-
-static bool g_blocking = true;
-void setBlocking(bool blocking) { g_blocking = blocking; }
-bool isBlocking() { return g_blocking; }
 
 Tensor *Tensor::addAndClear(Tensor *other) {
     require(dims.size == other->dims.size, "Tensor::addAndClear: element counts differ");
@@ -161,8 +168,7 @@ Tensor *Tensor::addAndClear(Tensor *other) {
         for (uint32 i = 0; i < dims.size; ++i) elements[i] += other->elements[i], other->elements[i] = 0.f;
         return this;
     }
-    throwOnStatus(crb_tensor_add_clear(elements, other->elements, dims.size, nullptr), __FILE__, __LINE__);
-    assertHip(__FILE__, __LINE__);
+    launched(crb_tensor_add_clear(elements, other->elements, dims.size, nullptr), __FILE__, __LINE__);
     return this;
 }
 
@@ -173,8 +179,7 @@ Tensor *Tensor::operator-(Tensor *other) {
         for (uint32 i = 0; i < dims.size; ++i) elements[i] -= other->elements[i];
         return this;
     }
-    throwOnStatus(crb_tensor_sub_inplace(elements, other->elements, dims.size, nullptr), __FILE__, __LINE__);
-    assertHip(__FILE__, __LINE__);
+    launched(crb_tensor_sub_inplace(elements, other->elements, dims.size, nullptr), __FILE__, __LINE__);
     return this;
 }
 
@@ -183,8 +188,7 @@ Tensor *Tensor::operator*(float factor) {
         for (uint32 i = 0; i < dims.size; ++i) elements[i] *= factor;
         return this;
     }
-    throwOnStatus(crb_tensor_scale_inplace(elements, factor, dims.size, nullptr), __FILE__, __LINE__);
-    assertHip(__FILE__, __LINE__);
+    launched(crb_tensor_scale_inplace(elements, factor, dims.size, nullptr), __FILE__, __LINE__);
     return this;
 }
 
@@ -193,8 +197,7 @@ Tensor *Tensor::constFill(float val) {
         for (uint32 i = 0; i < dims.size; ++i) elements[i] = val;
         return this;
     }
-    throwOnStatus(crb_tensor_fill(elements, val, dims.size, nullptr), __FILE__, __LINE__);
-    assertHip(__FILE__, __LINE__);
+    launched(crb_tensor_fill(elements, val, dims.size, nullptr), __FILE__, __LINE__);
     return this;
 }
 
