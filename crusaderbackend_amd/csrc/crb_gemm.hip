@@ -10,14 +10,15 @@ namespace crb {
 typedef TileCfg<128, 128, 16, 2, 2, 2> CfgLarge;
 typedef TileCfg<64, 64, 16, 2, 2, 2> CfgSmall;
 typedef TileCfg<64, 64, 64, 2, 2, 2> CfgSmallDeep;  // 64-wide K slabs: one workgroup per CU has nobody to hide its loads behind
-typedef TileCfg<64, 64, 32, 2, 2, 2, 2> CfgSmallAhead;  // loads run two slabs ahead: small tiles finish a slab faster than a load takes
+typedef TileCfg<64, 64, 32, 2, 2, 2, 2> CfgSmallAhead;
+typedef TileCfg<64, 64, 64, 2, 2, 1, 1, 2> CfgSmallDeep8;  // eight waves: two K groups per macro-tile, for grids of one workgroup per CU  // loads run two slabs ahead: small tiles finish a slab faster than a load takes
 
 static inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 // Tile choice by how many workgroups the grid gives a CU; when neither tile size fills the chip, K is split — with
 // large tiles only when each slice keeps a long contraction (the split costs a second pass over the result).
 // `dense` = the result rows are contiguous (ld == N), which the partial results of a split assume.
-enum GemmTile { TILE_LARGE, TILE_SMALL, TILE_SMALL_DEEP, TILE_SMALL_AHEAD };
+enum GemmTile { TILE_LARGE, TILE_SMALL, TILE_SMALL_DEEP, TILE_SMALL_AHEAD, TILE_SMALL_DEEP8 };
 struct GemmChoice {
     GemmTile tile;
     u32 want_splits;  // > 1: cut K this many times although the tile grid covers the chip
@@ -36,6 +37,9 @@ static GemmChoice choose_tiles(u32 M, u32 N, u32 K, u32 zdim, bool dense) {
         // other's loads (measured: pays from K = 1280, from 1024 when the tiles do not cover the CUs evenly) ...
         if (tiles_s >= 160 && K < 2048 && (K >= 1280 || (K >= 1024 && tiles_s > 256)) && zdim == 1 && dense) return {TILE_SMALL_AHEAD, 2};
         // ... a shorter one gets longer slabs, so that a slab's loads have a whole slab of MFMAs (2048 clocks) to arrive in
+        // ... with at most one tile per CU as eight waves (two K groups), so that every SIMD still holds two waves
+        // (1024^3: 32.0 -> 29.7 us, 1000^3: 30.7 -> 28.6; slabs of 32 or 128 and loads two slabs ahead measured the same)
+        if (tiles_s >= 160 && tiles_s <= 256 && K >= 512 && K < 2048) return {TILE_SMALL_DEEP8, 0};
         if (tiles_s >= 160 && K >= 512 && K < 2048) return {TILE_SMALL_DEEP, 0};
         if (tiles_s >= 160 && K < 2048) return {TILE_SMALL_AHEAD, 0};
         // one small tile per CU at most but a long contraction: two K slices per tile put two workgroups on every CU
@@ -87,6 +91,7 @@ static int run_tiles(const AOp &a, const BOp &b, const RowMajorEpi &e, u32 M, u3
     switch (c.tile) {
         case TILE_LARGE: return run_cfg<CfgLarge>(a, b, e, M, N, K, zdim, s, what, c.want_splits);
         case TILE_SMALL_DEEP: return run_cfg<CfgSmallDeep>(a, b, e, M, N, K, zdim, s, what, c.want_splits);
+        case TILE_SMALL_DEEP8: return run_cfg<CfgSmallDeep8>(a, b, e, M, N, K, zdim, s, what, c.want_splits);
         case TILE_SMALL_AHEAD: return run_cfg<CfgSmallAhead>(a, b, e, M, N, K, zdim, s, what, c.want_splits);
         default: return run_cfg<CfgSmall>(a, b, e, M, N, K, zdim, s, what, c.want_splits);
     }
@@ -100,6 +105,7 @@ size_t gemm_scratch_bytes(u32 M, u32 N, u32 K, u32 zdim) {
     switch (c.tile) {
         case TILE_LARGE: sp = split_for<CfgLarge>(M, N, K, zdim, c.want_splits, true); break;
         case TILE_SMALL_DEEP: sp = split_for<CfgSmallDeep>(M, N, K, zdim, c.want_splits, true); break;
+        case TILE_SMALL_DEEP8: sp = split_for<CfgSmallDeep8>(M, N, K, zdim, c.want_splits, true); break;
         case TILE_SMALL_AHEAD: sp = split_for<CfgSmallAhead>(M, N, K, zdim, c.want_splits, true); break;
         default: sp = split_for<CfgSmall>(M, N, K, zdim, c.want_splits, true); break;
     }

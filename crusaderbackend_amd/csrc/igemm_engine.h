@@ -39,9 +39,14 @@ struct IgemmDims {
 
 // PF_: how many K slabs ahead of the MFMAs the global loads run (1: the next slab's loads have one slab of MFMAs to
 // arrive in; 2: two register sets, two slabs in flight — for grids that leave a CU a single workgroup).
-template <int BM_, int BN_, int BK_, int WM_, int WN_, int OCC_, int PF_ = 1>
+// KG_: wave groups along K. 2: eight waves; both groups own the same macro-tile and each multiplies half of every staged
+// slab, so that a grid of one workgroup per CU still puts two waves on every SIMD; the second group's accumulators are
+// added to the first's through LDS before the epilogue (fixed order: bit-reproducible).
+template <int BM_, int BN_, int BK_, int WM_, int WN_, int OCC_, int PF_ = 1, int KG_ = 1>
 struct TileCfg {
-    static constexpr int BM = BM_, BN = BN_, BK = BK_, WM = WM_, WN = WN_, OCC = OCC_, PF = PF_;
+    static constexpr int BM = BM_, BN = BN_, BK = BK_, WM = WM_, WN = WN_, OCC = OCC_, PF = PF_, KG = KG_;
+    static constexpr int NTH = kThreads * KG_;  // threads per workgroup
+    static_assert(KG == 1 || (KG == 2 && BK_ % 16 == 0), "two wave groups split a slab into halves of whole 8-k groups");
     static_assert(PF == 1 || PF == 2, "prefetch distance");
     static constexpr int WTM = BM / WM, WTN = BN / WN;  // wave tile
     static constexpr int TM = WTM / 32, TN = WTN / 32;  // 32x32 MFMA blocks per wave tile
@@ -51,7 +56,7 @@ struct TileCfg {
 };
 
 // ---- global -> register -> LDS staging of one operand panel (ROWS x BK) -----------------------------
-template <class Op, int ROWS, int BK>
+template <class Op, int ROWS, int BK, int NTH = kThreads>
 struct PanelLoader {
     static constexpr bool KF = Op::kKFast;
     static constexpr bool VEC = Op::kVec;
@@ -59,11 +64,11 @@ struct PanelLoader {
     static constexpr int SIZE = KF ? ROWS * LD : BK * LD;
     // number of register-resident items per thread per slab
     static constexpr int ITEMS = VEC ? ROWS * BK / 4 : ROWS * BK;
-    static constexpr int NP = (ITEMS + kThreads - 1) / kThreads;
-    static_assert(ITEMS % kThreads == 0 || ITEMS < kThreads, "panel must split evenly over 256 threads");
+    static constexpr int NP = (ITEMS + NTH - 1) / NTH;
+    static_assert(ITEMS % NTH == 0 || ITEMS < NTH, "panel must split evenly over 256 threads");
     // panels with fewer items than threads are staged by the first ITEMS threads only
-    static __device__ __forceinline__ bool active() { return ITEMS >= kThreads || threadIdx.x < ITEMS; }
-    static_assert(VEC || KF || ROWS <= kThreads, "row-fast scalar staging needs ROWS <= 256");
+    static __device__ __forceinline__ bool active() { return ITEMS >= NTH || threadIdx.x < ITEMS; }
+    static_assert(VEC || KF || ROWS <= NTH, "row-fast scalar staging needs ROWS <= 256");
 
     // scalar, k-fast: thread owns k lane t%BK and rows t/BK + i*(256/BK): NP row states kept
     // scalar, row-fast: thread owns row t%ROWS and k's t/ROWS + i*(256/ROWS): one row state kept
@@ -78,7 +83,7 @@ struct PanelLoader {
         if constexpr (!VEC) {
             if constexpr (KF) {
 #pragma unroll
-                for (int i = 0; i < NP; ++i) rs[i] = op.prep_row(row0 + t / BK + i * (kThreads / BK));
+                for (int i = 0; i < NP; ++i) rs[i] = op.prep_row(row0 + t / BK + i * (NTH / BK));
             } else {
                 rs[0] = op.prep_row(row0 + t % ROWS);
             }
@@ -90,14 +95,14 @@ struct PanelLoader {
         if (!active()) return;
         if constexpr (VEC) {
             if constexpr (KF) {
-                constexpr int QK = BK / 4, RP = kThreads / QK;
+                constexpr int QK = BK / 4, RP = NTH / QK;
 #pragma unroll
                 for (int i = 0; i < NP; ++i) {
                     v4f v = op.fetch4(row0 + t / QK + i * RP, k0 + 4 * (t % QK), klimit);
                     reg[4 * i + 0] = v.x, reg[4 * i + 1] = v.y, reg[4 * i + 2] = v.z, reg[4 * i + 3] = v.w;
                 }
             } else {
-                constexpr int QR = ROWS / 4, KP = kThreads / QR;
+                constexpr int QR = ROWS / 4, KP = NTH / QR;
 #pragma unroll
                 for (int i = 0; i < NP; ++i) {
                     v4f v = op.fetch4(row0 + 4 * (t % QR), k0 + t / QR + i * KP, klimit);
@@ -110,7 +115,7 @@ struct PanelLoader {
 #pragma unroll
                 for (int i = 0; i < NP; ++i) reg[i] = op.fetch(rs[i], ks);
             } else {
-                constexpr int KP = kThreads / ROWS;
+                constexpr int KP = NTH / ROWS;
 #pragma unroll
                 for (int i = 0; i < NP; ++i) {
                     typename Op::KS ks = op.prep_k(k0 + t / ROWS + i * KP, klimit);
@@ -125,14 +130,14 @@ struct PanelLoader {
         if (!active()) return;
         if constexpr (VEC) {
             if constexpr (KF) {
-                constexpr int QK = BK / 4, RP = kThreads / QK;
+                constexpr int QK = BK / 4, RP = NTH / QK;
 #pragma unroll
                 for (int i = 0; i < NP; ++i) {
                     v4f v = {reg[4 * i], reg[4 * i + 1], reg[4 * i + 2], reg[4 * i + 3]};
                     *reinterpret_cast<v4f *>(lds + (t / QK + i * RP) * LD + 4 * (t % QK)) = v;
                 }
             } else {
-                constexpr int QR = ROWS / 4, KP = kThreads / QR;
+                constexpr int QR = ROWS / 4, KP = NTH / QR;
 #pragma unroll
                 for (int i = 0; i < NP; ++i) {
                     v4f v = {reg[4 * i], reg[4 * i + 1], reg[4 * i + 2], reg[4 * i + 3]};
@@ -142,9 +147,9 @@ struct PanelLoader {
         } else {
             if constexpr (KF) {
 #pragma unroll
-                for (int i = 0; i < NP; ++i) lds[(t / BK + i * (kThreads / BK)) * LD + t % BK] = reg[i];
+                for (int i = 0; i < NP; ++i) lds[(t / BK + i * (NTH / BK)) * LD + t % BK] = reg[i];
             } else {
-                constexpr int KP = kThreads / ROWS;
+                constexpr int KP = NTH / ROWS;
 #pragma unroll
                 for (int i = 0; i < NP; ++i) lds[(t / ROWS + i * KP) * LD + t % ROWS] = reg[i];
             }
@@ -203,10 +208,10 @@ __device__ __forceinline__ void swizzled_tile(u32 bid, u32 tiles_m, u32 tiles_n,
 }
 
 template <class Cfg, class AOp, class BOp, class Epi>
-__global__ void __launch_bounds__(kThreads, Cfg::OCC) igemm_kernel(AOp a, BOp b, Epi epi, IgemmDims d) {
+__global__ void __launch_bounds__(Cfg::NTH, Cfg::OCC) igemm_kernel(AOp a, BOp b, Epi epi, IgemmDims d) {
     constexpr int BM = Cfg::BM, BN = Cfg::BN, BK = Cfg::BK, TM = Cfg::TM, TN = Cfg::TN;
-    using LA = PanelLoader<AOp, BM, BK>;
-    using LB = PanelLoader<BOp, BN, BK>;
+    using LA = PanelLoader<AOp, BM, BK, Cfg::NTH>;
+    using LB = PanelLoader<BOp, BN, BK, Cfg::NTH>;
     __shared__ __attribute__((aligned(16))) float sA[2][LA::SIZE];
     __shared__ __attribute__((aligned(16))) float sB[2][LB::SIZE];
 
@@ -223,7 +228,8 @@ __global__ void __launch_bounds__(kThreads, Cfg::OCC) igemm_kernel(AOp a, BOp b,
     }
     epi.bind(z);
 
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int lane = threadIdx.x & 63, wave = (threadIdx.x >> 6) & 3;  // wave: position in the macro-tile (shared by both K groups)
+    const int kgroup = threadIdx.x >> 8;                               // which half of every slab this wave multiplies (KG = 2)
     const int wave_m = wave / Cfg::WN, wave_n = wave % Cfg::WN;
     const u32 row0 = tm * BM, col0 = tn * BN;
 
@@ -243,8 +249,10 @@ __global__ void __launch_bounds__(kThreads, Cfg::OCC) igemm_kernel(AOp a, BOp b,
     // the MFMAs of the slab held by LDS buffer `buf`
     auto multiply = [&](int buf) {
         const float *pa = sA[buf], *pb = sB[buf];
+        constexpr int GPW = BK / 8 / Cfg::KG;  // 8-k groups per wave per slab
 #pragma unroll
-        for (int g = 0; g < BK / 8; ++g) {
+        for (int gi = 0; gi < GPW; ++gi) {
+            const int g = Cfg::KG == 1 ? gi : kgroup * GPW + gi;
             float fa[4][TM], fb[4][TN];
             read_frags<AOp::kKFast, TM, LA::LD>(pa, wave_m * Cfg::WTM, g, lane, fa);
             read_frags<BOp::kKFast, TN, LB::LD>(pb, wave_n * Cfg::WTN, g, lane, fb);
@@ -319,6 +327,29 @@ __global__ void __launch_bounds__(kThreads, Cfg::OCC) igemm_kernel(AOp a, BOp b,
         }
     }
 
+    if constexpr (Cfg::KG == 2) {
+        // the second K group parks its accumulators in the staging space (idle now: the last slab's barrier has passed),
+        // the first adds them to its own and runs the epilogue alone
+        float *park = &sA[0][0];
+        constexpr int PER_WAVE = TM * TN * 16 * 64;
+        static_assert(4 * PER_WAVE <= 2 * LA::SIZE, "parking space");
+        if (kgroup == 1) {
+#pragma unroll
+            for (int mi = 0; mi < TM; ++mi)
+#pragma unroll
+                for (int ni = 0; ni < TN; ++ni)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) park[wave * PER_WAVE + ((mi * TN + ni) * 16 + r) * 64 + lane] = acc[mi][ni][r];
+        }
+        __syncthreads();
+        if (kgroup == 1) return;
+#pragma unroll
+        for (int mi = 0; mi < TM; ++mi)
+#pragma unroll
+            for (int ni = 0; ni < TN; ++ni)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) acc[mi][ni][r] += park[wave * PER_WAVE + ((mi * TN + ni) * 16 + r) * 64 + lane];
+    }
     // epilogue: accumulator register r of lane l is D[8*(r/4) + 4*(l/32) + r%4][l%32] of its block
     const int j = lane & 31, h = lane >> 5;
     if constexpr (!BOp::kKFast && TN == 2 && Epi::kPairStore) {
@@ -583,7 +614,7 @@ inline int launch_igemm(const AOp &a, const BOp &b, const Epi &epi, u32 M, u32 N
     const uint64_t tiles = uint64_t(d.tiles_m) * d.tiles_n;
     if (tiles > 0x7fffffffull || zdim > 65535u) return fail(CRB_EINVAL_SHAPE, "%s: launch grid too large", what);
     dim3 grid(u32(tiles), 1, zdim);
-    hipLaunchKernelGGL((igemm_kernel<Cfg, AOp, BOp, Epi>), grid, dim3(kThreads), 0, stream, a, b, epi, d);
+    hipLaunchKernelGGL((igemm_kernel<Cfg, AOp, BOp, Epi>), grid, dim3(Cfg::NTH), 0, stream, a, b, epi, d);
     return check_launch(what);
 }
 
