@@ -3,6 +3,7 @@
 #include "conv3x3_direct.h"
 #include "conv3x3_wgrad.h"
 #include "conv1x1_s2.h"
+#include "conv1x1_wgrad.h"
 #include "gemm_internal.h"
 #include "operands.h"
 
@@ -623,8 +624,11 @@ int crb_conv_dgrad(const float *W, const float *dY, float *dX, const crb_conv_ge
 
 size_t crb_conv_wgrad_workspace_bytes(const crb_conv_geom *g) {
     if (check_geom("crb_conv_wgrad_workspace_bytes", g)) return 0;
-    if (pointwise_shape(g))  // accumulate-NT GEMM form over the batch-concatenated contraction
-        return uint64_t(g->IH) * g->IW * g->N > 0x7fffffffull ? 0 : gemm_scratch_bytes(g->OC, g->IC, g->IH * g->IW * g->N, 1);
+    if (pointwise_shape(g)) {  // pixel-contraction kernel, or (unaligned / wide layers) the accumulate-NT GEMM form
+        const size_t gemm = uint64_t(g->IH) * g->IW * g->N > 0x7fffffffull ? 0 : gemm_scratch_bytes(g->OC, g->IC, g->IH * g->IW * g->N, 1);
+        if (!pw_wgrad_fits(g->IC, g->OC, g->IH * g->IW)) return gemm;
+        return std::max(gemm, pw_wgrad_plan(g->N, g->IC, g->OC, g->IH * g->IW).workspace_bytes);
+    }
     if (tiny2x2_shape(g)) return size_t(g->OC) * g->IC * 16 * sizeof(float);  // (oc, p) x (ic, p') product before the tap fold
     if (shortcut_shape(g)) return sc_wgrad_plan(g->N, g->IC, g->OC, g->OH, g->OW).workspace_bytes;
     {
@@ -642,6 +646,19 @@ int crb_conv_wgrad(const float *dY, const float *X, float *dW, const crb_conv_ge
     if (int st = check_geom("crb_conv_wgrad", g)) return st;
     if (workspace && !aligned16(workspace)) return fail(CRB_EWORKSPACE, "crb_conv_wgrad: workspace is not 16-byte aligned");
     hipStream_t s = hipStream_t(stream);
+    if (pointwise_shape(g) && pw_wgrad_fits(g->IC, g->OC, g->IH * g->IW) && aligned16(dY) && aligned16(X)) {
+        const PwWgradPlan pp = pw_wgrad_plan(g->N, g->IC, g->OC, g->IH * g->IW);
+        float *pws = static_cast<float *>(workspace);
+        if (pp.workspace_bytes) {
+            if (pws) {
+                if (workspace_bytes < pp.workspace_bytes)
+                    return fail(CRB_EWORKSPACE, "crb_conv_wgrad: workspace %zu bytes < required %zu", workspace_bytes, pp.workspace_bytes);
+            } else if (int sg = scratch_get(pp.workspace_bytes, s, "crb_conv_wgrad", &pws)) {
+                return sg;
+            }
+        }
+        return launch_pw_wgrad(dY, X, dW, pws, pp, g->IC, g->OC, g->IH * g->IW, s, "crb_conv_wgrad");
+    }
     if (pointwise_shape(g)) {
         if (!workspace) return crb_sgemm_nta(dY, X, dW, g->OC, g->IC, g->IH * g->IW, g->N, stream);
         ScratchScope scope(workspace, workspace_bytes);  // the GEMM's split scratch comes from the caller's block

@@ -301,7 +301,9 @@ POINTWISE = [(3, 24, 32, 32, 48), (2, 204, 32, 32, 48), (2, 108, 16, 16, 48), (4
              (2, 64, 32, 32, 64), (2, 17, 8, 8, 33), (2, 16, 12, 16, 16), (2, 16, 8, 12, 16), (1, 40, 24, 32, 70),
              # batches large enough to pass the workgroup-count gate of the staged 1x1 kernel
              (64, 204, 32, 32, 48), (64, 24, 32, 32, 48), (64, 108, 16, 16, 48), (96, 70, 16, 16, 130), (64, 150, 8, 8, 48),
-             (128, 37, 8, 8, 64), (48, 80, 32, 32, 20)]
+             (128, 37, 8, 8, 64), (48, 80, 32, 32, 20),
+             # pixel-contraction weight gradient: ragged last slice, 49..64 output channels, one 64-pixel run per image
+             (40, 50, 32, 32, 50), (3, 16, 8, 8, 64), (72, 342, 8, 8, 48)]
 
 
 @pytest.mark.parametrize("N,IC,H,W,OC", POINTWISE)
