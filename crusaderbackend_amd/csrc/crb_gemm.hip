@@ -69,11 +69,21 @@ static SplitPlan split_for(u32 M, u32 N, u32 K, u32 zdim, u32 want_splits, bool 
 // Runs C = A*B through the engine. `e` describes the final result; when the M x N tile grid is too small to occupy the
 // chip (and there is no batch), K is cut into slices whose partial results go to scratch and a second kernel combines
 // them in fixed order and applies the epilogue (bias / accumulate / ReLU).
-template <class Cfg, class AOp, class BOp>
-static int run_cfg(const AOp &a, const BOp &b, const RowMajorEpi &e, u32 M, u32 N, u32 K, u32 zdim, hipStream_t s,
-                   const char *what, u32 want_splits = 0) {
+template <class Cfg, class AOp, class BOp, class E>
+static int run_cfg(const AOp &a, const BOp &b, const E &e, u32 M, u32 N, u32 K, u32 zdim, hipStream_t s, const char *what,
+                   u32 want_splits = 0, bool *rowsum_done = nullptr) {
     const SplitPlan sp = split_for<Cfg>(M, N, K, zdim, want_splits, e.ld == N);
-    if (sp.splits == 1) return launch_igemm<Cfg>(a, b, e, M, N, K, zdim, 0, K, s, what);
+    if (sp.splits == 1) {
+        if constexpr (E::kRowSum) {
+            // the row sums of A ride along only with one unsplit, unbatched launch; otherwise the caller forms them itself
+            E e1 = e;
+            if (zdim != 1) e1.a_rowsum = nullptr;
+            if (rowsum_done) *rowsum_done = e1.a_rowsum != nullptr;
+            return launch_igemm<Cfg>(a, b, e1, M, N, K, zdim, 0, K, s, what);
+        } else {
+            return launch_igemm<Cfg>(a, b, e, M, N, K, zdim, 0, K, s, what);
+        }
+    }
     const size_t need = size_t(sp.splits) * M * N * sizeof(float);
     float *ws = nullptr;
     if (int st = scratch_get(need, s, what, &ws)) return st;
@@ -84,16 +94,16 @@ static int run_cfg(const AOp &a, const BOp &b, const RowMajorEpi &e, u32 M, u32 
                                 s, what);
 }
 
-template <class AOp, class BOp>
-static int run_tiles(const AOp &a, const BOp &b, const RowMajorEpi &e, u32 M, u32 N, u32 K, u32 zdim, hipStream_t s,
-                     const char *what) {
+template <class AOp, class BOp, class E>
+static int run_tiles(const AOp &a, const BOp &b, const E &e, u32 M, u32 N, u32 K, u32 zdim, hipStream_t s, const char *what,
+                     bool *rowsum_done = nullptr) {
     const GemmChoice c = choose_tiles(M, N, K, zdim, e.ld == N);
     switch (c.tile) {
-        case TILE_LARGE: return run_cfg<CfgLarge>(a, b, e, M, N, K, zdim, s, what, c.want_splits);
-        case TILE_SMALL_DEEP: return run_cfg<CfgSmallDeep>(a, b, e, M, N, K, zdim, s, what, c.want_splits);
-        case TILE_SMALL_DEEP8: return run_cfg<CfgSmallDeep8>(a, b, e, M, N, K, zdim, s, what, c.want_splits);
-        case TILE_SMALL_AHEAD: return run_cfg<CfgSmallAhead>(a, b, e, M, N, K, zdim, s, what, c.want_splits);
-        default: return run_cfg<CfgSmall>(a, b, e, M, N, K, zdim, s, what, c.want_splits);
+        case TILE_LARGE: return run_cfg<CfgLarge>(a, b, e, M, N, K, zdim, s, what, c.want_splits, rowsum_done);
+        case TILE_SMALL_DEEP: return run_cfg<CfgSmallDeep>(a, b, e, M, N, K, zdim, s, what, c.want_splits, rowsum_done);
+        case TILE_SMALL_DEEP8: return run_cfg<CfgSmallDeep8>(a, b, e, M, N, K, zdim, s, what, c.want_splits, rowsum_done);
+        case TILE_SMALL_AHEAD: return run_cfg<CfgSmallAhead>(a, b, e, M, N, K, zdim, s, what, c.want_splits, rowsum_done);
+        default: return run_cfg<CfgSmall>(a, b, e, M, N, K, zdim, s, what, c.want_splits, rowsum_done);
     }
 }
 
@@ -167,13 +177,24 @@ static int gemm_nn(const float *A, const float *B, float *C, u32 M, u32 N, u32 K
 }
 
 static int gemm_tn(const float *A, const float *B, float *C, u32 M, u32 N, u32 K, u32 batch, u32 flags,
-                   hipStream_t s, const char *what) {
-    if (tiny_gemm_fits(M, N, K, batch))  // A stored K x M, B (K x N) row-major
-        return launch_tiny_gemm(TinyGemmArgs{A, B, C, nullptr, nullptr, M, N, K, 1, M, N, 1, N, flags}, K, 0, 0, s, what);
+                   hipStream_t s, const char *what, float *a_rowsum = nullptr, bool *rowsum_done = nullptr) {
+    if (rowsum_done) *rowsum_done = false;
+    if (tiny_gemm_fits(M, N, K, batch)) {  // A stored K x M, B (K x N) row-major
+        TinyGemmArgs t{A, B, C, nullptr, nullptr, M, N, K, 1, M, N, 1, N, flags};
+        t.a_rowsum = a_rowsum;
+        if (rowsum_done) *rowsum_done = a_rowsum != nullptr;
+        return launch_tiny_gemm(t, K, 0, 0, s, what);
+    }
     RowMajorEpi e{C, nullptr, N, M * N, flags};
     if (M % 4 == 0 && N % 4 == 0 && aligned16(A) && aligned16(B)) {
         MatR<true> a{A, M, M, 0};
         MatR<true> b{B, N, N, K * N};
+        if (flags & EPI_ACCUM) {  // the dense layers' weight gradient
+            RowMajorAccEpi ea;
+            static_cast<RowMajorEpi &>(ea) = e;
+            ea.a_rowsum = a_rowsum;
+            return run_tiles(a, b, ea, M, N, K, batch, s, what, rowsum_done);
+        }
         return run_tiles(a, b, e, M, N, K, batch, s, what);
     }
     MatR<false> a{A, M, M, 0};
@@ -337,8 +358,10 @@ int crb_linear_wgrad(const float *dY, const float *X, float *dW, float *dB, uint
     if (int st = check_dims("crb_linear_wgrad", OUT, IN, batch, 1)) return st;
     hipStream_t s = hipStream_t(stream);
     // dW (OUT x IN) += dY^T (dY stored batch x OUT) * X (batch x IN)
-    if (int st = gemm_tn(dY, X, dW, OUT, IN, batch, 1, EPI_ACCUM, s, "crb_linear_wgrad")) return st;
-    if (dB) {
+    // the bias gradient (column sums of dY = row sums of the A operand) rides along with an unsplit product
+    bool db_done = false;
+    if (int st = gemm_tn(dY, X, dW, OUT, IN, batch, 1, EPI_ACCUM, s, "crb_linear_wgrad", dB, &db_done)) return st;
+    if (dB && !db_done) {
         hipLaunchKernelGGL(colsum_accum_kernel, dim3(ceil_div(OUT, 32)), dim3(256), 0, s, dY, dB, batch, OUT);
         return check_launch("crb_linear_wgrad(dB)");
     }

@@ -28,11 +28,15 @@ struct TinyGemmArgs {
     // K is then batch * kb_len. Without a batch kb_len = K.
     u32 a_bs, b_bs;
     FastDiv kb_len;
+    // optional second result: a_rowsum[i] += sum over k of A(i, k), formed by the workgroups of the first block column
+    // (lanes, then waves, in fixed order: bit-reproducible)
+    float *a_rowsum = nullptr;
 };
 
 template <bool KVEC>
 __global__ void __launch_bounds__(256) tiny_gemm_kernel(TinyGemmArgs a) {
     __shared__ __attribute__((aligned(16))) float red[4 * 256];
+    __shared__ float rsum[256];
     const u32 t = threadIdx.x, lane = t & 63, wave = t >> 6;
     const u32 li = lane & 15, g = lane >> 4;
     const u32 row0 = (blockIdx.x / a.tiles_n) * 16, col0 = (blockIdx.x % a.tiles_n) * 16;
@@ -40,6 +44,7 @@ __global__ void __launch_bounds__(256) tiny_gemm_kernel(TinyGemmArgs a) {
     const u32 ke = kb + a.k_per_wave < a.K ? kb + a.k_per_wave : a.K;
     const bool row_ok = row0 + li < a.M, col_ok = col0 + li < a.N;
     v4f acc = {0.f, 0.f, 0.f, 0.f};
+    float asum = 0.f;  // this lane's share of row li's sum of A
     if constexpr (KVEC) {
         // both operands contiguous along k, K % 4 == 0, 16-byte aligned rows
         const float *pa = a.A + size_t(row0 + li) * a.a_rs;
@@ -58,6 +63,7 @@ __global__ void __launch_bounds__(256) tiny_gemm_kernel(TinyGemmArgs a) {
             }
 #pragma unroll
             for (int u = 0; u < U; ++u) {
+                asum += (va[u].x + va[u].y) + (va[u].z + va[u].w);
                 acc = __builtin_amdgcn_mfma_f32_16x16x4f32(va[u].x, vb[u].x, acc, 0, 0, 0);
                 acc = __builtin_amdgcn_mfma_f32_16x16x4f32(va[u].y, vb[u].y, acc, 0, 0, 0);
                 acc = __builtin_amdgcn_mfma_f32_16x16x4f32(va[u].z, vb[u].z, acc, 0, 0, 0);
@@ -67,7 +73,7 @@ __global__ void __launch_bounds__(256) tiny_gemm_kernel(TinyGemmArgs a) {
     } else {
         const float *pa = a.A + size_t(row0 + li) * a.a_rs;
         const float *pb = a.B + size_t(col0 + li) * a.b_cs;
-        constexpr int U = 8;  // MFMA steps requested together
+        constexpr int U = 16;  // MFMA steps requested together
         for (u32 k = kb; k < ke; k += 4 * U) {
             float va[U], vb[U];
 #pragma unroll
@@ -80,11 +86,22 @@ __global__ void __launch_bounds__(256) tiny_gemm_kernel(TinyGemmArgs a) {
                 vb[u] = (in && col_ok) ? pb[size_t(nd) * a.b_bs + size_t(kr) * a.b_ks] : 0.f;
             }
 #pragma unroll
-            for (int u = 0; u < U; ++u) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(va[u], vb[u], acc, 0, 0, 0);
+            for (int u = 0; u < U; ++u) {
+                asum += va[u];
+                acc = __builtin_amdgcn_mfma_f32_16x16x4f32(va[u], vb[u], acc, 0, 0, 0);
+            }
         }
     }
     *reinterpret_cast<v4f *>(red + wave * 256 + lane * 4) = acc;
+    const bool do_rowsum = a.a_rowsum && col0 == 0;
+    if (do_rowsum) rsum[t] = asum;
     __syncthreads();
+    if (do_rowsum && t < 16 && row0 + t < a.M) {
+        float v = 0.f;
+#pragma unroll
+        for (int q = 0; q < 16; ++q) v += rsum[q * 16 + t];  // wave q / 4, k lane group q % 4
+        a.a_rowsum[row0 + t] += v;
+    }
     // thread t finishes element (row t / 16, column t % 16): register row % 4 of lane (row / 4) * 16 + column
     const u32 r = t >> 4, c = t & 15;
     const u32 row = row0 + r, col = col0 + c;

@@ -246,9 +246,55 @@ __global__ void __launch_bounds__(Cfg::NTH, Cfg::OCC) igemm_kernel(AOp a, BOp b,
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[mi][ni][r] = 0.0f;
 
+    // accumulating epilogues on interior tiles read the result's previous values a block (16 per lane, or 16 pairs) at a
+    // time, all loads of a block in flight together, instead of one memory round trip per element; a one-block wave
+    // tile requests them before the last slab is multiplied, so that they arrive behind its MFMAs
+    constexpr bool kPair = !BOp::kKFast && TN == 2 && Epi::kPairStore;
+    constexpr bool kOldEarly = Epi::kEarlyOld && TM * TN == 1;
+    float oldv[Epi::kPrefetchOld ? (kPair ? 32 : 16) : 1];
+    bool have_old = false, old_tried = false;
+    // block (mi, ni) of the wave tile (pair form: both ni of row block mi)
+    auto fetch_old_block = [&](int mi, int ni) {
+        if constexpr (Epi::kPrefetchOld) {
+            const int j = lane & 31, h = lane >> 5;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int id = 8 * (r / 4) + 4 * h + (r % 4);
+                const u32 row = row0 + wave_m * Cfg::WTM + (AOp::kKFast ? mi * 32 + id : id * TM + mi);
+                if constexpr (kPair) {
+                    const v2f o = *reinterpret_cast<const v2f *>(epi.at(row, col0 + wave_n * Cfg::WTN + j * 2));
+                    oldv[r] = o.x, oldv[16 + r] = o.y;
+                } else {
+                    oldv[r] = *epi.at(row, col0 + wave_n * Cfg::WTN + (BOp::kKFast ? ni * 32 + j : j * TN + ni));
+                }
+            }
+        }
+    };
+    const bool old_ok = Epi::kPrefetchOld && kgroup == 0 && epi.accum_interior(row0, col0, BM, BN, d.M, d.N) &&
+                        (!kPair || epi.pair_aligned(col0 + wave_n * Cfg::WTN));
+    auto fetch_old = [&]() {
+        old_tried = true;
+        if constexpr (kOldEarly) {
+            if (old_ok) fetch_old_block(0, 0), have_old = true;
+        }
+    };
+
+    // optional second result of epilogues that carry `a_rowsum`: a_rowsum[m] += sum over k of A(m, k), formed by the
+    // workgroups of the first tile column from the A panels they stage anyway, in ascending k (bit-reproducible);
+    // thread t < BM owns row t of the panel
+    bool do_rowsum = false;
+    if constexpr (Epi::kRowSum) do_rowsum = epi.a_rowsum && tn == 0 && threadIdx.x < BM;
+    float rowsum = 0.f;
+
     // the MFMAs of the slab held by LDS buffer `buf`
     auto multiply = [&](int buf) {
         const float *pa = sA[buf], *pb = sB[buf];
+        if constexpr (Epi::kRowSum) {
+            if (do_rowsum) {
+#pragma unroll
+                for (int k = 0; k < BK; ++k) rowsum += AOp::kKFast ? pa[threadIdx.x * LA::LD + k] : pa[k * LA::LD + threadIdx.x];
+            }
+        }
         constexpr int GPW = BK / 8 / Cfg::KG;  // 8-k groups per wave per slab
 #pragma unroll
         for (int gi = 0; gi < GPW; ++gi) {
@@ -291,6 +337,7 @@ __global__ void __launch_bounds__(Cfg::NTH, Cfg::OCC) igemm_kernel(AOp a, BOp b,
                 far_a.fetch(a, k0 + 2 * BK, kend);
                 far_b.fetch(b, k0 + 2 * BK, kend);
             }
+            if (k0 + BK >= kend) fetch_old();
             multiply(buf);
             if (k0 + BK < kend) {
                 near_a.commit(sA[buf ^ 1]);
@@ -317,6 +364,8 @@ __global__ void __launch_bounds__(Cfg::NTH, Cfg::OCC) igemm_kernel(AOp a, BOp b,
             if (more) {
                 la.fetch(a, k0 + BK, kend);
                 lb.fetch(b, k0 + BK, kend);
+            } else {
+                fetch_old();
             }
             multiply(buf);
             if (more) {
@@ -350,6 +399,10 @@ __global__ void __launch_bounds__(Cfg::NTH, Cfg::OCC) igemm_kernel(AOp a, BOp b,
 #pragma unroll
                 for (int r = 0; r < 16; ++r) acc[mi][ni][r] += park[wave * PER_WAVE + ((mi * TN + ni) * 16 + r) * 64 + lane];
     }
+    if constexpr (Epi::kRowSum) {
+        if (do_rowsum && row0 + threadIdx.x < d.M) epi.a_rowsum[row0 + threadIdx.x] += rowsum;
+    }
+    if (!old_tried) fetch_old();  // empty contraction range
     // epilogue: accumulator register r of lane l is D[8*(r/4) + 4*(l/32) + r%4][l%32] of its block
     const int j = lane & 31, h = lane >> 5;
     if constexpr (!BOp::kKFast && TN == 2 && Epi::kPairStore) {
@@ -358,26 +411,32 @@ __global__ void __launch_bounds__(Cfg::NTH, Cfg::OCC) igemm_kernel(AOp a, BOp b,
         const u32 col = col0 + wave_n * Cfg::WTN + j * 2;
         const typename Epi::ColS c0 = epi.prep_col(col, d.N), c1 = epi.prep_col(col + 1, d.N);
 #pragma unroll
-        for (int mi = 0; mi < TM; ++mi)
+        for (int mi = 0; mi < TM; ++mi) {
+            if (old_ok) fetch_old_block(mi, 0), have_old = true;
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
                 const int id = 8 * (r / 4) + 4 * h + (r % 4);
                 const u32 row = row0 + wave_m * Cfg::WTM + (AOp::kKFast ? mi * 32 + id : id * TM + mi);
-                if (row < d.M && c0.ok) epi.store2(row, c0, c1, acc[mi][0][r], acc[mi][1][r]);
+                if (row < d.M && c0.ok) epi.store2(row, c0, c1, acc[mi][0][r], acc[mi][1][r], have_old, oldv[r], oldv[kPair ? 16 + r : 0]);
             }
+        }
     } else {
 #pragma unroll
         for (int ni = 0; ni < TN; ++ni) {
             const u32 col = col0 + wave_n * Cfg::WTN + (BOp::kKFast ? ni * 32 + j : j * TN + ni);
             const typename Epi::ColS cs = epi.prep_col(col, d.N);
 #pragma unroll
-            for (int mi = 0; mi < TM; ++mi)
+            for (int mi = 0; mi < TM; ++mi) {
+                if constexpr (!kOldEarly) {
+                    if (old_ok) fetch_old_block(mi, ni), have_old = true;
+                }
 #pragma unroll
                 for (int r = 0; r < 16; ++r) {
                     const int id = 8 * (r / 4) + 4 * h + (r % 4);
                     const u32 row = row0 + wave_m * Cfg::WTM + (AOp::kKFast ? mi * 32 + id : id * TM + mi);
-                    if (row < d.M) epi.store(row, cs, acc[mi][ni][r]);
+                    if (row < d.M) epi.store(row, cs, acc[mi][ni][r], have_old, oldv[r]);
                 }
+            }
         }
     }
 }

@@ -277,22 +277,35 @@ struct RowMajorEpi {
         const bool ok = col < ncols;
         return {col, (ok && col_bias) ? col_bias[col >> col_bias_shift] : 0.0f, ok};
     }
-    __device__ __forceinline__ void store(u32 row, const ColS &c, float v) const {
+    // accumulating forms may hand in the previous value (`old`, requested a block at a time) instead of having it read here
+    static constexpr bool kPrefetchOld = true;
+    static constexpr bool kEarlyOld = false;  // the request does not move into the main loop
+    static constexpr bool kRowSum = false;
+    __device__ __forceinline__ bool accum_interior(u32 row0, u32 col0, u32 bm, u32 bn, u32 M, u32 N) const {
+        return (flags & EPI_ACCUM) && row0 + bm <= M && col0 + bn <= N;
+    }
+    __device__ __forceinline__ const float *at(u32 row, u32 col) const { return C + size_t(row) * ld + col; }
+    __device__ __forceinline__ bool pair_aligned(u32 col) const { return ld % 2 == 0 && (reinterpret_cast<uintptr_t>(C + col) & 7u) == 0; }
+    __device__ __forceinline__ void store(u32 row, const ColS &c, float v, bool have_old = false, float old = 0.f) const {
         if (!c.ok) return;
         float *p = C + size_t(row) * ld + c.col;
         v += c.bias;
         if (row_bias) v += row_bias[row];
-        if (flags & EPI_ACCUM) v += *p;
+        if (have_old)
+            v += old;
+        else if (flags & EPI_ACCUM)
+            v += *p;
         if (flags & EPI_RELU) v = v > 0.0f ? v : 0.0f;
         *p = v;
     }
     // Two neighbouring columns of one row (c1.col == c0.col + 1) as one 8-byte access where the address allows it.
     static constexpr bool kPairStore = true;
-    __device__ __forceinline__ void store2(u32 row, const ColS &c0, const ColS &c1, float v0, float v1) const {
+    __device__ __forceinline__ void store2(u32 row, const ColS &c0, const ColS &c1, float v0, float v1, bool have_old = false,
+                                           float old0 = 0.f, float old1 = 0.f) const {
         float *p = C + size_t(row) * ld + c0.col;
         if (!c1.ok || (reinterpret_cast<uintptr_t>(p) & 7u)) {
-            store(row, c0, v0);
-            store(row, c1, v1);
+            store(row, c0, v0, have_old, old0);
+            store(row, c1, v1, have_old, old1);
             return;
         }
         v0 += c0.bias, v1 += c1.bias;
@@ -300,13 +313,24 @@ struct RowMajorEpi {
             const float rb = row_bias[row];
             v0 += rb, v1 += rb;
         }
-        if (flags & EPI_ACCUM) {
+        if (have_old) {
+            v0 += old0, v1 += old1;
+        } else if (flags & EPI_ACCUM) {
             const v2f old = *reinterpret_cast<const v2f *>(p);
             v0 += old.x, v1 += old.y;
         }
         if (flags & EPI_RELU) v0 = v0 > 0.0f ? v0 : 0.0f, v1 = v1 > 0.0f ? v1 : 0.0f;
         *reinterpret_cast<v2f *>(p) = v2f{v0, v1};
     }
+};
+
+// The accumulating dense form (C += A*B with a short contraction, where the epilogue weighs as much as the product):
+// previous values of one-block wave tiles are requested before the last slab is multiplied, and the row sums of A can ride
+// along (a_rowsum[m] += sum_k A(m, k); null: not wanted; only for one unsplit, unbatched launch).
+struct RowMajorAccEpi : RowMajorEpi {
+    static constexpr bool kEarlyOld = true;
+    static constexpr bool kRowSum = true;
+    float *a_rowsum = nullptr;
 };
 
 // NCHW scatter: row = channel, col = n*HW + p  ->  T[(n*C + row)*HW + p], optional per-row bias, ReLU.
@@ -321,14 +345,20 @@ struct NchwEpi {
         bool ok;
     };
     static constexpr bool kPairStore = false;
-    __device__ __forceinline__ void store2(u32, const ColS &, const ColS &, float, float) const {}
+    static constexpr bool kPrefetchOld = false;
+    static constexpr bool kEarlyOld = false;
+    static constexpr bool kRowSum = false;
+    __device__ __forceinline__ void store2(u32, const ColS &, const ColS &, float, float, bool, float, float) const {}
     __device__ __forceinline__ void bind(u32 z) { T += size_t(z) * zstride; }
     __device__ __forceinline__ ColS prep_col(u32 col, u32 ncols) const {
         u32 n, p;
         hw.divmod(col, n, p);
         return {n * C * HW + p, col < ncols};
     }
-    __device__ __forceinline__ void store(u32 row, const ColS &c, float v) const {
+    __device__ __forceinline__ bool accum_interior(u32, u32, u32, u32, u32, u32) const { return false; }
+    __device__ __forceinline__ const float *at(u32, u32) const { return nullptr; }
+    __device__ __forceinline__ bool pair_aligned(u32) const { return false; }
+    __device__ __forceinline__ void store(u32 row, const ColS &c, float v, bool = false, float = 0.f) const {
         if (!c.ok) return;
         if (row_bias) v += row_bias[row];
         if (flags & EPI_RELU) v = v > 0.0f ? v : 0.0f;
