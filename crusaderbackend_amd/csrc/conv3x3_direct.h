@@ -66,7 +66,11 @@ struct DirectCfg {
     static constexpr int XR = MI ? IMGS * 6 : (FS == 1 ? ROWS : (DG2 ? ROWS + 1 : S * (ROWS - 1) + 3));
     static constexpr int ROW0_MUL = FW2 ? 2 : 1;
     static constexpr int ROW0_ADD = (DG2 || FS == 1) ? 0 : -1;
-    static constexpr int PSTEP = FW2 ? 2 : 1;     // LDS distance of neighbouring grid pixels
+    // Stride-2 forward: a staged row holds the input row's odd columns (with the left halo column -1 in front) and then
+    // its even columns, W floats each, so that neighbouring grid pixels are neighbouring floats for every tap (fw = 0 and
+    // 2 read the odd half, fw = 1 the even half) and a fragment read touches 16 consecutive banks per lane group, as at
+    // stride 1, instead of every other bank twice.
+    static constexpr int RSTEP = FW2 ? 2 : 1;     // staged rows between neighbouring grid rows
     static constexpr int XS = SW + 8;  // LDS row stride: 3 pad, left halo, SW interior (16-byte aligned), right halo, 3 pad
     // channel plane stride (floats): the four lane groups (lane/16) of a fragment read sit one plane apart;
     // 16 mod 32 (8 mod 32 for the 2-row blocks of W = 8) puts them on disjoint LDS banks. Multiple of 4.
@@ -97,13 +101,14 @@ struct DirectCfg {
         if (FS == 1) return 1;  // the pixel itself: interior starts one float past the lane's base
         if (DG2) return (fh == 0 ? 1 : 0) * XS + (fw == 0 ? 1 : 0) + 1;
         if (DGRAD) return (2 - fh) * XS + (2 - fw);
+        if (FW2) return fh * XS + (fw == 0 ? 0 : (fw == 2 ? 1 : W + 1));
         return fh * XS + fw;
     }
     // parity class 2*py + px of dX that tap (fh, fw) contributes to (stride-2 data gradient), else 0
     static constexpr int tap_phase(int tap) { return DG2 ? (tap / 3 == 1 ? 0 : 2) + (tap % 3 == 1 ? 0 : 1) : 0; }
     static constexpr int pix_off(int q) {
         if (MI) return ((q / 16) * 6 + (q % 16) / 4) * XS + q % 4;  // image q/16 of the stack, 6 staged rows each
-        return (q / W) * PSTEP * XS + (q % W) * PSTEP;
+        return (q / W) * RSTEP * XS + (q % W);
     }
 };
 
@@ -216,7 +221,12 @@ __device__ __forceinline__ void conv3x3_body(const DirectArgs &a, const u32 bid,
             const u32 e = t + i * kThreads;
             if (XQ % kThreads == 0 || e < XQ) {
                 const u32 q = e % (SW / 4), lr = (e / (SW / 4)) % XR, c = e / ((SW / 4) * XR);
-                *reinterpret_cast<v4f *>(dX + c * XP + lr * XS + 4 + 4 * q) = xreg[i];
+                if constexpr (Cfg::FW2) {  // columns 4q..4q+3: odd ones to the first half of the row, even ones to the second
+                    *reinterpret_cast<v2f *>(dX + c * XP + lr * XS + 4 + 2 * q) = v2f{xreg[i].y, xreg[i].w};
+                    *reinterpret_cast<v2f *>(dX + c * XP + lr * XS + 4 + W + 2 * q) = v2f{xreg[i].x, xreg[i].z};
+                } else {
+                    *reinterpret_cast<v4f *>(dX + c * XP + lr * XS + 4 + 4 * q) = xreg[i];
+                }
             }
         }
 #pragma unroll
