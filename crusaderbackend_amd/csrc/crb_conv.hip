@@ -141,6 +141,11 @@ static int try_direct(const float *Wt, const float *X, float *Y, const float *bi
             // too few 8-row tiles for two workgroups per CU: 4-row tiles
             if (C_OUT <= 16 && C_IN > 16 && N * (gH / 8) < 512) { CRB_TRY(32, 4, 16, 16, 2, 1, DG, 2, 2, 1) }
             // 33..48 output channels: a 48-wide tile instead of a quarter-empty 64-wide one
+            // image layers (3 input channels): one 4-channel chunk instead of an 8-channel one that is 5/8 zeros
+            // (3 -> 64, batch 128: 21.0 -> 13.4 us; 3 -> 16: 6.8 -> 4.6 us)
+            if (C_IN <= 4 && C_OUT > 32) { CRB_TRY(32, 8, 4, 64, 4, 4, DG, 2, 1, 1, 3, 4) }
+            if (C_IN <= 4 && C_OUT > 16) { CRB_TRY(32, 8, 4, 32, 4, 2, DG, 2, 1, 1, 3, 4) }
+            if (C_IN <= 4) { CRB_TRY(32, 8, 4, 16, 4, 1, DG, 2, 1, 1, 3, 4) }
             if (C_OUT > 32 && C_OUT <= 48 && N * (gH / 8) < 512) { CRB_TRY(32, 4, 8, 48, 2, 3, DG, 2, 2, 1) }
             if (C_OUT > 32 && C_OUT <= 48) { CRB_TRY(32, 8, 8, 48, 4, 3, DG, 2, 2, 1) }
             if (C_OUT > 32) { CRB_TRY(32, 8, 8, 64, 4, 4, DG, 2, 2, 1) }
