@@ -237,6 +237,10 @@ static int try_pointwise(const float *Wt, const float *X, float *Y, const float 
     // long contractions with few workgroups: half-height tiles, so two workgroups share a CU and one multiplies while
     // the other waits for its next channel chunk
     const bool half = C_IN > 64 && tiles * ceil_div(C_OUT, 48u) < 512;
+    auto good_half = [&](u32 oct) {  // the same test for half-height tiles (twice as many of them)
+        const u32 nt = ceil_div(C_OUT, oct);
+        return nt * oct * 3 <= C_OUT * 4 + 3 * 15 && 2 * tiles * nt >= 192;
+    };
     // a contraction of at most 48 channels (the data gradient of a bottleneck layer): one LDS-resident chunk, stores in
     // pixel groups (48 -> 204 at batch 64: 28.1 -> 25.6 us @32x32, 9.7 -> 8.9 us @16x16, 5.1 -> 4.5 us @8x8)
     const bool resident = DG && C_IN > 16 && C_IN <= 48;
@@ -258,7 +262,7 @@ static int try_pointwise(const float *Wt, const float *X, float *Y, const float 
         if (good(32)) { CRB_TRY(32, 8, 16, 32, 4, 2, DG, 2, 2, 1, 1) }
         if (good(16)) { CRB_TRY(32, 8, 16, 16, 4, 1, DG, 2, 2, 1, 1) }
     } else if (gW == 16) {
-        if (half && good(48)) { CRB_TRY(16, 4, 16, 48, 1, 3, DG, 2, 2, 1, 1) }
+        if (half && good_half(48)) { CRB_TRY(16, 4, 16, 48, 1, 3, DG, 2, 2, 1, 1) }
         if (good(64)) { CRB_TRY(16, 8, 16, 64, 2, 4, DG, 2, 2, 1, 1) }
         if (good(48)) { CRB_TRY(16, 8, 16, 48, 2, 3, DG, 2, 2, 1, 1) }
         if (good(32)) { CRB_TRY(16, 8, 16, 32, 2, 2, DG, 2, 2, 1, 1) }
