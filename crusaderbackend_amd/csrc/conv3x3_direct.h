@@ -36,19 +36,14 @@ namespace crb {
 // half the LDS, so more workgroups fit on a CU and overlap each other's staging.
 // FS_ = 3: 3x3 filter with pad 1. FS_ = 1: 1x1 filter, no padding, stride 1 (one tap, no halo) — the bottleneck layers,
 // which are bandwidth-bound: same staging and MFMA mapping, the contraction is just the channel chunk.
-// PFD_ > 1 (chunked configurations): the global loads of chunk c + PFD are issued while chunk c is multiplied (PFD register
-// sets in flight), for bandwidth-bound shapes whose chunks are multiplied faster than a load from HBM takes.
 // PGS_ > 1 (single-chunk configurations only): a wave finishes its pixel blocks in PGS groups, one after the other, and
 // stores each group as soon as it is complete, so the stores of all groups but the last overlap the MFMAs of the next.
-template <int W_, int ROWS_, int CI_, int OCT_, int PBW_, int OBW_, bool DGRAD_, int OCC_, int NBUF_ = 2, int S_ = 1, int FS_ = 3, int PGS_ = 1,
-          int PFD_ = 1>
+template <int W_, int ROWS_, int CI_, int OCT_, int PBW_, int OBW_, bool DGRAD_, int OCC_, int NBUF_ = 2, int S_ = 1, int FS_ = 3, int PGS_ = 1>
 struct DirectCfg {
     static constexpr int W = W_, ROWS = ROWS_, CI = CI_, OCT = OCT_, PBW = PBW_, OBW = OBW_, OCC = OCC_, NBUF = NBUF_, S = S_;
     static constexpr int FS = FS_, NT = FS_ * FS_;  // filter size, taps
     static constexpr int PGS = PGS_, PGC = PBW_ / PGS_;  // pixel-block groups per wave, blocks per group
     static constexpr bool STREAM_OUT = PGS_ > 1 || FS_ == 1;  // non-temporal output stores (see store_out)
-    static constexpr int PFD = PFD_;  // how many chunks ahead of the MFMAs the global loads run (register sets)
-    static_assert(PFD == 1 || PFD == 2 || PFD == 4, "prefetch distance");
     static constexpr bool DGRAD = DGRAD_;
     // W = 4: the grid is a 4x4 image and a tile is ROWS / 4 whole images stacked, each staged with its own halo rows
     static constexpr bool MI = W_ == 4;
@@ -172,13 +167,11 @@ __device__ __forceinline__ void conv3x3_body(const DirectArgs &a, const u32 bid,
     // filter slice: one (filter row j, chunk channel c) pair per item, 9 contiguous taps each
     constexpr int WQ = OCT * CI;
     constexpr int WNP = (WQ + kThreads - 1) / kThreads;
-    constexpr int NT = Cfg::NT, PFD = Cfg::PFD;
-    v4f xregs[PFD][XNP];
-    float wregs[PFD][WNP * NT];
+    constexpr int NT = Cfg::NT;
+    v4f xreg[XNP];
+    float wreg[WNP * NT];
 
-    auto fetch = [&](u32 c0, int set = 0) {
-        v4f *xreg = xregs[set];
-        float *wreg = wregs[set];
+    auto fetch = [&](u32 c0) {
 #pragma unroll
         for (int i = 0; i < XNP; ++i) {
             const u32 e = t + i * kThreads;
@@ -213,9 +206,7 @@ __device__ __forceinline__ void conv3x3_body(const DirectArgs &a, const u32 bid,
         }
     };
 
-    auto commit = [&](float *dX, float *dW, int set = 0) {
-        const v4f *xreg = xregs[set];
-        const float *wreg = wregs[set];
+    auto commit = [&](float *dX, float *dW) {
 #pragma unroll
         for (int i = 0; i < XNP; ++i) {
             const u32 e = t + i * kThreads;
@@ -361,25 +352,6 @@ __device__ __forceinline__ void conv3x3_body(const DirectArgs &a, const u32 bid,
         return;
     } else if constexpr (NBUF == 1) {
         compute(sX[0], sW[0], AllP0{}, AllPC{});
-    } else if constexpr (PFD > 1) {
-        // chunk c travels in register set c % PFD from its fetch (PFD chunks before it is multiplied) to its commit (one
-        // chunk before); LDS buffer c % 2
-        const u32 nchunk = (a.C_IN + CI - 1) / CI;
-#pragma unroll
-        for (int d = 1; d < PFD; ++d)
-            if (u32(d) < nchunk) fetch(d * CI, d);
-        for (u32 ch = 0; ch < nchunk; ch += PFD) {
-#pragma unroll
-            for (int j = 0; j < PFD; ++j) {
-                const u32 c = ch + j;
-                if (c < nchunk) {
-                    if (c + PFD < nchunk) fetch((c + PFD) * CI, j);
-                    compute(sX[j & 1], sW[j & 1], AllP0{}, AllPC{});
-                    if (c + 1 < nchunk) commit(sX[(j + 1) & 1], sW[(j + 1) & 1], (j + 1) % PFD);
-                    __syncthreads();
-                }
-            }
-        }
     } else {
         const u32 nchunk = (a.C_IN + CI - 1) / CI;
         for (u32 ch = 0; ch < nchunk; ++ch) {

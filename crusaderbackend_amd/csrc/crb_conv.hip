@@ -4,6 +4,7 @@
 #include "conv3x3_wgrad.h"
 #include "conv1x1_s2.h"
 #include "conv1x1_wgrad.h"
+#include "conv1x1_stream.h"
 #include "gemm_internal.h"
 #include "operands.h"
 
@@ -222,6 +223,11 @@ template <bool DG>
 static int try_pointwise(const float *Wt, const float *X, float *Y, const float *bias, u32 N, u32 C_IN, u32 C_OUT, u32 gH, u32 gW,
                          u32 relu, hipStream_t s, const char *what, bool &done, bool probe = false) {
     done = true;
+    // large layers whose short side (forward: the output channels; data gradient: the contraction) fits one wave: the
+    // activations go from global memory straight into the MFMAs (204 -> 48 @ 32x32, batch 64: forward 20.2 -> 17.0 us,
+    // data gradient 23.0 -> 17.6 us)
+    if (pw_stream_fits(N, DG ? C_IN : C_OUT, gH * gW))
+        return probe ? int(CRB_OK) : launch_pw_stream(DG, Wt, X, Y, bias, N, DG ? C_OUT : C_IN, DG ? C_IN : C_OUT, gH * gW, relu, s, what);
     if ((gW != 32 && gW != 16 && gW != 8) || gH % 8 != 0) {  // every configuration below tiles rows by 8 or 4
         done = false;
         return CRB_OK;

@@ -303,7 +303,9 @@ POINTWISE = [(3, 24, 32, 32, 48), (2, 204, 32, 32, 48), (2, 108, 16, 16, 48), (4
              (64, 204, 32, 32, 48), (64, 24, 32, 32, 48), (64, 108, 16, 16, 48), (96, 70, 16, 16, 130), (64, 150, 8, 8, 48),
              (128, 37, 8, 8, 64), (48, 80, 32, 32, 20),
              # pixel-contraction weight gradient: ragged last slice, 49..64 output channels, one 64-pixel run per image
-             (40, 50, 32, 32, 50), (3, 16, 8, 8, 64), (72, 342, 8, 8, 48)]
+             (40, 50, 32, 32, 50), (3, 16, 8, 8, 64), (72, 342, 8, 8, 48),
+             # streamed forward / data gradient: 16-byte pixel vectors (131072 pixels), two filter staging passes (IC > 256)
+             (128, 20, 32, 32, 24), (32, 300, 32, 32, 40)]
 
 
 @pytest.mark.parametrize("N,IC,H,W,OC", POINTWISE)
