@@ -76,6 +76,24 @@ def test_random_conv_geometries(dev, seed):
         assert np.array_equal(to_np(dX1), to_np(dX2)) and np.array_equal(to_np(dW1), to_np(dW2)), shape
 
 
+@pytest.mark.parametrize("seed", [31, 32])
+def test_random_large_pointwise_layers(dev, seed):
+    """1x1 layers with enough pixels per call for the kernels that stream the activations straight into the matrix
+    instructions (at least 32768 pixels, at most 64 channels on the short side) and for the pixel-contraction weight
+    gradient: ragged channel counts on both sides, 8- and 16-byte pixel vectors, more than one filter staging pass."""
+    rng = random.Random(seed)
+    for i in range(6):
+        H, W = rng.choice([(32, 32), (32, 32), (16, 32), (64, 16), (16, 16)])
+        N = rng.choice([32, 40, 64, 72, 136]) * (4 if H * W == 256 else (2 if H * W == 512 else 1))
+        IC, OC = rng.choice([5, 24, 50, 97, 204, 270, 300]), rng.choice([1, 12, 20, 33, 48, 50, 64])
+        if N * IC * H * W > 24_000_000:
+            N = max(32 * 1024 // (H * W), N // 2)
+        shape = (N, IC, H, W, OC, 1, 1, 1, 1, 0, 0)
+        bias = rng.random() < 0.5
+        print("pointwise", seed, i, shape, bias, flush=True)
+        run_layer(dev, *shape, bias=bias, seed=100 * seed + i, ws=rng.random() < 0.5)
+
+
 @pytest.mark.parametrize("seed", [21, 22])
 def test_random_gemm_shapes(dev, seed):
     rng = random.Random(seed)
