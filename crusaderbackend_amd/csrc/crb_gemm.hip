@@ -204,7 +204,7 @@ static int gemm_tn(const float *A, const float *B, float *C, u32 M, u32 N, u32 K
 
 static int gemm_nt(const float *A, const float *B, float *C, u32 M, u32 N, u32 K, const float *col_bias, u32 flags,
                    hipStream_t s, const char *what) {
-    if (tiny_gemm_fits(M, N, K, 1))  // A (M x K) row-major, B stored N x K
+    if (tiny_gemm_fits(M, N, K, 1, true))  // A (M x K) row-major, B stored N x K
         return launch_tiny_gemm(TinyGemmArgs{A, B, C, col_bias, nullptr, M, N, K, K, 1, 1, K, N, flags}, K, 0, 0, s, what);
     RowMajorEpi e{C, col_bias, N, 0, flags};
     if (K % 4 == 0 && aligned16(A) && aligned16(B)) {

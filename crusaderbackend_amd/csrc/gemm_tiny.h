@@ -121,8 +121,13 @@ __global__ void __launch_bounds__(256) tiny_gemm_kernel(TinyGemmArgs a) {
 // Whether the one-launch form takes a product: a small result, a contraction short enough that a quarter of it per wave is
 // a few dozen MFMA steps, and enough 16 x 16 blocks (or little enough work) that the chip is not left idle for long.
 // K: the whole contraction (batch * K for the K-concatenated accumulate-NT form); batch: independent products (must be 1).
-inline bool tiny_gemm_fits(u32 M, u32 N, u32 K, u32 batch) {
+// kfast: both operands are contiguous along k (the NT forms: 16-byte loads). Every block re-reads its operand rows from L2,
+// so beyond 2^27 multiply-adds (2^26 with scalar loads) the staged engine wins again (measured, batch 128: 1024 x 1024 one
+// launch 9.6 us against 12.9, 1024 x 4096 32.4 against 22.6; data-gradient form 1024 x 512 9.6 against 11.4, 1024 x 1024
+// 17.7 against 12.8).
+inline bool tiny_gemm_fits(u32 M, u32 N, u32 K, u32 batch, bool kfast = false) {
     if (batch != 1 || uint64_t(M) * N > 512u * 512u || K > 4096u) return false;
+    if (uint64_t(M) * N * K > (uint64_t(1) << (kfast ? 27 : 26))) return false;
     const u32 blocks = ceil_div(M, 16u) * ceil_div(N, 16u);
     return blocks >= 64u || uint64_t(M) * N * K <= (1u << 22);
 }
