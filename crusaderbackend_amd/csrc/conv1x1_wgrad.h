@@ -3,11 +3,11 @@
 // operands both lie pixel-contiguous in NCHW memory, read once each (the pass is bandwidth-bound).
 //
 // A workgroup owns ALL output channels (NOB blocks of 16, OC <= 16 * NOB), four blocks of 16 input channels (block
-// w * groups + g for wave w of group g) and a slice z of
-// the (image, 64-pixel run) tiles. Per tile it stages the dY planes and its 64 X planes in double-buffered LDS (16-byte
-// global loads of whole 256-byte runs); wave w multiplies ic block w against every oc block, so a staged dY value feeds
-// NOB MFMAs per wave and no accumulator is shared between waves (no cross-wave reduction). One partial result per
-// (ic group, z), summed in fixed order by the split reduction: bit-reproducible.
+// w * groups + g for wave w of group g) and a slice z of the (image, 64-pixel run) tiles. Per tile it stages the dY planes
+// and its 64 X planes in double-buffered LDS (16-byte global loads of whole 256-byte runs); wave w multiplies its ic block
+// against every oc block, so a staged dY value feeds NOB MFMAs per wave and no accumulator is shared between waves (no
+// cross-wave reduction). One partial result per (ic group, z), summed in fixed order by the split reduction:
+// bit-reproducible.
 //
 // v_mfma_f32_16x16x4_f32 (wave64, lane l): A = dY[oc = l%16][pixel 4s + l/16], B = X[pixel 4s + l/16][ic = l%16],
 // accumulator register r = dW[oc = 4*(l/16) + r][ic = l%16].
