@@ -422,7 +422,10 @@ def main():
     A = torch.rand(n, n, device=dev) * 2 - 1
     B = torch.rand(n, n, device=dev) * 2 - 1
     C = torch.empty(n, n, device=dev)
-    gemm_ms = event_time_ms(torch, lambda: capi.sgemm_nn(A, B, C, n, n, n), reps=10)
+    # three averages of ten launches: the first follows the allocations above, with the device clock still ramping up, and
+    # reads several per cent high; the smallest is reported and all three are kept in `extra`
+    gemm_runs = [event_time_ms(torch, lambda: capi.sgemm_nn(A, B, C, n, n, n), reps=10) for _ in range(3)]
+    gemm_ms = min(gemm_runs)
     gemm_tflops = 2.0 * n ** 3 / gemm_ms / 1e9
     del A, B, C
 
@@ -449,7 +452,7 @@ def main():
             "resnet56_conv_images_per_s": images_per_s,
             "resnet56_conv_images_per_s_kernel_only": BATCH / (kern_sum_ms / 1e3),
             "kernel_only_tflops": step_flops / kern_sum_ms / 1e9,
-            "sgemm_4096_tflops": gemm_tflops, "sgemm_4096_ms": gemm_ms,
+            "sgemm_4096_tflops": gemm_tflops, "sgemm_4096_ms": gemm_ms, "sgemm_4096_ms_runs": gemm_runs,
             "sgemm_4096_frac_peak": gemm_tflops / PEAK_FP32_MFMA_TFLOPS,
             "slice_sum_all_layers_ms": sum_ms, "slice_sum_items": len(slice_entries),
             "per_kernel": {k: {"ms": round(v["ms"], 5), "tflops": round(v["tflops"], 2), "gbs": round(v["gbs"], 1)}
