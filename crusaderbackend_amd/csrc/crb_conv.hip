@@ -2,6 +2,7 @@
 // standalone bias add, all as implicit GEMMs on the MFMA engine (no im2col buffer is materialised).
 #include "conv3x3_direct.h"
 #include "conv3x3_wgrad.h"
+#include "conv3x3_wgrad_image.h"
 #include "conv1x1_s2.h"
 #include "conv1x1_wgrad.h"
 #include "conv1x1_stream.h"
@@ -337,6 +338,11 @@ static bool wgrad_cfg2(const crb_conv_geom *g, bool run, const float *dY, const 
 }
 static bool wgrad_direct(const crb_conv_geom *g, bool run, const float *dY, const float *X, float *dW, float *ws,
                          hipStream_t s, WgradDirectPlan &plan, int &status) {
+    if (direct_shape(g, 1) && wgrad_image_fits(g->IC, g->OH, g->OW)) {  // image layers: (channel, tap) pairs on the MFMA columns
+        plan = wgrad_image_plan(g->N, g->IC, g->OC, g->OH);
+        if (run) status = launch_wgrad_image(dY, X, dW, ws, plan, g->IC, g->OC, g->OH, s, "crb_conv_wgrad");
+        return true;
+    }
     if (direct_shape(g, 1)) {
         if (g->OW == 32) return wgrad_cfg2<32, 8, 1, 2, 1>(g, run, dY, X, dW, ws, s, plan, status);
         if (g->OW == 16)

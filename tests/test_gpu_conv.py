@@ -125,6 +125,14 @@ def test_conv_vgg_stem_and_wide(dev):
     run_layer(dev, 2, 256, 4, 4, 512, 3, 3, 1, 1, 1, 1, bias=True, seed=8)
 
 
+# image layers (at most 3 input channels, 32 wide): the weight gradient with (channel, tap) pairs on the MFMA columns;
+# ragged output-channel blocks, 1-3 input channels, slices of one and of several tiles, a ragged last slice
+@pytest.mark.parametrize("N,IC,H,OC", [(128, 3, 32, 16), (128, 3, 32, 64), (5, 1, 8, 5), (7, 2, 16, 20), (200, 3, 32, 33), (1, 3, 8, 130)])
+def test_conv_image_layers(dev, N, IC, H, OC):
+    run_layer(dev, N, IC, H, 32, OC, 3, 3, 1, 1, 1, 1, bias=True, seed=19)
+    run_layer(dev, N, IC, H, 32, OC, 3, 3, 1, 1, 1, 1, bias=False, seed=20, ws=True)
+
+
 @pytest.mark.parametrize("IC,H,OC,s", RESNET)
 def test_conv_full_batch_adjoint(dev, IC, H, OC, s):
     """Size-independent property at the full benchmark batch (128): <conv(W,X), dY> = <X, dgrad(W,dY)> =
