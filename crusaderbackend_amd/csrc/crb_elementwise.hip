@@ -331,14 +331,27 @@ __global__ void __launch_bounds__(256) batchnorm_fwd_kernel(const float *__restr
     const BnGeom<FL> t(F);
     const bool cached = N <= G * kBnCache;
     const float *x = X + (t.on ? t.f : 0);
-    float xv[kBnCache];
+    // Cached sweeps load unconditionally (a sample past the batch reads row 0, a feature past the extent column 0) and drop
+    // what does not count afterwards: with a branch around every load the compiler puts each load next to its use, and a
+    // sweep becomes one memory round trip per sample instead of one in all.
+    float xv[kBnCache], av[kBnCache];
     float s = 0.f;
     if (cached) {
 #pragma unroll
         for (int i = 0; i < kBnCache; ++i) {
             const u32 n = t.g + G * i;
-            xv[i] = (t.on && n < N) ? x[size_t(n) * F] : 0.f;
+            xv[i] = x[size_t(n < N ? n : 0) * F];
         }
+        if (reluOut && addend) {  // the other summand of the residual connection: requested with the first sweep
+            const float *ad = addend + (t.on ? t.f : 0);
+#pragma unroll
+            for (int i = 0; i < kBnCache; ++i) {
+                const u32 n = t.g + G * i;
+                av[i] = ad[size_t(n < N ? n : 0) * F];
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < kBnCache; ++i) xv[i] = (t.on && t.g + G * i < N) ? xv[i] : 0.f;
 #pragma unroll
         for (int i = 0; i < kBnCache; ++i) s += xv[i];
     } else if (t.on) {
@@ -363,12 +376,12 @@ __global__ void __launch_bounds__(256) batchnorm_fwd_kernel(const float *__restr
     const float inv = 1.0f / sqrtf(v + 1e-8f), ga = gamma[t.f], be = beta[t.f];
     // outputs a caller does not need are not written: Y and xHat may be null; reluOut = max(Y + addend, 0) is optional
     // (addend: the other summand of a residual connection that closes right behind this normalisation, or null)
-    auto put = [&](u32 n, float xh) {
+    auto put = [&](u32 n, float xh, float add) {
         const float y = xh * ga + be;
         if (xHat) xHat[size_t(n) * F + t.f] = xh;
         if (Y) Y[size_t(n) * F + t.f] = y;
         if (reluOut) {
-            const float z = addend ? y + addend[size_t(n) * F + t.f] : y;
+            const float z = addend ? y + add : y;
             reluOut[size_t(n) * F + t.f] = z > 0.f ? z : 0.f;
         }
     };
@@ -376,10 +389,10 @@ __global__ void __launch_bounds__(256) batchnorm_fwd_kernel(const float *__restr
 #pragma unroll
         for (int i = 0; i < kBnCache; ++i) {
             const u32 n = t.g + G * i;
-            if (n < N) put(n, (xv[i] - m) * inv);
+            if (n < N) put(n, (xv[i] - m) * inv, (reluOut && addend) ? av[i] : 0.f);
         }
     } else {
-        for (u32 n = t.g; n < N; n += G) put(n, (x[size_t(n) * F] - m) * inv);
+        for (u32 n = t.g; n < N; n += G) put(n, (x[size_t(n) * F] - m) * inv, (reluOut && addend) ? addend[size_t(n) * F + t.f] : 0.f);
     }
     if (t.g == 0) mean[t.f] = m, var[t.f] = v;
 }
@@ -411,32 +424,25 @@ __global__ void __launch_bounds__(256) batchnorm_bwd_kernel(const float *__restr
     float xv[kBnCache], dv[kBnCache];
     float s = 0.f;
     if (cached) {
+        // every load of the sweep is issued, unconditionally (a sample past the batch reads row 0), before any is used: with
+        // a branch around a load the compiler puts it next to its use, one memory round trip per sample
+        float ev[SUM2 ? kBnCache : 1], mv[MASK ? kBnCache : 1];
 #pragma unroll
         for (int i = 0; i < kBnCache; ++i) {
             const u32 n = t.g + G * i;
-            const bool ok = t.on && n < N;
-            xv[i] = ok ? x[size_t(n) * F] : 0.f;
-            dv[i] = ok ? dy[size_t(n) * F] : 0.f;
+            const size_t row = size_t(n < N ? n : 0) * F;
+            xv[i] = x[row];
+            dv[i] = dy[row];
+            if (SUM2) ev[i] = dy2[row];
+            if (MASK) mv[i] = mk[row];
         }
-        if (SUM2) {  // all loads of the sweep are issued before any is used
-            float ev[kBnCache];
 #pragma unroll
-            for (int i = 0; i < kBnCache; ++i) {
-                const u32 n = t.g + G * i;
-                ev[i] = (t.on && n < N) ? dy2[size_t(n) * F] : 0.f;
-            }
-#pragma unroll
-            for (int i = 0; i < kBnCache; ++i) dv[i] = dv[i] + ev[i];
-        }
-        if (MASK) {
-            float mv[kBnCache];
-#pragma unroll
-            for (int i = 0; i < kBnCache; ++i) {
-                const u32 n = t.g + G * i;
-                mv[i] = (t.on && n < N) ? mk[size_t(n) * F] : 0.f;
-            }
-#pragma unroll
-            for (int i = 0; i < kBnCache; ++i) dv[i] = mv[i] > 0.f ? dv[i] : 0.f;
+        for (int i = 0; i < kBnCache; ++i) {
+            const bool ok = t.on && t.g + G * i < N;
+            if (SUM2) dv[i] = dv[i] + ev[i];
+            if (MASK) dv[i] = mv[i] > 0.f ? dv[i] : 0.f;
+            xv[i] = ok ? xv[i] : 0.f;
+            dv[i] = ok ? dv[i] : 0.f;
         }
 #pragma unroll
         for (int i = 0; i < kBnCache; ++i) s += xv[i];
