@@ -193,7 +193,10 @@ static int try_direct(const float *Wt, const float *X, float *Y, const float *bi
         }
     } else {
         if (gW == 32) {
-            if (C_OUT > 16) { CRB_TRY(32, 8, 8, 32, 4, 2, DG, 2, 2, 2) }
+            // forward only: the data gradient holds four parity classes per MFMA tile, and 32 of them do not fit the registers
+            if constexpr (!DG) {
+                if (C_OUT > 16) { CRB_TRY(32, 8, 8, 32, 4, 2, false, 2, 2, 2) }
+            }
             CRB_TRY(32, 8, 8, 16, 4, 1, DG, 2, 2, 2)
             CRB_TRY(32, 4, 8, 16, 2, 1, DG, 2, 2, 2)
         } else if (gW == 16) {

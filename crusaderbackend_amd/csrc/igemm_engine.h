@@ -405,6 +405,21 @@ __global__ void __launch_bounds__(Cfg::NTH, Cfg::OCC) igemm_kernel(AOp a, BOp b,
     if (!old_tried) fetch_old();  // empty contraction range
     // epilogue: accumulator register r of lane l is D[8*(r/4) + 4*(l/32) + r%4][l%32] of its block
     const int j = lane & 31, h = lane >> 5;
+    // the per-row bias of the 16 rows a lane holds of row block mi: requested together (a load in front of every store
+    // would be a memory round trip per element), live for that block only
+    float rowb[16];
+    auto fetch_row_bias = [&](int mi) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) rowb[r] = 0.f;
+        if (epi.has_row_bias()) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int id = 8 * (r / 4) + 4 * h + (r % 4);
+                const u32 row = row0 + wave_m * Cfg::WTM + (AOp::kKFast ? mi * 32 + id : id * TM + mi);
+                rowb[r] = epi.row_bias_at(row < d.M ? row : d.M - 1);
+            }
+        }
+    };
     if constexpr (!BOp::kKFast && TN == 2 && Epi::kPairStore) {
         // row-fast B: a lane's two blocks are neighbouring columns, stored (and, accumulating, loaded) as one 8-byte access,
         // so that a store instruction writes whole 256-byte runs instead of every other float of them
@@ -412,12 +427,13 @@ __global__ void __launch_bounds__(Cfg::NTH, Cfg::OCC) igemm_kernel(AOp a, BOp b,
         const typename Epi::ColS c0 = epi.prep_col(col, d.N), c1 = epi.prep_col(col + 1, d.N);
 #pragma unroll
         for (int mi = 0; mi < TM; ++mi) {
+            fetch_row_bias(mi);
             if (old_ok) fetch_old_block(mi, 0), have_old = true;
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
                 const int id = 8 * (r / 4) + 4 * h + (r % 4);
                 const u32 row = row0 + wave_m * Cfg::WTM + (AOp::kKFast ? mi * 32 + id : id * TM + mi);
-                if (row < d.M && c0.ok) epi.store2(row, c0, c1, acc[mi][0][r], acc[mi][1][r], have_old, oldv[r], oldv[kPair ? 16 + r : 0]);
+                if (row < d.M && c0.ok) epi.store2(row, c0, c1, acc[mi][0][r], acc[mi][1][r], rowb[r], have_old, oldv[r], oldv[kPair ? 16 + r : 0]);
             }
         }
     } else {
@@ -427,6 +443,7 @@ __global__ void __launch_bounds__(Cfg::NTH, Cfg::OCC) igemm_kernel(AOp a, BOp b,
             const typename Epi::ColS cs = epi.prep_col(col, d.N);
 #pragma unroll
             for (int mi = 0; mi < TM; ++mi) {
+                fetch_row_bias(mi);
                 if constexpr (!kOldEarly) {
                     if (old_ok) fetch_old_block(mi, ni), have_old = true;
                 }
@@ -434,7 +451,7 @@ __global__ void __launch_bounds__(Cfg::NTH, Cfg::OCC) igemm_kernel(AOp a, BOp b,
                 for (int r = 0; r < 16; ++r) {
                     const int id = 8 * (r / 4) + 4 * h + (r % 4);
                     const u32 row = row0 + wave_m * Cfg::WTM + (AOp::kKFast ? mi * 32 + id : id * TM + mi);
-                    if (row < d.M) epi.store(row, cs, acc[mi][ni][r], have_old, oldv[r]);
+                    if (row < d.M) epi.store(row, cs, acc[mi][ni][r], rowb[r], have_old, oldv[r]);
                 }
             }
         }

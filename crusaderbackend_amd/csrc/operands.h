@@ -286,11 +286,15 @@ struct RowMajorEpi {
     }
     __device__ __forceinline__ const float *at(u32 row, u32 col) const { return C + size_t(row) * ld + col; }
     __device__ __forceinline__ bool pair_aligned(u32 col) const { return ld % 2 == 0 && (reinterpret_cast<uintptr_t>(C + col) & 7u) == 0; }
-    __device__ __forceinline__ void store(u32 row, const ColS &c, float v, bool have_old = false, float old = 0.f) const {
+    // The per-row bias of a lane's rows is loaded by the caller in one batch (row_bias_at) and handed in as `rowb`: a load
+    // in front of every store would be a memory round trip per element.
+    __device__ __forceinline__ bool has_row_bias() const { return row_bias != nullptr; }
+    __device__ __forceinline__ float row_bias_at(u32 row) const { return row_bias[row]; }
+    __device__ __forceinline__ void store(u32 row, const ColS &c, float v, float rowb, bool have_old = false, float old = 0.f) const {
         if (!c.ok) return;
         float *p = C + size_t(row) * ld + c.col;
         v += c.bias;
-        if (row_bias) v += row_bias[row];
+        v += rowb;
         if (have_old)
             v += old;
         else if (flags & EPI_ACCUM)
@@ -300,19 +304,16 @@ struct RowMajorEpi {
     }
     // Two neighbouring columns of one row (c1.col == c0.col + 1) as one 8-byte access where the address allows it.
     static constexpr bool kPairStore = true;
-    __device__ __forceinline__ void store2(u32 row, const ColS &c0, const ColS &c1, float v0, float v1, bool have_old = false,
+    __device__ __forceinline__ void store2(u32 row, const ColS &c0, const ColS &c1, float v0, float v1, float rowb, bool have_old = false,
                                            float old0 = 0.f, float old1 = 0.f) const {
         float *p = C + size_t(row) * ld + c0.col;
         if (!c1.ok || (reinterpret_cast<uintptr_t>(p) & 7u)) {
-            store(row, c0, v0, have_old, old0);
-            store(row, c1, v1, have_old, old1);
+            store(row, c0, v0, rowb, have_old, old0);
+            store(row, c1, v1, rowb, have_old, old1);
             return;
         }
         v0 += c0.bias, v1 += c1.bias;
-        if (row_bias) {
-            const float rb = row_bias[row];
-            v0 += rb, v1 += rb;
-        }
+        v0 += rowb, v1 += rowb;
         if (have_old) {
             v0 += old0, v1 += old1;
         } else if (flags & EPI_ACCUM) {
@@ -348,7 +349,9 @@ struct NchwEpi {
     static constexpr bool kPrefetchOld = false;
     static constexpr bool kEarlyOld = false;
     static constexpr bool kRowSum = false;
-    __device__ __forceinline__ void store2(u32, const ColS &, const ColS &, float, float, bool, float, float) const {}
+    __device__ __forceinline__ void store2(u32, const ColS &, const ColS &, float, float, float, bool, float, float) const {}
+    __device__ __forceinline__ bool has_row_bias() const { return row_bias != nullptr; }
+    __device__ __forceinline__ float row_bias_at(u32 row) const { return row_bias[row]; }
     __device__ __forceinline__ void bind(u32 z) { T += size_t(z) * zstride; }
     __device__ __forceinline__ ColS prep_col(u32 col, u32 ncols) const {
         u32 n, p;
@@ -358,9 +361,9 @@ struct NchwEpi {
     __device__ __forceinline__ bool accum_interior(u32, u32, u32, u32, u32, u32) const { return false; }
     __device__ __forceinline__ const float *at(u32, u32) const { return nullptr; }
     __device__ __forceinline__ bool pair_aligned(u32) const { return false; }
-    __device__ __forceinline__ void store(u32 row, const ColS &c, float v, bool = false, float = 0.f) const {
+    __device__ __forceinline__ void store(u32 row, const ColS &c, float v, float rowb, bool = false, float = 0.f) const {
         if (!c.ok) return;
-        if (row_bias) v += row_bias[row];
+        v += rowb;
         if (flags & EPI_RELU) v = v > 0.0f ? v : 0.0f;
         T[c.off + row * HW] = v;
     }
