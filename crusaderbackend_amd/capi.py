@@ -130,6 +130,36 @@ def _stream(stream):
     return None if stream is None else stream.cuda_stream
 
 
+def prepared(name, *args):
+    """A zero-argument callable that issues entry point `name` with `args` converted once (tensors to their device
+    addresses, a ConvGeom to a reference to it, the rest as given, in the order of the C declaration). A timing loop over
+    the plain wrappers spends 3.5-4.5 us per call in argument conversion, which hides every kernel shorter than that; a
+    prepared call costs about a microsecond. The tensors and the geometry must outlive the callable."""
+    fn = getattr(load(), name)
+    conv, keep = [], []
+    for a in args:
+        if a is None or isinstance(a, int):
+            conv.append(a)
+        elif isinstance(a, ConvGeom):
+            keep.append(a)
+            conv.append(ctypes.byref(a))
+        elif hasattr(a, "data_ptr"):
+            keep.append(a)
+            conv.append(ctypes.c_void_p(a.data_ptr()))
+        elif hasattr(a, "cuda_stream"):
+            conv.append(ctypes.c_void_p(a.cuda_stream))
+        else:
+            conv.append(a)
+    conv = tuple(conv)
+
+    def call(_keep=keep):
+        st = fn(*conv)
+        if st != CRB_OK:
+            check(st)
+
+    return call
+
+
 # Thin helpers over torch CUDA tensors (device memory + streams only; no torch math).
 def sgemm_nn(A, B, C, M, N, K, batch=1, stream=None):
     check(load().crb_sgemm_nn(_p(A), _p(B), _p(C), M, N, K, batch, _stream(stream)))

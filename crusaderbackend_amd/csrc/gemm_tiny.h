@@ -43,6 +43,15 @@ __global__ void __launch_bounds__(256) tiny_gemm_kernel(TinyGemmArgs a) {
     const u32 kb = wave * a.k_per_wave;
     const u32 ke = kb + a.k_per_wave < a.K ? kb + a.k_per_wave : a.K;
     const bool row_ok = row0 + li < a.M, col_ok = col0 + li < a.N;
+    // What the epilogue adds to the element this thread finishes (row t / 16, column t % 16) is requested now: loaded at
+    // the end, bias and previous value would each cost a memory round trip of their own.
+    const u32 er = t >> 4, ec = t & 15;
+    const u32 erow = row0 + er, ecol = col0 + ec;
+    const bool e_ok = erow < a.M && ecol < a.N;
+    float *ep = a.C + size_t(e_ok ? erow : 0) * a.ldc + (e_ok ? ecol : 0);
+    const float e_cb = (a.col_bias && e_ok) ? a.col_bias[ecol] : 0.f;
+    const float e_rb = (a.row_bias && e_ok) ? a.row_bias[erow] : 0.f;
+    const float e_old = ((a.flags & EPI_ACCUM) && e_ok) ? *ep : 0.f;
     v4f acc = {0.f, 0.f, 0.f, 0.f};
     float asum = 0.f;  // this lane's share of row li's sum of A
     if constexpr (KVEC) {
@@ -103,19 +112,16 @@ __global__ void __launch_bounds__(256) tiny_gemm_kernel(TinyGemmArgs a) {
         a.a_rowsum[row0 + t] += v;
     }
     // thread t finishes element (row t / 16, column t % 16): register row % 4 of lane (row / 4) * 16 + column
-    const u32 r = t >> 4, c = t & 15;
-    const u32 row = row0 + r, col = col0 + c;
-    if (row >= a.M || col >= a.N) return;
-    const u32 e = ((r >> 2) * 16 + c) * 4 + (r & 3);
+    if (!e_ok) return;
+    const u32 e = ((er >> 2) * 16 + ec) * 4 + (er & 3);
     float v = red[e];
 #pragma unroll
     for (int w = 1; w < 4; ++w) v += red[w * 256 + e];
-    float *p = a.C + size_t(row) * a.ldc + col;
-    if (a.col_bias) v += a.col_bias[col];
-    if (a.row_bias) v += a.row_bias[row];
-    if (a.flags & EPI_ACCUM) v += *p;
+    if (a.col_bias) v += e_cb;
+    if (a.row_bias) v += e_rb;
+    if (a.flags & EPI_ACCUM) v += e_old;
     if (a.flags & EPI_RELU) v = v > 0.f ? v : 0.f;
-    *p = v;
+    *ep = v;
 }
 
 // Whether the one-launch form takes a product: a small result, a contraction short enough that a quarter of it per wave is
