@@ -28,10 +28,15 @@ def run(torch, capi, dev, event_time_ms, Layer):
         return torch.rand(*shape, device=dev) * 2 - 1
 
     def settled(fn, reps):
-        """GEMM-family rows: the smallest of three averages over `reps` launches. These rows follow tensor allocation and
-        host work during which the device clock drops, and its ramp back up takes longer than three warm-up launches: the
-        first average of such a row reads 5-15 % high."""
-        return min(event_time_ms(torch, fn, reps=reps) for _ in range(3))
+        """One row's time: the call is frozen (argument conversion done once: a plain wrapper call costs the host 3.5-4.5 us,
+        more than the shortest kernels take), repeated until the timed region is at least a millisecond, and the smallest
+        of three such averages is kept. Rows follow tensor allocation and host work during which the device clock drops,
+        and its ramp back up takes longer than three warm-up launches: a first average reads 5-15 % high."""
+        f = capi.frozen(fn)
+        ms = event_time_ms(torch, f, reps=reps)
+        if ms * reps < 1.0:
+            reps = min(4000, int(1.0 / ms) + 1)
+        return min(event_time_ms(torch, f, reps=reps) for _ in range(3))
 
     # config 1 + target GEMM
     for n in (1024, 4096):
@@ -47,7 +52,7 @@ def run(torch, capi, dev, event_time_ms, Layer):
                 if pname in ("bwd", "bwd_sliced") and key != "resnet56":  # the one-call forms of both gradients: residual-network shapes
                     continue
                 reps = 30 if L.flops < 2e9 else 10
-                entries[pname] = _entry(f"{name}.{pname}", event_time_ms(torch, fn, reps=reps), fl, L.bytes[pname])
+                entries[pname] = _entry(f"{name}.{pname}", settled(fn, reps), fl, L.bytes[pname])
                 out[key].append(entries[pname])
             # Bandwidth-bound shapes also get a cold-cache figure: the same call cycled over enough distinct buffer sets
             # (>= 640 MB in total, beyond L2 and the 256 MB memory-side cache) that no launch finds its operands cached.
@@ -93,9 +98,9 @@ def run(torch, capi, dev, event_time_ms, Layer):
         f_fwd = capi.prepared("crb_linear_fwd", X, W, bias, Y, b, IN, OUT, 0, None)
         f_dgrad = capi.prepared("crb_linear_dgrad", dY, W, dX, b, IN, OUT, None)
         f_wgrad = capi.prepared("crb_linear_wgrad", dY, X, dW, dB, b, IN, OUT, None)
-        out["vgg16"].append(_entry(f"fc{IN}-{OUT}.fwd", event_time_ms(torch, f_fwd, 100), fl, by))
-        out["vgg16"].append(_entry(f"fc{IN}-{OUT}.dgrad", event_time_ms(torch, f_dgrad, 100), fl, by))
-        out["vgg16"].append(_entry(f"fc{IN}-{OUT}.wgrad", event_time_ms(torch, f_wgrad, 100), fl, by))
+        out["vgg16"].append(_entry(f"fc{IN}-{OUT}.fwd", settled(f_fwd, 100), fl, by))
+        out["vgg16"].append(_entry(f"fc{IN}-{OUT}.dgrad", settled(f_dgrad, 100), fl, by))
+        out["vgg16"].append(_entry(f"fc{IN}-{OUT}.wgrad", settled(f_wgrad, 100), fl, by))
 
     # config 4: DenseNet-BC-100 (k = 12), batch 64: first / middle / last bottleneck of each stage + the 3x3
     dn = []
@@ -170,7 +175,7 @@ def run(torch, capi, dev, event_time_ms, Layer):
     out["elementwise"] = []
 
     def ew(name, fn, nbytes, reps=30):
-        ms = event_time_ms(torch, fn, reps=reps)
+        ms = settled(fn, reps)
         out["elementwise"].append({"name": name, "us": round(ms * 1e3, 2), "gflop": 0.0, "mbytes": round(nbytes / 1e6, 2), "ai": 0.0,
                                    "tflops": 0.0, "gbs": round(nbytes / ms / 1e6, 1), "bound": "hbm",
                                    "frac": round(nbytes / ms / 1e6 / PEAK_GBS, 4)})

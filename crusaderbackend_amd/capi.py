@@ -160,6 +160,58 @@ def prepared(name, *args):
     return call
 
 
+class _Recorder:
+    """Stands in for the library while `frozen` runs a wrapper once: passes every call through and notes the launching
+    ones (those that return a status) with their converted arguments."""
+
+    def __init__(self, lib):
+        self._lib, self.calls = lib, []
+
+    def __getattr__(self, name):
+        fn = getattr(self._lib, name)
+        if fn.restype is not ctypes.c_int or name == "crb_abi_version":
+            return fn  # size queries, error text: needed by the wrapper now, not part of the replay
+
+        def passthrough(*args):
+            self.calls.append((fn, args))
+            return fn(*args)
+
+        return passthrough
+
+
+def frozen(fn):
+    """Runs `fn` (any composition of the wrappers below) once and returns a zero-argument callable that re-issues the
+    same entry points with the same already-converted arguments. For timing loops over short kernels, like `prepared`,
+    without spelling the C argument list out. Every tensor `fn` touches must outlive the callable; host-side decisions
+    `fn` makes (workspace sizes, branches) are frozen with it."""
+    global _lib
+    real = load()
+    rec = _Recorder(real)
+    _lib = rec
+    try:
+        fn()
+    finally:
+        _lib = real
+    calls = tuple(rec.calls)
+    if not calls:  # `fn` does not go through the wrappers (already prepared calls): nothing to freeze
+        return fn
+    if len(calls) == 1:
+        f, a = calls[0]
+
+        def call():
+            st = f(*a)
+            if st != CRB_OK:
+                check(st)
+    else:
+        def call():
+            for f, a in calls:
+                st = f(*a)
+                if st != CRB_OK:
+                    check(st)
+    call.keep = fn  # the closure of `fn` holds the tensors
+    return call
+
+
 # Thin helpers over torch CUDA tensors (device memory + streams only; no torch math).
 def sgemm_nn(A, B, C, M, N, K, batch=1, stream=None):
     check(load().crb_sgemm_nn(_p(A), _p(B), _p(C), M, N, K, batch, _stream(stream)))

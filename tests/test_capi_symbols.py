@@ -40,3 +40,24 @@ def test_conv_geom_layout_matches_header():
     assert ctypes.sizeof(capi.ConvGeom) == 13 * 4
     g = capi.ConvGeom.make(128, 16, 32, 32, 32, 3, 3, 2, 2, 1, 1)
     assert (g.OH, g.OW) == (16, 16)
+
+
+def test_frozen_call_replays_the_launching_calls_only():
+    # null operands fail validation before any device work: the replay must issue the same call and raise the same error
+    seen = []
+
+    def wrapper():
+        seen.append(capi.gemm_workspace_bytes(64, 64, 64, 1))  # a size query: used by the wrapper, not replayed
+        lib = capi.load()
+        seen.append(lib.crb_sgemm_nn(None, None, None, 1, 1, 1, 1, None))
+
+    call = capi.frozen(wrapper)
+    assert seen[1] == capi.CRB_ENULL
+    assert capi.load() is not None and not isinstance(capi.load(), capi._Recorder)  # the library is back in place
+    try:
+        call()
+    except capi.CrbError as e:
+        assert "null operand" in str(e)
+    else:
+        raise AssertionError("the frozen call did not re-issue crb_sgemm_nn")
+    assert len(seen) == 2  # the wrapper itself did not run again

@@ -297,3 +297,19 @@ def test_batchnorm_relu_with_residual_parts_equals_separate_calls(dev, N, C, H, 
     d1, d2 = _nan(dev, N * F), _nan(dev, N * F)
     capi.tensor_relu_grad_copy2(d1, d2, R, dY, N * F, dY2=dY2)
     assert np.array_equal(to_np(d1).ravel(), to_np(dZ).ravel()) and np.array_equal(to_np(d2).ravel(), to_np(dZ).ravel())
+
+
+def test_prepared_and_frozen_calls_match_the_plain_wrapper(dev):
+    import torch
+    capi = _capi()
+    n = 4099
+    x = normal(11, n)
+    X = to_dev(x, dev)
+    want = np.maximum(x, 0)
+    for make in (lambda Y: capi.prepared("crb_relu_fwd", X, Y, n, None), lambda Y: capi.frozen(lambda: capi.relu_fwd(X, Y, n))):
+        Y = _nan(dev, n)
+        call = make(Y)
+        Y.fill_(float("nan"))
+        call()
+        torch.cuda.synchronize()
+        np.testing.assert_array_equal(to_np(Y), want)
