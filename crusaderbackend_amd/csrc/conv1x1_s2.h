@@ -10,7 +10,7 @@
 namespace crb {
 
 constexpr u32 kScMaxC = 64;  // channel limit of both kernels
-constexpr u32 kScTile = 64;  // output pixels per staged tile of the weight gradient
+constexpr u32 kScTile = 64;  // output pixels per staged tile of the weight gradient (32 when that is what fills the chip)
 
 // One thread per (image, output row, group of 4 input channels, output column): adjacent lanes write adjacent 8-byte pairs
 // {value, 0} of an even dX row and {0, 0} of the odd row below it. Summation over oc in ascending order.
@@ -45,15 +45,17 @@ __global__ void __launch_bounds__(256) sc_dgrad_kernel(const float *__restrict__
     }
 }
 
-// Workgroup z sums its run of 64-pixel tiles into part[z][oc][ic]. A tile is staged pixel-major in LDS (dY: 64 x OC, X at the
-// even positions: 64 x IC); a thread owns one output channel and four input channels (task = oc * IC/4 + ic/4; with at most
+// Workgroup z sums its run of PT-pixel tiles into part[z][oc][ic]. A tile is staged pixel-major in LDS (dY: PT x OC, X at the
+// even positions: PT x IC; every load of a tile is issued before the first is stored, a pixel past the end reads the last
+// one and is zeroed on the way to LDS); a thread owns one output channel and four input channels (task = oc * IC/4 + ic/4; with at most
 // 128 tasks the pixels of a tile are shared out over 256 / tasks subsets, combined in subset order at the end). Pixels in
 // ascending order within a thread: a fixed association.
+template <u32 PT>
 __global__ void __launch_bounds__(256) sc_wgrad_kernel(const float *__restrict__ dY, const float *__restrict__ X, float *__restrict__ part,
                                                        u32 IC, u32 OC, u32 OH, u32 OW, u32 total_px, u32 tiles_per_z, FastDiv d_ow,
                                                        FastDiv d_ohw) {
-    __shared__ float sY[kScTile][kScMaxC + 1];
-    __shared__ __attribute__((aligned(16))) float sX[kScTile][kScMaxC + 4];
+    __shared__ float sY[PT][kScMaxC + 1];
+    __shared__ __attribute__((aligned(16))) float sX[PT][kScMaxC + 4];
     __shared__ __attribute__((aligned(16))) v4f red[256];
     const u32 tasks = OC * (IC / 4);
     const u32 nsub = tasks <= 128 ? 256 / tasks : 1;     // pixel subsets per tile
@@ -65,21 +67,31 @@ __global__ void __launch_bounds__(256) sc_wgrad_kernel(const float *__restrict__
     v4f acc[4];
 #pragma unroll
     for (int k = 0; k < 4; ++k) acc[k] = v4f{0.f, 0.f, 0.f, 0.f};
-    const u32 p_lane = threadIdx.x % kScTile, c_lane = threadIdx.x / kScTile;  // staging: pixel of this lane, first channel
+    constexpr u32 CL = 256 / PT, NL = kScMaxC / CL;  // channel lanes of the staging; loads per lane and tensor at most
+    const u32 p_lane = threadIdx.x % PT, c_lane = threadIdx.x / PT;  // staging: pixel of this lane, first channel
     const u32 t_begin = blockIdx.x * tiles_per_z;
     for (u32 t = t_begin; t < t_begin + tiles_per_z; ++t) {
-        const u32 P = t * kScTile + p_lane;
+        const u32 P = t * PT + p_lane;
         const bool ok = P < total_px;
-        u32 n = 0, q = 0, oh = 0, ow = 0;
-        if (ok) {
-            d_ohw.divmod(P, n, q);
-            d_ow.divmod(q, oh, ow);
+        u32 n, q, oh, ow;
+        d_ohw.divmod(ok ? P : total_px - 1, n, q);
+        d_ow.divmod(q, oh, ow);
+        const float *dy = dY + size_t(n) * OC * OHW + q;
+        const float *x = X + (size_t(n) * IC * IH + 2 * oh) * IW + 2 * ow;
+        float vy[NL], vx[NL];
+#pragma unroll
+        for (u32 i = 0; i < NL; ++i) {
+            const u32 c = c_lane + i * CL;
+            vy[i] = dy[size_t(c < OC ? c : 0) * OHW];
+            vx[i] = x[size_t(c < IC ? c : 0) * IH * IW];
         }
         __syncthreads();  // the previous tile has been consumed
-        const float *dy = dY + size_t(n) * OC * OHW + q;
-        for (u32 c = c_lane; c < OC; c += 256 / kScTile) sY[p_lane][c] = ok ? dy[size_t(c) * OHW] : 0.f;
-        const float *x = X + (size_t(n) * IC * IH + 2 * oh) * IW + 2 * ow;
-        for (u32 c = c_lane; c < IC; c += 256 / kScTile) sX[p_lane][c] = ok ? x[size_t(c) * IH * IW] : 0.f;
+#pragma unroll
+        for (u32 i = 0; i < NL; ++i) {
+            const u32 c = c_lane + i * CL;
+            if (c < OC) sY[p_lane][c] = ok ? vy[i] : 0.f;
+            if (c < IC) sX[p_lane][c] = ok ? vx[i] : 0.f;
+        }
         __syncthreads();
         if (worker) {
 #pragma unroll
@@ -87,7 +99,7 @@ __global__ void __launch_bounds__(256) sc_wgrad_kernel(const float *__restrict__
                 const u32 task = task0 + k * 256;
                 if (k < per_thread && task < tasks) {
                     const u32 oc = task / icq_n, icq = task - oc * icq_n;
-                    for (u32 p = sub; p < kScTile; p += nsub) {
+                    for (u32 p = sub; p < PT; p += nsub) {
                         const float v = sY[p][oc];
                         const v4f xv = *reinterpret_cast<const v4f *>(&sX[p][4 * icq]);
                         acc[k].x += v * xv.x, acc[k].y += v * xv.y, acc[k].z += v * xv.z, acc[k].w += v * xv.w;
@@ -119,14 +131,15 @@ __global__ void __launch_bounds__(256) sc_wgrad_kernel(const float *__restrict__
 }
 
 struct ScWgradPlan {
-    u32 splits, tiles_per_z;
+    u32 splits, tiles_per_z, tile;  // tile: pixels per staged tile
     size_t workspace_bytes;
 };
 
 inline ScWgradPlan sc_wgrad_plan(u32 N, u32 IC, u32 OC, u32 OH, u32 OW) {
     ScWgradPlan p;
-    const u32 tiles = ceil_div(N * OH * OW, kScTile);
-    u32 splits = tiles < 256 ? tiles : 256;
+    p.tile = ceil_div(N * OH * OW, kScTile) < 512 ? kScTile / 2 : kScTile;  // few pixels: shorter tiles, one per workgroup
+    const u32 tiles = ceil_div(N * OH * OW, p.tile);
+    u32 splits = tiles < 512 ? tiles : 512;
     p.tiles_per_z = ceil_div(tiles, splits);
     p.splits = ceil_div(tiles, p.tiles_per_z);
     p.workspace_bytes = size_t(p.splits) * OC * IC * sizeof(float);
@@ -147,8 +160,12 @@ inline int launch_sc_dgrad(const float *W, const float *dY, float *dX, u32 N, u3
 // (dW == nullptr: the slices are left in part, unsummed)
 inline int launch_sc_wgrad(const float *dY, const float *X, float *dW, float *part, const ScWgradPlan &plan, u32 N, u32 IC, u32 OC,
                            u32 OH, u32 OW, hipStream_t s, const char *what) {
-    hipLaunchKernelGGL(sc_wgrad_kernel, dim3(plan.splits), dim3(256), 0, s, dY, X, part, IC, OC, OH, OW, N * OH * OW, plan.tiles_per_z,
-                       FastDiv(OW), FastDiv(OH * OW));
+    if (plan.tile == kScTile)
+        hipLaunchKernelGGL(sc_wgrad_kernel<kScTile>, dim3(plan.splits), dim3(256), 0, s, dY, X, part, IC, OC, OH, OW, N * OH * OW,
+                           plan.tiles_per_z, FastDiv(OW), FastDiv(OH * OW));
+    else
+        hipLaunchKernelGGL(sc_wgrad_kernel<kScTile / 2>, dim3(plan.splits), dim3(256), 0, s, dY, X, part, IC, OC, OH, OW, N * OH * OW,
+                           plan.tiles_per_z, FastDiv(OW), FastDiv(OH * OW));
     if (int st = check_launch(what)) return st;
     if (!dW) return CRB_OK;
     return launch_splitk_reduce(part, dW, OC * IC, plan.splits, ReduceEpi{nullptr, 1, 1, EPI_ACCUM}, s, what);

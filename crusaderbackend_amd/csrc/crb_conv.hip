@@ -650,6 +650,7 @@ int crb_conv_dgrad(const float *W, const float *dY, float *dX, const crb_conv_ge
     b.pH = g->pH, b.pW = g->pW;
     b.ihw.init(g->IH * g->IW), b.iw.init(g->IW), b.fhw.init(FHW), b.fw.init(g->FW);
     b.sH.init(g->sH), b.sW.init(g->sW);
+    b.unit_stride = g->sH == 1 && g->sW == 1;
     NchwEpi e{dX, nullptr, g->IC, g->IH * g->IW, 0u, FastDiv(g->IH * g->IW), 0u};
     return run_nchw(a, b, e, M, N, K, hipStream_t(stream), "crb_conv_dgrad");
 }

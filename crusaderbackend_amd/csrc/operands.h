@@ -224,6 +224,7 @@ struct DgradGather {
     u32 OH, OW, img_stride /* OC*OH*OW */, chan_stride /* OH*OW */;
     u32 pH, pW;
     FastDiv ihw, iw, fhw, fw, sH, sW;
+    bool unit_stride = false;  // sH == sW == 1: no division per element
     struct RowS {
         u32 off;
         int yp, xp;
@@ -249,12 +250,18 @@ struct DgradGather {
     }
     __device__ __forceinline__ float fetch(const RowS &r, const KS &k) const {
         const int th = r.yp - k.fh, tw = r.xp - k.fw;
-        if (!(r.ok && k.ok) || th < 0 || tw < 0) return 0.0f;
         u32 oh, rh, ow, rw;
-        sH.divmod(u32(th), oh, rh);
-        sW.divmod(u32(tw), ow, rw);
-        if (rh != 0 || rw != 0 || oh >= OH || ow >= OW) return 0.0f;
-        return dY[r.off + k.off + oh * OW + ow];
+        if (unit_stride) {
+            oh = u32(th), ow = u32(tw), rh = rw = 0;
+        } else {
+            sH.divmod(u32(th < 0 ? 0 : th), oh, rh);
+            sW.divmod(u32(tw < 0 ? 0 : tw), ow, rw);
+        }
+        const bool in = r.ok && k.ok && th >= 0 && tw >= 0 && rh == 0 && rw == 0 && oh < OH && ow < OW;
+        // the load is issued whatever `in` says (from element 0 when no output pixel feeds this tap): with a branch around
+        // it the loads of a staging pass are not in flight together
+        const float v = dY[in ? r.off + k.off + oh * OW + ow : 0u];
+        return in ? v : 0.0f;
     }
 };
 
