@@ -313,7 +313,9 @@ POINTWISE = [(3, 24, 32, 32, 48), (2, 204, 32, 32, 48), (2, 108, 16, 16, 48), (4
              # pixel-contraction weight gradient: ragged last slice, 49..64 output channels, one 64-pixel run per image
              (40, 50, 32, 32, 50), (3, 16, 8, 8, 64), (72, 342, 8, 8, 48),
              # streamed forward / data gradient: 16-byte pixel vectors (131072 pixels), two filter staging passes (IC > 256)
-             (128, 20, 32, 32, 24), (32, 300, 32, 32, 40)]
+             (128, 20, 32, 32, 24), (32, 300, 32, 32, 40),
+             # forward in chunks of 48 channels (contractions of 192 channels and more on 16x16 and 8x8 images)
+             (64, 288, 16, 16, 48), (72, 198, 8, 8, 40)]
 
 
 @pytest.mark.parametrize("N,IC,H,W,OC", POINTWISE)
