@@ -3,6 +3,7 @@
 // gradient, in-place subtract / scale, the momentum update with weight decay, and per-feature batch normalisation.
 // All are HBM-bound streaming kernels: 16-byte accesses where alignment allows, grid-stride loops, and reductions
 // with a fixed association (bit-reproducible, no atomics).
+#include <type_traits>
 #include "igemm_engine.h"
 
 namespace crb {
@@ -336,6 +337,10 @@ __global__ void __launch_bounds__(256) batchnorm_fwd_kernel(const float *__restr
     // sweep becomes one memory round trip per sample instead of one in all.
     float xv[kBnCache], av[kBnCache];
     float s = 0.f;
+    // scale and shift are requested with the first sweep and pinned behind the first reduction: requested where they are
+    // used, they would still be in flight when the store sweep starts, and every conditionally executed store block would
+    // wait for them again, and with them for the stores issued before it
+    float ga = gamma[t.on ? t.f : 0], be = beta[t.on ? t.f : 0];
     if (cached) {
 #pragma unroll
         for (int i = 0; i < kBnCache; ++i) {
@@ -350,6 +355,7 @@ __global__ void __launch_bounds__(256) batchnorm_fwd_kernel(const float *__restr
                 av[i] = ad[size_t(n < N ? n : 0) * F];
             }
         }
+        __builtin_amdgcn_sched_barrier(0);  // no use of a loaded value moves up between the loads
 #pragma unroll
         for (int i = 0; i < kBnCache; ++i) xv[i] = (t.on && t.g + G * i < N) ? xv[i] : 0.f;
 #pragma unroll
@@ -358,6 +364,7 @@ __global__ void __launch_bounds__(256) batchnorm_fwd_kernel(const float *__restr
         for (u32 n = t.g; n < N; n += G) s += x[size_t(n) * F];
     }
     const float m = t.reduce(s, red) / float(N);
+    asm volatile("" : "+v"(ga), "+v"(be));
     float q = 0.f;
     if (cached) {
 #pragma unroll
@@ -373,26 +380,43 @@ __global__ void __launch_bounds__(256) batchnorm_fwd_kernel(const float *__restr
     }
     const float v = t.reduce(q, red) / float(N);
     if (!t.on) return;
-    const float inv = 1.0f / sqrtf(v + 1e-8f), ga = gamma[t.f], be = beta[t.f];
+    const float inv = 1.0f / sqrtf(v + 1e-8f);
     // outputs a caller does not need are not written: Y and xHat may be null; reluOut = max(Y + addend, 0) is optional
     // (addend: the other summand of a residual connection that closes right behind this normalisation, or null)
-    auto put = [&](u32 n, float xh, float add) {
+    auto put = [&](u32 n, float xh, float add, auto has_xhat, auto has_y, auto has_relu) {
         const float y = xh * ga + be;
-        if (xHat) xHat[size_t(n) * F + t.f] = xh;
-        if (Y) Y[size_t(n) * F + t.f] = y;
-        if (reluOut) {
+        if constexpr (has_xhat.value) xHat[size_t(n) * F + t.f] = xh;
+        if constexpr (has_y.value) Y[size_t(n) * F + t.f] = y;
+        if constexpr (has_relu.value) {
             const float z = addend ? y + add : y;
             reluOut[size_t(n) * F + t.f] = z > 0.f ? z : 0.f;
         }
     };
-    if (cached) {
+    // Which outputs exist is decided once, outside the store sweep: with a test in front of every store the compiler's
+    // wait in front of the next block also covers the stores just issued (they count like loads), one round trip per sample.
+    auto sweep = [&](auto has_xhat, auto has_y, auto has_relu) {
+        if (cached) {
 #pragma unroll
-        for (int i = 0; i < kBnCache; ++i) {
-            const u32 n = t.g + G * i;
-            if (n < N) put(n, (xv[i] - m) * inv, (reluOut && addend) ? av[i] : 0.f);
+            for (int i = 0; i < kBnCache; ++i) {
+                const u32 n = t.g + G * i;
+                if (n < N) put(n, (xv[i] - m) * inv, (has_relu.value && addend) ? av[i] : 0.f, has_xhat, has_y, has_relu);
+            }
+        } else {
+            for (u32 n = t.g; n < N; n += G)
+                put(n, (x[size_t(n) * F] - m) * inv, (has_relu.value && addend) ? addend[size_t(n) * F + t.f] : 0.f, has_xhat, has_y, has_relu);
         }
-    } else {
-        for (u32 n = t.g; n < N; n += G) put(n, (x[size_t(n) * F] - m) * inv, (reluOut && addend) ? addend[size_t(n) * F + t.f] : 0.f);
+    };
+    using T = std::true_type;
+    using Fa = std::false_type;
+    switch ((xHat ? 1 : 0) | (Y ? 2 : 0) | (reluOut ? 4 : 0)) {
+        case 1: sweep(T{}, Fa{}, Fa{}); break;
+        case 2: sweep(Fa{}, T{}, Fa{}); break;
+        case 3: sweep(T{}, T{}, Fa{}); break;
+        case 4: sweep(Fa{}, Fa{}, T{}); break;
+        case 5: sweep(T{}, Fa{}, T{}); break;
+        case 6: sweep(Fa{}, T{}, T{}); break;
+        case 7: sweep(T{}, T{}, T{}); break;
+        default: break;
     }
     if (t.g == 0) mean[t.f] = m, var[t.f] = v;
 }
@@ -423,6 +447,7 @@ __global__ void __launch_bounds__(256) batchnorm_bwd_kernel(const float *__restr
     };
     float xv[kBnCache], dv[kBnCache];
     float s = 0.f;
+    float ga = gamma[t.on ? t.f : 0];  // requested with the sweep, pinned behind the first reduction
     if (cached) {
         // every load of the sweep is issued, unconditionally (a sample past the batch reads row 0), before any is used: with
         // a branch around a load the compiler puts it next to its use, one memory round trip per sample
@@ -436,6 +461,7 @@ __global__ void __launch_bounds__(256) batchnorm_bwd_kernel(const float *__restr
             if (SUM2) ev[i] = dy2[row];
             if (MASK) mv[i] = mk[row];
         }
+        __builtin_amdgcn_sched_barrier(0);  // no use of a loaded value moves up between the loads
 #pragma unroll
         for (int i = 0; i < kBnCache; ++i) {
             const bool ok = t.on && t.g + G * i < N;
@@ -450,6 +476,7 @@ __global__ void __launch_bounds__(256) batchnorm_bwd_kernel(const float *__restr
         for (u32 n = t.g; n < N; n += G) s += x[size_t(n) * F];
     }
     const float m = t.reduce(s, red) / float(N);
+    asm volatile("" : "+v"(ga));
     // one sweep for the remaining sums: sum d^2, sum dy*d, sum dy, sum d  (d = x - mean)
     float q = 0.f, sdd = 0.f, sdy = 0.f, sd = 0.f;
     if (cached) {
@@ -470,7 +497,7 @@ __global__ void __launch_bounds__(256) batchnorm_bwd_kernel(const float *__restr
     t.reduce4(q, Sdd, Sdy, Sd, red4);
     const float v = q / float(N);
     if (!t.on) return;
-    const float inv = 1.0f / sqrtf(v + 1e-8f), ga = gamma[t.f], invN = 1.0f / float(N);
+    const float inv = 1.0f / sqrtf(v + 1e-8f), invN = 1.0f / float(N);
     const float dVar = ga * Sdd * -0.5f * inv * inv * inv;
     const float dMean = ga * Sdy * -inv + dVar * (-2.0f * Sd) * invN;
     // the parameter gradients fall out of the same sums: dBeta = sum dy, dGamma = sum dy*xHat = inv * sum dy*(x - mean)
