@@ -38,11 +38,16 @@ namespace crb {
 // which are bandwidth-bound: same staging and MFMA mapping, the contraction is just the channel chunk.
 // PGS_ > 1 (single-chunk configurations only): a wave finishes its pixel blocks in PGS groups, one after the other, and
 // stores each group as soon as it is complete, so the stores of all groups but the last overlap the MFMAs of the next.
-template <int W_, int ROWS_, int CI_, int OCT_, int PBW_, int OBW_, bool DGRAD_, int OCC_, int NBUF_ = 2, int S_ = 1, int FS_ = 3, int PGS_ = 1>
+// KS_ = 2 (single-chunk configurations only): the contraction runs in two halves of the chunk's channels. The
+// first half's rows are requested first and multiplied (all pixel blocks) while the second half's are still arriving; the
+// second half then runs group by group with the stores in between, as with KS_ = 1.
+template <int W_, int ROWS_, int CI_, int OCT_, int PBW_, int OBW_, bool DGRAD_, int OCC_, int NBUF_ = 2, int S_ = 1, int FS_ = 3, int PGS_ = 1,
+          int KS_ = 1>
 struct DirectCfg {
     static constexpr int W = W_, ROWS = ROWS_, CI = CI_, OCT = OCT_, PBW = PBW_, OBW = OBW_, OCC = OCC_, NBUF = NBUF_, S = S_;
     static constexpr int FS = FS_, NT = FS_ * FS_;  // filter size, taps
     static constexpr int PGS = PGS_, PGC = PBW_ / PGS_;  // pixel-block groups per wave, blocks per group
+    static constexpr int KS = KS_;
     static constexpr bool STREAM_OUT = PGS_ > 1 || FS_ == 1;  // non-temporal output stores (see store_out)
     static constexpr bool DGRAD = DGRAD_;
     // W = 4: the grid is a 4x4 image and a tile is ROWS / 4 whole images stacked, each staged with its own halo rows
@@ -89,6 +94,7 @@ struct DirectCfg {
     static_assert((PBW * 16) % W == 0 || PBW == 1, "a wave's pixel blocks must start on a row boundary");
     static_assert(CI % 4 == 0, "chunk channel count");
     static_assert(PBW % PGS == 0 && (PGS == 1 || NBUF == 1), "pixel groups need a single-chunk configuration");
+    static_assert(KS == 1 || (KS == 2 && NBUF == 1 && (CI / 4) % 2 == 0 && !(W_ == 4)), "two-half contraction: single chunk, whole steps per half");
 
     // LDS offset of tap (fh, fw) relative to the lane's pixel base (which points one float left of the pixel)
     static constexpr int tap_off(int tap) {
@@ -112,6 +118,14 @@ struct DirectCfg {
 // lifetime (pixel groups), so that the write-back overlaps the remaining MFMAs: 16 -> 16 @ 32x32, batch 128 (8.4 MB of
 // output) 9.1 -> 8.6 us per launch; it changes nothing when all stores come at the end, and costs the stride-2 data
 // gradient 0.3 us. The 1x1 layers (bandwidth-bound, outputs of 12-50 MB) always stream: 204 -> 48 @ 32x32 21.5 -> 20.5 us.
+// Workgroup barrier that orders LDS accesses only: global loads requested before it stay in flight across it
+// (__syncthreads() fences every address space and so waits for them).
+__device__ __forceinline__ void lds_barrier() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
+
 template <bool STREAM>
 __device__ __forceinline__ void store_out(float *p, v4f v) {
     if constexpr (STREAM)
@@ -170,13 +184,23 @@ __device__ __forceinline__ void conv3x3_body(const DirectArgs &a, const u32 bid,
     constexpr int NT = Cfg::NT;
     v4f xreg[XNP];
     float wreg[WNP * NT];
+    bool xok[XNP], wok[WNP];  // two-half form: what a request that was issued regardless is worth
 
-    auto fetch = [&](u32 c0) {
+    auto fetch_x = [&](u32 c0, auto lo, auto hi) {
 #pragma unroll
-        for (int i = 0; i < XNP; ++i) {
+        for (int i = decltype(lo)::value; i < decltype(hi)::value; ++i) {
             const u32 e = t + i * kThreads;
             v4f v = {0.f, 0.f, 0.f, 0.f};
-            if (XQ % kThreads == 0 || e < XQ) {
+            if constexpr (Cfg::KS == 2) {
+                // Requested whatever the row is (a halo row outside the image or a channel past the extent reads row 0 of
+                // channel 0 and is zeroed on the way to LDS): behind a branch the compiler could not tell how many requests are
+                // in flight, and the wait for the first half would cover the second half too.
+                const u32 q = e % (SW / 4), lr = (e / (SW / 4)) % XR, c = e / ((SW / 4) * XR);
+                const int row = srow0 + int(lr);
+                const bool ok = row >= 0 && row < int(a.in_H) && c0 + c < a.C_IN && (XQ % kThreads == 0 || e < XQ);
+                xok[i] = ok;
+                v = *reinterpret_cast<const v4f *>(a.X + (size_t(n) * a.C_IN + (ok ? c0 + c : 0u)) * in_HW + (ok ? u32(row) : 0u) * SW + 4 * q);
+            } else if (XQ % kThreads == 0 || e < XQ) {
                 const u32 q = e % (SW / 4), lr = (e / (SW / 4)) % XR, c = e / ((SW / 4) * XR);
                 // stacked images: staged row lr is row lr % 6 - 1 of image lr / 6 (rows -1 and 4 are its halo)
                 const int row = Cfg::MI ? int(lr % 6) - 1 : srow0 + int(lr);
@@ -186,6 +210,8 @@ __device__ __forceinline__ void conv3x3_body(const DirectArgs &a, const u32 bid,
             }
             xreg[i] = v;
         }
+    };
+    auto fetch_w = [&](u32 c0) {
 #pragma unroll
         for (int i = 0; i < WNP; ++i) {
             const u32 e = t + i * kThreads;
@@ -196,7 +222,13 @@ __device__ __forceinline__ void conv3x3_body(const DirectArgs &a, const u32 bid,
                                           : a.Wt + ((size_t(oc0) + j) * a.C_IN + c0 + c) * NT;
             // channels past the tensor's extent (ragged last chunk / last channel tile) are staged as zeros
             const bool ok = (WQ % kThreads == 0 || e < WQ) && c0 + c < a.C_IN && oc0 + j < a.C_OUT;
-            if (ok) {  // one branch around the 9 contiguous loads keeps them mergeable into wide loads
+            if constexpr (Cfg::KS == 2) {
+                static_assert(!Cfg::DGRAD || Cfg::KS == 1, "two-half form: forward filter addressing only");
+                wok[i] = ok;
+                const float *src0 = a.Wt + ((size_t(oc0) + (ok ? j : 0u)) * a.C_IN + c0 + (ok ? c : 0u)) * NT;
+#pragma unroll
+                for (int tap = 0; tap < NT; ++tap) wreg[i * NT + tap] = src0[tap];
+            } else if (ok) {  // one branch around the 9 contiguous loads keeps them mergeable into wide loads
 #pragma unroll
                 for (int tap = 0; tap < NT; ++tap) wreg[i * NT + tap] = src[tap];
             } else {
@@ -206,29 +238,46 @@ __device__ __forceinline__ void conv3x3_body(const DirectArgs &a, const u32 bid,
         }
     };
 
-    auto commit = [&](float *dX, float *dW) {
+    using std::integral_constant;
+    typedef integral_constant<int, 0> XLo;
+    typedef integral_constant<int, XNP> XHi;
+    auto fetch = [&](u32 c0) {
+        fetch_x(c0, XLo{}, XHi{});
+        fetch_w(c0);
+    };
+
+    auto commit_x = [&](float *dX, auto lo, auto hi) {
 #pragma unroll
-        for (int i = 0; i < XNP; ++i) {
+        for (int i = decltype(lo)::value; i < decltype(hi)::value; ++i) {
             const u32 e = t + i * kThreads;
             if (XQ % kThreads == 0 || e < XQ) {
                 const u32 q = e % (SW / 4), lr = (e / (SW / 4)) % XR, c = e / ((SW / 4) * XR);
                 if constexpr (Cfg::FW2) {  // columns 4q..4q+3: odd ones to the first half of the row, even ones to the second
                     *reinterpret_cast<v2f *>(dX + c * XP + lr * XS + 4 + 2 * q) = v2f{xreg[i].y, xreg[i].w};
                     *reinterpret_cast<v2f *>(dX + c * XP + lr * XS + 4 + W + 2 * q) = v2f{xreg[i].x, xreg[i].z};
+                } else if constexpr (Cfg::KS == 2) {
+                    *reinterpret_cast<v4f *>(dX + c * XP + lr * XS + 4 + 4 * q) = xok[i] ? xreg[i] : v4f{0.f, 0.f, 0.f, 0.f};
                 } else {
                     *reinterpret_cast<v4f *>(dX + c * XP + lr * XS + 4 + 4 * q) = xreg[i];
                 }
             }
         }
+    };
+    auto commit_w = [&](float *dW) {
 #pragma unroll
         for (int i = 0; i < WNP; ++i) {
             const u32 e = t + i * kThreads;
             if (WQ % kThreads == 0 || e < WQ) {
                 const u32 j = Cfg::DGRAD ? e % OCT : e / CI, c = Cfg::DGRAD ? e / OCT : e % CI;
 #pragma unroll
-                for (int tap = 0; tap < NT; ++tap) dW[j * WSTR + tap * Cfg::CIP + c] = wreg[i * NT + tap];
+                for (int tap = 0; tap < NT; ++tap)
+                    dW[j * WSTR + tap * Cfg::CIP + c] = (Cfg::KS == 2 && !wok[i]) ? 0.f : wreg[i * NT + tap];
             }
         }
+    };
+    auto commit = [&](float *dX, float *dW) {
+        commit_x(dX, XLo{}, XHi{});
+        commit_w(dW);
     };
 
     // ---- zero the halo columns of both buffers once (never overwritten afterwards) ---------------------
@@ -264,15 +313,15 @@ __device__ __forceinline__ void conv3x3_body(const DirectArgs &a, const u32 bid,
 #pragma unroll
             for (int o = 0; o < OBW; ++o) acc[ph][p][o] = v4f{0.f, 0.f, 0.f, 0.f};
 
-    constexpr int CQ = Cfg::CQ;
-    // MFMAs of one chunk for the pixel blocks [P0, P0 + PC) of this wave
-    auto compute = [&](const float *cx, const float *cw, auto p0c, auto pcc) {
+    // MFMAs of one chunk for the pixel blocks [P0, P0 + PC) of this wave, channel quads [Q0, Q0 + QN) of every tap
+    auto compute_k = [&](const float *cx, const float *cw, auto p0c, auto pcc, auto q0c, auto qnc) {
         constexpr int P0 = decltype(p0c)::value, PC = decltype(pcc)::value;
+        constexpr int Q0 = decltype(q0c)::value, CQ = decltype(qnc)::value, NSTEP = CQ * Cfg::NT;
         constexpr int MPS = PC * OBW, PF = (8 / MPS) < 1 ? 1 : ((8 / MPS) > 4 ? 4 : (8 / MPS));  // read-ahead (steps)
         const float *px = cx + xbase, *pw = cw + wbase;
         float av[PF + 1][PC], bv[PF + 1][OBW];
         auto read_step = [&](int s, int slot) {
-            const int tap = s / CQ, cq = s % CQ;
+            const int tap = s / CQ, cq = Q0 + s % CQ;
             const int xo = cq * 4 * XP + Cfg::tap_off(tap);
 #pragma unroll
             for (int p = 0; p < PC; ++p) av[slot][p] = px[xo + Cfg::pix_off((P0 + p) * 16)];
@@ -294,9 +343,11 @@ __device__ __forceinline__ void conv3x3_body(const DirectArgs &a, const u32 bid,
             __builtin_amdgcn_sched_barrier(0);
         }
     };
-    using std::integral_constant;
     typedef integral_constant<int, 0> AllP0;
     typedef integral_constant<int, PBW> AllPC;
+    auto compute = [&](const float *cx, const float *cw, auto p0c, auto pcc) {
+        compute_k(cx, cw, p0c, pcc, integral_constant<int, 0>{}, integral_constant<int, Cfg::CQ>{});
+    };
 
     // ---- epilogue for the pixel blocks [p_lo, p_lo + p_cnt): a lane holds 4 consecutive grid pixels of one output channel ----
     auto store = [&](int p_lo, int p_cnt) {
@@ -335,6 +386,35 @@ __device__ __forceinline__ void conv3x3_body(const DirectArgs &a, const u32 bid,
     };
 
     // ---- main loop over input-channel chunks (double-buffered) ---------------------------------------------
+    if constexpr (Cfg::KS == 2) {
+        // items [0, XH) of a thread's rows cover the first half of the channels (items run channel-major over the workgroup)
+        constexpr int HQ = Cfg::CQ / 2;
+        constexpr int XH = ((CI / 2) * XR * (SW / 4) + kThreads - 1) / kThreads;
+        typedef integral_constant<int, XH> XMid;
+        fetch_w(0);
+        __builtin_amdgcn_sched_barrier(0);
+        fetch_x(0, XLo{}, XMid{});
+        __builtin_amdgcn_sched_barrier(0);  // the second half's requests stay behind the first half's
+        fetch_x(0, XMid{}, XHi{});
+        __builtin_amdgcn_sched_barrier(0);
+        commit_w(sW[0]);
+        commit_x(sX[0], XLo{}, XMid{});
+        lds_barrier();
+        compute_k(sX[0], sW[0], AllP0{}, AllPC{}, integral_constant<int, 0>{}, integral_constant<int, HQ>{});
+        commit_x(sX[0], XMid{}, XHi{});
+        lds_barrier();
+        auto group = [&](auto g) {
+            constexpr int G = decltype(g)::value;
+            compute_k(sX[0], sW[0], integral_constant<int, G * Cfg::PGC>{}, integral_constant<int, Cfg::PGC>{}, integral_constant<int, HQ>{},
+                      integral_constant<int, Cfg::CQ - HQ>{});
+            store(G * Cfg::PGC, Cfg::PGC);
+        };
+        group(integral_constant<int, 0>{});
+        if constexpr (Cfg::PGS > 1) group(integral_constant<int, 1>{});
+        if constexpr (Cfg::PGS > 2) group(integral_constant<int, 2>{});
+        if constexpr (Cfg::PGS > 3) group(integral_constant<int, 3>{});
+        return;
+    }
     fetch(0);
     commit(sX[0], sW[0]);
     __syncthreads();
