@@ -118,14 +118,6 @@ struct DirectCfg {
 // lifetime (pixel groups), so that the write-back overlaps the remaining MFMAs: 16 -> 16 @ 32x32, batch 128 (8.4 MB of
 // output) 9.1 -> 8.6 us per launch; it changes nothing when all stores come at the end, and costs the stride-2 data
 // gradient 0.3 us. The 1x1 layers (bandwidth-bound, outputs of 12-50 MB) always stream: 204 -> 48 @ 32x32 21.5 -> 20.5 us.
-// Workgroup barrier that orders LDS accesses only: global loads requested before it stay in flight across it
-// (__syncthreads() fences every address space and so waits for them).
-__device__ __forceinline__ void lds_barrier() {
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
-    __builtin_amdgcn_s_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
-}
-
 template <bool STREAM>
 __device__ __forceinline__ void store_out(float *p, v4f v) {
     if constexpr (STREAM)

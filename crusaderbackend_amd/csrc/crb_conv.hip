@@ -277,8 +277,11 @@ static int try_pointwise(const float *Wt, const float *X, float *Y, const float 
         if (good(32)) { CRB_TRY(32, 8, 16, 32, 4, 2, DG, 2, 2, 1, 1) }
         if (good(16)) { CRB_TRY(32, 8, 16, 16, 4, 1, DG, 2, 2, 1, 1) }
     } else if (gW == 16) {
-        // contractions of 192 channels and more: chunks of 48, a third of the chunk hand-overs (288 -> 48 @16x16: 12.0 -> 11.2 us)
-        if (!DG && C_IN >= 192 && half && good_half(48)) { CRB_TRY(16, 4, 48, 48, 1, 3, DG, 2, 2, 1, 1) }
+        // long contractions on few pixels: many small workgroups (16 output channels, four rows), three to a CU, so that one
+        // waits for its next chunk while the others multiply (batch 64: 108 -> 48 6.6 -> 5.9 us, 204 -> 48 9.9 -> 8.4 us,
+        // 288 -> 48 in chunks of 48 channels 11.2 -> 9.9 us)
+        if (!DG && C_IN >= 256 && N * (gH / 4) * ceil_div(C_OUT, 16u) >= 512) { CRB_TRY(16, 4, 48, 16, 1, 1, DG, 3, 2, 1, 1) }
+        if (!DG && C_IN > 64 && N * (gH / 4) * ceil_div(C_OUT, 16u) >= 512) { CRB_TRY(16, 4, 16, 16, 1, 1, DG, 3, 2, 1, 1) }
         if (half && good_half(48)) { CRB_TRY(16, 4, 16, 48, 1, 3, DG, 2, 2, 1, 1) }
         if (good(64)) { CRB_TRY(16, 8, 16, 64, 2, 4, DG, 2, 2, 1, 1) }
         if (good(48)) { CRB_TRY(16, 8, 16, 48, 2, 3, DG, 2, 2, 1, 1) }

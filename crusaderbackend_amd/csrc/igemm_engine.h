@@ -30,6 +30,14 @@ constexpr u32 kXcds = 8;
 
 enum : u32 { EPI_ACCUM = 1u, EPI_RELU = 2u };
 
+// Workgroup barrier that orders LDS accesses only: global loads requested before it stay in flight across it
+// (__syncthreads() fences every address space and so waits for them).
+__device__ __forceinline__ void lds_barrier() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
+
 struct IgemmDims {
     u32 M, N, K;
     u32 tiles_m, tiles_n;
