@@ -510,3 +510,11 @@ def test_shortcut_weight_gradients_join_the_postponed_sum(dev):
     torch.cuda.synchronize()
     for dX1, dW1, dX2, dW2 in layers:
         assert np.array_equal(to_np(dX1), to_np(dX2)) and np.array_equal(to_np(dW1), to_np(dW2))
+
+
+# 32-wide forward with 9..16 input and at most 16 output channels: the contraction in two halves (the second half of the rows
+# is committed to LDS behind the first half's MFMAs), rows requested unconditionally — ragged channel counts on both sides,
+# image heights that are and are not a whole number of 8-row tiles (the latter take another configuration), odd batches.
+@pytest.mark.parametrize("N,IC,H,OC", [(3, 12, 32, 10), (5, 16, 32, 16), (2, 9, 8, 1), (1, 13, 16, 16), (2, 16, 24, 7), (2, 12, 12, 12)])
+def test_conv_forward_two_half_contraction(dev, N, IC, H, OC):
+    run_layer(dev, N, IC, H, 32, OC, 3, 3, 1, 1, 1, 1, bias=True, seed=61)
