@@ -109,3 +109,30 @@ def test_random_gemm_shapes(dev, seed):
         gemm_cases.run_tn(dev, M, N, K, batch, seed=i + 1)
         gemm_cases.run_nt(dev, M, N, K, seed=i + 2)
         gemm_cases.run_nta(dev, M, N, max(1, K // 16), batch, seed=i + 3)
+
+
+@pytest.mark.parametrize("seed", [7, 8])
+def test_random_full_batch_layers(dev, seed):
+    """Layer shapes at batches of 64 to 128, where the workgroup-count gates of the kernel choice open (resident chunks, the
+    two-half forward, many-small-workgroup 1x1 tiles, streamed 1x1 layers, shortcut kernels, 4x4-image tiles): 3x3 at stride
+    1 and 2 and 1x1 at stride 1 and 2 on 4- to 32-wide grids, channel counts on and off the 16-channel blocks."""
+    rng = random.Random(seed)
+    done = 0
+    while done < 30:
+        W = rng.choice([4, 8, 16, 32])
+        H = rng.choice([W, W, W // 2 if W > 4 else W, 8])
+        F = rng.choice([3, 3, 1])
+        s = rng.choice([1, 1, 1, 2]) if (W >= 8 or F == 1) else 1
+        p = 1 if F == 3 else 0
+        IC = rng.choice([3, 9, 12, 16, 24, 32, 48, 64, 100, 128, 204, 256])
+        OC = rng.choice([10, 12, 16, 32, 48, 64, 96, 128])
+        N = rng.choice([64, 96, 128])
+        if N * max(IC, OC) * H * W > 12_000_000:
+            N = 64
+        if N * max(IC, OC) * H * W > 12_000_000:
+            IC = min(IC, 64)
+        shape = (N, IC, H * s, W * s, OC, F, F, s, s, p, p)
+        bias, own_ws = rng.random() < 0.5, rng.random() < 0.5
+        print("full batch", seed, done, shape, bias, own_ws, flush=True)
+        run_layer(dev, *shape, bias=bias, seed=1000 * seed + done, ws=own_ws)
+        done += 1
