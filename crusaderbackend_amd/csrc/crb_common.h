@@ -32,6 +32,7 @@ inline int scratch_get(size_t bytes, hipStream_t stream, const char *what, T **o
 int scratch_bind(void *ptr, size_t bytes, hipStream_t stream);
 void arena_release();
 // While alive, every scratch_get of this thread is served from [ptr, ptr + bytes) or refused; nothing is allocated.
+// Requests inside one scope get consecutive blocks (256-byte steps), never the same memory twice.
 struct ScratchScope {
     ScratchScope(void *ptr, size_t bytes);
     ~ScratchScope();
@@ -39,7 +40,7 @@ struct ScratchScope {
     ScratchScope &operator=(const ScratchScope &) = delete;
   private:
     void *prev_ptr;
-    size_t prev_bytes;
+    size_t prev_bytes, prev_used;
 };
 
 // Exact floor(n / d) for any n, d in [1, 2^32): round-up magic multiply (Granlund-Montgomery).

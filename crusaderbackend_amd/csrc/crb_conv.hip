@@ -780,8 +780,9 @@ int crb_conv_wgrad_noalloc(const float *dY, const float *X, float *dW, const crb
     void *ptr = nullptr;
     if (int st = static_scratch_ptr("crb_conv_wgrad_noalloc", &ptr)) return st;
     // every scratch request below this call is served from the built-in buffer or refused: nothing allocates
+    // (no explicit workspace is passed down, so the scope is the one owner of the buffer and hands out disjoint blocks)
     ScratchScope scope(ptr, kStaticScratchBytes);
-    return crb_conv_wgrad(dY, X, dW, g, ptr, kStaticScratchBytes, stream);
+    return crb_conv_wgrad(dY, X, dW, g, nullptr, 0, stream);
 }
 
 size_t crb_conv_fwd_workspace_bytes(const crb_conv_geom *g, int operands_aligned16) {
@@ -792,7 +793,7 @@ size_t crb_conv_fwd_workspace_bytes(const crb_conv_geom *g, int operands_aligned
         if (done) return 0;
     }
     if (pointwise_shape(g)) return gemm_scratch_bytes(g->OC, g->IH * g->IW, g->IC, g->N);
-    if (tiny2x2_shape(g) && operands_aligned16) return gemm_scratch_bytes(g->N, g->OC * 4, g->IC * 4, 1);
+    if (tiny2x2_shape(g) && operands_aligned16) return gemm_scratch_bytes(g->N, g->OC * 4, g->IC * 4, 1, false);
     if (operands_aligned16 && (direct_shape(g, 1) || direct_shape(g, 2))) {
         if (g->sH == 1)
             try_direct<false, 1>(nullptr, nullptr, nullptr, nullptr, g->N, g->IC, g->OC, g->OH, g->OW, g->IH, 0, nullptr, "", done, true);
@@ -811,7 +812,7 @@ size_t crb_conv_dgrad_workspace_bytes(const crb_conv_geom *g, int operands_align
         if (done) return 0;
     }
     if (pointwise_shape(g)) return gemm_scratch_bytes(g->IC, g->IH * g->IW, g->OC, g->N);
-    if (tiny2x2_shape(g) && operands_aligned16) return gemm_scratch_bytes(g->N, g->IC * 4, g->OC * 4, 1);
+    if (tiny2x2_shape(g) && operands_aligned16) return gemm_scratch_bytes(g->N, g->IC * 4, g->OC * 4, 1, false);
     if (operands_aligned16 && (direct_shape(g, 1) || direct_shape(g, 2))) {
         if (g->sH == 1)
             try_direct<true, 1>(nullptr, nullptr, nullptr, nullptr, g->N, g->OC, g->IC, g->OH, g->OW, g->OH, 0, nullptr, "", done, true);

@@ -108,8 +108,8 @@ static int run_tiles(const AOp &a, const BOp &b, const E &e, u32 M, u32 N, u32 K
 }
 
 // Scratch bytes run_tiles asks for on a dense M x N result with contraction length K (0: the contraction is not cut).
-size_t gemm_scratch_bytes(u32 M, u32 N, u32 K, u32 zdim) {
-    if (tiny_gemm_fits(M, N, K, zdim)) return 0;  // one launch, no partial results
+size_t gemm_scratch_bytes(u32 M, u32 N, u32 K, u32 zdim, bool one_launch_form) {
+    if (one_launch_form && tiny_gemm_fits(M, N, K, zdim)) return 0;  // one launch, no partial results
     const GemmChoice c = choose_tiles(M, N, K, zdim, true);
     SplitPlan sp;
     switch (c.tile) {

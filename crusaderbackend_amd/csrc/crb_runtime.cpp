@@ -48,18 +48,23 @@ static std::vector<std::pair<int, void *>> g_retired;  // (device, block)
 
 static thread_local void *g_scope_ptr = nullptr;
 static thread_local size_t g_scope_bytes = 0;
+static thread_local size_t g_scope_used = 0;  // bytes of the open scope already handed out
 
-ScratchScope::ScratchScope(void *ptr, size_t bytes) : prev_ptr(g_scope_ptr), prev_bytes(g_scope_bytes) {
-    g_scope_ptr = ptr, g_scope_bytes = bytes;
+ScratchScope::ScratchScope(void *ptr, size_t bytes) : prev_ptr(g_scope_ptr), prev_bytes(g_scope_bytes), prev_used(g_scope_used) {
+    g_scope_ptr = ptr, g_scope_bytes = bytes, g_scope_used = 0;
 }
-ScratchScope::~ScratchScope() { g_scope_ptr = prev_ptr, g_scope_bytes = prev_bytes; }
+ScratchScope::~ScratchScope() { g_scope_ptr = prev_ptr, g_scope_bytes = prev_bytes, g_scope_used = prev_used; }
 
 int scratch_get(size_t bytes, hipStream_t stream, const char *what, void **out) {
     *out = nullptr;
     if (g_scope_ptr) {
-        if (bytes > g_scope_bytes)
-            return fail(CRB_EWORKSPACE, "%s: needs %zu bytes of scratch, the buffer this call may use holds %zu", what, bytes, g_scope_bytes);
-        *out = g_scope_ptr;
+        // every request inside one scope gets a block of its own (256-byte steps), so two requests of one call never alias
+        const size_t at = (g_scope_used + 255) & ~size_t(255);
+        if (at > g_scope_bytes || bytes > g_scope_bytes - at)
+            return fail(CRB_EWORKSPACE, "%s: needs %zu bytes of scratch, the buffer this call may use holds %zu (%zu already in use)",
+                        what, bytes, g_scope_bytes, at);
+        *out = static_cast<char *>(g_scope_ptr) + at;
+        g_scope_used = at + bytes;
         return CRB_OK;
     }
     int dev = 0;
@@ -77,8 +82,12 @@ int scratch_get(size_t bytes, hipStream_t stream, const char *what, void **out) 
         return CRB_OK;
     }
     // growing means hipMalloc, which a stream capture cannot record
+    // (a capture query that fails — the legacy stream while another stream captures in global mode — counts as capturing)
     hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
-    if (hipStreamIsCapturing(stream, &cap) != hipSuccess) (void)hipGetLastError();
+    if (hipStreamIsCapturing(stream, &cap) != hipSuccess) {
+        (void)hipGetLastError();
+        cap = hipStreamCaptureStatusActive;
+    }
     if (cap != hipStreamCaptureStatusNone)
         return fail(CRB_EWORKSPACE,
                     "%s: needs %zu bytes of scratch while the stream is being captured; bind a workspace to the stream "

@@ -16,6 +16,8 @@ int conv2x2_fwd(const float *W, const float *X, float *Y, const float *bias, u32
 int conv2x2_dgrad(const float *W, const float *dY, float *dX, u32 N, u32 IC, u32 OC, hipStream_t s, const char *what);
 // G: scratch of OC*4 x IC*4 floats.
 // Scratch bytes the GEMM family asks for on a dense M x N result per batch entry with contraction length K (0: none).
-size_t gemm_scratch_bytes(u32 M, u32 N, u32 K, u32 zdim);
+// one_launch_form = false: the caller goes to the tiled engine directly and never takes the one-launch small-product kernel
+// (the 2x2-image convolutions), so the split plan of the tiles applies whatever the size.
+size_t gemm_scratch_bytes(u32 M, u32 N, u32 K, u32 zdim, bool one_launch_form = true);
 int conv2x2_wgrad(const float *dY, const float *X, float *dW, float *G, u32 N, u32 IC, u32 OC, hipStream_t s, const char *what);
 }  // namespace crb

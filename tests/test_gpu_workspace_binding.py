@@ -149,3 +149,55 @@ def test_pointwise_wgrad_honours_the_workspace_argument(dev):
     with pytest.raises(capi.CrbError) as ei:
         capi.conv_wgrad(to_dev(dY, dev), to_dev(X, dev), dW, g, workspace=ws[: need // 8])
     assert ei.value.status == capi.CRB_EWORKSPACE
+
+
+# (N, IC, H, OC, F, stride, pad, operands 16-byte aligned): 2x2 images (products over (channel, pixel) pairs on the tiled
+# engine), 1x1 layers the batched GEMM forms take (odd image size; operands off the 16-byte grid), the general gather path,
+# direct-kernel shapes on operands off the grid (which then take the general path too)
+EXACT_SHAPES = [(128, 64, 2, 64, 3, 1, 1, True), (128, 512, 2, 512, 3, 1, 1, True), (8, 40, 2, 24, 3, 1, 1, True),
+                (64, 24, 16, 48, 1, 1, 0, False), (4, 96, 7, 40, 1, 1, 0, True), (2, 300, 6, 20, 1, 1, 0, False),
+                (2, 64, 12, 48, 5, 1, 2, True), (3, 20, 9, 12, 3, 2, 1, True), (16, 16, 32, 16, 3, 1, 1, False),
+                (8, 16, 16, 32, 1, 2, 0, True)]
+
+
+@pytest.mark.parametrize("shape", EXACT_SHAPES, ids=lambda s: "x".join(map(str, s[:7])) + ("" if s[7] else "-unaligned"))
+def test_a_workspace_of_exactly_the_queried_size_serves_every_conv_entry_point(dev, shape):
+    """What the *_workspace_bytes queries return is what a call needs: each entry point runs on a bound block of exactly
+    that size (a bound block is never grown, so a query that under-reports shows as CRB_EWORKSPACE)."""
+    import torch
+    from crusaderbackend_amd import capi
+
+    N, IC, H, OC, F, st, p, aligned = shape
+    g = capi.ConvGeom.make(N, IC, H, H, OC, F, F, st, st, p, p)
+    X, W, dY, b = normal(1, N, IC, H, H), he_normal(2, OC, IC, F, F), normal(3, N, OC, g.OH, g.OW), normal(4, OC)
+
+    def place(a):  # aligned: as allocated; otherwise 4 bytes past a 16-byte boundary
+        if aligned:
+            return to_dev(a, dev)
+        buf = torch.empty(a.size + 1, device=dev)
+        buf[1:].copy_(torch.from_numpy(a.reshape(-1)))
+        return buf[1:].view(*a.shape)
+
+    Xd, Wd, dYd, bd = place(X), to_dev(W, dev), place(dY), to_dev(b, dev)
+    Y, dX = place(np.zeros_like(dY)), place(np.zeros_like(X))
+    dW = torch.zeros(OC, IC, F, F, device=dev)
+    s = torch.cuda.Stream(device=dev)
+    need = {"fwd": capi.conv_fwd_workspace_bytes(g, aligned), "dgrad": capi.conv_dgrad_workspace_bytes(g, aligned),
+            "wgrad": capi.conv_wgrad_workspace_bytes(g)}
+    torch.cuda.synchronize()
+    try:
+        for name in ("fwd", "dgrad", "wgrad"):
+            ws = torch.empty(max(need[name], 256) // 4, device=dev)  # nothing needed: a token block, still never grown
+            capi.bind_workspace(ws, stream=s)
+            if name == "fwd":
+                capi.conv_fwd(Wd, Xd, Y, bd, g, stream=s)
+            elif name == "dgrad":
+                capi.conv_dgrad(Wd, dYd, dX, g, stream=s)
+            else:
+                capi.conv_wgrad(dYd, Xd, dW, g, stream=s)
+            s.synchronize()
+    finally:
+        capi.bind_workspace(None, stream=s)
+    assert_close(to_np(Y), orc.conv(W, X, b, st, st, p, p), IC * F * F, f"conv fwd {shape}")
+    assert_close(to_np(dX), orc.convDerive(W, dY, (H, H), st, st, p, p), OC * F * F, f"conv dgrad {shape}")
+    assert_close(to_np(dW), orc.convError(dY, X, np.zeros_like(W), st, st, p, p), N * g.OH * g.OW, f"conv wgrad {shape}")

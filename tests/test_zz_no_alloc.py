@@ -91,3 +91,45 @@ def test_noalloc_refuses_what_does_not_fit_and_bad_arguments(dev):
     with pytest.raises(capi.CrbError) as ei:
         capi.conv_wgrad_noalloc(dY, X, dW, bad)
     assert ei.value.status == capi.CRB_EINVAL_SHAPE
+
+
+def test_noalloc_records_into_a_graph_with_nothing_bound_and_no_arena(dev):
+    """The property the entry point exists for: it runs where nothing may be allocated. A capture on a fresh stream (no
+    workspace bound, the library holds no arena for it) refuses any growth, so an allocation would surface as
+    CRB_EWORKSPACE; the graph is replayed with eager work in between and checked against crb_conv_wgrad every time.
+    Shapes: a direct 3x3 layer, a 1x1 layer on the pixel-contraction kernel, and a 1x1 layer whose operands are off the
+    16-byte grid (the accumulate-NT GEMM form, its split scratch served through the scope)."""
+    import torch
+    from crusaderbackend_amd import capi
+
+    cases = []
+    for i, (N, IC, H, OC, F, st, p, off) in enumerate(((64, 16, 32, 16, 3, 1, 1, 0), (64, 64, 16, 48, 1, 1, 0, 0), (64, 24, 16, 48, 1, 1, 0, 1))):
+        g = capi.ConvGeom.make(N, IC, H, H, OC, F, F, st, st, p, p)
+        X, dY, dW0 = normal(50 + i, N, IC, H, H), normal(60 + i, N, OC, g.OH, g.OW), he_normal(70 + i, OC, IC, F, F)
+
+        def place(a):
+            buf = torch.empty(a.size + off, device=dev)
+            buf[off:].copy_(torch.from_numpy(a.reshape(-1)))
+            return buf[off:].view(*a.shape)
+
+        Xd, dYd = place(X), place(dY)
+        assert capi.conv_wgrad_workspace_bytes(g) > 0
+        want = to_dev(dW0, dev)
+        ws = torch.empty(capi.conv_wgrad_workspace_bytes(g) // 4, device=dev)
+        capi.conv_wgrad(dYd, Xd, want, g, workspace=ws)
+        cases.append((g, Xd, dYd, dW0, want, to_dev(dW0, dev)))
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream(device=dev)  # fresh: nothing bound, no arena
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        for g, Xd, dYd, _, _, got in cases:
+            capi.conv_wgrad_noalloc(dYd, Xd, got, g, stream=torch.cuda.current_stream())
+    torch.cuda.synchronize()
+    for replay in range(3):
+        for _, _, _, dW0, _, got in cases:  # eager work between the replays: reset the accumulated-into tensors
+            got.copy_(torch.from_numpy(dW0))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        for g, _, _, _, want, got in cases:
+            assert torch.equal(got, want), (replay, g.IC, g.OC, g.FH)
