@@ -55,10 +55,13 @@ def parse():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--report", type=str, default=None, help="also time every benchmark configuration and write a JSON report")
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
-    ap.add_argument("--traffic", action="store_true",
-                    help="only run every (layer, pass) call of the workload three times, each group behind a one-float fill "
-                         "launch as a separator, and print the order: under rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE the "
-                         "dispatch list then splits into calls (profiles/resnet56_conv_step_b128.md is built from it)")
+    ap.add_argument("--no-configs", action="store_true",
+                    help="skip the `configs` block (one figure per other benchmark configuration; a few seconds of GPU time)")
+    ap.add_argument("--traffic", nargs="?", const="resnet56", default=None, choices=("resnet56", "densenet"),
+                    help="only run every (layer, pass) call of the workload (default) or of the DenseNet-BC-100 shapes of the "
+                         "report three times, each group behind a one-float fill launch as a separator, and print the order: "
+                         "under rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE the dispatch list then splits into calls "
+                         "(profiles/resnet56_conv_step_b128.md and profiles/densenet_bc100_hbm_bytes_per_call.md are built from it)")
     ap.add_argument("--calibrate", action="store_true",
                     help="only run a plain streaming kernel of known size (a += b on 64 Mi floats: reads 512 MiB, writes "
                          "256 MiB per launch) so hardware byte counters can be scaled against it, then exit")
@@ -66,15 +69,20 @@ def parse():
 
 
 class Layer:
-    def __init__(self, torch, capi, dev, name, IC, H, OC, s, mult, seed, batch=BATCH, F=3, pad=1, bias=False):
+    def __init__(self, torch, capi, dev, name, IC, H, OC, s, mult, seed, batch=BATCH, F=3, pad=1, bias=False, device_rng=False):
         self.name, self.mult = name, mult
         self.g = capi.ConvGeom.make(batch, IC, H, H, OC, F, F, s, s, pad, pad)
         g = self.g
-        gen = torch.Generator(device="cpu").manual_seed(seed)
-        self.X = torch.randn(batch, IC, H, H, generator=gen).to(dev)
-        self.W = (torch.randn(OC, IC, F, F, generator=gen) * math.sqrt(2.0 / (IC * F * F))).to(dev)
-        self.dY = torch.randn(batch, OC, g.OH, g.OW, generator=gen).to(dev)
-        self.b = torch.randn(OC, generator=gen).to(dev) if bias else None
+        # device_rng: values drawn on the GPU (timing-only layers: many tensors, nothing compared with a CPU result)
+        gen = torch.Generator(device=dev if device_rng else "cpu").manual_seed(seed)
+
+        def randn(*shape):
+            return torch.randn(*shape, generator=gen, device=dev) if device_rng else torch.randn(*shape, generator=gen).to(dev)
+
+        self.X = randn(batch, IC, H, H)
+        self.W = randn(OC, IC, F, F) * math.sqrt(2.0 / (IC * F * F))
+        self.dY = randn(batch, OC, g.OH, g.OW)
+        self.b = randn(OC) if bias else None
         self.Y = torch.empty(batch, OC, g.OH, g.OW, device=dev)
         self.dX = torch.empty(batch, IC, H, H, device=dev)
         self.dW = torch.zeros(OC, IC, F, F, device=dev)
@@ -169,16 +177,19 @@ TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "resnet56_conv_step_b128.md")
 
 
 def measured_hbm_bytes():
-    """{call key: bytes per call} and the commit the counters were taken at, from the tracked profile summary ({} if absent)."""
-    table, commit = {}, None
+    """{call key: bytes per call}, the commit the counters were taken at and the hash of the kernel sources they were taken
+    on, from the tracked profile summary ({} if absent)."""
+    table, commit, src_hash = {}, None, None
     try:
         lines = open(TRAFFIC_PROFILE).read().splitlines()
     except OSError:
-        return table, commit
+        return table, commit, src_hash
     on = False
     for ln in lines:
         if ln.startswith("Counters taken at commit"):
             commit = ln.split("`")[1] if "`" in ln else None
+        if ln.startswith("Kernel source hash"):
+            src_hash = ln.split("`")[1] if "`" in ln else None
         if ln.startswith("## HBM bytes per call"):
             on = True
             continue
@@ -190,7 +201,7 @@ def measured_hbm_bytes():
                 table[cells[0].strip("`")] = float(cells[-1]) * 1e6  # last column: total MB per call
             except (ValueError, IndexError):
                 pass
-    return table, commit
+    return table, commit, src_hash
 
 
 def device_clock_khz():
@@ -306,12 +317,23 @@ def main():
         print(json.dumps({"calibrate": "add_inplace_kernel", "floats": n, "read_bytes": 8 * n, "write_bytes": 4 * n}))
         return
 
-    layers = [Layer(torch, capi, dev, n, IC, H, OC, s, m, seed=10 + i) for i, (n, IC, H, OC, s, m) in enumerate(RESNET56)]
+    if args.traffic == "densenet":
+        # benchmark configuration 4: first / middle / last bottleneck of each stage and the stage's 3x3 layer, batch 64
+        layers = []
+        for (H, base) in ((32, 24), (16, 108), (8, 150)):
+            for i in (0, 8, 15):
+                layers.append(Layer(torch, capi, dev, f"1x1_{base + 12 * i}-48@{H}", base + 12 * i, H, 48, 1, 1, seed=300 + i, batch=64, F=1,
+                                    pad=0, bias=True, device_rng=True))
+            layers.append(Layer(torch, capi, dev, f"3x3_48-12@{H}", 48, H, 12, 1, 1, seed=400, batch=64, F=3, pad=1, bias=True, device_rng=True))
+    else:
+        layers = [Layer(torch, capi, dev, n, IC, H, OC, s, m, seed=10 + i) for i, (n, IC, H, OC, s, m) in enumerate(RESNET56)]
     if args.traffic:
         sep = torch.zeros(1, device=dev)
         order = []
         for L in layers:
             for pname, fn, _, _ in L.passes():
+                if args.traffic == "densenet" and pname not in ("fwd", "dgrad", "wgrad"):
+                    continue
                 for _ in range(2):  # untimed: lets every kernel of the call load its code and grow nothing later
                     fn()
                 torch.cuda.synchronize()
@@ -321,7 +343,7 @@ def main():
                 capi.tensor_fill(sep, 0.0, 1)  # closing separator
                 torch.cuda.synchronize()
                 order.append(f"{L.name}.{pname}")
-        print(json.dumps({"traffic_order": order, "calls_per_group": 3,
+        print(json.dumps({"traffic_order": order, "calls_per_group": 3, "algorithmic_bytes": {f"{L.name}.{p}": L.bytes[p] for L in layers for p in ("fwd", "dgrad", "wgrad")},
                           "separator": "a fill of 1 float before and after each group of three calls"}))
         return
     step_flops = sum(3 * L.mult * L.flops for L in layers)
@@ -416,12 +438,21 @@ def main():
     sum_ms = event_time_ms(torch, lambda: capi.sum_slices_multi(slice_table), reps=20) if slice_table is not None else 0.0
     dom = max(per, key=lambda k: per[k]["ms"] * per[k]["mult"])
     d = per[dom]
-    hbm_bytes, hbm_commit = measured_hbm_bytes()
+    hbm_bytes, hbm_commit, hbm_src_hash = measured_hbm_bytes()
+    from crusaderbackend_amd import bench_report
+
+    if hbm_src_hash is None:
+        src_note = "the profile records no kernel source hash"
+    elif hbm_src_hash == bench_report.csrc_hash():
+        src_note = "kernel sources (crusaderbackend_amd/csrc) unchanged since"
+    else:
+        src_note = "WARNING: kernel sources (crusaderbackend_amd/csrc) have changed since the counters were taken (hash %s then, %s now)" % (
+            hbm_src_hash, bench_report.csrc_hash())
     roofline = {
         "bound": "mfma", "kernel": dom, "achieved": d["tflops"], "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s",
         "frac": d["tflops"] / PEAK_FP32_MFMA_TFLOPS, "traffic": hbm_bytes.get(dom),
         "traffic_unit": "bytes per call (FETCH_SIZE and WRITE_SIZE of rocprofv3 --pmc, scaled against a copy kernel)",
-        "traffic_source": "profiles/resnet56_conv_step_b128.md, table 'HBM bytes per call', counters taken at commit %s (not measured by this run)" % hbm_commit,
+        "traffic_source": "profiles/resnet56_conv_step_b128.md, table 'HBM bytes per call', counters taken at commit %s (not measured by this run); %s" % (hbm_commit, src_note),
         "algorithmic_bytes": d["bytes"],
         "flops_per_launch": d["flops"], "avg_launch_ms": d["ms"],
         "share_of_step": d["ms"] * d["mult"] / sum(v["ms"] * v["mult"] for v in per.values()),
@@ -436,9 +467,13 @@ def main():
     # three averages of ten launches: the first follows the allocations above, with the device clock still ramping up, and
     # reads several per cent high; the smallest is reported and all three are kept in `extra`
     gemm_runs = [event_time_ms(torch, lambda: capi.sgemm_nn(A, B, C, n, n, n), reps=10) for _ in range(3)]
-    gemm_ms = min(gemm_runs)
+    gemm_ms, gemm_ms_mean = min(gemm_runs), sum(gemm_runs) / len(gemm_runs)
     gemm_tflops = 2.0 * n ** 3 / gemm_ms / 1e9
     del A, B, C
+    torch.cuda.empty_cache()
+
+    # the other benchmark configurations, one figure each (the full per-call tables: --report)
+    configs = None if args.no_configs else bench_report.compact(torch, capi, dev, event_time_ms, Layer)
 
     clock_khz = device_clock_khz()
 
@@ -465,6 +500,8 @@ def main():
             "kernel_only_tflops": step_flops / kern_sum_ms / 1e9,
             "sgemm_4096_tflops": gemm_tflops, "sgemm_4096_ms": gemm_ms, "sgemm_4096_ms_runs": gemm_runs,
             "sgemm_4096_frac_peak": gemm_tflops / PEAK_FP32_MFMA_TFLOPS,
+            "sgemm_4096_ms_mean": gemm_ms_mean, "sgemm_4096_tflops_mean": 2.0 * 4096 ** 3 / gemm_ms_mean / 1e9,
+            "sgemm_4096_frac_peak_mean": 2.0 * 4096 ** 3 / gemm_ms_mean / 1e9 / PEAK_FP32_MFMA_TFLOPS,
             "slice_sum_all_layers_ms": sum_ms, "slice_sum_items": len(slice_entries),
             "per_kernel": {k: {"ms": round(v["ms"], 5), "tflops": round(v["tflops"], 2), "gbs": round(v["gbs"], 1)}
                            for k, v in per.items()},
@@ -474,11 +511,11 @@ def main():
             "peak_from_reported_clock_tflops": props.multi_processor_count * clock_khz * 1e3 * 256 / 1e12,
         },
     }
+    if configs is not None:
+        out["configs"] = configs
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(RESNET56)
     if args.report:
-        from crusaderbackend_amd import bench_report
-
         rep = bench_report.run(torch, capi, dev, event_time_ms, Layer)
         with open(args.report, "w") as f:
             json.dump(rep, f, indent=1)
