@@ -47,11 +47,12 @@ VGG16_CONVS = [(3, 32, 64), (64, 32, 64), (64, 16, 128), (128, 16, 128), (128, 8
 def _settled(torch, capi, event_time_ms, fn, reps):
     """One row's time: the call is frozen (argument conversion done once: a plain wrapper call costs the host 3.5-4.5 us,
     more than the shortest kernels take), repeated until the timed region is at least a millisecond, three such averages.
-    Returns (smallest, mean): rows follow tensor allocation and host work during which the device clock drops, and its
-    ramp back up takes longer than three warm-up launches, so a first average reads 5-15 % high; the smallest is the
-    row's figure and the mean is reported next to it."""
+    Returns (smallest, mean). Rows follow tensor allocation and host work during which the device clock drops, and its
+    ramp back up takes tens of milliseconds (a dense layer timed right after its tensors were made read 13 % longer than
+    the same call timed a little later), so a row first runs untimed for about 20 ms."""
     f = capi.frozen(fn)
     ms = event_time_ms(torch, f, reps=reps)
+    event_time_ms(torch, f, reps=max(1, min(8000, int(20.0 / max(ms, 1e-4)))), warm=0)
     if ms * reps < 1.0:
         reps = min(4000, int(1.0 / ms) + 1)
     runs = [event_time_ms(torch, f, reps=reps) for _ in range(3)]

@@ -51,6 +51,9 @@ static GemmChoice choose_tiles(u32 M, u32 N, u32 K, u32 zdim, bool dense) {
         if (sp.splits > 1 && sp.k_per_z >= 512) return {TILE_LARGE, 0};
     }
     if (K >= 32768) return {TILE_SMALL_AHEAD, 0};  // very long contraction: slices stay long after the split
+    // tall and skinny (the im2col shape of a 64-channel layer): one column of 64x64 tiles, two per CU; with 64-wide slabs and
+    // eight waves a tile's nine slabs are nine hand-overs instead of 36 (32768 x 64 x 576: 29.3 -> 27.7 us)
+    if (M >= 8192 && N > 32 && N <= 64 && K >= 512 && K < 2048 && zdim == 1) return {TILE_SMALL_DEEP8, 0};
     return {TILE_SMALL, 0};
 }
 

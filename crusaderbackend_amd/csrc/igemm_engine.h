@@ -334,6 +334,7 @@ __global__ void __launch_bounds__(Cfg::NTH, Cfg::OCC) igemm_kernel(AOp a, BOp b,
                 la2.fetch(a, kbeg + BK, kend);
                 lb2.fetch(b, kbeg + BK, kend);
             }
+            fetch_old();  // (one-block wave tiles of the accumulating dense form) behind the first slabs: they arrive with them
             la.commit(sA[0]);
             lb.commit(sB[0]);
         }
@@ -345,7 +346,7 @@ __global__ void __launch_bounds__(Cfg::NTH, Cfg::OCC) igemm_kernel(AOp a, BOp b,
                 far_a.fetch(a, k0 + 2 * BK, kend);
                 far_b.fetch(b, k0 + 2 * BK, kend);
             }
-            if (k0 + BK >= kend) fetch_old();
+            if (k0 + BK >= kend && !old_tried) fetch_old();
             multiply(buf);
             if (k0 + BK < kend) {
                 near_a.commit(sA[buf ^ 1]);
@@ -522,8 +523,9 @@ __device__ __forceinline__ void reduce_vec_block(const float *__restrict__ parti
     // the result's previous value (accumulating forms) is requested before the slices, not after their sum, so that it
     // does not cost a memory round trip of its own at the end
     const u32 j = block * OUTS + threadIdx.x;
-    float prev = 0.f;
+    float prev = 0.f, bias_v = 0.f;
     if ((e.flags & EPI_ACCUM) && threadIdx.x < OUTS && j < count) prev = C[j];
+    if (e.bias && threadIdx.x < OUTS && j < count) bias_v = e.bias[bdiv.div(j) % e.bias_mod];  // likewise: behind the sum it would be a round trip of its own
     float4 s0 = make_float4(0.f, 0.f, 0.f, 0.f), s1 = s0;
     auto add = [](float4 &s, const float4 &v) { s.x += v.x, s.y += v.y, s.z += v.z, s.w += v.w; };
     if (i < count) {
@@ -561,7 +563,7 @@ __device__ __forceinline__ void reduce_vec_block(const float *__restrict__ parti
         float r = red[threadIdx.x];
 #pragma unroll
         for (u32 k = 1; k < ZL; ++k) r += red[k * RS + threadIdx.x];
-        if (e.bias) r += e.bias[bdiv.div(j) % e.bias_mod];
+        if (e.bias) r += bias_v;
         if (e.flags & EPI_ACCUM) r += prev;
         if (e.flags & EPI_RELU) r = r > 0.f ? r : 0.f;
         C[j] = r;
