@@ -138,6 +138,8 @@ class Layer:
         self._dgrad = c.prepared("crb_conv_dgrad", self.W, self.dY, self.dX, self.g, None)
         self._wgrad = c.prepared("crb_conv_wgrad", self.dY, self.X, self.dW, self.g, ws, nbytes, None)
         self._bwd = c.prepared("crb_conv_bwd", self.W, self.dY, self.X, self.dX, self.dW, self.g, ws, nbytes, None)
+        self._bwd_sliced = [c.prepared("crb_conv_bwd_sliced", self.W, self.dY, self.X, self.dX, self.g, w, w.numel() * w.element_size(), None)
+                            for w in self.ws_each]
 
     def fwd(self):
         self._fwd()
@@ -152,7 +154,7 @@ class Layer:
         self._bwd()
 
     def bwd_sliced(self, k=0):
-        self.capi.conv_bwd_sliced(self.W, self.dY, self.X, self.dX, self.g, self.ws_each[k])
+        self._bwd_sliced[k]()
 
     def slice_entries(self):
         return [(ws, dW, self.n_slices) for ws, dW in zip(self.ws_each, self.dW_each)]

@@ -72,7 +72,7 @@ def _densenet_pairs(torch, capi, dev, Layer, device_rng=False):
     return pairs
 
 
-def _densenet_step(torch, event_time_ms, pairs):
+def _densenet_step(torch, capi, event_time_ms, pairs):
     """Config 4 as a whole: forward in network order, then conv / convDerive / convError as separate calls per layer in
     reverse order; also the 1x1 layers alone and the 3x3 layers alone."""
     def dn_step(kinds):
@@ -92,6 +92,25 @@ def _densenet_step(torch, event_time_ms, pairs):
     def work(idx):
         return (sum(3 * p[idx].flops for p in pairs), sum(p[idx].bytes["fwd"] + p[idx].bytes["dgrad"] + p[idx].bytes["wgrad"] for p in pairs))
 
+    # The same work as a training step needs it: per layer the forward call and ONE backward call that leaves the weight
+    # gradient as slices (crb_conv_bwd_sliced), and one crb_sum_slices_multi over all 96 layers at the end of the step.
+    sliced = [L for p in pairs for L in p if L.n_slices]
+    table = capi.slice_sum_table([e for L in sliced for e in L.slice_entries()]) if sliced else None
+
+    def streamlined():
+        for pw, c3 in pairs:
+            pw.fwd(), c3.fwd()
+        for pw, c3 in reversed(pairs):
+            for L in (c3, pw):
+                if L.n_slices:
+                    L.bwd_sliced(0)
+                else:
+                    L.bwd()
+        if table is not None:
+            capi.sum_slices_multi(table)
+
+    sl_ms = min(event_time_ms(torch, streamlined, reps=5, warm=2) for _ in range(2))
+
     all_ms = min(event_time_ms(torch, dn_step(("1x1", "3x3")), reps=5, warm=2) for _ in range(2))
     pw_ms = min(event_time_ms(torch, dn_step(("1x1",)), reps=5, warm=2) for _ in range(2))
     c3_ms = min(event_time_ms(torch, dn_step(("3x3",)), reps=5, warm=2) for _ in range(2))
@@ -104,6 +123,8 @@ def _densenet_step(torch, event_time_ms, pairs):
         "pointwise_frac_hbm": round(pw_by / pw_ms / 1e6 / PEAK_GBS, 4), "pointwise_tflops": round(pw_fl / pw_ms / 1e9, 2),
         "conv3x3_us": round(c3_ms * 1e3, 1), "conv3x3_gflop": round(c3_fl / 1e9, 2), "conv3x3_tflops": round(c3_fl / c3_ms / 1e9, 2),
         "conv3x3_frac_mfma": round(c3_fl / c3_ms / 1e9 / PEAK_TF, 4),
+        "one_backward_call_us": round(sl_ms * 1e3, 1), "one_backward_call_tflops": round((pw_fl + c3_fl) / sl_ms / 1e9, 2),
+        "one_backward_call_images_per_s": round(64 / sl_ms * 1e3, 1), "one_backward_call_layers_sliced": len(sliced),
     }
 
 
@@ -194,13 +215,16 @@ def compact(torch, capi, dev, event_time_ms, Layer):
     torch.cuda.empty_cache()
     # config 4: the whole DenseNet-BC-100 convolution step
     pairs = _densenet_pairs(torch, capi, dev, Layer, device_rng=True)
-    d = _densenet_step(torch, event_time_ms, pairs)
+    d = _densenet_step(torch, capi, event_time_ms, pairs)
     del pairs
     torch.cuda.empty_cache()
     out["4_densenet_bc100_conv_step_b64"] = {
         "ms": round(d["us"] / 1e3, 4), "tflops": d["tflops"], "images_per_s": d["images_per_s"],
         "pointwise": {"ms": round(d["pointwise_us"] / 1e3, 4), "gbs": d["pointwise_gbs"], "bound": "hbm", "frac": d["pointwise_frac_hbm"]},
         "conv3x3": {"ms": round(d["conv3x3_us"] / 1e3, 4), "tflops": d["conv3x3_tflops"], "bound": "mfma", "frac": d["conv3x3_frac_mfma"]},
+        "one_backward_call_per_layer": {"ms": round(d["one_backward_call_us"] / 1e3, 4), "tflops": d["one_backward_call_tflops"],
+                                        "images_per_s": d["one_backward_call_images_per_s"],
+                                        "what": "crb_conv_fwd + crb_conv_bwd_sliced per layer, one crb_sum_slices_multi per step"},
         "what": "48 x (1x1 IC->48, 3x3 48->12), conv / convDerive / convError as separate calls, every layer on tensors of its own"}
     # config 5
     for e in _dense_rows(torch, capi, dev, settled):
@@ -277,7 +301,7 @@ def run(torch, capi, dev, event_time_ms, Layer):
 
     # config 4 as a whole: the convolution work of one DenseNet-BC-100 training step at batch 64
     pairs = _densenet_pairs(torch, capi, dev, Layer)
-    out["densenet_full_step"] = _densenet_step(torch, event_time_ms, pairs)
+    out["densenet_full_step"] = _densenet_step(torch, capi, event_time_ms, pairs)
     del pairs
     torch.cuda.empty_cache()
 

@@ -158,6 +158,7 @@ inline PwWgradPlan pw_wgrad_plan(u32 N, u32 IC, u32 OC, u32 HW) {
     return p;
 }
 
+// dW == nullptr (a split plan only): the slices are left in ws, unsummed.
 inline int launch_pw_wgrad(const float *dY, const float *X, float *dW, float *ws, const PwWgradPlan &p, u32 IC, u32 OC, u32 HW,
                            hipStream_t s, const char *what) {
     PwWgradArgs a;
@@ -172,7 +173,7 @@ inline int launch_pw_wgrad(const float *dY, const float *X, float *dW, float *ws
     else
         hipLaunchKernelGGL(pw_wgrad_kernel<4>, dim3(u32(wgs)), dim3(kThreads), 0, s, a);
     if (int st = check_launch(what)) return st;
-    if (p.splits > 1) return launch_splitk_reduce(ws, dW, OC * IC, p.splits, ReduceEpi{nullptr, 1, 1, EPI_ACCUM}, s, what);
+    if (p.splits > 1 && dW) return launch_splitk_reduce(ws, dW, OC * IC, p.splits, ReduceEpi{nullptr, 1, 1, EPI_ACCUM}, s, what);
     return CRB_OK;
 }
 

@@ -445,13 +445,25 @@ static bool bwd_fused(const crb_conv_geom *g, bool run, const float *Wt, const f
     typedef DirectCfg<16, 8, 16, 16, 2, 1, true, 2, 2, 2> D16s2c;           // chunks of 16
     typedef DirectCfg<8, 8, 8, 32, 1, 2, true, 2, 2, 2> D8s2;
     typedef DirectCfg<8, 8, 16, 32, 1, 2, true, 2, 2, 2> D8s2c;
+    // growth-12 dense layers (48 -> 12): the data gradient reads 9..12 channels and writes 33..48; the configurations are
+    // the ones try_direct<true, 1> picks for these shapes
+    typedef DirectCfg<32, 4, 12, 48, 2, 3, true, 2, 1, 1, 3, 2> D32g;
+    typedef DirectCfg<16, 4, 12, 48, 1, 3, true, 2, 1, 1> D16g;
+    typedef DirectCfg<8, 8, 16, 16, 1, 1, true, 2, 2, 1> D8g;
     typedef WgradCfg<32, 8, 1, 2, 1> W32a;
     typedef WgradCfg<16, 16, 1, 2, 1> W16a;
     typedef WgradCfg<8, 8, 4, 2, 1> W8a;
+    typedef WgradCfg<16, 8, 1, 2, 1> W16b;  // what crb_conv_wgrad falls back to when the image height or the batch does not fit
+    typedef WgradCfg<8, 8, 2, 2, 1> W8b;
     typedef WgradCfg<16, 8, 1, 1, 2> W16s2;
     typedef WgradCfg<8, 8, 2, 1, 2> W8s2;
     const u32 ci = g->OC, co = g->IC;  // channels the data gradient reads / writes
     if (direct_shape(g, 1)) {
+        if (ci > 8 && ci <= 12 && co > 32 && co <= 48) {
+            if (g->OW == 32) return CRB_PAIR(D32g, W32a);
+            if (g->OW == 16) return CRB_PAIR(D16g, W16a) || CRB_PAIR(D16g, W16b);
+            if (g->OW == 8) return CRB_PAIR(D8g, W8a) || CRB_PAIR(D8g, W8b);
+        }
         if (g->OW == 32 && ci <= 16 && ci > 8 && co <= 16) return CRB_PAIR(D32a, W32a);
         if (g->OW == 16 && co > 16 && co <= 64 && ci > 8)
             return one_chunk_w16(g->N, ci, co, g->OH) ? CRB_PAIR(D16r, W16a) : CRB_PAIR(D16a, W16a);
@@ -854,7 +866,12 @@ uint32_t crb_conv_bwd_slices(const crb_conv_geom *g) {
     if (check_geom("crb_conv_bwd_slices", g)) return 0;
     WgradDirectPlan dp;
     int st = CRB_OK;
-    if (pointwise_shape(g) || tiny2x2_shape(g)) return 0;
+    if (pointwise_shape(g)) {  // the pixel-contraction weight gradient leaves one slice per pixel range
+        if (!pw_wgrad_fits(g->IC, g->OC, g->IH * g->IW)) return 0;
+        const u32 n = pw_wgrad_plan(g->N, g->IC, g->OC, g->IH * g->IW).splits;
+        return n > 1 ? n : 0;
+    }
+    if (tiny2x2_shape(g)) return 0;
     if (shortcut_shape(g)) {
         const u32 n = sc_wgrad_plan(g->N, g->IC, g->OC, g->OH, g->OW).splits;
         return n > 1 ? n : 0;
@@ -873,6 +890,13 @@ int crb_conv_bwd_sliced(const float *W, const float *dY, const float *X, float *
     int st = CRB_OK;
     float *ws = static_cast<float *>(workspace);
     hipStream_t s = hipStream_t(stream);
+    if (pointwise_shape(g)) {
+        const PwWgradPlan pp = pw_wgrad_plan(g->N, g->IC, g->OC, g->IH * g->IW);
+        if (workspace_bytes < pp.workspace_bytes)
+            return fail(CRB_EWORKSPACE, "crb_conv_bwd_sliced: workspace %zu bytes < required %zu", workspace_bytes, pp.workspace_bytes);
+        if (int sd = crb_conv_dgrad(W, dY, dX, g, stream)) return sd;
+        return launch_pw_wgrad(dY, X, nullptr, ws, pp, g->IC, g->OC, g->IH * g->IW, s, "crb_conv_bwd_sliced");
+    }
     if (shortcut_shape(g)) {
         const ScWgradPlan sp = sc_wgrad_plan(g->N, g->IC, g->OC, g->OH, g->OW);
         if (workspace_bytes < sp.workspace_bytes)

@@ -331,7 +331,10 @@ BWD_CASES = [(8, 16, 32, 16, 3, 1, 1), (128, 16, 32, 16, 3, 1, 1), (8, 32, 16, 3
              (8, 32, 16, 64, 3, 2, 1), (128, 32, 16, 64, 3, 2, 1),
              (6, 12, 32, 14, 3, 1, 1), (6, 24, 16, 40, 3, 1, 1), (6, 64, 8, 48, 3, 1, 1), (3, 64, 8, 64, 3, 1, 1),
              (4, 3, 32, 16, 3, 1, 1), (4, 64, 32, 64, 3, 1, 1), (4, 128, 8, 128, 3, 1, 1), (4, 8, 12, 8, 3, 1, 1),
-             (4, 16, 16, 8, 5, 1, 2), (4, 24, 8, 12, 1, 1, 0), (4, 32, 2, 32, 3, 1, 1), (4, 32, 4, 32, 3, 1, 1)]
+             (4, 16, 16, 8, 5, 1, 2), (4, 24, 8, 12, 1, 1, 0), (4, 32, 2, 32, 3, 1, 1), (4, 32, 4, 32, 3, 1, 1),
+             # growth-12 dense layers: both gradients in one launch at the three image sizes (and sizes off the tile grid)
+             (8, 48, 32, 12, 3, 1, 1), (64, 48, 32, 12, 3, 1, 1), (8, 48, 16, 12, 3, 1, 1), (64, 48, 16, 12, 3, 1, 1),
+             (8, 48, 8, 12, 3, 1, 1), (64, 48, 8, 12, 3, 1, 1), (6, 40, 8, 10, 3, 1, 1), (3, 48, 24, 12, 3, 1, 1), (5, 36, 16, 9, 3, 1, 1)]
 
 
 @pytest.mark.parametrize("N,IC,H,OC,F,s,p", BWD_CASES)
@@ -381,7 +384,8 @@ def test_conv_bwd_sliced_then_one_sum_equals_bwd(dev):
     import torch
     capi = _capi()
     specs = [(128, 16, 32, 16, 1), (128, 32, 16, 32, 1), (128, 64, 8, 64, 1), (128, 16, 32, 32, 2), (128, 32, 16, 64, 2),
-             (16, 64, 32, 64, 1), (32, 128, 8, 128, 1), (8, 16, 32, 16, 1), (64, 48, 16, 12, 1)]
+             (16, 64, 32, 64, 1), (32, 128, 8, 128, 1), (8, 16, 32, 16, 1), (64, 48, 16, 12, 1), (64, 48, 32, 12, 1), (64, 48, 8, 12, 1),
+             (6, 40, 8, 10, 1)]
     layers, entries = [], []
     for i, (N, IC, H, OC, s) in enumerate(specs):
         g = capi.ConvGeom.make(N, IC, H, H, OC, 3, 3, s, s, 1, 1)
@@ -427,7 +431,7 @@ def test_conv_bwd_sliced_many_items_and_errors(dev):
     for (ws, dst, n), ref in zip(entries, refs):
         assert_close(to_np(dst), ref, n, "slice sum")
     # geometries without a sliced form
-    assert capi.conv_bwd_slices(capi.ConvGeom.make(4, 24, 8, 8, 12, 1, 1, 1, 1, 0, 0)) == 0
+    assert capi.conv_bwd_slices(capi.ConvGeom.make(4, 8, 8, 8, 12, 1, 1, 1, 1, 0, 0)) == 0
     assert capi.conv_bwd_slices(capi.ConvGeom.make(4, 16, 12, 12, 8, 3, 3, 1, 1, 1, 1)) == 0
     t = torch.zeros(1 << 16, device=dev)
     p = t.data_ptr()
@@ -510,6 +514,35 @@ def test_shortcut_weight_gradients_join_the_postponed_sum(dev):
     torch.cuda.synchronize()
     for dX1, dW1, dX2, dW2 in layers:
         assert np.array_equal(to_np(dX1), to_np(dX2)) and np.array_equal(to_np(dW1), to_np(dW2))
+
+
+def test_pointwise_weight_gradients_join_the_postponed_sum(dev):
+    """1x1 stride-1 layers (dense-network bottlenecks) have a sliced form too: dX at once, dW after crb_sum_slices_multi, both
+    exactly as crb_conv_bwd gives them; the growth-12 3x3 layers behind them run both gradients in one launch."""
+    import torch
+    capi = _capi()
+    layers, entries = [], []
+    for i, (N, IC, H, OC) in enumerate([(64, 24, 32, 48), (64, 204, 32, 48), (64, 108, 16, 48), (64, 150, 8, 48), (8, 40, 8, 20), (3, 330, 8, 48)]):
+        g = capi.ConvGeom.make(N, IC, H, H, OC, 1, 1)
+        n_slices = capi.conv_bwd_slices(g)
+        assert n_slices > 1, (N, IC, H, OC)
+        X, W = to_dev(normal(10 + i, N, IC, H, H), dev), to_dev(he_normal(30 + i, OC, IC, 1, 1), dev)
+        dY, dW0 = to_dev(normal(50 + i, N, OC, H, H), dev), normal(70 + i, OC, IC, 1, 1)
+        ws = torch.empty(capi.conv_wgrad_workspace_bytes(g) // 4, dtype=torch.float32, device=dev)
+        assert ws.numel() >= n_slices * OC * IC
+        dX1, dW1 = _nan(dev, N, IC, H, H), to_dev(dW0, dev)
+        capi.conv_bwd(W, dY, X, dX1, dW1, g)
+        dX2, dW2 = _nan(dev, N, IC, H, H), to_dev(dW0, dev)
+        capi.conv_bwd_sliced(W, dY, X, dX2, g, ws)
+        layers.append((dX1, dW1, dX2, dW2))
+        entries.append((ws, dW2, n_slices))
+    capi.sum_slices_multi(capi.slice_sum_table(entries))
+    torch.cuda.synchronize()
+    for dX1, dW1, dX2, dW2 in layers:
+        assert np.array_equal(to_np(dX1), to_np(dX2)) and np.array_equal(to_np(dW1), to_np(dW2))
+    with pytest.raises(capi.CrbError) as ei:  # too small a workspace is refused before anything is launched
+        capi.conv_bwd_sliced(W, dY, X, dX2, g, ws[:16])
+    assert ei.value.status == capi.CRB_EWORKSPACE
 
 
 # 32-wide forward with 9..16 input and at most 16 output channels: the contraction in two halves (the second half of the rows
