@@ -55,14 +55,31 @@ constexpr int kPwsThreads = 512;  // eight waves: the filter matrix is staged on
 // Staging of the filter matrix W (OC x IC, rows contiguous) for contraction/input channels [c0, c0 + kc), kc <= 256:
 // thread t owns column t % 256 and the rows t / 256, t / 256 + 2, ... of the ROWS staged ones; all of a thread's loads are
 // in flight together (one memory round trip), and there is no division in the address arithmetic.
-// dst[column * col_stride + row * row_stride]; rows or columns past the tensor's extent are staged as zeros.
-template <int ROWS>
-__device__ __forceinline__ void pws_stage(float *dst, const float *W, u32 OC, u32 IC, u32 c0, u32 kc, u32 cols, u32 row_stride, u32 col_stride) {
+// dst[at(column, row)]; rows or columns past the tensor's extent are staged as zeros.
+template <int ROWS, class At>
+__device__ __forceinline__ void pws_stage(float *dst, const float *W, u32 OC, u32 IC, u32 c0, u32 kc, u32 cols, At at) {
     static_assert(kPwsThreads == 512 && ROWS % 2 == 0, "two row phases of 256 columns");
     const u32 col = threadIdx.x & 255u, r0 = threadIdx.x >> 8;
     if (col >= cols) return;
     // every load is issued (clamped to a valid element) and the value dropped afterwards: a branch around a load would
     // put a wait for the previous one in front of it
+    float v[ROWS / 2];
+    const u32 ccol = col < kc ? col : kc - 1;
+#pragma unroll
+    for (int i = 0; i < ROWS / 2; ++i) {
+        const u32 row = r0 + 2 * i;
+        v[i] = W[size_t(row < OC ? row : OC - 1) * IC + c0 + ccol];
+    }
+#pragma unroll
+    for (int i = 0; i < ROWS / 2; ++i) dst[at(col, r0 + 2 * i)] = (col < kc && r0 + 2 * i < OC) ? v[i] : 0.f;
+}
+
+// The same staging to dst[column * col_stride + row * row_stride].
+template <int ROWS>
+__device__ __forceinline__ void pws_stage(float *dst, const float *W, u32 OC, u32 IC, u32 c0, u32 kc, u32 cols, u32 row_stride, u32 col_stride) {
+    static_assert(kPwsThreads == 512 && ROWS % 2 == 0, "two row phases of 256 columns");
+    const u32 col = threadIdx.x & 255u, r0 = threadIdx.x >> 8;
+    if (col >= cols) return;
     float v[ROWS / 2];
     const u32 ccol = col < kc ? col : kc - 1;
 #pragma unroll
@@ -77,17 +94,23 @@ __device__ __forceinline__ void pws_stage(float *dst, const float *W, u32 OC, u3
 template <int NOB>
 struct PwsFwdLds {
     static constexpr int KC = NOB <= 3 ? 256 : 192;                              // contraction channels staged per pass
-    // row stride == 17 mod 32: the lane groups l/16 = 0, 1 of a half-wave meet in one bank only, and the staging stores
-    // (consecutive lanes on consecutive rows) spread over all banks
-    static constexpr int WP = (NOB <= 1 ? 16 : (NOB <= 3 ? 48 : 80)) + 1;
-    static constexpr int FLOATS = (KC + 4) * WP;  // one channel step past the staged rows may be read (never used)
+    // Ws holds one row of NOB * 16 output channels per contraction channel; channel c sits at (c / 2) * PS + (c % 2) * S1.
+    // S1 == 16 mod 32: a fragment read's two lane groups of a half-wave (channels 4s and 4s + 1, or 4s + 2 and 4s + 3,
+    // sixteen consecutive output channels each) cover all 32 banks once. PS odd: the staging stores (consecutive lanes on
+    // consecutive channels) of a half-wave are sixteen channel pairs whose starts p * PS are distinct mod 32 and never
+    // 16 apart, so they cover all 32 banks once as well.
+    static constexpr int S1 = NOB <= 1 ? 16 : (NOB <= 3 ? 48 : 80);
+    static constexpr int PS = 2 * S1 + 1;
+    static constexpr int FLOATS = (KC / 2 + 2) * PS;  // one channel step past the staged rows may be read (never used)
+    static __device__ __forceinline__ u32 at(u32 c) { return (c >> 1) * u32(PS) + (c & 1u) * u32(S1); }
 };
 
 template <int NOB, int PV>
 __global__ void __launch_bounds__(kPwsThreads, 1) pw_fwd_stream_kernel(PwStreamArgs a) {
     typedef typename PixVec<PV>::T XV;
-    constexpr int KC = PwsFwdLds<NOB>::KC, WP = PwsFwdLds<NOB>::WP, D = kPwsDepth;
-    __shared__ __attribute__((aligned(16))) float Ws[PwsFwdLds<NOB>::FLOATS];  // Ws[ic][oc]
+    typedef PwsFwdLds<NOB> LdsW;
+    constexpr int KC = LdsW::KC, D = kPwsDepth;
+    __shared__ __attribute__((aligned(16))) float Ws[LdsW::FLOATS];  // Ws[ic][oc], see PwsFwdLds
     const u32 t = threadIdx.x, lane = t & 63, wave = t >> 6, j = lane & 15, k = lane >> 4;
     const u32 task = blockIdx.x * (kPwsThreads / 64) + wave;
     const bool on = task < a.tasks;  // idle waves still help staging and meet the barriers
@@ -111,29 +134,35 @@ __global__ void __launch_bounds__(kPwsThreads, 1) pw_fwd_stream_kernel(PwStreamA
             bias_v[o][r] = (a.bias && oc < a.OC) ? a.bias[oc] : 0.f;
         }
 
+    // Channel step s of a pass that starts at channel c0: this lane's channel is c0 + 4 s + k; past the tensor's extent it
+    // reads the last channel and is zeroed at use (its filter values are zero, but 0 * inf is not). Past the pass it reads
+    // one dummy line, so that every iteration issues the same loads and the wait in front of a use covers exactly the
+    // loads issued before it.
+    XV xq[D];
+    auto issue_at = [&](u32 c0, u32 steps, u32 s, int slot) {
+        const u32 ch = c0 + 4 * s + k;
+        const float *p = s < steps ? xrun + size_t(ch < a.IC ? ch : a.IC - 1) * a.HW : a.X;
+        xq[slot] = *reinterpret_cast<const XV *>(p);
+    };
+    // (Requesting the first pass's activations before the filters are staged was measured and is not done: the staging's
+    // own loads then queue behind them, 204 -> 48 @ 32x32 at batch 64 took 17.6 instead of 15.3 us.)
+
     for (u32 c0 = 0; c0 < a.IC; c0 += KC) {
         const u32 kc = a.IC - c0 < u32(KC) ? a.IC - c0 : u32(KC);
         const u32 steps = (kc + 3) / 4, kc4 = steps * 4;
         if (c0) __syncthreads();  // every wave is done with the previous pass's filters
         // consecutive threads take consecutive contraction channels of one filter row (contiguous in memory)
-        pws_stage<NOB * 16>(Ws, a.Wt, a.OC, a.IC, c0, kc, kc4, 1, WP);
+        pws_stage<NOB * 16>(Ws, a.Wt, a.OC, a.IC, c0, kc, kc4, [](u32 col, u32 row) { return LdsW::at(col) + row; });
         __syncthreads();
         if (!on) continue;
 
-        // Channel step s: this lane's channel is c0 + 4 s + k; past the tensor's extent it reads the last channel and is
-        // zeroed at use (its filter values are zero, but 0 * inf is not). Past the pass it reads one dummy line, so that
-        // every iteration issues the same loads and the wait in front of a use covers exactly the loads issued before it.
-        XV xq[D];
-        auto issue = [&](u32 s, int slot) {
-            const u32 ch = c0 + 4 * s + k;
-            const float *p = s < steps ? xrun + size_t(ch < a.IC ? ch : a.IC - 1) * a.HW : a.X;
-            xq[slot] = *reinterpret_cast<const XV *>(p);
-        };
-        const float *wl = Ws + k * WP + j;
+        auto issue = [&](u32 s, int slot) { issue_at(c0, steps, s, slot); };
+        // this lane's filter values of step s: channel 4 s + k, output channels 16 o + j
+        const float *wl = Ws + (k >> 1) * LdsW::PS + (k & 1u) * LdsW::S1 + j;
         float av[2][NOB];
         auto read_a = [&](u32 s, int slot) {
 #pragma unroll
-            for (int o = 0; o < NOB; ++o) av[slot][o] = wl[(4 * s) * WP + o * 16];
+            for (int o = 0; o < NOB; ++o) av[slot][o] = wl[(2 * s) * LdsW::PS + o * 16];
         };
 #pragma unroll
         for (int i = 0; i < D; ++i) issue(i, i);
