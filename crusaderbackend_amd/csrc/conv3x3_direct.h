@@ -145,7 +145,7 @@ struct DirectArgs {
 template <class Cfg>
 __device__ __forceinline__ void conv3x3_body(const DirectArgs &a, const u32 bid, float *smem) {
     constexpr int W = Cfg::W, ROWS = Cfg::ROWS, CI = Cfg::CI, OCT = Cfg::OCT, PBW = Cfg::PBW, OBW = Cfg::OBW;
-    constexpr int XS = Cfg::XS, XR = Cfg::XR, XP = Cfg::XP, NSTEP = Cfg::NSTEP, WSTR = Cfg::WSTR, SW = Cfg::SW;
+    constexpr int XS = Cfg::XS, XR = Cfg::XR, XP = Cfg::XP, WSTR = Cfg::WSTR, SW = Cfg::SW;
     constexpr int NBUF = Cfg::NBUF, NPH = Cfg::NPH;
     float(*sX)[Cfg::X_SIZE] = reinterpret_cast<float(*)[Cfg::X_SIZE]>(smem);
     float(*sW)[Cfg::W_SIZE] = reinterpret_cast<float(*)[Cfg::W_SIZE]>(smem + NBUF * Cfg::X_SIZE);

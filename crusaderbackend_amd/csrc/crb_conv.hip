@@ -370,7 +370,9 @@ static bool wgrad_direct(const crb_conv_geom *g, bool run, const float *dY, cons
                    wgrad_cfg2<4, 4, 4, 2, 1>(g, run, dY, X, dW, ws, s, plan, status);
     } else if (direct_shape(g, 2)) {
         if (g->OW == 32) return wgrad_cfg2<32, 4, 1, 1, 2>(g, run, dY, X, dW, ws, s, plan, status);
-        if (g->OW == 16) return wgrad_cfg2<16, 8, 1, 1, 2>(g, run, dY, X, dW, ws, s, plan, status);
+        if (g->OW == 16)
+            return wgrad_cfg2<16, 4, 1, 2, 2>(g, run, dY, X, dW, ws, s, plan, status) ||
+                   wgrad_cfg2<16, 8, 1, 1, 2>(g, run, dY, X, dW, ws, s, plan, status);
         if (g->OW == 8)
             return wgrad_cfg2<8, 8, 2, 1, 2>(g, run, dY, X, dW, ws, s, plan, status) ||
                    wgrad_cfg2<8, 4, 2, 1, 2>(g, run, dY, X, dW, ws, s, plan, status);
@@ -443,8 +445,6 @@ static bool bwd_fused(const crb_conv_geom *g, bool run, const float *Wt, const f
     typedef DirectCfg<8, 8, 16, 32, 1, 2, true, 2, 2, 1> D8a;
     typedef DirectCfg<16, 8, 8, 16, 2, 1, true, 2, 2, 2> D16s2;             // chunks of 8
     typedef DirectCfg<16, 8, 16, 16, 2, 1, true, 2, 2, 2> D16s2c;           // chunks of 16
-    typedef DirectCfg<8, 8, 8, 32, 1, 2, true, 2, 2, 2> D8s2;
-    typedef DirectCfg<8, 8, 16, 32, 1, 2, true, 2, 2, 2> D8s2c;
     // growth-12 dense layers (48 -> 12): the data gradient reads 9..12 channels and writes 33..48; the configurations are
     // the ones try_direct<true, 1> picks for these shapes
     typedef DirectCfg<32, 4, 12, 48, 2, 3, true, 2, 1, 1, 3, 2> D32g;
@@ -455,8 +455,7 @@ static bool bwd_fused(const crb_conv_geom *g, bool run, const float *Wt, const f
     typedef WgradCfg<8, 8, 4, 2, 1> W8a;
     typedef WgradCfg<16, 8, 1, 2, 1> W16b;  // what crb_conv_wgrad falls back to when the image height or the batch does not fit
     typedef WgradCfg<8, 8, 2, 2, 1> W8b;
-    typedef WgradCfg<16, 8, 1, 1, 2> W16s2;
-    typedef WgradCfg<8, 8, 2, 1, 2> W8s2;
+    typedef WgradCfg<16, 4, 1, 2, 2> W16s2;  // 4-row tiles: 51 KB of LDS, so that a workgroup of each kind shares a CU (8-row tiles: 92 KB)
     const u32 ci = g->OC, co = g->IC;  // channels the data gradient reads / writes
     if (direct_shape(g, 1)) {
         if (ci > 8 && ci <= 12 && co > 32 && co <= 48) {
@@ -470,8 +469,9 @@ static bool bwd_fused(const crb_conv_geom *g, bool run, const float *Wt, const f
         if (g->OW == 8 && co <= 64 && ci > 8) return CRB_PAIR(D8a, W8a);
     } else if (direct_shape(g, 2)) {
         if (g->OW == 16 && co <= 16) return s2_dgrad_w16_c16(g->N, ci, co, g->OH) ? CRB_PAIR(D16s2c, W16s2) : CRB_PAIR(D16s2, W16s2);
-        if (g->OW == 8 && co > 16)  // here the data gradient is the longer half
-            return s2_dgrad_w8_c16(g->N, ci, co) ? CRB_PAIR(D8s2c, W8s2, true) : CRB_PAIR(D8s2, W8s2, true);
+        // 8-wide stride-2 layers (32 -> 64) run the two gradients as two launches: the weight gradient's 8-row tiles of two
+        // images need 92 KB of LDS, so a CU held one workgroup of the pair at a time and the one launch took as long as
+        // both (15.1 us against 6.8 + 6.4), and tile shapes small enough for two to share a CU were slower still
     }
 #undef CRB_PAIR
     return false;
