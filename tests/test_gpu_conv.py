@@ -120,6 +120,15 @@ def test_conv_densenet_layers_full_batch(dev, IC, H):
     run_layer(dev, 64, 48, H, H, 12, 3, 3, 1, 1, 1, 1, seed=16)
 
 
+@pytest.mark.parametrize("H,base", [(32, 24), (16, 108), (8, 150)])
+def test_conv_densenet_every_bottleneck_width_full_batch(dev, H, base):
+    """benchmark configuration 4, every one of its 48 bottleneck layers at its own batch (64) and with the bias the dense block
+    gives them (seann/operands/prefabs/DenseBlock.cuh:53): IC = base + 12 i, i = 0..15, per stage."""
+    for i in range(16):
+        run_layer(dev, 64, base + 12 * i, H, H, 48, 1, 1, 1, 1, 0, 0, bias=True, seed=200 + i, ws=bool(i & 1))
+    run_layer(dev, 64, 48, H, H, 12, 3, 3, 1, 1, 1, 1, bias=True, seed=17, ws=True)
+
+
 def test_conv_vgg_stem_and_wide(dev):
     run_layer(dev, 4, 3, 32, 32, 64, 3, 3, 1, 1, 1, 1, bias=True, seed=7)
     run_layer(dev, 2, 256, 4, 4, 512, 3, 3, 1, 1, 1, 1, bias=True, seed=8)
