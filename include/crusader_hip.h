@@ -177,8 +177,9 @@ int crb_conv_bias(float *Y, const float *bias, uint32_t N, uint32_t C, uint32_t 
 /* Both gradients of a convolution layer in one call: dX as crb_conv_dgrad writes it and dW as crb_conv_wgrad accumulates
  * it (same workspace rule: crb_conv_wgrad_workspace_bytes(g) bytes, or NULL for the library arena). Replaces the pair of
  * calls Conv2D::xGrads / Conv2D::paramGrads make back to back (seann/operands/seblas/Conv2D.cu:18-29: convDerive, then
- * convError): the two are independent, and for the layer shapes of CIFAR residual networks they run as one launch that
- * shares the chip; other shapes run the two calls one after the other. Results are identical to the separate calls.
+ * convError): the two are independent, and for the 3x3 layer shapes of CIFAR residual networks (stride 1, and the 16 -> 32
+ * stride-2 transition) and the growth-12 layers of dense networks (48 -> 12) they run as one launch that shares the chip;
+ * other shapes run the two calls one after the other. Results are identical to the separate calls.
  * dX must not overlap X or dY. */
 int crb_conv_bwd(const float *W, const float *dY, const float *X, float *dX, float *dW, const crb_conv_geom *g, void *workspace,
                  size_t workspace_bytes, void *stream);
@@ -187,7 +188,9 @@ int crb_conv_bwd(const float *W, const float *dY, const float *X, float *dX, flo
  * runs (no counterpart in the reference). crb_conv_bwd_sliced writes dX as crb_conv_bwd does and leaves the weight
  * gradient of this call as crb_conv_bwd_slices(g) partial sums ("slices", each OC*IC*FH*FW floats, one after the other)
  * in `workspace` (caller-owned, crb_conv_wgrad_workspace_bytes(g) bytes, 16-byte aligned, not shared with another pending
- * call). crb_conv_bwd_slices returns 0 for geometries without a sliced form: use crb_conv_bwd for those.
+ * call). Geometries with a sliced form: 3x3 / pad 1 layers on the direct kernels, 1x1 / stride 1 layers on the
+ * pixel-contraction kernel (at most 64 output channels, at least 16 input channels, whole 64-pixel runs), 1x1 / stride 2
+ * shortcuts. crb_conv_bwd_slices returns 0 for geometries without one: use crb_conv_bwd for those.
  * crb_sum_slices_multi then completes any number of such gradients in one launch: for every item,
  * dst[i] += sum over z of slices[z*count + i]; `items` is host memory. The summation order per element is the one
  * crb_conv_wgrad / crb_conv_bwd use internally, so the results are bit-identical to theirs. */
