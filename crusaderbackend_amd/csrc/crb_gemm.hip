@@ -1,6 +1,7 @@
 // C-ABI entry points of the GEMM and dense-layer families (fp32, row-major) on the MFMA engine.
 #include "gemm_internal.h"
 #include "gemm_tiny.h"
+#include "igemm_dma.h"
 #include "operands.h"
 
 namespace crb {
@@ -110,9 +111,45 @@ static int run_tiles(const AOp &a, const BOp &b, const E &e, u32 M, u32 N, u32 K
     }
 }
 
+// ---- products of plain dense matrices on the direct-to-LDS kernel (igemm_dma.h) ---------------------------------------------
+// Taken when the contraction is a multiple of 32, the operands are 16-byte friendly and the tile grid fills the chip in
+// whole rounds; everything else stays on the register-staged engine. Returns 0: not taken; 1: 128 x 128 tiles; 2: 64 x 64.
+static int choose_dma(u32 M, u32 N, u32 K, u32 zdim) {
+    if (K % 32 || K < 256) return 0;  // whole 32-deep slabs; a short contraction is mostly prologue and epilogue
+    const uint64_t tiles_l = uint64_t(ceil_div(M, 128)) * ceil_div(N, 128) * zdim;
+    const uint64_t tiles_s = uint64_t(ceil_div(M, 64)) * ceil_div(N, 64) * zdim;
+    // One 128 x 128 tile per CU already runs close to the MFMA rate, so the time goes by whole rounds of 256 tiles: taken
+    // when the last round is (nearly) full. Measured against the register-staged engine, NN / NT / TN alike:
+    // 2048^3 138 vs 150 us, 4096 x 4096 x 256 76 vs 83, 4096^3 1025 vs 1070; 3072^3 (2.25 rounds) 583 vs 494.
+    if (M >= 128 && N >= 128 && tiles_l >= 256 && tiles_l * 10 >= ceil_div(tiles_l, 256) * 256 * 9) return 1;
+    // 64 x 64 tiles, two per CU: rounds of 512 (512 x 4096 x 1024 40.3 vs 42.8 us, 32768 x 64 x 576 25.3 vs 26.4;
+    // 1024^3 the same as the engine, 1536^3 and 1280 x 1024 x 1024 slower)
+    if (M >= 64 && N >= 64 && K >= 512 && tiles_s >= 512 && tiles_s * 20 >= ceil_div(tiles_s, 512) * 512 * 19) return 2;
+    return 0;
+}
+
+// Runs the product through the direct-to-LDS kernel when the operands allow it and the shape is one it wins on. Returns
+// false when it did not take the problem (the caller goes on to the engine); `status` is the launch status otherwise.
+template <bool AKF, bool BKF, class E>
+static bool try_dma(const DmaOperand &a, const DmaOperand &b, const E &e, u32 M, u32 N, u32 K, u32 zdim, hipStream_t s, const char *what,
+                    int &status, bool *rowsum_done = nullptr) {
+    if (!dma_operand_ok(a, AKF) || !dma_operand_ok(b, BKF)) return false;
+    const int tile = choose_dma(M, N, K, zdim);
+    if (!tile) return false;
+    E e1 = e;
+    if constexpr (E::kRowSum) {
+        if (zdim != 1 || AKF) e1.a_rowsum = nullptr;  // the row sums ride along with one unbatched launch on a row-fast A only
+        if (rowsum_done) *rowsum_done = e1.a_rowsum != nullptr;
+    }
+    status = tile == 1 ? launch_igemm_dma<DmaLarge, AKF, BKF>(a, b, e1, M, N, K, zdim, s, what)
+                       : launch_igemm_dma<DmaSmall, AKF, BKF>(a, b, e1, M, N, K, zdim, s, what);
+    return true;
+}
+
 // Scratch bytes run_tiles asks for on a dense M x N result with contraction length K (0: the contraction is not cut).
 size_t gemm_scratch_bytes(u32 M, u32 N, u32 K, u32 zdim, bool one_launch_form) {
     if (one_launch_form && tiny_gemm_fits(M, N, K, zdim)) return 0;  // one launch, no partial results
+    // (the direct-to-LDS kernel never cuts the contraction: a problem it takes needs no scratch, one it leaves needs the engine's)
     const GemmChoice c = choose_tiles(M, N, K, zdim, true);
     SplitPlan sp;
     switch (c.tile) {
@@ -170,6 +207,8 @@ static int gemm_nn(const float *A, const float *B, float *C, u32 M, u32 N, u32 K
     RowMajorEpi e{C, col_bias, N, M * N, flags};
     e.row_bias = row_bias;
     if (K % 4 == 0 && N % 4 == 0 && aligned16(A) && aligned16(B)) {
+        int st = CRB_OK;
+        if (try_dma<true, false>(DmaOperand{A, M, K, 0, 0, 0}, DmaOperand{B, N, N, K * N, 0, 0}, e, M, N, K, batch, s, what, st)) return st;
         MatK<true> a{A, M, K, 0};
         MatR<true> b{B, N, N, K * N};
         return run_tiles(a, b, e, M, N, K, batch, s, what);
@@ -192,12 +231,16 @@ static int gemm_tn(const float *A, const float *B, float *C, u32 M, u32 N, u32 K
     if (M % 4 == 0 && N % 4 == 0 && aligned16(A) && aligned16(B)) {
         MatR<true> a{A, M, M, 0};
         MatR<true> b{B, N, N, K * N};
+        int st = CRB_OK;
+        const DmaOperand da{A, M, M, 0, 0, 0}, db{B, N, N, K * N, 0, 0};
         if (flags & EPI_ACCUM) {  // the dense layers' weight gradient
             RowMajorAccEpi ea;
             static_cast<RowMajorEpi &>(ea) = e;
             ea.a_rowsum = a_rowsum;
+            if (try_dma<false, false>(da, db, ea, M, N, K, batch, s, what, st, rowsum_done)) return st;
             return run_tiles(a, b, ea, M, N, K, batch, s, what, rowsum_done);
         }
+        if (try_dma<false, false>(da, db, e, M, N, K, batch, s, what, st)) return st;
         return run_tiles(a, b, e, M, N, K, batch, s, what);
     }
     MatR<false> a{A, M, M, 0};
@@ -211,6 +254,8 @@ static int gemm_nt(const float *A, const float *B, float *C, u32 M, u32 N, u32 K
         return launch_tiny_gemm(TinyGemmArgs{A, B, C, col_bias, nullptr, M, N, K, K, 1, 1, K, N, flags}, K, 0, 0, s, what);
     RowMajorEpi e{C, col_bias, N, 0, flags};
     if (K % 4 == 0 && aligned16(A) && aligned16(B)) {
+        int st = CRB_OK;
+        if (try_dma<true, true>(DmaOperand{A, M, K, 0, 0, 0}, DmaOperand{B, N, K, 0, 0, 0}, e, M, N, K, 1, s, what, st)) return st;
         MatK<true> a{A, M, K, 0};
         MatK<true> b{B, N, K, 0};
         return run_tiles(a, b, e, M, N, K, 1, s, what);
@@ -329,6 +374,9 @@ int crb_sgemm_nta(const float *A, const float *B, float *C, uint32_t M, uint32_t
     if (tiny_gemm_fits(M, N, KK, 1))  // the batch concatenated along the contraction
         return launch_tiny_gemm(TinyGemmArgs{A, B, C, nullptr, nullptr, M, N, KK, K, 1, 1, K, N, EPI_ACCUM}, K, M * K, N * K, s, "crb_sgemm_nta");
     if (K % 4 == 0 && aligned16(A) && aligned16(B)) {
+        int st = CRB_OK;
+        if (K % 32 == 0 && try_dma<true, true>(DmaOperand{A, M, K, 0, K, M * K}, DmaOperand{B, N, K, 0, K, N * K}, e, M, N, KK, 1, s, "crb_sgemm_nta", st))
+            return st;
         MatKCat<true> a{A, M, K, M * K, FastDiv(K)};
         MatKCat<true> b{B, N, K, N * K, FastDiv(K)};
         return run_tiles(a, b, e, M, N, KK, 1, s, "crb_sgemm_nta");

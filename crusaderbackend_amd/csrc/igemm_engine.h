@@ -429,6 +429,60 @@ __global__ void __launch_bounds__(Cfg::NTH, Cfg::OCC) igemm_kernel(AOp a, BOp b,
             }
         }
     };
+    // A whole tile takes stores that test and read nothing: bounds tests and a conditional read of the previous value in
+    // front of every store keep each store waiting for the one before it. Previous values (accumulating forms) and row
+    // biases are requested a block at a time, then the block's 16 stores follow one another.
+    const bool whole = row0 + BM <= d.M && col0 + BN <= d.N;
+    if constexpr (!BOp::kKFast && TN == 2 && Epi::kPairStore) {
+        if (whole && epi.pair_aligned(col0 + wave_n * Cfg::WTN)) {
+            const u32 col = col0 + wave_n * Cfg::WTN + j * 2;
+            const typename Epi::ColS c0 = epi.prep_col(col, d.N), c1 = epi.prep_col(col + 1, d.N);
+            const bool accumulates = epi.accumulates();
+            if constexpr (Epi::kPrefetchOld) {
+#pragma unroll
+                for (int r = 0; r < (kPair ? 32 : 16); ++r) oldv[r] = 0.f;
+            }
+#pragma unroll
+            for (int mi = 0; mi < TM; ++mi) {
+                fetch_row_bias(mi);
+                if (accumulates) fetch_old_block(mi, 0);
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int id = 8 * (r / 4) + 4 * h + (r % 4);
+                    const u32 row = row0 + wave_m * Cfg::WTM + (AOp::kKFast ? mi * 32 + id : id * TM + mi);
+                    epi.put2(row, c0, c1, acc[mi][0][r], acc[mi][1][r], rowb[r], Epi::kPrefetchOld ? oldv[r] : 0.f,
+                             Epi::kPrefetchOld ? oldv[kPair ? 16 + r : 0] : 0.f);
+                }
+            }
+            return;
+        }
+    } else {
+        if (whole) {
+            const bool accumulates = epi.accumulates();
+            if constexpr (Epi::kPrefetchOld) {
+                if (!have_old) {
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) oldv[r] = 0.f;
+                }
+            }
+#pragma unroll
+            for (int ni = 0; ni < TN; ++ni) {
+                const typename Epi::ColS cs = epi.prep_col(col0 + wave_n * Cfg::WTN + (BOp::kKFast ? ni * 32 + j : j * TN + ni), d.N);
+#pragma unroll
+                for (int mi = 0; mi < TM; ++mi) {
+                    fetch_row_bias(mi);
+                    if (accumulates && !have_old) fetch_old_block(mi, ni);  // have_old: the one block was requested in the main loop
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) {
+                        const int id = 8 * (r / 4) + 4 * h + (r % 4);
+                        const u32 row = row0 + wave_m * Cfg::WTM + (AOp::kKFast ? mi * 32 + id : id * TM + mi);
+                        epi.put(row, cs, acc[mi][ni][r], rowb[r], Epi::kPrefetchOld ? oldv[r] : 0.f);
+                    }
+                }
+            }
+            return;
+        }
+    }
     if constexpr (!BOp::kKFast && TN == 2 && Epi::kPairStore) {
         // row-fast B: a lane's two blocks are neighbouring columns, stored (and, accumulating, loaded) as one 8-byte access,
         // so that a store instruction writes whole 256-byte runs instead of every other float of them

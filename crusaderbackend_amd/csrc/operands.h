@@ -292,6 +292,16 @@ struct RowMajorEpi {
         return (flags & EPI_ACCUM) && row0 + bm <= M && col0 + bn <= N;
     }
     __device__ __forceinline__ const float *at(u32 row, u32 col) const { return C + size_t(row) * ld + col; }
+    __device__ __forceinline__ bool accumulates() const { return (flags & EPI_ACCUM) != 0u; }
+    // A store that tests and reads nothing: the caller has checked the bounds and hands in the previous value (0 when the
+    // form does not accumulate). Same order of additions as store().
+    __device__ __forceinline__ void put(u32 row, const ColS &c, float v, float rowb, float old) const {
+        v += c.bias;
+        v += rowb;
+        v += old;
+        if (flags & EPI_RELU) v = v > 0.0f ? v : 0.0f;
+        C[size_t(row) * ld + c.col] = v;
+    }
     __device__ __forceinline__ bool pair_aligned(u32 col) const { return ld % 2 == 0 && (reinterpret_cast<uintptr_t>(C + col) & 7u) == 0; }
     // The per-row bias of a lane's rows is loaded by the caller in one batch (row_bias_at) and handed in as `rowb`: a load
     // in front of every store would be a memory round trip per element.
@@ -308,6 +318,14 @@ struct RowMajorEpi {
             v += *p;
         if (flags & EPI_RELU) v = v > 0.0f ? v : 0.0f;
         *p = v;
+    }
+    // the same for two neighbouring columns at an 8-byte aligned address
+    __device__ __forceinline__ void put2(u32 row, const ColS &c0, const ColS &c1, float v0, float v1, float rowb, float old0, float old1) const {
+        v0 += c0.bias, v1 += c1.bias;
+        v0 += rowb, v1 += rowb;
+        v0 += old0, v1 += old1;
+        if (flags & EPI_RELU) v0 = v0 > 0.0f ? v0 : 0.0f, v1 = v1 > 0.0f ? v1 : 0.0f;
+        *reinterpret_cast<v2f *>(C + size_t(row) * ld + c0.col) = v2f{v0, v1};
     }
     // Two neighbouring columns of one row (c1.col == c0.col + 1) as one 8-byte access where the address allows it.
     static constexpr bool kPairStore = true;
@@ -374,6 +392,13 @@ struct NchwEpi {
         if (flags & EPI_RELU) v = v > 0.0f ? v : 0.0f;
         T[c.off + row * HW] = v;
     }
+    __device__ __forceinline__ bool accumulates() const { return false; }
+    __device__ __forceinline__ void put(u32 row, const ColS &c, float v, float rowb, float) const {  // bounds checked by the caller
+        v += rowb;
+        if (flags & EPI_RELU) v = v > 0.0f ? v : 0.0f;
+        T[c.off + row * HW] = v;
+    }
+    __device__ __forceinline__ void put2(u32, const ColS &, const ColS &, float, float, float, float, float) const {}
 };
 
 }  // namespace crb

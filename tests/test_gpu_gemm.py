@@ -154,6 +154,47 @@ def test_linear_relu_flag(dev):
     assert_close(to_np(Y), np.maximum(orc.linear(X, W, b), 0), IN, "linear+relu")
 
 
+# Shapes whose tile grid fills the chip in whole rounds and whose contraction is a multiple of 32 run on the kernel that
+# loads operand panels straight into LDS: 128 x 128 tiles (the first three), 64 x 64 tiles (the rest); ragged edge tiles included.
+DIRECT_TO_LDS = [(2048, 2048, 256), (2040, 2044, 288), (1024, 4096, 320), (512, 4096, 512), (508, 4092, 544), (32768, 64, 576)]
+
+
+@pytest.mark.parametrize("M,N,K", DIRECT_TO_LDS)
+def test_sgemm_forms_on_chip_filling_shapes(dev, M, N, K):
+    run_nn(dev, M, N, K, 1, seed=71)
+    run_nt(dev, M, N, K, seed=72)
+    run_tn(dev, M, N, K, 1, seed=73)
+    run_nta(dev, M, N, K // 2 if K % 64 == 0 else K, 2 if K % 64 == 0 else 1, seed=74)
+
+
+def test_sgemm_nn_batched_on_chip_filling_shape(dev):
+    run_nn(dev, 512, 1024, 256, 4, seed=75)
+    run_tn(dev, 512, 1024, 256, 4, seed=76)
+
+
+@pytest.mark.parametrize("batch,IN,OUT", [(2048, 256, 2048), (512, 512, 4096), (2040, 288, 2044), (2048, 1024, 2048)])
+def test_linear_family_on_chip_filling_shapes(dev, batch, IN, OUT):
+    """Bias, ReLU, accumulation and the bias gradient riding along, on the whole-tile and the edge-tile epilogues."""
+    capi, orc = _capi(), _oracle()
+    X, W, b = normal(1, batch, IN), normal(2, OUT, IN, std=(2.0 / IN) ** 0.5), normal(3, OUT)
+    dY = normal(4, batch, OUT)
+    Y = _empty(dev, batch, OUT)
+    capi.linear_fwd(to_dev(X, dev), to_dev(W, dev), to_dev(b, dev), Y, batch, IN, OUT)
+    ref = orc.linear(X, W, b, threads=8)
+    assert_close(to_np(Y), ref, IN, "linear")
+    capi.linear_fwd(to_dev(X, dev), to_dev(W, dev), to_dev(b, dev), Y, batch, IN, OUT, flags=capi.CRB_FLAG_RELU)
+    assert_close(to_np(Y), np.maximum(ref, 0), IN, "linear+relu")
+    dX = _empty(dev, batch, IN)
+    capi.linear_dgrad(to_dev(dY, dev), to_dev(W, dev), dX, batch, IN, OUT)
+    assert_close(to_np(dX), orc.linearXGrad(dY, W, threads=8), OUT, "linearXGrad")
+    dW0, dB0 = normal(5, OUT, IN), normal(6, OUT)
+    dW, dB = to_dev(dW0, dev), to_dev(dB0, dev)
+    capi.linear_wgrad(to_dev(dY, dev), to_dev(X, dev), dW, dB, batch, IN, OUT)
+    rW, rB = orc.linearParamGrad(dY, X, dW0, dB0, threads=8)
+    assert_close(to_np(dW), rW, batch, "linearParamGrad dW")
+    assert_close(to_np(dB), rB, batch, "linearParamGrad dB")
+
+
 def test_error_paths(dev):
     import torch
     capi = _capi()
@@ -267,7 +308,7 @@ def test_dense_sweep_configuration_full_size(dev):
     run_nn(dev, 32768, 64, 576, 1, seed=9)
 
 
-@pytest.mark.parametrize("M,N,K", [(128, 128, 64), (260, 132, 516), (64, 1024, 2048)])
+@pytest.mark.parametrize("M,N,K", [(128, 128, 64), (260, 132, 516), (64, 1024, 2048), (2048, 2048, 256)])
 def test_gemm_operands_aligned_to_4_bytes_only(dev, M, N, K):
     """Every operand one float past a 16-byte boundary, sizes that would otherwise take the 16-byte-load paths."""
     import torch
