@@ -114,18 +114,34 @@ static int run_tiles(const AOp &a, const BOp &b, const E &e, u32 M, u32 N, u32 K
 // ---- products of plain dense matrices on the direct-to-LDS kernel (igemm_dma.h) ---------------------------------------------
 // Taken when the contraction is a multiple of 32, the operands are 16-byte friendly and the tile grid fills the chip in
 // whole rounds; everything else stays on the register-staged engine. Returns 0: not taken; 1: 128 x 128 tiles; 2: 64 x 64.
-static int choose_dma(u32 M, u32 N, u32 K, u32 zdim) {
-    if (K % 32 || K < 256) return 0;  // whole 32-deep slabs; a short contraction is mostly prologue and epilogue
+struct DmaChoice {
+    int tile;    // 0: not taken; 1: 128 x 128 tiles; 2: 64 x 64
+    u32 splits;  // > 1: the contraction is cut into this many slices (dense, unbatched results only)
+};
+static DmaChoice choose_dma(u32 M, u32 N, u32 K, u32 zdim) {
+    if (K % 32 || K < 256) return {0, 1};  // whole 32-deep slabs; a short contraction is mostly prologue and epilogue
     const uint64_t tiles_l = uint64_t(ceil_div(M, 128)) * ceil_div(N, 128) * zdim;
     const uint64_t tiles_s = uint64_t(ceil_div(M, 64)) * ceil_div(N, 64) * zdim;
     // One 128 x 128 tile per CU already runs close to the MFMA rate, so the time goes by whole rounds of 256 tiles: taken
     // when the last round is (nearly) full. Measured against the register-staged engine, NN / NT / TN alike:
     // 2048^3 138 vs 150 us, 4096 x 4096 x 256 76 vs 83, 4096^3 1025 vs 1070; 3072^3 (2.25 rounds) 583 vs 494.
-    if (M >= 128 && N >= 128 && tiles_l >= 256 && tiles_l * 10 >= ceil_div(tiles_l, 256) * 256 * 9) return 1;
+    if (M >= 128 && N >= 128 && tiles_l >= 256 && tiles_l * 10 >= ceil_div(tiles_l, 256) * 256 * 9) return {1, 1};
     // 64 x 64 tiles, two per CU: rounds of 512 (512 x 4096 x 1024 40.3 vs 42.8 us, 32768 x 64 x 576 25.3 vs 26.4;
     // 1024^3 the same as the engine, 1536^3 and 1280 x 1024 x 1024 slower)
-    if (M >= 64 && N >= 64 && K >= 512 && tiles_s >= 512 && tiles_s * 20 >= ceil_div(tiles_s, 512) * 512 * 19) return 2;
-    return 0;
+    if (M >= 64 && N >= 64 && K >= 512 && tiles_s >= 512 && tiles_s * 20 >= ceil_div(tiles_s, 512) * 512 * 19) return {2, 1};
+    // Few tiles and a long contraction: K is cut so that tiles x slices make one round (partial results to scratch, summed
+    // in fixed order by the split reduction). Measured against the engine's own split plans, M x N x K: 256 x 4096 x 4096
+    // 78 vs 85 us, 512 x 512 x 4096 26.4 vs 29.5, 128 x 2048 x 2048 15.6 vs 17.4, 256 x 1024 x 8192 43.9 vs 50.9; with fewer
+    // than 16 tiles the engine's deeper cuts win (128 x 128 x 8192: 10.5 vs 15.8).
+    if (zdim == 1 && K >= 1024) {
+        if (M >= 128 && N >= 128 && tiles_l >= 64 && tiles_l <= 128 && K / u32(256 / tiles_l) >= 1024) return {1, u32(256 / tiles_l)};
+        if (M >= 64 && N >= 64 && tiles_s >= 16 && tiles_s <= 128) {
+            u32 splits = u32(512 / tiles_s);
+            if (splits > 16) splits = 16;
+            if (K / splits >= 256) return {2, splits};
+        }
+    }
+    return {0, 1};
 }
 
 // Runs the product through the direct-to-LDS kernel when the operands allow it and the shape is one it wins on. Returns
@@ -133,23 +149,44 @@ static int choose_dma(u32 M, u32 N, u32 K, u32 zdim) {
 template <bool AKF, bool BKF, class E>
 static bool try_dma(const DmaOperand &a, const DmaOperand &b, const E &e, u32 M, u32 N, u32 K, u32 zdim, hipStream_t s, const char *what,
                     int &status, bool *rowsum_done = nullptr) {
-    if (!dma_operand_ok(a, AKF) || !dma_operand_ok(b, BKF)) return false;
-    const int tile = choose_dma(M, N, K, zdim);
-    if (!tile) return false;
+    if (K % 32 || !dma_operand_ok(a, AKF) || !dma_operand_ok(b, BKF)) return false;
+    const DmaChoice c = choose_dma(M, N, K, zdim);
+    if (!c.tile) return false;
+    if (c.splits > 1) {
+        if (zdim != 1 || e.ld != N || a.cat_k || b.cat_k) return false;
+        const u32 k_per_z = ceil_div(ceil_div(K, c.splits), 32u) * 32u, splits = ceil_div(K, k_per_z);
+        float *ws = nullptr;
+        if ((status = scratch_get(size_t(splits) * M * N * sizeof(float), s, what, &ws))) return true;
+        RowMajorEpi pe{ws, nullptr, N, M * N, 0u};
+        status = c.tile == 1 ? launch_igemm_dma<DmaLarge, AKF, BKF>(a, b, pe, M, N, K, splits, k_per_z, s, what)
+                             : launch_igemm_dma<DmaSmall, AKF, BKF>(a, b, pe, M, N, K, splits, k_per_z, s, what);
+        if (status) return true;
+        status = e.row_bias ? launch_splitk_reduce(ws, e.C, M * N, splits, ReduceEpi{e.row_bias, N, M, e.flags}, s, what)
+                            : launch_splitk_reduce(ws, e.C, M * N, splits, ReduceEpi{e.col_bias, 1u << e.col_bias_shift, N >> e.col_bias_shift, e.flags}, s, what);
+        return true;
+    }
     E e1 = e;
     if constexpr (E::kRowSum) {
         if (zdim != 1 || AKF) e1.a_rowsum = nullptr;  // the row sums ride along with one unbatched launch on a row-fast A only
         if (rowsum_done) *rowsum_done = e1.a_rowsum != nullptr;
     }
-    status = tile == 1 ? launch_igemm_dma<DmaLarge, AKF, BKF>(a, b, e1, M, N, K, zdim, s, what)
-                       : launch_igemm_dma<DmaSmall, AKF, BKF>(a, b, e1, M, N, K, zdim, s, what);
+    status = c.tile == 1 ? launch_igemm_dma<DmaLarge, AKF, BKF>(a, b, e1, M, N, K, zdim, 0, s, what)
+                         : launch_igemm_dma<DmaSmall, AKF, BKF>(a, b, e1, M, N, K, zdim, 0, s, what);
     return true;
 }
 
 // Scratch bytes run_tiles asks for on a dense M x N result with contraction length K (0: the contraction is not cut).
 size_t gemm_scratch_bytes(u32 M, u32 N, u32 K, u32 zdim, bool one_launch_form) {
     if (one_launch_form && tiny_gemm_fits(M, N, K, zdim)) return 0;  // one launch, no partial results
-    // (the direct-to-LDS kernel never cuts the contraction: a problem it takes needs no scratch, one it leaves needs the engine's)
+    // the direct-to-LDS kernel needs friendly operands, which a size query cannot see: the larger of its need and the engine's
+    size_t dma_need = 0;
+    if (one_launch_form) {  // (callers that name the tiled engine directly never take the direct-to-LDS kernel)
+        const DmaChoice dc = choose_dma(M, N, K, zdim);
+        if (dc.tile && dc.splits > 1) {
+            const u32 k_per_z = ceil_div(ceil_div(K, dc.splits), 32u) * 32u;
+            dma_need = size_t(ceil_div(K, k_per_z)) * M * N * sizeof(float);
+        }
+    }
     const GemmChoice c = choose_tiles(M, N, K, zdim, true);
     SplitPlan sp;
     switch (c.tile) {
@@ -159,7 +196,8 @@ size_t gemm_scratch_bytes(u32 M, u32 N, u32 K, u32 zdim, bool one_launch_form) {
         case TILE_SMALL_AHEAD: sp = split_for<CfgSmallAhead>(M, N, K, zdim, c.want_splits, true); break;
         default: sp = split_for<CfgSmall>(M, N, K, zdim, c.want_splits, true); break;
     }
-    return sp.splits > 1 ? size_t(sp.splits) * M * N * sizeof(float) : 0;
+    const size_t eng = sp.splits > 1 ? size_t(sp.splits) * M * N * sizeof(float) : 0;
+    return eng > dma_need ? eng : dma_need;
 }
 
 static int check_dims(const char *what, u32 M, u32 N, u32 K, u32 batch) {

@@ -32,7 +32,8 @@ struct DmaOperand {
 
 struct DmaDims {
     u32 M, N, K;
-    u32 tiles_m, tiles_n;  // blockIdx.z is the batch index
+    u32 tiles_m, tiles_n;
+    u32 k_per_z;  // 0: blockIdx.z is a batch index; otherwise it names a slice of the contraction, this many long (multiple of 32)
 };
 
 template <int BM_, int BN_, int WM_, int WN_, int S_, int OCC_>
@@ -64,8 +65,13 @@ __global__ void __launch_bounds__(kThreads, Cfg::OCC) igemm_dma_kernel(DmaOperan
     u32 tm, tn;
     swizzled_tile(blockIdx.x, d.tiles_m, d.tiles_n, tm, tn);
     const u32 z = blockIdx.z;
-    const u32 kbeg = 0, kend = d.K;
-    a.base += size_t(z) * a.zstride, b.base += size_t(z) * b.zstride;
+    u32 kbeg = 0, kend = d.K;
+    if (d.k_per_z) {
+        kbeg = z * d.k_per_z;
+        kend = kbeg + d.k_per_z < d.K ? kbeg + d.k_per_z : d.K;
+    } else {
+        a.base += size_t(z) * a.zstride, b.base += size_t(z) * b.zstride;
+    }
     epi.bind(z);
 
     const u32 t = threadIdx.x, lane = t & 63, wave = t >> 6;
@@ -244,11 +250,12 @@ inline bool dma_operand_ok(const DmaOperand &op, bool kfast) {
 }
 
 template <class Cfg, bool AKF, bool BKF, class Epi>
-inline int launch_igemm_dma(const DmaOperand &a, const DmaOperand &b, const Epi &e, u32 M, u32 N, u32 K, u32 zdim,
+inline int launch_igemm_dma(const DmaOperand &a, const DmaOperand &b, const Epi &e, u32 M, u32 N, u32 K, u32 zdim, u32 k_per_z,
                             hipStream_t s, const char *what) {
     DmaDims d;
     d.M = M, d.N = N, d.K = K;
     d.tiles_m = ceil_div(M, u32(Cfg::BM)), d.tiles_n = ceil_div(N, u32(Cfg::BN));
+    d.k_per_z = k_per_z;
     const uint64_t tiles = uint64_t(d.tiles_m) * d.tiles_n;
     if (tiles > 0x7fffffffull || zdim > 65535u) return fail(CRB_EINVAL_SHAPE, "%s: launch grid too large", what);
     hipLaunchKernelGGL((igemm_dma_kernel<Cfg, AKF, BKF, Epi>), dim3(u32(tiles), 1, zdim), dim3(kThreads), 0, s, a, b, e, d);

@@ -214,6 +214,31 @@ def test_split_k_paths(dev, M, N, K):
     run_nt(dev, M, N, K, seed=43)
 
 
+@pytest.mark.parametrize("M,N,K", [(256, 2048, 2048), (512, 512, 4096), (128, 2048, 2048), (250, 1020, 2048), (128, 512, 8192)])
+def test_split_k_on_the_direct_to_lds_kernel(dev, M, N, K):
+    """Few tiles, contraction a multiple of 32: slices of K on the kernel that loads straight into LDS (128-wide and 64-wide tiles,
+    ragged edges), every form, and the dense-layer epilogues (bias, ReLU, accumulate with the bias gradient) behind the slice sum."""
+    run_nn(dev, M, N, K, 1, seed=45)
+    run_tn(dev, M, N, K, 1, seed=46)
+    run_nt(dev, M, N, K, seed=47)
+    capi, orc = _capi(), _oracle()
+    X, W, b = normal(1, M, K), normal(2, N, K, std=(2.0 / K) ** 0.5), normal(3, N)
+    Y = _empty(dev, M, N)
+    capi.linear_fwd(to_dev(X, dev), to_dev(W, dev), to_dev(b, dev), Y, M, K, N, flags=capi.CRB_FLAG_RELU)
+    assert_close(to_np(Y), np.maximum(orc.linear(X, W, b, threads=8), 0), K, "linear + bias + relu behind the slice sum")
+    Y2 = _empty(dev, M, N)
+    capi.linear_fwd(to_dev(X, dev), to_dev(W, dev), to_dev(b, dev), Y2, M, K, N, flags=capi.CRB_FLAG_RELU)
+    assert np.array_equal(to_np(Y), to_np(Y2)), "bit-reproducible"
+    # weight gradient dW (M x N) += dY^T (K x M) * X (K x N), dB += column sums of dY: batch = K
+    dY, Xb = normal(4, K, M), normal(5, K, N)
+    dW0, dB0 = normal(6, M, N), normal(7, M)
+    dW, dB = to_dev(dW0, dev), to_dev(dB0, dev)
+    capi.linear_wgrad(to_dev(dY, dev), to_dev(Xb, dev), dW, dB, K, N, M)
+    rW, rB = orc.linearParamGrad(dY, Xb, dW0, dB0, threads=8)
+    assert_close(to_np(dW), rW, K, "linearParamGrad dW behind the slice sum")
+    assert_close(to_np(dB), rB, K, "linearParamGrad dB")
+
+
 def test_split_k_nta_small_output_and_bias_epilogue(dev):
     run_nta(dev, 48, 24, 1024, 64, seed=44)
     capi, orc = _capi(), _oracle()
