@@ -115,7 +115,7 @@ static int run_tiles(const AOp &a, const BOp &b, const E &e, u32 M, u32 N, u32 K
 // Taken when the contraction is a multiple of 32, the operands are 16-byte friendly and the tile grid fills the chip in
 // whole rounds; everything else stays on the register-staged engine. Returns 0: not taken; 1: 128 x 128 tiles; 2: 64 x 64.
 struct DmaChoice {
-    int tile;    // 0: not taken; 1: 128 x 128 tiles; 2: 64 x 64
+    int tile;    // 0: not taken; 1: 128 x 128 tiles; 2: 64 x 64; 3: 64 x 64 as eight waves
     u32 splits;  // > 1: the contraction is cut into this many slices (dense, unbatched results only)
 };
 static DmaChoice choose_dma(u32 M, u32 N, u32 K, u32 zdim) {
@@ -129,6 +129,10 @@ static DmaChoice choose_dma(u32 M, u32 N, u32 K, u32 zdim) {
     // 64 x 64 tiles, two per CU: rounds of 512 (512 x 4096 x 1024 40.3 vs 42.8 us, 32768 x 64 x 576 25.3 vs 26.4;
     // 1024^3 the same as the engine, 1536^3 and 1280 x 1024 x 1024 slower)
     if (M >= 64 && N >= 64 && K >= 512 && tiles_s >= 512 && tiles_s * 20 >= ceil_div(tiles_s, 512) * 512 * 19) return {2, 1};
+    // At most one 64 x 64 tile per CU: the same tile as an eight-wave workgroup, two waves per SIMD (1024^3 24.0-24.8 us
+    // against the engine's eight-wave tiles at 24.1-25.9, 1024 x 1024 x 2048 44.6-46.1 against 45.6-47.5, 896^3 21.4-21.8
+    // against 21.4-22.8); longer contractions are better cut (below)
+    if (M >= 64 && N >= 64 && K >= 512 && K <= 2048 && tiles_s >= 160 && tiles_s <= 256) return {3, 1};
     // Few tiles and a long contraction: K is cut so that tiles x slices make one round (partial results to scratch, summed
     // in fixed order by the split reduction). Measured against the engine's own split plans, M x N x K: 256 x 4096 x 4096
     // 78 vs 85 us, 512 x 512 x 4096 26.4 vs 29.5, 128 x 2048 x 2048 15.6 vs 17.4, 256 x 1024 x 8192 43.9 vs 50.9; with fewer
@@ -158,8 +162,9 @@ static bool try_dma(const DmaOperand &a, const DmaOperand &b, const E &e, u32 M,
         float *ws = nullptr;
         if ((status = scratch_get(size_t(splits) * M * N * sizeof(float), s, what, &ws))) return true;
         RowMajorEpi pe{ws, nullptr, N, M * N, 0u};
-        status = c.tile == 1 ? launch_igemm_dma<DmaLarge, AKF, BKF>(a, b, pe, M, N, K, splits, k_per_z, s, what)
-                             : launch_igemm_dma<DmaSmall, AKF, BKF>(a, b, pe, M, N, K, splits, k_per_z, s, what);
+        status = c.tile == 1   ? launch_igemm_dma<DmaLarge, AKF, BKF>(a, b, pe, M, N, K, splits, k_per_z, s, what)
+                 : c.tile == 2 ? launch_igemm_dma<DmaSmall, AKF, BKF>(a, b, pe, M, N, K, splits, k_per_z, s, what)
+                               : launch_igemm_dma<DmaSmall8, AKF, BKF>(a, b, pe, M, N, K, splits, k_per_z, s, what);
         if (status) return true;
         status = e.row_bias ? launch_splitk_reduce(ws, e.C, M * N, splits, ReduceEpi{e.row_bias, N, M, e.flags}, s, what)
                             : launch_splitk_reduce(ws, e.C, M * N, splits, ReduceEpi{e.col_bias, 1u << e.col_bias_shift, N >> e.col_bias_shift, e.flags}, s, what);
@@ -170,8 +175,9 @@ static bool try_dma(const DmaOperand &a, const DmaOperand &b, const E &e, u32 M,
         if (zdim != 1 || AKF) e1.a_rowsum = nullptr;  // the row sums ride along with one unbatched launch on a row-fast A only
         if (rowsum_done) *rowsum_done = e1.a_rowsum != nullptr;
     }
-    status = c.tile == 1 ? launch_igemm_dma<DmaLarge, AKF, BKF>(a, b, e1, M, N, K, zdim, 0, s, what)
-                         : launch_igemm_dma<DmaSmall, AKF, BKF>(a, b, e1, M, N, K, zdim, 0, s, what);
+    status = c.tile == 1   ? launch_igemm_dma<DmaLarge, AKF, BKF>(a, b, e1, M, N, K, zdim, 0, s, what)
+             : c.tile == 2 ? launch_igemm_dma<DmaSmall, AKF, BKF>(a, b, e1, M, N, K, zdim, 0, s, what)
+                           : launch_igemm_dma<DmaSmall8, AKF, BKF>(a, b, e1, M, N, K, zdim, 0, s, what);
     return true;
 }
 

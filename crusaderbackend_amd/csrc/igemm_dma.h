@@ -36,14 +36,18 @@ struct DmaDims {
     u32 k_per_z;  // 0: blockIdx.z is a batch index; otherwise it names a slice of the contraction, this many long (multiple of 32)
 };
 
-template <int BM_, int BN_, int WM_, int WN_, int S_, int OCC_>
+// KG_ = 2: an eight-wave workgroup; both groups of four waves own the whole tile and each multiplies half of every slab
+// (two waves per SIMD, so one wave's fragment reads hide behind the other's MFMAs even with one workgroup on the CU); the
+// second group's accumulators are added to the first's through LDS before the epilogue.
+template <int BM_, int BN_, int WM_, int WN_, int S_, int OCC_, int KG_ = 1>
 struct DmaCfg {
-    static constexpr int BM = BM_, BN = BN_, WM = WM_, WN = WN_, S = S_, OCC = OCC_, BK = 32;
+    static constexpr int BM = BM_, BN = BN_, WM = WM_, WN = WN_, S = S_, OCC = OCC_, BK = 32, KG = KG_, THREADS = 256 * KG_;
     static constexpr int WTM = BM / WM, WTN = BN / WN, TM = WTM / 32, TN = WTN / 32;
     static_assert(WM * WN == 4 && TM >= 1 && TN >= 1 && TM * 32 * WM == BM && TN * 32 * WN == BN, "tile shape");
     static constexpr int A_FLOATS = BM * BK, B_FLOATS = BK * BN, STAGE = A_FLOATS + B_FLOATS;
-    static constexpr int A_PW = A_FLOATS / 256 / 4, B_PW = B_FLOATS / 256 / 4;  // 1 KB load instructions per wave per slab
-    static_assert(A_FLOATS % 1024 == 0 && B_FLOATS % 1024 == 0, "whole load instructions per wave");
+    static constexpr int A_PW = A_FLOATS / THREADS / 4, B_PW = B_FLOATS / THREADS / 4;  // 1 KB load instructions per wave per slab
+    static_assert(A_FLOATS % (4 * THREADS) == 0 && B_FLOATS % (4 * THREADS) == 0 && (KG == 1 || KG == 2), "whole load instructions per wave");
+    static_assert(KG == 1 || 4 * TM * TN * 16 * 64 <= S * STAGE, "room to hand over the second group's accumulators");
     static constexpr int LPS = A_PW + B_PW;
     static_assert((S - 2) * LPS <= 63, "the counter wait must fit its field");
 };
@@ -57,7 +61,7 @@ __device__ __forceinline__ void dma_wait() {
 }
 
 template <class Cfg, bool AKF, bool BKF, class Epi>
-__global__ void __launch_bounds__(kThreads, Cfg::OCC) igemm_dma_kernel(DmaOperand a, DmaOperand b, Epi epi, DmaDims d) {
+__global__ void __launch_bounds__(Cfg::THREADS, Cfg::OCC) igemm_dma_kernel(DmaOperand a, DmaOperand b, Epi epi, DmaDims d) {
     constexpr int BM = Cfg::BM, BN = Cfg::BN, BK = Cfg::BK, S = Cfg::S, TM = Cfg::TM, TN = Cfg::TN;
     constexpr int A_PW = Cfg::A_PW, B_PW = Cfg::B_PW;
     __shared__ __attribute__((aligned(1024))) float smem[S * Cfg::STAGE];
@@ -74,8 +78,9 @@ __global__ void __launch_bounds__(kThreads, Cfg::OCC) igemm_dma_kernel(DmaOperan
     }
     epi.bind(z);
 
-    const u32 t = threadIdx.x, lane = t & 63, wave = t >> 6;
-    const int wave_m = wave / Cfg::WN, wave_n = wave % Cfg::WN;
+    const u32 t = threadIdx.x, lane = t & 63, wave = t >> 6;  // the loads are shared out over all waves
+    const u32 kgroup = wave >> 2;                              // which half of a slab this wave multiplies (KG == 2)
+    const int wave_m = (wave & 3) / Cfg::WN, wave_n = (wave & 3) % Cfg::WN;
     const u32 row0 = tm * BM, col0 = tn * BN;
 
     // ---- where this lane's load instructions fetch from (slab offset added per slab) ---------------------------------
@@ -147,7 +152,8 @@ __global__ void __launch_bounds__(kThreads, Cfg::OCC) igemm_dma_kernel(DmaOperan
             }
         }
 #pragma unroll
-        for (int g = 0; g < BK / 8; ++g) {
+        for (int gi = 0; gi < BK / 8 / Cfg::KG; ++gi) {
+            const int g = Cfg::KG == 1 ? gi : int(kgroup) * (BK / 8 / Cfg::KG) + gi;
             float fa[4][TM], fb[4][TN];
 #pragma unroll
             for (int mi = 0; mi < TM; ++mi) {
@@ -183,6 +189,28 @@ __global__ void __launch_bounds__(kThreads, Cfg::OCC) igemm_dma_kernel(DmaOperan
 
     if constexpr (Epi::kRowSum && !AKF) {
         if (do_rowsum && row0 + t < d.M) epi.a_rowsum[row0 + t] += rowsum;
+    }
+    if constexpr (Cfg::KG == 2) {
+        // the second group hands its accumulators over through the ring (idle now: the barrier says every wave has read the
+        // last slab), the first adds them to its own and runs the epilogue alone
+        constexpr int PER_WAVE = TM * TN * 16 * 64;
+        lds_barrier();
+        if (kgroup == 1) {
+#pragma unroll
+            for (int mi = 0; mi < TM; ++mi)
+#pragma unroll
+                for (int ni = 0; ni < TN; ++ni)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) smem[(wave & 3) * PER_WAVE + ((mi * TN + ni) * 16 + r) * 64 + lane] = acc[mi][ni][r];
+        }
+        lds_barrier();
+        if (kgroup == 1) return;
+#pragma unroll
+        for (int mi = 0; mi < TM; ++mi)
+#pragma unroll
+            for (int ni = 0; ni < TN; ++ni)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) acc[mi][ni][r] += smem[wave * PER_WAVE + ((mi * TN + ni) * 16 + r) * 64 + lane];
     }
     // ---- epilogue: accumulator register r of lane l is D[8*(r/4) + 4*(l/32) + r%4][l%32] of its 32 x 32 block -------------
     if (row0 + BM <= d.M && col0 + BN <= d.N) {
@@ -241,6 +269,7 @@ __global__ void __launch_bounds__(kThreads, Cfg::OCC) igemm_dma_kernel(DmaOperan
 
 typedef DmaCfg<128, 128, 2, 2, 2, 2> DmaLarge;  // 64 KB of LDS: two workgroups per CU, one slab in flight each
 typedef DmaCfg<64, 64, 2, 2, 4, 2> DmaSmall;    // 64 KB of LDS: two workgroups per CU, three slabs in flight each
+typedef DmaCfg<64, 64, 2, 2, 4, 2, 2> DmaSmall8;  // the same tile as eight waves, for grids of at most one tile per CU
 
 // Whether an operand can be loaded this way: 16-byte aligned rows (or k rows) and, row-fast, whole 4-float chunks.
 inline bool dma_operand_ok(const DmaOperand &op, bool kfast) {
@@ -258,7 +287,7 @@ inline int launch_igemm_dma(const DmaOperand &a, const DmaOperand &b, const Epi 
     d.k_per_z = k_per_z;
     const uint64_t tiles = uint64_t(d.tiles_m) * d.tiles_n;
     if (tiles > 0x7fffffffull || zdim > 65535u) return fail(CRB_EINVAL_SHAPE, "%s: launch grid too large", what);
-    hipLaunchKernelGGL((igemm_dma_kernel<Cfg, AKF, BKF, Epi>), dim3(u32(tiles), 1, zdim), dim3(kThreads), 0, s, a, b, e, d);
+    hipLaunchKernelGGL((igemm_dma_kernel<Cfg, AKF, BKF, Epi>), dim3(u32(tiles), 1, zdim), dim3(Cfg::THREADS), 0, s, a, b, e, d);
     return check_launch(what);
 }
 

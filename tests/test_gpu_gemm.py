@@ -155,8 +155,10 @@ def test_linear_relu_flag(dev):
 
 
 # Shapes whose tile grid fills the chip in whole rounds and whose contraction is a multiple of 32 run on the kernel that
-# loads operand panels straight into LDS: 128 x 128 tiles (the first three), 64 x 64 tiles (the rest); ragged edge tiles included.
-DIRECT_TO_LDS = [(2048, 2048, 256), (2040, 2044, 288), (1024, 4096, 320), (512, 4096, 512), (508, 4092, 544), (32768, 64, 576)]
+# loads operand panels straight into LDS: 128 x 128 tiles (the first three), 64 x 64 tiles (the next three), the latter as
+# eight-wave workgroups when there is at most one per CU (the last two); ragged edge tiles included.
+DIRECT_TO_LDS = [(2048, 2048, 256), (2040, 2044, 288), (1024, 4096, 320), (512, 4096, 512), (508, 4092, 544), (32768, 64, 576),
+                 (1000, 1020, 544), (768, 1024, 1024)]
 
 
 @pytest.mark.parametrize("M,N,K", DIRECT_TO_LDS)
