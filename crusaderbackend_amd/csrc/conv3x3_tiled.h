@@ -1,0 +1,280 @@
+// 3x3 / pad 1 / stride 1 convolution (forward and data gradient) for gfx950 on images of ANY extent: the layers whose width is
+// not one of the widths the width-specialised direct kernels are built for (56, 28, 14, 7, 24, 12 ...).
+//
+// The output image is cut into TH x TW pixel tiles (ragged at the right and bottom edges). A 256-thread workgroup owns one
+// tile of one image and OCT output channels and walks the input channels in chunks of CI: per chunk the (TH + 2) x (TW + 2)
+// input window (halo included, zero outside the image) of CI channels and the matching OCT x CI x 9 filter slice are staged
+// in double-buffered LDS (global -> registers -> LDS, the next chunk's loads in flight while this one is multiplied) and
+// fed to v_mfma_f32_32x32x2_f32 with the filters on the row operand and the pixels on the column operand.
+//
+// Contraction order inside a chunk is the filters' own memory order, k = channel * 9 + tap, so a filter row is a straight
+// copy of global memory (16-byte loads and LDS stores when the tensor allows). An MFMA consumes two k per step, one per lane
+// half; lane half h takes k = s + h * KC / 2 (KC = 9 CI), i.e. the same tap of channel c + CI / 2: both halves share every
+// compile-time address offset, the half is a per-lane base. Filter fragments are read four steps at a time (one 16-byte
+// LDS read, row stride 4 mod 32 floats ... 28 mod 32: eight consecutive rows cover all banks), pixel fragments one float per
+// step at `lane base + immediate` (the tap shift and the channel plane are the immediate).
+//
+// v_mfma_f32_32x32x2_f32 (wave64, lane l): A[i = l%32][k = l/32], B[k = l/32][j = l%32], accumulator register r =
+// D[i = 8*(r/4) + 4*(l/32) + r%4][j = l%32]: i = output channel, j = pixel, so the 32 lanes of a half-wave store 32
+// consecutive pixels (TW of them per image row) of one output channel per instruction.
+//
+// Data gradient: the same computation on dY with the filter's channel roles swapped and its taps mirrored
+// (dX(y, x) = sum dY(y + 1 - fh, x + 1 - fw) W[oc][ic][fh][fw]): only the filter staging and the immediates differ.
+#pragma once
+#include <type_traits>
+
+#include "igemm_engine.h"
+
+namespace crb {
+
+template <int TH_, int TW_, int OCT_, int WP_, int CI_, bool DGRAD_, int OCC_>
+struct TiledCfg {
+    static constexpr int TH = TH_, TW = TW_, OCT = OCT_, WP = WP_, WO = 4 / WP_, CI = CI_, OCC = OCC_;
+    static constexpr bool DGRAD = DGRAD_;
+    static constexpr int PIX = TH * TW, NPB = PIX / 32, NOB = OCT / 32;  // 32-pixel and 32-channel MFMA blocks
+    static constexpr int PB = NPB / WP, OB = NOB / WO;                  // blocks per wave
+    static constexpr int RB = 32 / TW;                                  // image rows per pixel block
+    static constexpr int XR = TH + 2, XC = TW + 2, XS = TW + 4;          // staged rows, columns; LDS row stride
+    static constexpr int XP = XR * XS;                                  // channel plane stride
+    static constexpr int X_SIZE = CI * XP;
+    static constexpr int KC = CI * 9, KH = KC / 2;                      // contraction per chunk, per lane half
+    static constexpr int WSTR = KC + 4;                                 // filter row stride: 12 or 20 mod 32 for CI = 8 / 16
+    static constexpr int W_SIZE = OCT * WSTR;
+    static constexpr int SMEM_FLOATS = 2 * (X_SIZE + W_SIZE);
+    static_assert(TW == 8 || TW == 16 || TW == 32, "tile width");
+    static_assert(WP * WO == 4 && NPB % WP == 0 && NOB % WO == 0 && PB >= 1 && OB >= 1, "wave tiling");
+    static_assert(PIX % 32 == 0 && OCT % 32 == 0 && (TH % RB) == 0, "whole MFMA blocks");
+    static_assert(CI % 8 == 0 && KH % 4 == 0 && (WSTR % 8) == 4, "16-byte filter fragments, conflict-free rows");
+};
+
+struct TiledArgs {
+    const float *Wt;    // filters, OC x IC x 3 x 3 of the forward convolution
+    const float *X;     // input of this pass  (forward: X, data gradient: dY), N x C_IN x H x W
+    float *Y;           // output of this pass (forward: Y, data gradient: dX), N x C_OUT x H x W
+    const float *bias;  // per output channel or nullptr
+    u32 C_IN, C_OUT, H, W;
+    u32 tiles_x, tiles_per_img, oc_tiles, tiles_total;  // tiles_total = N * tiles_per_img
+    u32 relu;
+};
+
+// WVEC (forward only): filter rows are staged with 16-byte loads (C_IN % 4 == 0 and a 16-byte aligned tensor).
+template <class Cfg, bool WVEC>
+__global__ void __launch_bounds__(kThreads, Cfg::OCC) conv3x3_tiled_kernel(TiledArgs a) {
+    constexpr int TH = Cfg::TH, TW = Cfg::TW, OCT = Cfg::OCT, CI = Cfg::CI, PB = Cfg::PB, OB = Cfg::OB;
+    constexpr int XR = Cfg::XR, XC = Cfg::XC, XS = Cfg::XS, XP = Cfg::XP, KC = Cfg::KC, KH = Cfg::KH, WSTR = Cfg::WSTR;
+    __shared__ __attribute__((aligned(16))) float smem[Cfg::SMEM_FLOATS];
+    float(*sX)[Cfg::X_SIZE] = reinterpret_cast<float(*)[Cfg::X_SIZE]>(smem);
+    float(*sW)[Cfg::W_SIZE] = reinterpret_cast<float(*)[Cfg::W_SIZE]>(smem + 2 * Cfg::X_SIZE);
+
+    const u32 t = threadIdx.x, bid = blockIdx.x;
+    // Workgroups are dealt round-robin to the 8 XCDs: the oc_tiles workgroups that read the same input window get ids 8
+    // apart, land on the same XCD back to back and share the window through its L2.
+    const u32 xcd = bid % kXcds, slot = bid / kXcds;
+    const u32 oct = slot % a.oc_tiles, rest = (slot / a.oc_tiles) * kXcds + xcd;
+    if (rest >= a.tiles_total) return;
+    const u32 n = rest / a.tiles_per_img, tile = rest % a.tiles_per_img;
+    const int y0 = int(tile / a.tiles_x) * TH, x0 = int(tile % a.tiles_x) * TW;
+    const u32 oc0 = oct * OCT;
+    const u32 HW = a.H * a.W;
+
+    // ---- staging: thread t owns items t, t + 256, ... of the window (channel, row, column) and of the filter slice --------
+    // An item's byte offset from the chunk's (uniform) base address does not depend on the chunk: computed once. Loads are
+    // issued whatever the item is worth (offset 0 when it is nothing) and the value is judged when it goes to LDS: with a
+    // select behind every load, each load would wait for the one before it.
+    constexpr int XQ = CI * XR * XC, XNP = (XQ + kThreads - 1) / kThreads;
+    constexpr int WITEMS = WVEC ? OCT * KC / 4 : OCT * KC, WNP = (WITEMS + kThreads - 1) / kThreads;
+    constexpr u32 kNone = ~0u;
+    float xreg[XNP];
+    u32 xoff[XNP], woff[WNP];
+    typedef typename std::conditional<WVEC, v4f, float>::type WItem;
+    WItem wreg[WNP];
+    const char *xin = reinterpret_cast<const char *>(a.X + size_t(n) * a.C_IN * HW);
+#pragma unroll
+    for (int i = 0; i < XNP; ++i) {
+        const u32 e = t + i * kThreads;
+        const u32 c = e / (XR * XC), lr = (e / XC) % XR, lc = e % XC;
+        const int y = y0 - 1 + int(lr), x = x0 - 1 + int(lc);
+        const bool ok = (XQ % kThreads == 0 || e < XQ) && y >= 0 && y < int(a.H) && x >= 0 && x < int(a.W);
+        xoff[i] = ok ? (c * HW + u32(y) * a.W + u32(x)) * 4u : kNone;
+    }
+    // filter slice of chunk c0: LDS row j (output channel oc0 + j) holds k = c * 9 + tap for the chunk's channels c.
+    // forward: row j is KC consecutive floats of Wt[oc0 + j] from channel c0 on; data gradient: the OCT * 9 consecutive floats
+    // Wt[c0 + c][oc0 ..] hold (row j, tap) for contraction channel c.
+#pragma unroll
+    for (int i = 0; i < WNP; ++i) {
+        const u32 e = t + i * kThreads;
+        bool ok = WITEMS % kThreads == 0 || e < WITEMS;
+        u32 off;
+        if constexpr (Cfg::DGRAD) {
+            const u32 c = e / (OCT * 9), f = e % (OCT * 9);
+            ok = ok && oc0 * 9 + f < a.C_OUT * 9;
+            off = c * a.C_OUT * 9 + f;
+        } else if constexpr (WVEC) {
+            const u32 j = e / (KC / 4), q = e % (KC / 4);
+            ok = ok && oc0 + j < a.C_OUT;
+            off = j * a.C_IN * 9 + 4 * q;
+        } else {
+            const u32 j = e / KC, k = e % KC;
+            ok = ok && oc0 + j < a.C_OUT;
+            off = j * a.C_IN * 9 + k;
+        }
+        woff[i] = ok ? off * 4u : kNone;
+    }
+    // whether item e of the filter slice lies inside the tensor's channels in chunk c0 (ragged last chunk)
+    auto w_in_chunk = [&](u32 e, u32 c0) -> bool {
+        if constexpr (Cfg::DGRAD) return c0 + e / (OCT * 9) < a.C_IN;
+        else if constexpr (WVEC) return c0 * 9 + 4 * (e % (KC / 4)) < a.C_IN * 9;  // a 16-byte item never straddles the end: C_IN % 4 == 0
+        else return c0 * 9 + e % KC < a.C_IN * 9;
+    };
+    auto fetch = [&](u32 c0) {
+        const char *xc = xin + size_t(c0) * HW * 4;
+        const char *wc = reinterpret_cast<const char *>(Cfg::DGRAD ? a.Wt + (size_t(c0) * a.C_OUT + oc0) * 9 : a.Wt + (size_t(oc0) * a.C_IN + c0) * 9);
+#pragma unroll
+        for (int i = 0; i < XNP; ++i) {
+            const bool ok = xoff[i] != kNone && c0 + (t + i * kThreads) / (XR * XC) < a.C_IN;
+            xreg[i] = *reinterpret_cast<const float *>(xc + (ok ? xoff[i] : 0u));
+        }
+#pragma unroll
+        for (int i = 0; i < WNP; ++i) {
+            const bool ok = woff[i] != kNone && w_in_chunk(t + i * kThreads, c0);
+            wreg[i] = *reinterpret_cast<const WItem *>(wc + (ok ? woff[i] : 0u));
+        }
+    };
+    auto commit = [&](float *dx, float *dw, u32 c0) {
+#pragma unroll
+        for (int i = 0; i < XNP; ++i) {
+            const u32 e = t + i * kThreads, c = e / (XR * XC);
+            const bool ok = xoff[i] != kNone && c0 + c < a.C_IN;
+            if (XQ % kThreads == 0 || e < XQ) dx[c * XP + ((e / XC) % XR) * XS + e % XC] = ok ? xreg[i] : 0.f;
+        }
+#pragma unroll
+        for (int i = 0; i < WNP; ++i) {
+            const u32 e = t + i * kThreads;
+            const bool ok = woff[i] != kNone && w_in_chunk(e, c0);
+            if (WITEMS % kThreads == 0 || e < WITEMS) {
+                if constexpr (Cfg::DGRAD) {
+                    const u32 c = e / (OCT * 9), f = e % (OCT * 9);
+                    dw[(f / 9) * WSTR + c * 9 + f % 9] = ok ? wreg[i] : 0.f;
+                } else if constexpr (WVEC) {
+                    *reinterpret_cast<v4f *>(dw + (e / (KC / 4)) * WSTR + 4 * (e % (KC / 4))) = ok ? wreg[i] : v4f{0.f, 0.f, 0.f, 0.f};
+                } else {
+                    dw[(e / KC) * WSTR + e % KC] = ok ? wreg[i] : 0.f;
+                }
+            }
+        }
+    };
+
+    // ---- per-lane fragment addressing ---------------------------------------------------------------------------------------
+    const int lane = t & 63, wave = t >> 6, j32 = lane & 31, h = lane >> 5;
+    const int wp = wave % Cfg::WP, wo = wave / Cfg::WP;
+    // this lane's pixel in the wave's first pixel block; block p is RB * p image rows further down
+    const int pix = wp * PB * 32 + j32, prow = pix / TW, pcol = pix % TW;
+    const int xbase = h * (CI / 2) * XP + prow * XS + pcol;
+    const int wbase = (wo * OB * 32 + j32) * WSTR + h * KH;
+
+    v16f acc[OB][PB];
+#pragma unroll
+    for (int o = 0; o < OB; ++o)
+#pragma unroll
+        for (int p = 0; p < PB; ++p)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[o][p][r] = 0.f;
+
+    // Fragments are read one group of four steps ahead of the MFMAs that consume them (two register sets; the scheduler is
+    // fenced so that it neither undoes the pipeline nor hoists every read of the chunk to its top).
+    auto compute = [&](const float *cx, const float *cw) {
+        const float *xfrag = cx + xbase, *wfrag = cw + wbase;
+        v4f wv[2][OB];
+        float xv[2][4][PB];
+        auto read_group = [&](int sq, int set) {
+#pragma unroll
+            for (int o = 0; o < OB; ++o) wv[set][o] = *reinterpret_cast<const v4f *>(wfrag + o * 32 * WSTR + 4 * sq);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const int s = 4 * sq + e, c = s / 9, tap = s % 9;
+                const int fh = Cfg::DGRAD ? 2 - tap / 3 : tap / 3, fw = Cfg::DGRAD ? 2 - tap % 3 : tap % 3;
+#pragma unroll
+                for (int p = 0; p < PB; ++p) xv[set][e][p] = xfrag[c * XP + (p * Cfg::RB + fh) * XS + fw];
+            }
+        };
+        read_group(0, 0);
+#pragma unroll
+        for (int sq = 0; sq < KH / 4; ++sq) {
+            if (sq + 1 < KH / 4) read_group(sq + 1, (sq + 1) & 1);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+#pragma unroll
+                for (int o = 0; o < OB; ++o)
+#pragma unroll
+                    for (int p = 0; p < PB; ++p)
+                        acc[o][p] = __builtin_amdgcn_mfma_f32_32x32x2f32(wv[sq & 1][o][e], xv[sq & 1][e][p], acc[o][p], 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+
+    // ---- main loop over input-channel chunks (double-buffered) -------------------------------------------------------------
+    const u32 nchunk = (a.C_IN + CI - 1) / CI;
+    fetch(0);
+    commit(sX[0], sW[0], 0);
+    __syncthreads();
+    for (u32 ch = 0; ch < nchunk; ++ch) {
+        const u32 b = ch & 1;
+        const bool more = ch + 1 < nchunk;
+        if (more) fetch((ch + 1) * CI);
+        compute(sX[b], sW[b]);
+        if (more) commit(sX[b ^ 1], sW[b ^ 1], (ch + 1) * CI);
+        __syncthreads();
+    }
+
+    // ---- epilogue: register r of block (o, p) is output channel ocb + 8*(r/4) + 4h + r%4 at this lane's pixel ----------------
+#pragma unroll
+    for (int o = 0; o < OB; ++o) {
+        const u32 ocb = oc0 + (wo * OB + o) * 32 + 4 * h;
+        float bv[16];
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const u32 oc = ocb + 8 * (r / 4) + (r % 4);
+            bv[r] = (a.bias && oc < a.C_OUT) ? a.bias[oc] : 0.f;  // requested together, ahead of the stores
+        }
+#pragma unroll
+        for (int p = 0; p < PB; ++p) {
+            const int y = y0 + prow + p * Cfg::RB, x = x0 + pcol;
+            const bool pok = y < int(a.H) && x < int(a.W);
+            float *dst = a.Y + size_t(n) * a.C_OUT * HW + size_t(pok ? y : 0) * a.W + (pok ? x : 0);
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const u32 oc = ocb + 8 * (r / 4) + (r % 4);
+                float v = acc[o][p][r] + bv[r];
+                if (a.relu) v = v > 0.f ? v : 0.f;
+                if (pok && oc < a.C_OUT) dst[size_t(oc) * HW] = v;
+            }
+        }
+    }
+}
+
+template <class Cfg>
+inline int launch_tiled(const float *Wt, const float *X, float *Y, const float *bias, u32 N, u32 C_IN, u32 C_OUT, u32 H, u32 W, u32 relu,
+                        hipStream_t s, const char *what) {
+    TiledArgs a;
+    a.Wt = Wt, a.X = X, a.Y = Y, a.bias = bias;
+    a.C_IN = C_IN, a.C_OUT = C_OUT, a.H = H, a.W = W;
+    a.tiles_x = ceil_div(W, u32(Cfg::TW));
+    a.tiles_per_img = a.tiles_x * ceil_div(H, u32(Cfg::TH));
+    a.oc_tiles = ceil_div(C_OUT, u32(Cfg::OCT));
+    const uint64_t tiles = uint64_t(N) * a.tiles_per_img;
+    const uint64_t wgs = uint64_t(ceil_div(u32(tiles > 0xffffffffull ? 0xffffffffu : tiles), kXcds)) * kXcds * a.oc_tiles;
+    if (tiles > 0x7fffffffull || wgs > 0x7fffffffull) return fail(CRB_EINVAL_SHAPE, "%s: launch grid too large", what);
+    a.tiles_total = u32(tiles);
+    a.relu = relu;
+    // an item's byte offset inside its image / inside the filter tensor is kept in 32 bits
+    if (uint64_t(C_IN) * H * W * 4 > 0xffffffffull || uint64_t(C_IN) * C_OUT * 36 > 0xffffffffull)
+        return fail(CRB_EINVAL_SHAPE, "%s: image or filter tensor beyond 4 GB", what);
+    if (!Cfg::DGRAD && C_IN % 4 == 0 && reinterpret_cast<uintptr_t>(Wt) % 16 == 0)
+        hipLaunchKernelGGL((conv3x3_tiled_kernel<Cfg, !Cfg::DGRAD>), dim3(u32(wgs)), dim3(kThreads), 0, s, a);
+    else
+        hipLaunchKernelGGL((conv3x3_tiled_kernel<Cfg, false>), dim3(u32(wgs)), dim3(kThreads), 0, s, a);
+    return check_launch(what);
+}
+
+}  // namespace crb

@@ -1,6 +1,7 @@
 // C-ABI entry points of the convolution family: forward, data gradient, weight gradient and the
 // standalone bias add, all as implicit GEMMs on the MFMA engine (no im2col buffer is materialised).
 #include "conv3x3_direct.h"
+#include "conv3x3_tiled.h"
 #include "conv3x3_wgrad.h"
 #include "conv3x3_wgrad_image.h"
 #include "conv1x1_s2.h"
@@ -223,6 +224,26 @@ static int try_direct(const float *Wt, const float *X, float *Y, const float *bi
 #undef CRB_TRY
     done = false;
     return CRB_OK;
+}
+
+// 3x3 / pad 1 / stride 1 on images of any extent (conv3x3_tiled.h), <TH, TW, OCT, WP, CI, DGRAD, OCC>: 128-pixel tiles of the
+// shape that pads the image least, 32 output channels per workgroup (measured at batch 32-128 on 56 / 28 / 14 / 48 / 24 / 12
+// wide images with 32-256 channels: within 3 % of the best of eighteen tile shapes everywhere; 256-pixel and 64- or
+// 128-channel tiles and chunks of 16 channels were 5-80 % slower), 8 x 8 tiles with 64 channels for images up to 8 x 8.
+// Against the implicit-GEMM engine, forward / data gradient: 64->64 @56x56 batch 32 157 / 168 -> 93 / 99 us,
+// 128->128 @28 146 / 184 -> 93 / 99, 256->256 @14 124 / 143 -> 96 / 97, 512->512 @7 141 / 162 -> 118 / 141,
+// 64->64 @24 batch 64 84 / 99 -> 40 / 40, 32->32 @48 72 / 80 -> 37 / 37.
+template <bool DG>
+static int launch_tiled_any(const float *Wt, const float *X, float *Y, const float *bias, u32 N, u32 C_IN, u32 C_OUT, u32 H, u32 W, u32 relu,
+                            hipStream_t s, const char *what) {
+#define CRB_TILED(TH, TW, OCT, WP) return launch_tiled<TiledCfg<TH, TW, OCT, WP, 8, DG, 2>>(Wt, X, Y, bias, N, C_IN, C_OUT, H, W, relu, s, what)
+    if (H <= 8 && W <= 8) CRB_TILED(8, 8, 64, 2);
+    auto padded = [&](u32 th, u32 tw) { return uint64_t(ceil_div(H, th)) * th * ceil_div(W, tw) * tw; };
+    const uint64_t p816 = padded(8, 16), p168 = padded(16, 8), p432 = padded(4, 32);
+    if (p816 <= p168 && p816 <= p432) CRB_TILED(8, 16, 32, 4);
+    if (p168 <= p432) CRB_TILED(16, 8, 32, 4);
+    CRB_TILED(4, 32, 32, 4);
+#undef CRB_TILED
 }
 
 // Direct kernel configurations for 1x1 / stride 1 / no padding layers <W, ROWS, CI, OCT, PBW, OBW, DGRAD, OCC, NBUF, S, FS=1>.
@@ -629,6 +650,8 @@ int crb_conv_fwd(const float *W, const float *X, float *Y, const float *bias_or_
                                                    flags & CRB_FLAG_RELU, s, "crb_conv_fwd", done);
         if (done) return st;
     }
+    if (direct_shape(g, 1))  // any other extent (and operands that are only 4-byte aligned)
+        return launch_tiled_any<false>(W, X, Y, bias_or_null, g->N, g->IC, g->OC, g->OH, g->OW, flags & CRB_FLAG_RELU, s, "crb_conv_fwd");
     if (K % 4 == 0 && aligned16(W)) {
         MatK<true> a{W, M, K, 0};
         return run_nchw(a, b, e, M, N, K, s, "crb_conv_fwd");
@@ -661,6 +684,8 @@ int crb_conv_dgrad(const float *W, const float *dY, float *dX, const crb_conv_ge
     }
     if (shortcut_shape(g) && aligned16(dX))
         return launch_sc_dgrad(W, dY, dX, g->N, g->IC, g->OC, g->OH, g->OW, hipStream_t(stream), "crb_conv_dgrad");
+    if (direct_shape(g, 1))  // any other extent (and operands that are only 4-byte aligned)
+        return launch_tiled_any<true>(W, dY, dX, nullptr, g->N, g->OC, g->IC, g->OH, g->OW, 0, hipStream_t(stream), "crb_conv_dgrad");
     const u32 FHW = g->FH * g->FW;
     const u32 M = g->IC, N = g->N * g->IH * g->IW, K = g->OC * FHW;
     SepK a{W, g->IC, FHW, g->IC * FHW, 1, FastDiv(FHW)};
@@ -813,6 +838,7 @@ size_t crb_conv_fwd_workspace_bytes(const crb_conv_geom *g, int operands_aligned
             try_direct<false, 2>(nullptr, nullptr, nullptr, nullptr, g->N, g->IC, g->OC, g->OH, g->OW, g->IH, 0, nullptr, "", done, true);
         if (done) return 0;
     }
+    if (direct_shape(g, 1)) return 0;  // the tiled kernel
     return nchw_scratch_bytes(g->OC, g->N * g->OH * g->OW, g->IC * g->FH * g->FW);
 }
 
@@ -833,6 +859,7 @@ size_t crb_conv_dgrad_workspace_bytes(const crb_conv_geom *g, int operands_align
         if (done) return 0;
     }
     if (shortcut_shape(g) && operands_aligned16) return 0;
+    if (direct_shape(g, 1)) return 0;  // the tiled kernel
     return nchw_scratch_bytes(g->IC, g->N * g->IH * g->IW, g->OC * g->FH * g->FW);
 }
 

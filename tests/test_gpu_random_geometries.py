@@ -76,6 +76,54 @@ def test_random_conv_geometries(dev, seed):
         assert np.array_equal(to_np(dX1), to_np(dX2)) and np.array_equal(to_np(dW1), to_np(dW2)), shape
 
 
+# 3x3 / pad 1 / stride 1 on extents that none of the width-specialised kernels takes: the tiled kernel, every tile shape
+# (8 x 16, 16 x 8, 4 x 32 and 8 x 8 by which pads least), ragged right and bottom edges, ragged channel chunks and tiles
+OFF_GRID = [(2, 64, 56, 56, 64), (2, 128, 28, 28, 128), (3, 256, 14, 14, 96), (8, 130, 7, 7, 70), (4, 3, 24, 40, 16), (1, 20, 33, 5, 100),
+            (2, 12, 5, 33, 33), (5, 8, 1, 1, 8), (3, 9, 3, 3, 5), (2, 36, 12, 12, 64), (1, 17, 60, 17, 31), (2, 4, 9, 100, 12)]
+
+
+@pytest.mark.parametrize("shape", OFF_GRID, ids=lambda s: "x".join(map(str, s)))
+def test_3x3_layers_off_the_width_grid(dev, shape):
+    N, IC, IH, IW, OC = shape
+    run_layer(dev, N, IC, IH, IW, OC, 3, 3, 1, 1, 1, 1, bias=True, seed=sum(shape))
+
+
+@pytest.mark.parametrize("seed", [41, 42])
+def test_random_3x3_layers_of_any_extent(dev, seed):
+    rng = random.Random(seed)
+    for i in range(30):
+        N, IC, OC = rng.choice([1, 2, 3, 5]), rng.choice([1, 3, 4, 8, 9, 16, 20, 33, 64]), rng.choice([1, 5, 8, 31, 32, 33, 64, 65, 100])
+        IH, IW = rng.randint(1, 40), rng.randint(1, 70)
+        print("3x3", seed, i, (N, IC, IH, IW, OC), flush=True)
+        run_layer(dev, N, IC, IH, IW, OC, 3, 3, 1, 1, 1, 1, bias=rng.random() < 0.5, seed=100 * seed + i)
+
+
+def test_3x3_off_grid_operands_aligned_to_4_bytes_only(dev):
+    """The tiled kernel makes no alignment demands (scalar window loads; the 16-byte filter loads are chosen from the filter
+    tensor's own address): every operand one float past a 16-byte boundary."""
+    import torch
+    from crusaderbackend_amd import capi
+    from oracle import seblas_oracle as orc
+    from tests.util import assert_close
+    N, IC, H, W_, OC = 2, 16, 14, 22, 40
+    g = capi.ConvGeom.make(N, IC, H, W_, OC, 3, 3, 1, 1, 1, 1)
+    X, W, dY, b = normal(1, N, IC, H, W_), he_normal(2, OC, IC, 3, 3), normal(3, N, OC, H, W_), normal(4, OC)
+
+    def shifted(a):
+        buf = torch.empty(a.size + 1, dtype=torch.float32, device=dev)
+        v = buf[1:].view(*a.shape)
+        v.copy_(to_dev(a, dev))
+        assert v.data_ptr() % 16 == 4
+        return v
+
+    Y = shifted(np.full((N, OC, H, W_), np.nan, np.float32))
+    capi.conv_fwd(shifted(W), shifted(X), Y, shifted(b), g)
+    assert_close(to_np(Y), orc.conv(W, X, b, 1, 1, 1, 1, threads=8), IC * 9, "fwd, 4-byte aligned")
+    dX = shifted(np.full((N, IC, H, W_), np.nan, np.float32))
+    capi.conv_dgrad(shifted(W), shifted(dY), dX, g)
+    assert_close(to_np(dX), orc.convDerive(W, dY, (H, W_), 1, 1, 1, 1, threads=8), OC * 9, "dgrad, 4-byte aligned")
+
+
 @pytest.mark.parametrize("seed", [31, 32])
 def test_random_large_pointwise_layers(dev, seed):
     """1x1 layers with enough pixels per call for the kernels that stream the activations straight into the matrix
