@@ -82,6 +82,41 @@ static int run_nchw(const AOp &a, const BOp &b, NchwEpi e, u32 M, u32 N, u32 K, 
     return launch_splitk_reduce(ws, e.T, count, sp.splits, ReduceEpi{e.row_bias, e.HW, e.C, e.flags}, s, what);
 }
 
+// Data gradient at stride > 1 through the engine, one residue class of input pixels per launch (operands.h: ClassTaps,
+// ClassGather, NchwClassEpi). Classes no tap reaches (filters smaller than the stride) are zero-filled.
+static int dgrad_by_classes(const float *W, const float *dY, float *dX, const crb_conv_geom *g, hipStream_t s) {
+    const char *what = "crb_conv_dgrad";
+    const u32 FHW = g->FH * g->FW;
+    bool empty_class = false;
+    for (u32 py = 0; py < g->sH && py < g->IH; ++py)
+        for (u32 px = 0; px < g->sW && px < g->IW; ++px)
+            if ((py + g->pH) % g->sH >= g->FH || (px + g->pW) % g->sW >= g->FW) empty_class = true;
+    if (empty_class) {
+        const uint64_t count = uint64_t(g->N) * g->IC * g->IH * g->IW;
+        if (int st = crb_tensor_fill(dX, 0.f, uint32_t(count), s)) return st;
+    }
+    for (u32 py = 0; py < g->sH && py < g->IH; ++py)
+        for (u32 px = 0; px < g->sW && px < g->IW; ++px) {
+            const u32 fh0 = (py + g->pH) % g->sH, fw0 = (px + g->pW) % g->sW;
+            if (fh0 >= g->FH || fw0 >= g->FW) continue;
+            const u32 nfh = ceil_div(g->FH - fh0, g->sH), nfw = ceil_div(g->FW - fw0, g->sW);
+            const u32 CH = ceil_div(g->IH - py, g->sH), CW = ceil_div(g->IW - px, g->sW);  // the class's pixel grid
+            const u32 M = g->IC, N = g->N * CH * CW, K = g->OC * nfh * nfw;
+            ClassTaps a{W, g->IC, FHW, g->IC * FHW, fh0 * g->FW + fw0, g->sH * g->FW, g->sW, FastDiv(nfh * nfw), FastDiv(nfw)};
+            ClassGather b;
+            b.dY = dY, b.npix = N;
+            b.OH = g->OH, b.OW = g->OW, b.img_stride = g->OC * g->OH * g->OW, b.chan_stride = g->OH * g->OW;
+            b.qh = int((py + g->pH) / g->sH), b.qw = int((px + g->pW) / g->sW);
+            b.chw.init(CH * CW), b.cw.init(CW), b.ntap.init(nfh * nfw), b.nfw.init(nfw);
+            NchwClassEpi e;
+            e.T = dX, e.C = g->IC, e.HW = g->IH * g->IW, e.W = g->IW;
+            e.sH = g->sH, e.sW = g->sW, e.py = py, e.px = px;
+            e.chw.init(CH * CW), e.cw.init(CW);
+            if (int st = run_by_m(a, b, e, M, N, K, 1, 0, K, s, what)) return st;
+        }
+    return CRB_OK;
+}
+
 // Scratch bytes run_nchw asks for (0: the contraction is not cut).
 static size_t nchw_scratch_bytes(u32 M, u32 N, u32 K) {
     const u32 bm = M <= 32 ? 32 : (M <= 64 ? 64 : 128);
@@ -687,6 +722,7 @@ int crb_conv_dgrad(const float *W, const float *dY, float *dX, const crb_conv_ge
     if (direct_shape(g, 1))  // any other extent (and operands that are only 4-byte aligned)
         return launch_tiled_any<true>(W, dY, dX, nullptr, g->N, g->OC, g->IC, g->OH, g->OW, 0, hipStream_t(stream), "crb_conv_dgrad");
     const u32 FHW = g->FH * g->FW;
+    if (g->sH > 1 || g->sW > 1) return dgrad_by_classes(W, dY, dX, g, hipStream_t(stream));
     const u32 M = g->IC, N = g->N * g->IH * g->IW, K = g->OC * FHW;
     SepK a{W, g->IC, FHW, g->IC * FHW, 1, FastDiv(FHW)};
     DgradGather b;
@@ -860,6 +896,7 @@ size_t crb_conv_dgrad_workspace_bytes(const crb_conv_geom *g, int operands_align
     }
     if (shortcut_shape(g) && operands_aligned16) return 0;
     if (direct_shape(g, 1)) return 0;  // the tiled kernel
+    if (g->sH > 1 || g->sW > 1) return 0;  // one launch per residue class, none of them cut
     return nchw_scratch_bytes(g->IC, g->N * g->IH * g->IW, g->OC * g->FH * g->FW);
 }
 

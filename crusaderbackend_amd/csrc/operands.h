@@ -265,6 +265,78 @@ struct DgradGather {
     }
 };
 
+// ---- strided data gradient, one residue class of input pixels at a time -----------------------------------------
+// At stride (sH, sW) the input pixel (y, x) is reached only through the taps fh = (y + pH) mod sH + i sH,
+// fw = (x + pW) mod sW + j sW. All pixels of one residue class (y mod sH, x mod sW) = (py, px) therefore share one tap
+// subset, and their gradient is a unit-stride correlation of dY with that subset:
+//   dX[n, ic, sH y'' + py, sW x'' + px] = sum over (oc, i, j) of dY[n, oc, y'' + qh - i, x'' + qw - j] W[oc, ic, fh0 + i sH, fw0 + j sW]
+// with fh0 = (py + pH) mod sH, qh = (py + pH) / sH (likewise fw0, qw). The gather over all taps multiplies
+// (sH sW - 1) / (sH sW) structural zeros; the classes multiply none.
+// A operand: rows = input channels, k = (oc, i, j) over the class's taps.
+struct ClassTaps {
+    static constexpr bool kKFast = true, kVec = false;
+    const float *W;
+    u32 rows /* IC */, rstride /* FH*FW */, oc_stride /* IC*FH*FW */;
+    u32 tap0 /* fh0*FW + fw0 */, tap_i /* sH*FW */, tap_j /* sW */;
+    FastDiv ntap /* nfh*nfw */, nfw;
+    struct RowS {
+        u32 off;
+        bool ok;
+    };
+    struct KS {
+        u32 off;
+        bool ok;
+    };
+    __device__ __forceinline__ void bind(u32) {}
+    __device__ __forceinline__ RowS prep_row(u32 row) const { return {row * rstride, row < rows}; }
+    __device__ __forceinline__ KS prep_k(u32 k, u32 klimit) const {
+        u32 oc, r, i, j;
+        ntap.divmod(k, oc, r);
+        nfw.divmod(r, i, j);
+        return {oc * oc_stride + tap0 + i * tap_i + j * tap_j, k < klimit};
+    }
+    __device__ __forceinline__ float fetch(const RowS &r, const KS &k) const { return (r.ok && k.ok) ? W[r.off + k.off] : 0.0f; }
+};
+
+// B operand: columns are the class's pixels (n, y'', x''); k = (oc, i, j).
+struct ClassGather {
+    static constexpr bool kKFast = false, kVec = false;
+    const float *dY;
+    u32 npix;  // N * CH * CW pixels of the class
+    u32 OH, OW, img_stride /* OC*OH*OW */, chan_stride /* OH*OW */;
+    int qh, qw;
+    FastDiv chw, cw, ntap, nfw;
+    struct RowS {
+        u32 off;
+        int y, x;  // y'' + qh, x'' + qw
+        bool ok;
+    };
+    struct KS {
+        u32 off;
+        int i, j;
+        bool ok;
+    };
+    __device__ __forceinline__ void bind(u32) {}
+    __device__ __forceinline__ RowS prep_row(u32 col) const {
+        u32 n, p, y, x;
+        chw.divmod(col, n, p);
+        cw.divmod(p, y, x);
+        return {n * img_stride, int(y) + qh, int(x) + qw, col < npix};
+    }
+    __device__ __forceinline__ KS prep_k(u32 k, u32 klimit) const {
+        u32 oc, r, i, j;
+        ntap.divmod(k, oc, r);
+        nfw.divmod(r, i, j);
+        return {oc * chan_stride, int(i), int(j), k < klimit};
+    }
+    __device__ __forceinline__ float fetch(const RowS &r, const KS &k) const {
+        const int oh = r.y - k.i, ow = r.x - k.j;
+        const bool in = r.ok && k.ok && oh >= 0 && ow >= 0 && oh < int(OH) && ow < int(OW);
+        const float v = dY[in ? r.off + k.off + u32(oh) * OW + u32(ow) : 0u];  // issued regardless: no branch around a load
+        return in ? v : 0.0f;
+    }
+};
+
 // ---- epilogues ----------------------------------------------------------------------------------------
 // Row-major result C[z*zstride + row*ld + col], optional per-column bias (dense layer) or per-row bias (1x1
 // convolution as a batched GEMM), optional accumulate (C += v) and ReLU.
@@ -399,6 +471,41 @@ struct NchwEpi {
         T[c.off + row * HW] = v;
     }
     __device__ __forceinline__ void put2(u32, const ColS &, const ColS &, float, float, float, float, float) const {}
+};
+
+// NCHW scatter of one residue class: row = channel, col = (n, y'', x'') -> T[(n*C + row)*H*W + (sH y'' + py)*W + sW x'' + px].
+struct NchwClassEpi {
+    float *T;
+    u32 C, HW, W;          // channels, pixels per plane, row length of the full tensor
+    u32 sH, sW, py, px;
+    FastDiv chw, cw;       // pixels per image and per row of the class
+    struct ColS {
+        u32 off;
+        bool ok;
+    };
+    static constexpr bool kPairStore = false;
+    static constexpr bool kPrefetchOld = false;
+    static constexpr bool kEarlyOld = false;
+    static constexpr bool kRowSum = false;
+    __device__ __forceinline__ void store2(u32, const ColS &, const ColS &, float, float, float, bool, float, float) const {}
+    __device__ __forceinline__ void put2(u32, const ColS &, const ColS &, float, float, float, float, float) const {}
+    __device__ __forceinline__ bool has_row_bias() const { return false; }
+    __device__ __forceinline__ float row_bias_at(u32) const { return 0.f; }
+    __device__ __forceinline__ void bind(u32) {}
+    __device__ __forceinline__ ColS prep_col(u32 col, u32 ncols) const {
+        u32 n, p, y, x;
+        chw.divmod(col, n, p);
+        cw.divmod(p, y, x);
+        return {n * C * HW + (sH * y + py) * W + sW * x + px, col < ncols};
+    }
+    __device__ __forceinline__ bool accum_interior(u32, u32, u32, u32, u32, u32) const { return false; }
+    __device__ __forceinline__ const float *at(u32, u32) const { return nullptr; }
+    __device__ __forceinline__ bool pair_aligned(u32) const { return false; }
+    __device__ __forceinline__ bool accumulates() const { return false; }
+    __device__ __forceinline__ void store(u32 row, const ColS &c, float v, float, bool = false, float = 0.f) const {
+        if (c.ok) T[c.off + row * HW] = v;
+    }
+    __device__ __forceinline__ void put(u32 row, const ColS &c, float v, float, float) const { T[c.off + row * HW] = v; }
 };
 
 }  // namespace crb
