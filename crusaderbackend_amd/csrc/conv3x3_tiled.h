@@ -253,6 +253,11 @@ __global__ void __launch_bounds__(kThreads, Cfg::OCC) conv3x3_tiled_kernel(Tiled
     }
 }
 
+// An item's byte offset inside its image / inside the filter tensor is kept in 32 bits.
+inline bool tiled_fits(u32 C_IN, u32 C_OUT, u32 H, u32 W) {
+    return uint64_t(C_IN) * H * W * 4 <= 0xffffffffull && uint64_t(C_IN) * C_OUT * 36 <= 0xffffffffull;
+}
+
 template <class Cfg>
 inline int launch_tiled(const float *Wt, const float *X, float *Y, const float *bias, u32 N, u32 C_IN, u32 C_OUT, u32 H, u32 W, u32 relu,
                         hipStream_t s, const char *what) {
@@ -267,9 +272,7 @@ inline int launch_tiled(const float *Wt, const float *X, float *Y, const float *
     if (tiles > 0x7fffffffull || wgs > 0x7fffffffull) return fail(CRB_EINVAL_SHAPE, "%s: launch grid too large", what);
     a.tiles_total = u32(tiles);
     a.relu = relu;
-    // an item's byte offset inside its image / inside the filter tensor is kept in 32 bits
-    if (uint64_t(C_IN) * H * W * 4 > 0xffffffffull || uint64_t(C_IN) * C_OUT * 36 > 0xffffffffull)
-        return fail(CRB_EINVAL_SHAPE, "%s: image or filter tensor beyond 4 GB", what);
+    if (!tiled_fits(C_IN, C_OUT, H, W)) return fail(CRB_EINVAL_SHAPE, "%s: image or filter tensor beyond 4 GB", what);
     if (!Cfg::DGRAD && C_IN % 4 == 0 && reinterpret_cast<uintptr_t>(Wt) % 16 == 0)
         hipLaunchKernelGGL((conv3x3_tiled_kernel<Cfg, !Cfg::DGRAD>), dim3(u32(wgs)), dim3(kThreads), 0, s, a);
     else

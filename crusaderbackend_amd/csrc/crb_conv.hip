@@ -685,7 +685,7 @@ int crb_conv_fwd(const float *W, const float *X, float *Y, const float *bias_or_
                                                    flags & CRB_FLAG_RELU, s, "crb_conv_fwd", done);
         if (done) return st;
     }
-    if (direct_shape(g, 1))  // any other extent (and operands that are only 4-byte aligned)
+    if (direct_shape(g, 1) && tiled_fits(g->IC, g->OC, g->IH, g->IW))  // any other extent (and operands that are only 4-byte aligned)
         return launch_tiled_any<false>(W, X, Y, bias_or_null, g->N, g->IC, g->OC, g->OH, g->OW, flags & CRB_FLAG_RELU, s, "crb_conv_fwd");
     if (K % 4 == 0 && aligned16(W)) {
         MatK<true> a{W, M, K, 0};
@@ -719,7 +719,7 @@ int crb_conv_dgrad(const float *W, const float *dY, float *dX, const crb_conv_ge
     }
     if (shortcut_shape(g) && aligned16(dX))
         return launch_sc_dgrad(W, dY, dX, g->N, g->IC, g->OC, g->OH, g->OW, hipStream_t(stream), "crb_conv_dgrad");
-    if (direct_shape(g, 1))  // any other extent (and operands that are only 4-byte aligned)
+    if (direct_shape(g, 1) && tiled_fits(g->OC, g->IC, g->IH, g->IW))  // any other extent (and operands that are only 4-byte aligned)
         return launch_tiled_any<true>(W, dY, dX, nullptr, g->N, g->OC, g->IC, g->OH, g->OW, 0, hipStream_t(stream), "crb_conv_dgrad");
     const u32 FHW = g->FH * g->FW;
     if (g->sH > 1 || g->sW > 1) return dgrad_by_classes(W, dY, dX, g, hipStream_t(stream));
@@ -874,7 +874,7 @@ size_t crb_conv_fwd_workspace_bytes(const crb_conv_geom *g, int operands_aligned
             try_direct<false, 2>(nullptr, nullptr, nullptr, nullptr, g->N, g->IC, g->OC, g->OH, g->OW, g->IH, 0, nullptr, "", done, true);
         if (done) return 0;
     }
-    if (direct_shape(g, 1)) return 0;  // the tiled kernel
+    if (direct_shape(g, 1) && tiled_fits(g->IC, g->OC, g->IH, g->IW)) return 0;  // the tiled kernel
     return nchw_scratch_bytes(g->OC, g->N * g->OH * g->OW, g->IC * g->FH * g->FW);
 }
 
@@ -895,7 +895,7 @@ size_t crb_conv_dgrad_workspace_bytes(const crb_conv_geom *g, int operands_align
         if (done) return 0;
     }
     if (shortcut_shape(g) && operands_aligned16) return 0;
-    if (direct_shape(g, 1)) return 0;  // the tiled kernel
+    if (direct_shape(g, 1) && tiled_fits(g->OC, g->IC, g->IH, g->IW)) return 0;  // the tiled kernel
     if (g->sH > 1 || g->sW > 1) return 0;  // one launch per residue class, none of them cut
     return nchw_scratch_bytes(g->IC, g->N * g->IH * g->IW, g->OC * g->FH * g->FW);
 }
