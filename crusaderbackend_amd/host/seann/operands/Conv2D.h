@@ -17,6 +17,7 @@ public:
     bool gradsFused = false;      // xGrads computes the filter gradient too (fuseGrads())
     bool filterGradDone = false;  // ... and has done so since the last forward / paramGrads
     Tensor *gradSlices = nullptr;  // deferSliceSum(): xGrads leaves the filter gradient here as partial sums
+    OperandBase *fusedRelu = nullptr;  // the ReLU behind this operand whose passes it computes (absorbReLU)
 
     Conv2D(shape4 filterShape, uint32 strideH, uint32 strideW, uint32 padH, uint32 padW, bool WITH_BIAS)
         : filterShape(filterShape), strideH(strideH), strideW(strideW), padH(padH), padW(padW), WITH_BIAS(WITH_BIAS) {}
@@ -45,6 +46,12 @@ public:
         if (WITH_BIAS) out.push_back(bias);
     }
     void fuseGrads() override { gradsFused = true; }
+    // forward writes max(conv, 0) straight into the ReLU's output; xGrads masks the ReLU's output gradient by that output
+    // (positive exactly where the convolution's own result was) before it runs the convolution's gradients
+    bool absorbReLU(OperandBase *relu) override {
+        fusedRelu = relu;
+        return true;
+    }
     void deferSliceSum(std::vector<seblas::SliceSumItem> &items) override;
     uint32 OPERAND_ID() override { return OPR_SEBLAS_CONV2D; }
     // info: filter dims, strides, paddings, has-bias flag (36 bytes); params: filter, then bias (Conv2D.cu:59-80)

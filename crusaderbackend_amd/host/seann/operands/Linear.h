@@ -13,6 +13,7 @@ public:
     NetParam *biases{};
     uint32 INPUT_SIZE{};
     uint32 OUTPUT_SIZE;
+    OperandBase *fusedRelu = nullptr;  // the ReLU behind this operand whose passes it computes (absorbReLU)
 
     explicit Linear(uint32 OUTPUT_SIZE) : OUTPUT_SIZE(OUTPUT_SIZE) {}
 
@@ -37,6 +38,11 @@ public:
     void collectNetParams(std::vector<NetParam *> &out) override {
         out.push_back(weights);
         out.push_back(biases);
+    }
+    // forward writes max(., 0) straight into the ReLU's output; xGrads masks the ReLU's output gradient by that output
+    bool absorbReLU(OperandBase *relu) override {
+        fusedRelu = relu;
+        return true;
     }
     uint32 OPERAND_ID() override { return OPR_SEBLAS_LINEAR; }
     // info: OUTPUT_SIZE; params: weights, then biases (Linear.cu:62-75)

@@ -27,11 +27,13 @@ void Conv2D::initNetParams(OptimizerInfo *info, shape4 inShape) {
 
 void Conv2D::forward() {  // Conv2D.cu:8-16
     filterGradDone = false;
-    conv(filter->data(), X->A, Y->A, int(strideH), int(strideW), int(padH), int(padW), WITH_BIAS ? bias->data() : nullptr);
+    conv(filter->data(), X->A, fusedRelu ? fusedRelu->Y->A : Y->A, int(strideH), int(strideW), int(padH), int(padW),
+         WITH_BIAS ? bias->data() : nullptr, fusedRelu != nullptr);
 }
 
 void Conv2D::xGrads() {  // Conv2D.cu:18-22
     foldReserve();
+    if (fusedRelu) reluGradFast(fusedRelu->Y->A, fusedRelu->Y->dA, Y->dA);
     if (gradSlices) {  // both gradients in one call, the filter gradient as partial sums that the caller completes
         convBackwardSliced(filter->data(), Y->dA, X->A, X->dA, gradSlices, int(strideH), int(strideW), int(padH), int(padW));
         filterGradDone = true;
@@ -84,12 +86,15 @@ void Linear::initNetParams(OptimizerInfo *info, shape4 inShape) {  // Linear.cu:
     biases = new NetParam(info, OUTPUT_SIZE, 1);
 }
 
-void Linear::forward() { linear(X->A, weights->data(), biases->data(), Y->A); }  // Linear.cu:17-19
+void Linear::forward() {  // Linear.cu:17-19
+    linear(X->A, weights->data(), biases->data(), fusedRelu ? fusedRelu->Y->A : Y->A, fusedRelu != nullptr);
+}
 
 void Linear::paramGrads() { linearParamGrad(Y->dA, X->A, weights->grad(), biases->grad()); }  // :21-23
 
 void Linear::xGrads() {  // Linear.cu:35-40
     foldReserve();
+    if (fusedRelu) reluGradFast(fusedRelu->Y->A, fusedRelu->Y->dA, Y->dA);
     linearXGrad(Y->dA, weights->data(), X->dA);
 }
 

@@ -55,7 +55,7 @@ Tensor *sgemmNTA(Tensor *A, Tensor *B, Tensor *C) {
     return C;
 }
 
-Tensor *linear(Tensor *X, Tensor *W, Tensor *B, Tensor *Y) {
+Tensor *linear(Tensor *X, Tensor *W, Tensor *B, Tensor *Y, bool relu) {
     const uint32 M = Y->dims.h;                                  // cuLinear.cu:1053
     const uint32 N = Y->dims.n * Y->dims.w;                      // :1054
     require(W->dims.w == X->dims.h, "linear: W.w != X.h");       // :1056
@@ -63,7 +63,7 @@ Tensor *linear(Tensor *X, Tensor *W, Tensor *B, Tensor *Y) {
     require(Y->dims.w == 1 && B->dims.w == 1 && X->dims.w == 1, "linear: X, B, Y must have w == 1");  // :1058
     require(X->dims.n == Y->dims.n, "linear: batch mismatch");   // :1059
     require(W->dims.h == M, "linear: W.h != Y.h");
-    finish(crb_linear_fwd(X->elements, W->elements, B->elements, Y->elements, N, W->dims.w, M, 0, nullptr), __FILE__,
+    finish(crb_linear_fwd(X->elements, W->elements, B->elements, Y->elements, N, W->dims.w, M, relu ? CRB_FLAG_RELU : 0u, nullptr), __FILE__,
            __LINE__);
     return Y;
 }
@@ -106,10 +106,10 @@ static crb_conv_geom geom(Tensor *filters, Tensor *features, Tensor *featureOut,
     return g;
 }
 
-Tensor *conv(Tensor *A, Tensor *B, Tensor *C, int strideH, int strideW, int padH, int padW, Tensor *biases) {
+Tensor *conv(Tensor *A, Tensor *B, Tensor *C, int strideH, int strideW, int padH, int padW, Tensor *biases, bool relu) {
     crb_conv_geom g = geom(A, B, C, strideH, strideW, padH, padW);
     if (biases) require(biases->dims.size == g.OC, "conv: biases must hold OC elements");
-    finish(crb_conv_fwd(A->elements, B->elements, C->elements, biases ? biases->elements : nullptr, &g, 0, nullptr),
+    finish(crb_conv_fwd(A->elements, B->elements, C->elements, biases ? biases->elements : nullptr, &g, relu ? CRB_FLAG_RELU : 0u, nullptr),
            __FILE__, __LINE__);
     return C;
 }

@@ -19,12 +19,12 @@ Tensor *sgemmNT(Tensor *A, Tensor *B, Tensor *C);   // C = A * B^T
 Tensor *sgemmNTA(Tensor *A, Tensor *B, Tensor *C);  // C += sum_n A[n] * B[n]^T
 
 // cuLinear.cu:1052-1113
-Tensor *linear(Tensor *X, Tensor *W, Tensor *B, Tensor *Y);
+Tensor *linear(Tensor *X, Tensor *W, Tensor *B, Tensor *Y, bool relu = false);  // relu: max(., 0) applied in the same pass (not in the reference)
 Tensor *linearXGrad(Tensor *dY, Tensor *W, Tensor *dX);
 Tensor *linearParamGrad(Tensor *dY, Tensor *X, Tensor *dW, Tensor *dB);  // returns dW
 
 // cuConv.cu:757-818. A: filters OC x IC x FH x FW.
-Tensor *conv(Tensor *A, Tensor *B, Tensor *C, int strideH, int strideW, int padH, int padW, Tensor *biases);
+Tensor *conv(Tensor *A, Tensor *B, Tensor *C, int strideH, int strideW, int padH, int padW, Tensor *biases, bool relu = false);
 Tensor *convDerive(Tensor *A, Tensor *B, Tensor *C, int strideH, int strideW, int padH, int padW);
 // A: errors N x OC x OH x OW, B: inputs N x IC x IH x IW, C: filter grads (accumulated). Returns A, as the
 // reference does (cuConv.cu:805).
