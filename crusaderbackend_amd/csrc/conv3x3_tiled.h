@@ -27,14 +27,22 @@
 
 namespace crb {
 
-template <int TH_, int TW_, int OCT_, int WP_, int CI_, bool DGRAD_, int OCC_>
+template <int TH_, int TW_, int OCT_, int WP_, int CI_, bool DGRAD_, int OCC_, int S_ = 1>
 struct TiledCfg {
-    static constexpr int TH = TH_, TW = TW_, OCT = OCT_, WP = WP_, WO = 4 / WP_, CI = CI_, OCC = OCC_;
+    static constexpr int TH = TH_, TW = TW_, OCT = OCT_, WP = WP_, WO = 4 / WP_, CI = CI_, OCC = OCC_, S = S_;
     static constexpr bool DGRAD = DGRAD_;
     static constexpr int PIX = TH * TW, NPB = PIX / 32, NOB = OCT / 32;  // 32-pixel and 32-channel MFMA blocks
     static constexpr int PB = NPB / WP, OB = NOB / WO;                  // blocks per wave
     static constexpr int RB = 32 / TW;                                  // image rows per pixel block
-    static constexpr int XR = TH + 2, XC = TW + 2, XS = TW + 4;          // staged rows, columns; LDS row stride
+    // staged rows and columns of the input window; LDS row stride. Stride 2 (forward only): a staged row holds the window's
+    // even columns (input columns 2 x0 - 1, 2 x0 + 1, ...: taps fw = 0 and 2) and then, HALF floats further, its odd columns
+    // (tap fw = 1), so that neighbouring pixels read neighbouring floats for every tap.
+    static constexpr int XR = S * (TH - 1) + 3, XC = S * (TW - 1) + 3;
+    static constexpr int HALF = TW + 2;
+    static constexpr int XS = S == 1 ? TW + 4 : 2 * TW + 4;
+    static constexpr int col_pos(int lc) { return S == 1 ? lc : (lc % 2) * HALF + lc / 2; }
+    static constexpr int tap_off(int fh, int fw) { return S == 1 ? fh * XS + fw : fh * XS + (fw == 1 ? HALF : fw / 2); }
+    static_assert(S == 1 || (S == 2 && !DGRAD_), "stride 2: forward only");
     static constexpr int XP = XR * XS;                                  // channel plane stride
     static constexpr int X_SIZE = CI * XP;
     static constexpr int KC = CI * 9, KH = KC / 2;                      // contraction per chunk, per lane half
@@ -52,7 +60,8 @@ struct TiledArgs {
     const float *X;     // input of this pass  (forward: X, data gradient: dY), N x C_IN x H x W
     float *Y;           // output of this pass (forward: Y, data gradient: dX), N x C_OUT x H x W
     const float *bias;  // per output channel or nullptr
-    u32 C_IN, C_OUT, H, W;
+    u32 C_IN, C_OUT, H, W;  // H, W: extent of the output (the pixel grid)
+    u32 IH, IW;             // extent of the staged tensor (H, W at stride 1)
     u32 tiles_x, tiles_per_img, oc_tiles, tiles_total;  // tiles_total = N * tiles_per_img
     u32 relu;
 };
@@ -75,7 +84,7 @@ __global__ void __launch_bounds__(kThreads, Cfg::OCC) conv3x3_tiled_kernel(Tiled
     const u32 n = rest / a.tiles_per_img, tile = rest % a.tiles_per_img;
     const int y0 = int(tile / a.tiles_x) * TH, x0 = int(tile % a.tiles_x) * TW;
     const u32 oc0 = oct * OCT;
-    const u32 HW = a.H * a.W;
+    const u32 HW = a.H * a.W, IHW = a.IH * a.IW;
 
     // ---- staging: thread t owns items t, t + 256, ... of the window (channel, row, column) and of the filter slice --------
     // An item's byte offset from the chunk's (uniform) base address does not depend on the chunk: computed once. Loads are
@@ -88,14 +97,14 @@ __global__ void __launch_bounds__(kThreads, Cfg::OCC) conv3x3_tiled_kernel(Tiled
     u32 xoff[XNP], woff[WNP];
     typedef typename std::conditional<WVEC, v4f, float>::type WItem;
     WItem wreg[WNP];
-    const char *xin = reinterpret_cast<const char *>(a.X + size_t(n) * a.C_IN * HW);
+    const char *xin = reinterpret_cast<const char *>(a.X + size_t(n) * a.C_IN * IHW);
 #pragma unroll
     for (int i = 0; i < XNP; ++i) {
         const u32 e = t + i * kThreads;
         const u32 c = e / (XR * XC), lr = (e / XC) % XR, lc = e % XC;
-        const int y = y0 - 1 + int(lr), x = x0 - 1 + int(lc);
-        const bool ok = (XQ % kThreads == 0 || e < XQ) && y >= 0 && y < int(a.H) && x >= 0 && x < int(a.W);
-        xoff[i] = ok ? (c * HW + u32(y) * a.W + u32(x)) * 4u : kNone;
+        const int y = Cfg::S * y0 - 1 + int(lr), x = Cfg::S * x0 - 1 + int(lc);
+        const bool ok = (XQ % kThreads == 0 || e < XQ) && y >= 0 && y < int(a.IH) && x >= 0 && x < int(a.IW);
+        xoff[i] = ok ? (c * IHW + u32(y) * a.IW + u32(x)) * 4u : kNone;
     }
     // filter slice of chunk c0: LDS row j (output channel oc0 + j) holds k = c * 9 + tap for the chunk's channels c.
     // forward: row j is KC consecutive floats of Wt[oc0 + j] from channel c0 on; data gradient: the OCT * 9 consecutive floats
@@ -127,7 +136,7 @@ __global__ void __launch_bounds__(kThreads, Cfg::OCC) conv3x3_tiled_kernel(Tiled
         else return c0 * 9 + e % KC < a.C_IN * 9;
     };
     auto fetch = [&](u32 c0) {
-        const char *xc = xin + size_t(c0) * HW * 4;
+        const char *xc = xin + size_t(c0) * IHW * 4;
         const char *wc = reinterpret_cast<const char *>(Cfg::DGRAD ? a.Wt + (size_t(c0) * a.C_OUT + oc0) * 9 : a.Wt + (size_t(oc0) * a.C_IN + c0) * 9);
 #pragma unroll
         for (int i = 0; i < XNP; ++i) {
@@ -145,7 +154,7 @@ __global__ void __launch_bounds__(kThreads, Cfg::OCC) conv3x3_tiled_kernel(Tiled
         for (int i = 0; i < XNP; ++i) {
             const u32 e = t + i * kThreads, c = e / (XR * XC);
             const bool ok = xoff[i] != kNone && c0 + c < a.C_IN;
-            if (XQ % kThreads == 0 || e < XQ) dx[c * XP + ((e / XC) % XR) * XS + e % XC] = ok ? xreg[i] : 0.f;
+            if (XQ % kThreads == 0 || e < XQ) dx[c * XP + ((e / XC) % XR) * XS + Cfg::col_pos(e % XC)] = ok ? xreg[i] : 0.f;
         }
 #pragma unroll
         for (int i = 0; i < WNP; ++i) {
@@ -169,7 +178,7 @@ __global__ void __launch_bounds__(kThreads, Cfg::OCC) conv3x3_tiled_kernel(Tiled
     const int wp = wave % Cfg::WP, wo = wave / Cfg::WP;
     // this lane's pixel in the wave's first pixel block; block p is RB * p image rows further down
     const int pix = wp * PB * 32 + j32, prow = pix / TW, pcol = pix % TW;
-    const int xbase = h * (CI / 2) * XP + prow * XS + pcol;
+    const int xbase = h * (CI / 2) * XP + Cfg::S * prow * XS + pcol;
     const int wbase = (wo * OB * 32 + j32) * WSTR + h * KH;
 
     v16f acc[OB][PB];
@@ -194,7 +203,7 @@ __global__ void __launch_bounds__(kThreads, Cfg::OCC) conv3x3_tiled_kernel(Tiled
                 const int s = 4 * sq + e, c = s / 9, tap = s % 9;
                 const int fh = Cfg::DGRAD ? 2 - tap / 3 : tap / 3, fw = Cfg::DGRAD ? 2 - tap % 3 : tap % 3;
 #pragma unroll
-                for (int p = 0; p < PB; ++p) xv[set][e][p] = xfrag[c * XP + (p * Cfg::RB + fh) * XS + fw];
+                for (int p = 0; p < PB; ++p) xv[set][e][p] = xfrag[c * XP + Cfg::S * p * Cfg::RB * XS + Cfg::tap_off(fh, fw)];
             }
         };
         read_group(0, 0);
@@ -260,10 +269,11 @@ inline bool tiled_fits(u32 C_IN, u32 C_OUT, u32 H, u32 W) {
 
 template <class Cfg>
 inline int launch_tiled(const float *Wt, const float *X, float *Y, const float *bias, u32 N, u32 C_IN, u32 C_OUT, u32 H, u32 W, u32 relu,
-                        hipStream_t s, const char *what) {
+                        hipStream_t s, const char *what, u32 IH = 0, u32 IW = 0) {
     TiledArgs a;
     a.Wt = Wt, a.X = X, a.Y = Y, a.bias = bias;
     a.C_IN = C_IN, a.C_OUT = C_OUT, a.H = H, a.W = W;
+    a.IH = IH ? IH : H, a.IW = IW ? IW : W;
     a.tiles_x = ceil_div(W, u32(Cfg::TW));
     a.tiles_per_img = a.tiles_x * ceil_div(H, u32(Cfg::TH));
     a.oc_tiles = ceil_div(C_OUT, u32(Cfg::OCT));
@@ -272,7 +282,7 @@ inline int launch_tiled(const float *Wt, const float *X, float *Y, const float *
     if (tiles > 0x7fffffffull || wgs > 0x7fffffffull) return fail(CRB_EINVAL_SHAPE, "%s: launch grid too large", what);
     a.tiles_total = u32(tiles);
     a.relu = relu;
-    if (!tiled_fits(C_IN, C_OUT, H, W)) return fail(CRB_EINVAL_SHAPE, "%s: image or filter tensor beyond 4 GB", what);
+    if (!tiled_fits(C_IN, C_OUT, a.IH, a.IW)) return fail(CRB_EINVAL_SHAPE, "%s: image or filter tensor beyond 4 GB", what);
     if (!Cfg::DGRAD && C_IN % 4 == 0 && reinterpret_cast<uintptr_t>(Wt) % 16 == 0)
         hipLaunchKernelGGL((conv3x3_tiled_kernel<Cfg, !Cfg::DGRAD>), dim3(u32(wgs)), dim3(kThreads), 0, s, a);
     else

@@ -88,6 +88,17 @@ def test_3x3_layers_off_the_width_grid(dev, shape):
     run_layer(dev, N, IC, IH, IW, OC, 3, 3, 1, 1, 1, 1, bias=True, seed=sum(shape))
 
 
+# 3x3 / pad 1 / stride 2 off the width grid: tiled forward (odd / even window columns de-interleaved in LDS), data gradient by
+# residue classes; odd and even extents, ragged tiles and channel chunks
+OFF_GRID_S2 = [(2, 64, 56, 56, 128), (3, 16, 7, 7, 24), (2, 9, 15, 22, 33), (1, 128, 28, 28, 40), (4, 8, 5, 64, 8), (2, 40, 24, 24, 64)]
+
+
+@pytest.mark.parametrize("shape", OFF_GRID_S2, ids=lambda s: "x".join(map(str, s)))
+def test_3x3_stride_2_layers_off_the_width_grid(dev, shape):
+    N, IC, IH, IW, OC = shape
+    run_layer(dev, N, IC, IH, IW, OC, 3, 3, 2, 2, 1, 1, bias=True, seed=sum(shape))
+
+
 @pytest.mark.parametrize("seed", [41, 42])
 def test_random_3x3_layers_of_any_extent(dev, seed):
     rng = random.Random(seed)
