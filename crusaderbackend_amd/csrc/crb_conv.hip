@@ -2,6 +2,7 @@
 // standalone bias add, all as implicit GEMMs on the MFMA engine (no im2col buffer is materialised).
 #include "conv3x3_direct.h"
 #include "conv3x3_tiled.h"
+#include "conv3x3_tiled_wgrad.h"
 #include "conv3x3_wgrad.h"
 #include "conv3x3_wgrad_image.h"
 #include "conv1x1_s2.h"
@@ -386,6 +387,38 @@ static bool tiny2x2_shape(const crb_conv_geom *g) {
     return direct_shape(g, 1) && g->IH == 2 && g->IW == 2 && uint64_t(g->OC) * g->IC * 16 <= 0x7fffffffull;
 }
 
+// Weight gradient of 3x3 / pad 1 / stride 1 layers on any extent (conv3x3_tiled_wgrad.h), <TH, TW, NOB, NIB, OCC>: 64-pixel tiles of
+// the shape that pads the image least, blocks of 64 x 64 channels (32 on a side with at most 32 channels).
+// `run` = false only computes the plan (workspace size).
+static bool wgrad_tiled(const crb_conv_geom *g, bool run, const float *dY, const float *X, float *dW, float *ws, hipStream_t s,
+                        TiledWgradPlan &plan, int &status) {
+    // (images below 12 x 12 pad their 8 x 8 tiles too much: the engine's flat pixel contraction is as fast or faster there)
+    if (!direct_shape(g, 1) || !tiled_wgrad_fits(g->N, g->IC, g->OC, g->OH, g->OW) || g->OH * g->OW < 144) return false;
+    const u32 H = g->OH, W = g->OW;
+    auto padded = [&](u32 th, u32 tw) { return uint64_t(ceil_div(H, th)) * th * ceil_div(W, tw) * tw; };
+    const uint64_t p416 = padded(4, 16), p88 = padded(8, 8), p232 = padded(2, 32);
+    const int shape = (p416 <= p88 && p416 <= p232) ? 0 : (p88 <= p232 ? 1 : 2);
+#define CRB_TW(TH, TW, NOB, NIB)                                                                                        \
+    {                                                                                                                   \
+        typedef TiledWgradCfg<TH, TW, NOB, NIB> C;                                                                      \
+        plan = tiled_wgrad_plan<C>(g->N, g->IC, g->OC, H, W);                                                           \
+        if (run) status = launch_tiled_wgrad<C>(dY, X, dW, ws, plan, g->IC, g->OC, H, W, s, "crb_conv_wgrad");          \
+        return true;                                                                                                    \
+    }
+#define CRB_TW_SHAPES(NOB, NIB)            \
+    {                                      \
+        if (shape == 0) CRB_TW(4, 16, NOB, NIB) \
+        if (shape == 1) CRB_TW(8, 8, NOB, NIB)  \
+        CRB_TW(2, 32, NOB, NIB)            \
+    }
+    if (g->OC > 32 && g->IC > 32) CRB_TW_SHAPES(2, 2)
+    if (g->OC > 32) CRB_TW_SHAPES(2, 1)
+    if (g->IC > 32) CRB_TW_SHAPES(1, 2)
+    CRB_TW_SHAPES(1, 1)
+#undef CRB_TW_SHAPES
+#undef CRB_TW
+}
+
 // ---- direct 3x3 / pad 1 weight gradient (stride 1 and 2) ---------------------------------------------------------
 // One entry per configuration <W, TR, TI, OCC>; `run` = false only computes the plan (workspace size).
 constexpr u32 kWgradTargetWgs = 256;  // one workgroup per CU: pairs x splits (two per CU for wide layers, see wgrad_direct_plan)
@@ -761,8 +794,10 @@ size_t crb_conv_wgrad_workspace_bytes(const crb_conv_geom *g) {
     if (shortcut_shape(g)) return sc_wgrad_plan(g->N, g->IC, g->OC, g->OH, g->OW).workspace_bytes;
     {
         WgradDirectPlan dp;
+        TiledWgradPlan tp;
         int st = 0;
         if (wgrad_direct(g, false, nullptr, nullptr, nullptr, nullptr, nullptr, dp, st)) return dp.workspace_bytes;
+        if (wgrad_tiled(g, false, nullptr, nullptr, nullptr, nullptr, nullptr, tp, st)) return tp.workspace_bytes;
     }
     const WgradPlan p = wgrad_plan(g);
     return p.splits > 1 ? size_t(p.splits) * p.M * p.Ncols * sizeof(float) : 0;
@@ -829,6 +864,24 @@ int crb_conv_wgrad(const float *dY, const float *X, float *dW, const crb_conv_ge
                 }
             }
             wgrad_direct(g, true, dY, X, dW, dws, s, dp, st);
+            return st;
+        }
+    }
+    {
+        // the shapes no width-specialised kernel takes (those keep their own workspace size, whatever the alignment)
+        TiledWgradPlan tp;
+        WgradDirectPlan dp;
+        int st = CRB_OK;
+        if (!wgrad_direct(g, false, nullptr, nullptr, nullptr, nullptr, nullptr, dp, st) &&
+            wgrad_tiled(g, false, nullptr, nullptr, nullptr, nullptr, nullptr, tp, st)) {
+            float *tws = static_cast<float *>(workspace);
+            if (tws) {
+                if (workspace_bytes < tp.workspace_bytes)
+                    return fail(CRB_EWORKSPACE, "crb_conv_wgrad: workspace %zu bytes < required %zu", workspace_bytes, tp.workspace_bytes);
+            } else if (int sg = scratch_get(tp.workspace_bytes, s, "crb_conv_wgrad", &tws)) {
+                return sg;
+            }
+            wgrad_tiled(g, true, dY, X, dW, tws, s, tp, st);
             return st;
         }
     }

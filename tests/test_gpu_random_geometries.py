@@ -76,10 +76,12 @@ def test_random_conv_geometries(dev, seed):
         assert np.array_equal(to_np(dX1), to_np(dX2)) and np.array_equal(to_np(dW1), to_np(dW2)), shape
 
 
-# 3x3 / pad 1 / stride 1 on extents that none of the width-specialised kernels takes: the tiled kernel, every tile shape
-# (8 x 16, 16 x 8, 4 x 32 and 8 x 8 by which pads least), ragged right and bottom edges, ragged channel chunks and tiles
+# 3x3 / pad 1 / stride 1 on extents that none of the width-specialised kernels takes: the tiled kernels, every tile shape
+# (forward / data gradient 8 x 16, 16 x 8, 4 x 32 and 8 x 8, weight gradient 4 x 16, 8 x 8 and 2 x 32, by which pads least) and
+# every channel blocking of the weight gradient, ragged right and bottom edges, ragged channel chunks and blocks
 OFF_GRID = [(2, 64, 56, 56, 64), (2, 128, 28, 28, 128), (3, 256, 14, 14, 96), (8, 130, 7, 7, 70), (4, 3, 24, 40, 16), (1, 20, 33, 5, 100),
-            (2, 12, 5, 33, 33), (5, 8, 1, 1, 8), (3, 9, 3, 3, 5), (2, 36, 12, 12, 64), (1, 17, 60, 17, 31), (2, 4, 9, 100, 12)]
+            (2, 12, 5, 33, 33), (5, 8, 1, 1, 8), (3, 9, 3, 3, 5), (2, 36, 12, 12, 64), (1, 17, 60, 17, 31), (2, 4, 9, 100, 12),
+            (2, 40, 20, 20, 24), (9, 33, 13, 29, 33)]
 
 
 @pytest.mark.parametrize("shape", OFF_GRID, ids=lambda s: "x".join(map(str, s)))

@@ -157,7 +157,7 @@ def test_pointwise_wgrad_honours_the_workspace_argument(dev):
 EXACT_SHAPES = [(128, 64, 2, 64, 3, 1, 1, True), (128, 512, 2, 512, 3, 1, 1, True), (8, 40, 2, 24, 3, 1, 1, True),
                 (64, 24, 16, 48, 1, 1, 0, False), (4, 96, 7, 40, 1, 1, 0, True), (2, 300, 6, 20, 1, 1, 0, False),
                 (2, 64, 12, 48, 5, 1, 2, True), (3, 20, 9, 12, 3, 2, 1, True), (16, 16, 32, 16, 3, 1, 1, False),
-                (8, 16, 16, 32, 1, 2, 0, True)]
+                (8, 16, 16, 32, 1, 2, 0, True), (4, 40, 14, 48, 3, 1, 1, True), (3, 24, 20, 70, 3, 1, 1, False), (2, 16, 15, 24, 3, 2, 1, True)]
 
 
 @pytest.mark.parametrize("shape", EXACT_SHAPES, ids=lambda s: "x".join(map(str, s[:7])) + ("" if s[7] else "-unaligned"))
