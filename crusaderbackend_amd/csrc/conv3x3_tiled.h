@@ -177,7 +177,14 @@ __global__ void __launch_bounds__(kThreads, Cfg::OCC) conv3x3_tiled_kernel(Tiled
     const int lane = t & 63, wave = t >> 6, j32 = lane & 31, h = lane >> 5;
     const int wp = wave % Cfg::WP, wo = wave / Cfg::WP;
     // this lane's pixel in the wave's first pixel block; block p is RB * p image rows further down
-    const int pix = wp * PB * 32 + j32, prow = pix / TW, pcol = pix % TW;
+    // A wave with one pixel block takes image rows that are SPREAD apart instead of adjacent ones, so that the rows of a
+    // fragment read land on disjoint banks (16-wide tiles: rows r and r + 4, 80 floats = 16 banks apart; 8-wide tiles: rows
+    // r, r + 2, r + 4, r + 6, 24 floats apart: banks +24, +16, +8); adjacent rows overlapped on 2 to 4 banks.
+    constexpr bool kSpread = PB == 1 && TW < 32 && Cfg::S == 1;
+    constexpr int kRowStep = !kSpread ? 1 : (TW == 16 ? TH / 2 : 2);
+    const int pix = wp * PB * 32 + j32, pcol = pix % TW;
+    const int prow = !kSpread ? pix / TW : (TW == 16 ? wp + kRowStep * (j32 / TW) : (wp / 2) * 8 + wp % 2 + kRowStep * (j32 / TW));
+    static_assert(!kSpread || (TW == 16 && Cfg::NPB == TH / 2) || (TW == 8 && TH % 8 == 0), "row spreading covers the tile");
     const int xbase = h * (CI / 2) * XP + Cfg::S * prow * XS + pcol;
     const int wbase = (wo * OB * 32 + j32) * WSTR + h * KH;
 
