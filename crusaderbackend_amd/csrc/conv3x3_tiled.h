@@ -27,9 +27,11 @@
 
 namespace crb {
 
-template <int TH_, int TW_, int OCT_, int WP_, int CI_, bool DGRAD_, int OCC_, int S_ = 1>
+// F_: filter size (3, or 5 with pad 2 at stride 1); the header's "3x3", "9" and "halo of one" read F x F, F * F and F / 2.
+template <int TH_, int TW_, int OCT_, int WP_, int CI_, bool DGRAD_, int OCC_, int S_ = 1, int F_ = 3>
 struct TiledCfg {
     static constexpr int TH = TH_, TW = TW_, OCT = OCT_, WP = WP_, WO = 4 / WP_, CI = CI_, OCC = OCC_, S = S_;
+    static constexpr int F = F_, NT = F_ * F_, PAD = F_ / 2;
     static constexpr bool DGRAD = DGRAD_;
     static constexpr int PIX = TH * TW, NPB = PIX / 32, NOB = OCT / 32;  // 32-pixel and 32-channel MFMA blocks
     static constexpr int PB = NPB / WP, OB = NOB / WO;                  // blocks per wave
@@ -37,16 +39,17 @@ struct TiledCfg {
     // staged rows and columns of the input window; LDS row stride. Stride 2 (forward only): a staged row holds the window's
     // even columns (input columns 2 x0 - 1, 2 x0 + 1, ...: taps fw = 0 and 2) and then, HALF floats further, its odd columns
     // (tap fw = 1), so that neighbouring pixels read neighbouring floats for every tap.
-    static constexpr int XR = S * (TH - 1) + 3, XC = S * (TW - 1) + 3;
+    static constexpr int XR = S * (TH - 1) + F, XC = S * (TW - 1) + F;
     static constexpr int HALF = TW + 2;
-    static constexpr int XS = S == 1 ? TW + 4 : 2 * TW + 4;
+    static constexpr int XS = S == 1 ? TW + 4 : 2 * TW + 4;  // >= XC for both filter sizes
     static constexpr int col_pos(int lc) { return S == 1 ? lc : (lc % 2) * HALF + lc / 2; }
     static constexpr int tap_off(int fh, int fw) { return S == 1 ? fh * XS + fw : fh * XS + (fw == 1 ? HALF : fw / 2); }
-    static_assert(S == 1 || (S == 2 && !DGRAD_), "stride 2: forward only");
+    static_assert(S == 1 || (S == 2 && !DGRAD_ && F == 3), "stride 2: forward only, 3 x 3 only");
+    static_assert(F == 3 || F == 5, "filter size");
     static constexpr int XP = XR * XS;                                  // channel plane stride
     static constexpr int X_SIZE = CI * XP;
-    static constexpr int KC = CI * 9, KH = KC / 2;                      // contraction per chunk, per lane half
-    static constexpr int WSTR = KC + 4;                                 // filter row stride: 12 or 20 mod 32 for CI = 8 / 16
+    static constexpr int KC = CI * NT, KH = KC / 2;                     // contraction per chunk, per lane half
+    static constexpr int WSTR = KC + 4;                                 // filter row stride: 12 mod 32 (3 x 3 and 5 x 5 with CI = 8), 20 (CI = 16)
     static constexpr int W_SIZE = OCT * WSTR;
     static constexpr int SMEM_FLOATS = 2 * (X_SIZE + W_SIZE);
     static_assert(TW == 8 || TW == 16 || TW == 32, "tile width");
@@ -71,6 +74,7 @@ template <class Cfg, bool WVEC>
 __global__ void __launch_bounds__(kThreads, Cfg::OCC) conv3x3_tiled_kernel(TiledArgs a) {
     constexpr int TH = Cfg::TH, TW = Cfg::TW, OCT = Cfg::OCT, CI = Cfg::CI, PB = Cfg::PB, OB = Cfg::OB;
     constexpr int XR = Cfg::XR, XC = Cfg::XC, XS = Cfg::XS, XP = Cfg::XP, KC = Cfg::KC, KH = Cfg::KH, WSTR = Cfg::WSTR;
+    constexpr int F = Cfg::F, NT = Cfg::NT;
     __shared__ __attribute__((aligned(16))) float smem[Cfg::SMEM_FLOATS];
     float(*sX)[Cfg::X_SIZE] = reinterpret_cast<float(*)[Cfg::X_SIZE]>(smem);
     float(*sW)[Cfg::W_SIZE] = reinterpret_cast<float(*)[Cfg::W_SIZE]>(smem + 2 * Cfg::X_SIZE);
@@ -102,7 +106,7 @@ __global__ void __launch_bounds__(kThreads, Cfg::OCC) conv3x3_tiled_kernel(Tiled
     for (int i = 0; i < XNP; ++i) {
         const u32 e = t + i * kThreads;
         const u32 c = e / (XR * XC), lr = (e / XC) % XR, lc = e % XC;
-        const int y = Cfg::S * y0 - 1 + int(lr), x = Cfg::S * x0 - 1 + int(lc);
+        const int y = Cfg::S * y0 - Cfg::PAD + int(lr), x = Cfg::S * x0 - Cfg::PAD + int(lc);
         const bool ok = (XQ % kThreads == 0 || e < XQ) && y >= 0 && y < int(a.IH) && x >= 0 && x < int(a.IW);
         xoff[i] = ok ? (c * IHW + u32(y) * a.IW + u32(x)) * 4u : kNone;
     }
@@ -115,29 +119,29 @@ __global__ void __launch_bounds__(kThreads, Cfg::OCC) conv3x3_tiled_kernel(Tiled
         bool ok = WITEMS % kThreads == 0 || e < WITEMS;
         u32 off;
         if constexpr (Cfg::DGRAD) {
-            const u32 c = e / (OCT * 9), f = e % (OCT * 9);
-            ok = ok && oc0 * 9 + f < a.C_OUT * 9;
-            off = c * a.C_OUT * 9 + f;
+            const u32 c = e / (OCT * NT), f = e % (OCT * NT);
+            ok = ok && oc0 * NT + f < a.C_OUT * NT;
+            off = c * a.C_OUT * NT + f;
         } else if constexpr (WVEC) {
             const u32 j = e / (KC / 4), q = e % (KC / 4);
             ok = ok && oc0 + j < a.C_OUT;
-            off = j * a.C_IN * 9 + 4 * q;
+            off = j * a.C_IN * NT + 4 * q;
         } else {
             const u32 j = e / KC, k = e % KC;
             ok = ok && oc0 + j < a.C_OUT;
-            off = j * a.C_IN * 9 + k;
+            off = j * a.C_IN * NT + k;
         }
         woff[i] = ok ? off * 4u : kNone;
     }
     // whether item e of the filter slice lies inside the tensor's channels in chunk c0 (ragged last chunk)
     auto w_in_chunk = [&](u32 e, u32 c0) -> bool {
-        if constexpr (Cfg::DGRAD) return c0 + e / (OCT * 9) < a.C_IN;
-        else if constexpr (WVEC) return c0 * 9 + 4 * (e % (KC / 4)) < a.C_IN * 9;  // a 16-byte item never straddles the end: C_IN % 4 == 0
-        else return c0 * 9 + e % KC < a.C_IN * 9;
+        if constexpr (Cfg::DGRAD) return c0 + e / (OCT * NT) < a.C_IN;
+        else if constexpr (WVEC) return c0 * NT + 4 * (e % (KC / 4)) < a.C_IN * NT;  // a 16-byte item never straddles the end: C_IN % 4 == 0
+        else return c0 * NT + e % KC < a.C_IN * NT;
     };
     auto fetch = [&](u32 c0) {
         const char *xc = xin + size_t(c0) * IHW * 4;
-        const char *wc = reinterpret_cast<const char *>(Cfg::DGRAD ? a.Wt + (size_t(c0) * a.C_OUT + oc0) * 9 : a.Wt + (size_t(oc0) * a.C_IN + c0) * 9);
+        const char *wc = reinterpret_cast<const char *>(Cfg::DGRAD ? a.Wt + (size_t(c0) * a.C_OUT + oc0) * NT : a.Wt + (size_t(oc0) * a.C_IN + c0) * NT);
 #pragma unroll
         for (int i = 0; i < XNP; ++i) {
             const bool ok = xoff[i] != kNone && c0 + (t + i * kThreads) / (XR * XC) < a.C_IN;
@@ -162,8 +166,8 @@ __global__ void __launch_bounds__(kThreads, Cfg::OCC) conv3x3_tiled_kernel(Tiled
             const bool ok = woff[i] != kNone && w_in_chunk(e, c0);
             if (WITEMS % kThreads == 0 || e < WITEMS) {
                 if constexpr (Cfg::DGRAD) {
-                    const u32 c = e / (OCT * 9), f = e % (OCT * 9);
-                    dw[(f / 9) * WSTR + c * 9 + f % 9] = ok ? wreg[i] : 0.f;
+                    const u32 c = e / (OCT * NT), f = e % (OCT * NT);
+                    dw[(f / NT) * WSTR + c * NT + f % NT] = ok ? wreg[i] : 0.f;
                 } else if constexpr (WVEC) {
                     *reinterpret_cast<v4f *>(dw + (e / (KC / 4)) * WSTR + 4 * (e % (KC / 4))) = ok ? wreg[i] : v4f{0.f, 0.f, 0.f, 0.f};
                 } else {
@@ -207,8 +211,8 @@ __global__ void __launch_bounds__(kThreads, Cfg::OCC) conv3x3_tiled_kernel(Tiled
             for (int o = 0; o < OB; ++o) wv[set][o] = *reinterpret_cast<const v4f *>(wfrag + o * 32 * WSTR + 4 * sq);
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
-                const int s = 4 * sq + e, c = s / 9, tap = s % 9;
-                const int fh = Cfg::DGRAD ? 2 - tap / 3 : tap / 3, fw = Cfg::DGRAD ? 2 - tap % 3 : tap % 3;
+                const int s = 4 * sq + e, c = s / NT, tap = s % NT;
+                const int fh = Cfg::DGRAD ? F - 1 - tap / F : tap / F, fw = Cfg::DGRAD ? F - 1 - tap % F : tap % F;
 #pragma unroll
                 for (int p = 0; p < PB; ++p) xv[set][e][p] = xfrag[c * XP + Cfg::S * p * Cfg::RB * XS + Cfg::tap_off(fh, fw)];
             }
@@ -270,8 +274,8 @@ __global__ void __launch_bounds__(kThreads, Cfg::OCC) conv3x3_tiled_kernel(Tiled
 }
 
 // An item's byte offset inside its image / inside the filter tensor is kept in 32 bits.
-inline bool tiled_fits(u32 C_IN, u32 C_OUT, u32 H, u32 W) {
-    return uint64_t(C_IN) * H * W * 4 <= 0xffffffffull && uint64_t(C_IN) * C_OUT * 36 <= 0xffffffffull;
+inline bool tiled_fits(u32 C_IN, u32 C_OUT, u32 H, u32 W, u32 taps = 9) {
+    return uint64_t(C_IN) * H * W * 4 <= 0xffffffffull && uint64_t(C_IN) * C_OUT * taps * 4 <= 0xffffffffull;
 }
 
 template <class Cfg>
@@ -289,7 +293,7 @@ inline int launch_tiled(const float *Wt, const float *X, float *Y, const float *
     if (tiles > 0x7fffffffull || wgs > 0x7fffffffull) return fail(CRB_EINVAL_SHAPE, "%s: launch grid too large", what);
     a.tiles_total = u32(tiles);
     a.relu = relu;
-    if (!tiled_fits(C_IN, C_OUT, a.IH, a.IW)) return fail(CRB_EINVAL_SHAPE, "%s: image or filter tensor beyond 4 GB", what);
+    if (!tiled_fits(C_IN, C_OUT, a.IH, a.IW, Cfg::NT)) return fail(CRB_EINVAL_SHAPE, "%s: image or filter tensor beyond 4 GB", what);
     if (!Cfg::DGRAD && C_IN % 4 == 0 && reinterpret_cast<uintptr_t>(Wt) % 16 == 0)
         hipLaunchKernelGGL((conv3x3_tiled_kernel<Cfg, !Cfg::DGRAD>), dim3(u32(wgs)), dim3(kThreads), 0, s, a);
     else

@@ -101,6 +101,16 @@ def test_3x3_stride_2_layers_off_the_width_grid(dev, shape):
     run_layer(dev, N, IC, IH, IW, OC, 3, 3, 2, 2, 1, 1, bias=True, seed=sum(shape))
 
 
+# 5x5 / pad 2 / stride 1: the tiled kernel with 25 taps (forward and data gradient), any extent
+FIVE_BY_FIVE = [(4, 16, 28, 28, 32), (2, 3, 32, 32, 6), (3, 20, 9, 14, 50), (2, 64, 12, 12, 64), (1, 8, 5, 3, 9), (2, 33, 17, 40, 31)]
+
+
+@pytest.mark.parametrize("shape", FIVE_BY_FIVE, ids=lambda s: "x".join(map(str, s)))
+def test_5x5_same_padding_layers(dev, shape):
+    N, IC, IH, IW, OC = shape
+    run_layer(dev, N, IC, IH, IW, OC, 5, 5, 1, 1, 2, 2, bias=True, seed=sum(shape))
+
+
 @pytest.mark.parametrize("seed", [41, 42])
 def test_random_3x3_layers_of_any_extent(dev, seed):
     rng = random.Random(seed)

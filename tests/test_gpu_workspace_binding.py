@@ -105,15 +105,16 @@ def test_conv_queries_and_general_path_on_a_bound_workspace(dev):
     for (N, IC, H, OC, F, st, p) in ((128, 16, 32, 16, 3, 1, 1), (128, 16, 32, 32, 3, 2, 1), (64, 204, 32, 48, 1, 1, 0)):
         g = capi.ConvGeom.make(N, IC, H, H, OC, F, F, st, st, p, p)
         assert capi.conv_fwd_workspace_bytes(g) == 0 and capi.conv_dgrad_workspace_bytes(g) == 0
-    # 5x5 filters on 12x12 images, few pixels: the general path cuts the contraction
-    N, IC, H, OC = 2, 64, 12, 48
-    g = capi.ConvGeom.make(N, IC, H, H, OC, 5, 5, 1, 1, 2, 2)
+    # 5x5 filters with pad 1 on 12x12 images (no kernel of their own), few pixels: the general path cuts the contraction
+    N, IC, H, OC = 4, 64, 12, 48
+    g = capi.ConvGeom.make(N, IC, H, H, OC, 5, 5, 1, 1, 1, 1)
+    OH = g.OH
     nf, nd, nw, nb = (capi.conv_fwd_workspace_bytes(g), capi.conv_dgrad_workspace_bytes(g), capi.conv_wgrad_workspace_bytes(g),
-                      capi.conv_bias_grad_workspace_bytes(N, OC, H * H))
+                      capi.conv_bias_grad_workspace_bytes(N, OC, OH * OH))
     assert nf > 0 and nd > 0 and nw > 0 and nb > 0
-    X, W, dY, b = normal(1, N, IC, H, H), he_normal(2, OC, IC, 5, 5), normal(3, N, OC, H, H), normal(4, OC)
+    X, W, dY, b = normal(1, N, IC, H, H), he_normal(2, OC, IC, 5, 5), normal(3, N, OC, OH, OH), normal(4, OC)
     Xd, Wd, dYd, bd = to_dev(X, dev), to_dev(W, dev), to_dev(dY, dev), to_dev(b, dev)
-    Y, dX = torch.empty(N, OC, H, H, device=dev), torch.empty(N, IC, H, H, device=dev)
+    Y, dX = torch.empty(N, OC, OH, OH, device=dev), torch.empty(N, IC, H, H, device=dev)
     dW, dB = torch.zeros(OC, IC, 5, 5, device=dev), torch.zeros(OC, device=dev)
     ws = torch.empty(max(nf, nd, nw, nb) // 4, device=dev)
     torch.cuda.synchronize()
@@ -122,14 +123,14 @@ def test_conv_queries_and_general_path_on_a_bound_workspace(dev):
         capi.conv_fwd(Wd, Xd, Y, bd, g, stream=s)
         capi.conv_dgrad(Wd, dYd, dX, g, stream=s)
         capi.conv_wgrad(dYd, Xd, dW, g, stream=s)  # workspace argument NULL: the bound block serves it
-        capi.conv_bias_grad(dYd, dB, N, OC, H * H, stream=s)
+        capi.conv_bias_grad(dYd, dB, N, OC, OH * OH, stream=s)
         s.synchronize()
     finally:
         capi.bind_workspace(None, stream=s)
-    assert_close(to_np(Y), orc.conv(W, X, b, 1, 1, 2, 2), IC * 25, "conv fwd (bound workspace)")
-    assert_close(to_np(dX), orc.convDerive(W, dY, (H, H), 1, 1, 2, 2), OC * 25, "conv dgrad (bound workspace)")
-    assert_close(to_np(dW), orc.convError(dY, X, np.zeros_like(W), 1, 1, 2, 2), N * H * H, "conv wgrad (bound workspace)")
-    assert_close(to_np(dB), dY.astype(np.float64).sum(axis=(0, 2, 3)), N * H * H, "conv bias grad (bound workspace)")
+    assert_close(to_np(Y), orc.conv(W, X, b, 1, 1, 1, 1), IC * 25, "conv fwd (bound workspace)")
+    assert_close(to_np(dX), orc.convDerive(W, dY, (H, H), 1, 1, 1, 1), OC * 25, "conv dgrad (bound workspace)")
+    assert_close(to_np(dW), orc.convError(dY, X, np.zeros_like(W), 1, 1, 1, 1), N * OH * OH, "conv wgrad (bound workspace)")
+    assert_close(to_np(dB), dY.astype(np.float64).sum(axis=(0, 2, 3)), N * OH * OH, "conv bias grad (bound workspace)")
 
 
 def test_pointwise_wgrad_honours_the_workspace_argument(dev):
