@@ -215,10 +215,10 @@ inline TiledWgradPlan tiled_wgrad_plan(u32 N, u32 IC, u32 OC, u32 H, u32 W) {
     return p;
 }
 
-// The tensors' planes are addressed with 32-bit element offsets inside one image.
+// The tensors' planes are addressed with 32-bit byte offsets inside one image; the tile list is indexed in 32 bits.
 inline bool tiled_wgrad_fits(u32 N, u32 IC, u32 OC, u32 H, u32 W) {
     const uint64_t mx = IC > OC ? IC : OC;
-    return mx * H * W <= 0x7fffffffull && uint64_t(N) * ceil_div(H, 2u) * ceil_div(W, 8u) <= 0x7fffffffull;
+    return mx * H * W * 4 <= 0xffffffffull && uint64_t(N) * ceil_div(H, 2u) * ceil_div(W, 8u) <= 0x7fffffffull;
 }
 
 // The partial results go to ws (plan.workspace_bytes); dW += their sum in fixed order.
