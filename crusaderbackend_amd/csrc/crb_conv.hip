@@ -269,6 +269,17 @@ static int try_direct(const float *Wt, const float *X, float *Y, const float *bi
 // Against the implicit-GEMM engine, forward / data gradient: 64->64 @56x56 batch 32 157 / 168 -> 93 / 99 us,
 // 128->128 @28 146 / 184 -> 93 / 99, 256->256 @14 124 / 143 -> 96 / 97, 512->512 @7 141 / 162 -> 118 / 141,
 // 64->64 @24 batch 64 84 / 99 -> 40 / 40, 32->32 @48 72 / 80 -> 37 / 37.
+// Whether the tiled kernel is the better choice for a 3x3 (or 5x5) pass that reads C_IN channels and writes C_OUT on an
+// H x W pixel grid: not with fewer than 5 contraction channels (a chunk of 8 would be mostly zeros: 3 -> 64 @224 batch 8
+// 82 us against the engine's 43), and not when the grid is a handful of workgroups under a long contraction, which the
+// engine cuts over K (256 -> 256 @14 batch 4: 62 against 31 us). Checked on 35 random shapes (3-256 channels, 7-224 wide, batch 1-64)
+// against the engine: forward -58 ... +2 %, data gradient -72 ... +8 %.
+static bool tiled_pays(u32 N, u32 C_IN, u32 C_OUT, u32 H, u32 W, u32 taps) {
+    if (C_IN < 5) return false;
+    const uint64_t wgs = uint64_t(N) * ceil_div(H, 8u) * ceil_div(W, 16u) * ceil_div(C_OUT, 32u);
+    return wgs >= 192 || (wgs >= 48 && C_IN * taps < 1152);  // (a few dozen workgroups at most: 96 -> 24 @7x7 batch 4 25 against 16 us)
+}
+
 // S = 2 (forward only): H, W are the output's extent, IH, IW the input's. F = 5: 5x5 / pad 2 / stride 1 (16 -> 32 @28x28 batch 64:
 // forward 48 -> 21 us, data gradient 111 -> 39 us against the engine).
 template <bool DG, int S = 1, int F = 3>
@@ -405,10 +416,14 @@ static bool wgrad_tiled(const crb_conv_geom *g, bool run, const float *dY, const
     auto padded = [&](u32 th, u32 tw) { return uint64_t(ceil_div(H, th)) * th * ceil_div(W, tw) * tw; };
     const uint64_t p416 = padded(4, 16), p88 = padded(8, 8), p232 = padded(2, 32);
     const int shape = (p416 <= p88 && p416 <= p232) ? 0 : (p88 <= p232 ? 1 : 2);
+    // blocks of 32 channels at least three quarters full on both sides, and at least four tiles per workgroup (below that the
+    // engine's flat pixel contraction is as fast or faster: 3 -> 64 @224 batch 8 99 against 143 us, 8 -> 8 @100 33 against 43)
+    if (g->IC < 24 || g->OC < 24) return false;
 #define CRB_TW(TH, TW, NOB, NIB)                                                                                        \
     {                                                                                                                   \
         typedef TiledWgradCfg<TH, TW, NOB, NIB> C;                                                                      \
         plan = tiled_wgrad_plan<C>(g->N, g->IC, g->OC, H, W);                                                           \
+        if (uint64_t(plan.tiles_total) * plan.pairs < 1024) return false;                                               \
         if (run) status = launch_tiled_wgrad<C>(dY, X, dW, ws, plan, g->IC, g->OC, H, W, s, "crb_conv_wgrad");          \
         return true;                                                                                                    \
     }
@@ -733,11 +748,11 @@ int crb_conv_fwd(const float *W, const float *X, float *Y, const float *bias_or_
                                                    flags & CRB_FLAG_RELU, s, "crb_conv_fwd", done);
         if (done) return st;
     }
-    if (direct_shape(g, 1) && tiled_fits(g->IC, g->OC, g->IH, g->IW))  // any other extent (and operands that are only 4-byte aligned)
+    if (direct_shape(g, 1) && tiled_fits(g->IC, g->OC, g->IH, g->IW) && tiled_pays(g->N, g->IC, g->OC, g->OH, g->OW, 9))
         return launch_tiled_any<false>(W, X, Y, bias_or_null, g->N, g->IC, g->OC, g->OH, g->OW, flags & CRB_FLAG_RELU, s, "crb_conv_fwd");
-    if (tiled_5x5_shape(g))
+    if (tiled_5x5_shape(g) && tiled_pays(g->N, g->IC, g->OC, g->OH, g->OW, 25))
         return launch_tiled_any<false, 1, 5>(W, X, Y, bias_or_null, g->N, g->IC, g->OC, g->OH, g->OW, flags & CRB_FLAG_RELU, s, "crb_conv_fwd");
-    if (tiled_s2_shape(g))
+    if (tiled_s2_shape(g) && tiled_pays(g->N, g->IC, g->OC, g->OH, g->OW, 9))
         return launch_tiled_any<false, 2>(W, X, Y, bias_or_null, g->N, g->IC, g->OC, g->OH, g->OW, flags & CRB_FLAG_RELU, s, "crb_conv_fwd",
                                           g->IH, g->IW);
     if (K % 4 == 0 && aligned16(W)) {
@@ -772,9 +787,9 @@ int crb_conv_dgrad(const float *W, const float *dY, float *dX, const crb_conv_ge
     }
     if (shortcut_shape(g) && aligned16(dX))
         return launch_sc_dgrad(W, dY, dX, g->N, g->IC, g->OC, g->OH, g->OW, hipStream_t(stream), "crb_conv_dgrad");
-    if (direct_shape(g, 1) && tiled_fits(g->OC, g->IC, g->IH, g->IW))  // any other extent (and operands that are only 4-byte aligned)
+    if (direct_shape(g, 1) && tiled_fits(g->OC, g->IC, g->IH, g->IW) && tiled_pays(g->N, g->OC, g->IC, g->IH, g->IW, 9))
         return launch_tiled_any<true>(W, dY, dX, nullptr, g->N, g->OC, g->IC, g->OH, g->OW, 0, hipStream_t(stream), "crb_conv_dgrad");
-    if (tiled_5x5_shape(g))
+    if (tiled_5x5_shape(g) && tiled_pays(g->N, g->OC, g->IC, g->IH, g->IW, 25))
         return launch_tiled_any<true, 1, 5>(W, dY, dX, nullptr, g->N, g->OC, g->IC, g->OH, g->OW, 0, hipStream_t(stream), "crb_conv_dgrad");
     const u32 FHW = g->FH * g->FW;
     if (g->sH > 1 || g->sW > 1) return dgrad_by_classes(W, dY, dX, g, hipStream_t(stream));
@@ -949,7 +964,9 @@ size_t crb_conv_fwd_workspace_bytes(const crb_conv_geom *g, int operands_aligned
             try_direct<false, 2>(nullptr, nullptr, nullptr, nullptr, g->N, g->IC, g->OC, g->OH, g->OW, g->IH, 0, nullptr, "", done, true);
         if (done) return 0;
     }
-    if ((direct_shape(g, 1) && tiled_fits(g->IC, g->OC, g->IH, g->IW)) || tiled_s2_shape(g) || tiled_5x5_shape(g)) return 0;  // the tiled kernel
+    if ((direct_shape(g, 1) && tiled_fits(g->IC, g->OC, g->IH, g->IW) && tiled_pays(g->N, g->IC, g->OC, g->OH, g->OW, 9)) ||
+        ((tiled_s2_shape(g) || tiled_5x5_shape(g)) && tiled_pays(g->N, g->IC, g->OC, g->OH, g->OW, g->FH * g->FW)))
+        return 0;  // the tiled kernel
     return nchw_scratch_bytes(g->OC, g->N * g->OH * g->OW, g->IC * g->FH * g->FW);
 }
 
@@ -970,7 +987,9 @@ size_t crb_conv_dgrad_workspace_bytes(const crb_conv_geom *g, int operands_align
         if (done) return 0;
     }
     if (shortcut_shape(g) && operands_aligned16) return 0;
-    if ((direct_shape(g, 1) && tiled_fits(g->OC, g->IC, g->IH, g->IW)) || tiled_5x5_shape(g)) return 0;  // the tiled kernel
+    if ((direct_shape(g, 1) && tiled_fits(g->OC, g->IC, g->IH, g->IW) && tiled_pays(g->N, g->OC, g->IC, g->IH, g->IW, 9)) ||
+        (tiled_5x5_shape(g) && tiled_pays(g->N, g->OC, g->IC, g->IH, g->IW, 25)))
+        return 0;  // the tiled kernel
     if (g->sH > 1 || g->sW > 1) return 0;  // one launch per residue class, none of them cut
     return nchw_scratch_bytes(g->IC, g->N * g->IH * g->IW, g->OC * g->FH * g->FW);
 }
