@@ -118,6 +118,19 @@ static int dgrad_by_classes(const float *W, const float *dY, float *dX, const cr
     return CRB_OK;
 }
 
+// The class launches do not cut the contraction, so a class must bring enough tiles of its own: with fewer the one gather
+// over all taps, cut over K, is faster in spite of the zeros it multiplies (64 -> 64 @16x16 7x7 stride 2 batch 4, 8 tiles a
+// class: 360 against 29 us; 256 -> 32 @28 7x7 stride 2 batch 32, 98 tiles: 261 against 411).
+static bool dgrad_classes_pay(const crb_conv_geom *g) {
+    const u32 CH = ceil_div(g->IH, g->sH), CW = ceil_div(g->IW, g->sW);
+    const u32 bm = g->IC <= 32 ? 32 : (g->IC <= 64 ? 64 : 128);
+    const uint64_t tiles = uint64_t(ceil_div(g->IC, bm)) * ceil_div(g->N * CH * CW, 128u);
+    if (tiles < 48) return false;
+    // Each class writes every sW-th float of a row, and there are sH * sW launches: beyond stride 2 that only pays under a
+    // long contraction (256 -> 16 @32 4x4 stride 3 batch 32, K = 256: 107 against 77 us; 16 -> 32 @64 4x4 stride 3, K = 512: 73 against 142).
+    return (g->sH <= 2 && g->sW <= 2) || g->OC * g->FH * g->FW >= 512;
+}
+
 // Scratch bytes run_nchw asks for (0: the contraction is not cut).
 static size_t nchw_scratch_bytes(u32 M, u32 N, u32 K) {
     const u32 bm = M <= 32 ? 32 : (M <= 64 ? 64 : 128);
@@ -277,7 +290,11 @@ static int try_direct(const float *Wt, const float *X, float *Y, const float *bi
 static bool tiled_pays(u32 N, u32 C_IN, u32 C_OUT, u32 H, u32 W, u32 taps) {
     if (C_IN < 5) return false;
     const uint64_t wgs = uint64_t(N) * ceil_div(H, 8u) * ceil_div(W, 16u) * ceil_div(C_OUT, 32u);
-    return wgs >= 192 || (wgs >= 48 && C_IN * taps < 1152);  // (a few dozen workgroups at most: 96 -> 24 @7x7 batch 4 25 against 16 us)
+    // short contractions from a few dozen workgroups on (96 -> 24 @7x7 batch 4, four workgroups: 25 against 16 us); long ones
+    // need two workgroups per CU (256 -> 256 @28 stride 2 batch 16, 256 workgroups: 82 against 69 us; batch 32 -> 512 channels,
+    // 1024 workgroups: 237 against 292)
+    // (with at most 16 output channels the engine's 32-row tile is mostly empty: 128 -> 3 @20 batch 64, 384 workgroups, 50 against 90 us)
+    return C_IN * taps < 1152 ? wgs >= 48 : (wgs >= 512 || (wgs >= 192 && C_OUT <= 16));
 }
 
 // S = 2 (forward only): H, W are the output's extent, IH, IW the input's. F = 5: 5x5 / pad 2 / stride 1 (16 -> 32 @28x28 batch 64:
@@ -792,7 +809,7 @@ int crb_conv_dgrad(const float *W, const float *dY, float *dX, const crb_conv_ge
     if (tiled_5x5_shape(g) && tiled_pays(g->N, g->OC, g->IC, g->IH, g->IW, 25))
         return launch_tiled_any<true, 1, 5>(W, dY, dX, nullptr, g->N, g->OC, g->IC, g->OH, g->OW, 0, hipStream_t(stream), "crb_conv_dgrad");
     const u32 FHW = g->FH * g->FW;
-    if (g->sH > 1 || g->sW > 1) return dgrad_by_classes(W, dY, dX, g, hipStream_t(stream));
+    if ((g->sH > 1 || g->sW > 1) && dgrad_classes_pay(g)) return dgrad_by_classes(W, dY, dX, g, hipStream_t(stream));
     const u32 M = g->IC, N = g->N * g->IH * g->IW, K = g->OC * FHW;
     SepK a{W, g->IC, FHW, g->IC * FHW, 1, FastDiv(FHW)};
     DgradGather b;
@@ -990,7 +1007,7 @@ size_t crb_conv_dgrad_workspace_bytes(const crb_conv_geom *g, int operands_align
     if ((direct_shape(g, 1) && tiled_fits(g->OC, g->IC, g->IH, g->IW) && tiled_pays(g->N, g->OC, g->IC, g->IH, g->IW, 9)) ||
         (tiled_5x5_shape(g) && tiled_pays(g->N, g->OC, g->IC, g->IH, g->IW, 25)))
         return 0;  // the tiled kernel
-    if (g->sH > 1 || g->sW > 1) return 0;  // one launch per residue class, none of them cut
+    if ((g->sH > 1 || g->sW > 1) && dgrad_classes_pay(g)) return 0;  // one launch per residue class, none of them cut
     return nchw_scratch_bytes(g->IC, g->N * g->IH * g->IW, g->OC * g->FH * g->FW);
 }
 
