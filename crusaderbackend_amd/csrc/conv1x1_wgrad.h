@@ -126,14 +126,26 @@ __global__ void __launch_bounds__(kThreads, kPwOcc) pw_wgrad_kernel(PwWgradArgs 
     float *out = a.out + size_t(z) * a.OC * a.IC * (a.accumulate ? 0 : 1);
     const u32 ic = ib * 16 + li;
     if (ic >= a.IC) return;
+    // dW's old values are requested together, the stores follow (a read in front of every store would make each store wait for
+    // the one before it)
+    float old[NOB][4];
 #pragma unroll
     for (int o = 0; o < NOB; ++o)
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
             const u32 oc = o * 16 + 4 * kq + r;
-            if (oc >= a.OC) continue;
-            float *dst = out + size_t(oc) * a.IC + ic;
-            *dst = a.accumulate ? *dst + acc[o][r] : acc[o][r];
+            old[o][r] = (a.accumulate && oc < a.OC) ? out[size_t(oc) * a.IC + ic] : 0.f;
+        }
+#pragma unroll
+    for (int o = 0; o < NOB; ++o)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) asm volatile("" : "+v"(old[o][r]));
+#pragma unroll
+    for (int o = 0; o < NOB; ++o)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const u32 oc = o * 16 + 4 * kq + r;
+            if (oc < a.OC) out[size_t(oc) * a.IC + ic] = old[o][r] + acc[o][r];
         }
 }
 

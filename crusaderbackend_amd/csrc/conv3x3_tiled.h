@@ -64,9 +64,11 @@ struct TiledArgs {
     float *Y;           // output of this pass (forward: Y, data gradient: dX), N x C_OUT x H x W
     const float *bias;  // per output channel or nullptr
     u32 C_IN, C_OUT, H, W;  // H, W: extent of the output (the pixel grid)
-    u32 IH, IW;             // extent of the staged tensor (H, W at stride 1)
+    u32 IH, IW;             // extent of the staged tensor
     u32 tiles_x, tiles_per_img, oc_tiles, tiles_total;  // tiles_total = N * tiles_per_img
     u32 relu;
+    u32 pad;  // the window of pixel (y, x) starts at staged (S y - pad, S x - pad): the layer's padding for the forward pass,
+              // F - 1 - padding for the data gradient
 };
 
 // WVEC (forward only): filter rows are staged with 16-byte loads (C_IN % 4 == 0 and a 16-byte aligned tensor).
@@ -106,7 +108,7 @@ __global__ void __launch_bounds__(kThreads, Cfg::OCC) conv3x3_tiled_kernel(Tiled
     for (int i = 0; i < XNP; ++i) {
         const u32 e = t + i * kThreads;
         const u32 c = e / (XR * XC), lr = (e / XC) % XR, lc = e % XC;
-        const int y = Cfg::S * y0 - Cfg::PAD + int(lr), x = Cfg::S * x0 - Cfg::PAD + int(lc);
+        const int y = Cfg::S * y0 - int(a.pad) + int(lr), x = Cfg::S * x0 - int(a.pad) + int(lc);
         const bool ok = (XQ % kThreads == 0 || e < XQ) && y >= 0 && y < int(a.IH) && x >= 0 && x < int(a.IW);
         xoff[i] = ok ? (c * IHW + u32(y) * a.IW + u32(x)) * 4u : kNone;
     }
@@ -257,6 +259,9 @@ __global__ void __launch_bounds__(kThreads, Cfg::OCC) conv3x3_tiled_kernel(Tiled
             const u32 oc = ocb + 8 * (r / 4) + (r % 4);
             bv[r] = (a.bias && oc < a.C_OUT) ? a.bias[oc] : 0.f;  // requested together, ahead of the stores
         }
+        // ... and awaited here: a wait for them further down would also wait for every store issued before it
+#pragma unroll
+        for (int r = 0; r < 16; ++r) asm volatile("" : "+v"(bv[r]));
 #pragma unroll
         for (int p = 0; p < PB; ++p) {
             const int y = y0 + prow + p * Cfg::RB, x = x0 + pcol;
@@ -280,11 +285,12 @@ inline bool tiled_fits(u32 C_IN, u32 C_OUT, u32 H, u32 W, u32 taps = 9) {
 
 template <class Cfg>
 inline int launch_tiled(const float *Wt, const float *X, float *Y, const float *bias, u32 N, u32 C_IN, u32 C_OUT, u32 H, u32 W, u32 relu,
-                        hipStream_t s, const char *what, u32 IH = 0, u32 IW = 0) {
+                        hipStream_t s, const char *what, u32 IH = 0, u32 IW = 0, int pad = -1) {
     TiledArgs a;
     a.Wt = Wt, a.X = X, a.Y = Y, a.bias = bias;
     a.C_IN = C_IN, a.C_OUT = C_OUT, a.H = H, a.W = W;
     a.IH = IH ? IH : H, a.IW = IW ? IW : W;
+    a.pad = pad < 0 ? u32(Cfg::PAD) : u32(pad);
     a.tiles_x = ceil_div(W, u32(Cfg::TW));
     a.tiles_per_img = a.tiles_x * ceil_div(H, u32(Cfg::TH));
     a.oc_tiles = ceil_div(C_OUT, u32(Cfg::OCT));

@@ -1,5 +1,5 @@
-// Weight gradient of a 3x3 / pad 1 / stride 1 convolution for gfx950 on images of ANY extent:
-// dW[oc][ic][fh][fw] = sum over (n, y, x) of dY[n][oc][y][x] * X[n][ic][y + fh - 1][x + fw - 1].
+// Weight gradient of a 3x3 / stride 1 convolution (padding p = 0, 1 or 2 on both axes) for gfx950 on images of ANY extent:
+// dW[oc][ic][fh][fw] = sum over (n, y, x) of dY[n][oc][y][x] * X[n][ic][y + fh - p][x + fw - p].
 //
 // For each of the nine taps this is an (OC x IC) product whose contraction index is the pixel. A 256-thread workgroup owns
 // a block of 32 NOB output channels x 32 NIB input channels for all nine taps and a slice z of the (image, TH x TW pixel
@@ -10,8 +10,8 @@
 // each writes a partial result of its own. Partial results [z * PS + part][OC][IC][9] are summed in fixed order by the
 // split reduction: bit-reproducible.
 //
-// LDS is single-buffered (two workgroups per CU cover each other's staging); plane strides are odd, so the 32 lanes of a
-// fragment read (32 planes, one float each) land on 32 different banks.
+// LDS holds two tiles: the next one is requested before the current one is multiplied and stored behind it. Plane strides are
+// odd, so the 32 lanes of a fragment read (32 planes, one float each) land on 32 different banks.
 //
 // v_mfma_f32_32x32x2_f32 (wave64, lane l): A[i = l%32][k = l/32] = dY[oc = i][pixel], B[k = l/32][j = l%32] = X[pixel + tap][ic = j],
 // accumulator register r = dW[oc = 8*(r/4) + 4*(l/32) + r%4][ic = l%32]. Within a group of 8 pixels (one image row of the
@@ -40,9 +40,10 @@ struct TiledWgradCfg {
 
 struct TiledWgradArgs {
     const float *dY;  // N x OC x H x W
-    const float *X;   // N x IC x H x W
+    const float *X;   // N x IC x XH x XW
     float *out;       // partial results [z * PS + part][OC][IC][9]
-    u32 OC, IC, H, W;
+    u32 OC, IC, H, W;  // H, W: extent of dY (the pixel grid)
+    u32 XH, XW, pad;   // extent of X; the window of dY pixel (y, x) starts at X (y - pad, x - pad)
     u32 tiles_x, tiles_per_img, tiles_total;
     u32 ic_tiles, pairs, splits;
 };
@@ -65,7 +66,7 @@ __global__ void __launch_bounds__(Cfg::NT, 1) wgrad3x3_tiled_kernel(TiledWgradAr
         pair = bid % a.pairs, z = bid / a.pairs;
     }
     const u32 oc0 = (pair / a.ic_tiles) * OCT, ic0 = (pair % a.ic_tiles) * ICT;
-    const u32 HW = a.H * a.W;
+    const u32 HW = a.H * a.W, XHW = a.XH * a.XW;
     // slice z takes tiles [z T / splits, (z + 1) T / splits): sizes differ by at most one
     const u32 t_begin = u32(uint64_t(z) * a.tiles_total / a.splits), t_end = u32(uint64_t(z + 1) * a.tiles_total / a.splits);
 
@@ -96,7 +97,7 @@ __global__ void __launch_bounds__(Cfg::NT, 1) wgrad3x3_tiled_kernel(TiledWgradAr
         const int y0 = int(tl / a.tiles_x) * TH, x0 = int(tl % a.tiles_x) * TW;
         // uniform bases, 32-bit byte offsets per item
         const char *dyn = reinterpret_cast<const char *>(a.dY + (size_t(n) * a.OC + oc0) * HW);
-        const char *xn = reinterpret_cast<const char *>(a.X + (size_t(n) * a.IC + ic0) * HW);
+        const char *xn = reinterpret_cast<const char *>(a.X + (size_t(n) * a.IC + ic0) * XHW);
         yok = xok = 0;
 #pragma unroll
         for (int i = 0; i < YNP; ++i) {
@@ -109,10 +110,10 @@ __global__ void __launch_bounds__(Cfg::NT, 1) wgrad3x3_tiled_kernel(TiledWgradAr
 #pragma unroll
         for (int i = 0; i < XNP; ++i) {
             const u32 e = t + i * NT, j = e / (XR * XC), lr = (e / XC) % XR, lc = e % XC;
-            const int y = y0 - 1 + int(lr), x = x0 - 1 + int(lc);
-            const bool ok = (XQ % NT == 0 || e < XQ) && ic0 + j < a.IC && y >= 0 && y < int(a.H) && x >= 0 && x < int(a.W);
+            const int y = y0 - int(a.pad) + int(lr), x = x0 - int(a.pad) + int(lc);
+            const bool ok = (XQ % NT == 0 || e < XQ) && ic0 + j < a.IC && y >= 0 && y < int(a.XH) && x >= 0 && x < int(a.XW);
             xok |= ok ? (1u << i) : 0u;
-            xreg[i] = *reinterpret_cast<const float *>(xn + (ok ? (j * HW + u32(y) * a.W + u32(x)) * 4u : 0u));
+            xreg[i] = *reinterpret_cast<const float *>(xn + (ok ? (j * XHW + u32(y) * a.XW + u32(x)) * 4u : 0u));
         }
     };
     constexpr int NITEM = YNP + XNP;
@@ -224,10 +225,11 @@ inline bool tiled_wgrad_fits(u32 N, u32 IC, u32 OC, u32 H, u32 W) {
 // The partial results go to ws (plan.workspace_bytes); dW += their sum in fixed order.
 template <class Cfg>
 inline int launch_tiled_wgrad(const float *dY, const float *X, float *dW, float *ws, const TiledWgradPlan &p, u32 IC, u32 OC, u32 H, u32 W,
-                              hipStream_t s, const char *what) {
+                              u32 XH, u32 XW, u32 pad, hipStream_t s, const char *what) {
     TiledWgradArgs a;
     a.dY = dY, a.X = X, a.out = ws;
     a.OC = OC, a.IC = IC, a.H = H, a.W = W;
+    a.XH = XH, a.XW = XW, a.pad = pad;
     a.tiles_x = p.tiles_x, a.tiles_per_img = p.tiles_per_img, a.tiles_total = p.tiles_total;
     a.ic_tiles = p.ic_tiles, a.pairs = p.pairs, a.splits = p.splits;
     const uint64_t wgs = p.splits >= kXcds ? uint64_t(ceil_div(p.splits, kXcds)) * kXcds * p.pairs : uint64_t(p.splits) * p.pairs;

@@ -310,14 +310,30 @@ __device__ __forceinline__ void wgrad3x3_body(const WgradArgs &a, const u32 bid,
         }
         return;
     }
+    // (dW's old values are requested together and the stores follow: a read in front of every store would make each store wait
+    // for the one before it)
+    constexpr int NE = (2304 + NT - 1) / NT;
+    float *dst[NE];
+    float old[NE];
 #pragma unroll
-    for (int i = 0; i < (2304 + NT - 1) / NT; ++i) {
-        const u32 e = t + i * NT;             // e = oc*144 + ic*9 + tap
-        if (2304 % NT != 0 && e >= 2304u) continue;
+    for (int i = 0; i < NE; ++i) {
+        const u32 e = t + i * NT;                // e = oc*144 + ic*9 + tap
         const u32 oc = e / 144, rest = e % 144;  // rest = ic*9 + tap: contiguous in dW for one oc
-        if (ob * 16 + oc >= a.OC || ib * 16 + rest / 9 >= a.IC) continue;
-        float *dst = out + (size_t(ob * 16 + oc) * a.IC + ib * 16) * 9 + rest;
-        *dst = a.accumulate ? *dst + tr[e] : tr[e];
+        const bool ok = (2304 % NT == 0 || e < 2304u) && ob * 16 + oc < a.OC && ib * 16 + rest / 9 < a.IC;
+        dst[i] = ok ? out + (size_t(ob * 16 + oc) * a.IC + ib * 16) * 9 + rest : nullptr;
+        old[i] = 0.f;
+    }
+    if (a.accumulate) {
+#pragma unroll
+        for (int i = 0; i < NE; ++i)
+            if (dst[i]) old[i] = *dst[i];
+#pragma unroll
+        for (int i = 0; i < NE; ++i) asm volatile("" : "+v"(old[i]));
+    }
+#pragma unroll
+    for (int i = 0; i < NE; ++i) {
+        const u32 e = t + i * NT;
+        if (dst[i]) *dst[i] = old[i] + tr[(2304 % NT == 0 || e < 2304u) ? e : 0];
     }
 }
 

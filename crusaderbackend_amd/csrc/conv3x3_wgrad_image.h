@@ -141,14 +141,22 @@ __global__ void __launch_bounds__(kThreads, 2) wgrad3x3_image_kernel(ImgWgradArg
     float *out = a.out + size_t(z) * a.OC * K9 * (a.accumulate ? 0 : 1);
     // thread t: register r = t / 64 of lane l = t % 64: output channel 4 (l / 16) + r, column 16 b + l % 16
     const u32 r = t >> 6, l = t & 63;
+    // dW's old values are requested together, the stores follow (a read in front of every store would make each store wait for
+    // the one before it)
+    float old[NB];
+#pragma unroll
+    for (int b = 0; b < NB; ++b) {
+        const u32 oc = ob * 16 + 4 * (l >> 4) + r, n = b * 16 + (l & 15);
+        old[b] = (a.accumulate && oc < a.OC && n < K9) ? out[size_t(oc) * K9 + n] : 0.f;
+    }
+#pragma unroll
+    for (int b = 0; b < NB; ++b) asm volatile("" : "+v"(old[b]));
 #pragma unroll
     for (int b = 0; b < NB; ++b) {
         const u32 e = b * 256 + l * 4 + r;
         const float v = ((red[e] + red[NB * 256 + e]) + red[2 * NB * 256 + e]) + red[3 * NB * 256 + e];
         const u32 oc = ob * 16 + 4 * (l >> 4) + r, n = b * 16 + (l & 15);
-        if (oc >= a.OC || n >= K9) continue;
-        float *dst = out + size_t(oc) * K9 + n;
-        *dst = a.accumulate ? *dst + v : v;
+        if (oc < a.OC && n < K9) out[size_t(oc) * K9 + n] = old[b] + v;
     }
 }
 

@@ -289,6 +289,17 @@ static int try_direct(const float *Wt, const float *X, float *Y, const float *bi
 // against the engine: forward -58 ... +2 %, data gradient -72 ... +8 %.
 static bool tiled_pays(u32 N, u32 C_IN, u32 C_OUT, u32 H, u32 W, u32 taps) {
     if (C_IN < 5) return false;
+    // a contraction under 64 long into more than 16 output channels on 8192 pixels or more: the engine's 32-row tiles are full,
+    // its flat pixel list wastes nothing and fills the chip (6 -> 128 @10x10 batch 128: 16.6 against 14.1 us, 6 -> 64 @30x30
+    // batch 64: 18.8 against 15.9; but 6 -> 256 @64x64 batch 1: 8.0 against 13.5)
+    if (C_IN * taps < 64 && C_OUT > 16 && uint64_t(N) * H * W >= 8192) return false;
+    // a contraction from 2304 on a grid the tiles fill less than 60 % (256 -> 256 @18x18 batch 16, 51 % full: 132 against 105 us;
+    // shorter contractions still gain at that fill: 64 -> 256 @18x18 batch 16 40 against 46, 128 -> 256 @12x12 batch 32 52 against 60)
+    if (C_IN * taps >= 2304) {
+        auto padded = [&](u32 th, u32 tw) { return uint64_t(ceil_div(H, th)) * th * ceil_div(W, tw) * tw; };
+        const uint64_t best = (H <= 8 && W <= 8) ? 64 : std::min(padded(8, 16), std::min(padded(16, 8), padded(4, 32)));
+        if (5 * uint64_t(H) * W < 3 * best) return false;
+    }
     const uint64_t wgs = uint64_t(N) * ceil_div(H, 8u) * ceil_div(W, 16u) * ceil_div(C_OUT, 32u);
     // short contractions from a few dozen workgroups on (96 -> 24 @7x7 batch 4, four workgroups: 25 against 16 us); long ones
     // need two workgroups per CU (256 -> 256 @28 stride 2 batch 16, 256 workgroups: 82 against 69 us; batch 32 -> 512 channels,
@@ -301,9 +312,9 @@ static bool tiled_pays(u32 N, u32 C_IN, u32 C_OUT, u32 H, u32 W, u32 taps) {
 // forward 48 -> 21 us, data gradient 111 -> 39 us against the engine).
 template <bool DG, int S = 1, int F = 3>
 static int launch_tiled_any(const float *Wt, const float *X, float *Y, const float *bias, u32 N, u32 C_IN, u32 C_OUT, u32 H, u32 W, u32 relu,
-                            hipStream_t s, const char *what, u32 IH = 0, u32 IW = 0) {
+                            hipStream_t s, const char *what, u32 IH = 0, u32 IW = 0, int pad = -1) {
 #define CRB_TILED(TH, TW, OCT, WP) \
-    return launch_tiled<TiledCfg<TH, TW, OCT, WP, 8, DG, 2, S, F>>(Wt, X, Y, bias, N, C_IN, C_OUT, H, W, relu, s, what, IH, IW)
+    return launch_tiled<TiledCfg<TH, TW, OCT, WP, 8, DG, 2, S, F>>(Wt, X, Y, bias, N, C_IN, C_OUT, H, W, relu, s, what, IH, IW, pad)
     if (H <= 8 && W <= 8) CRB_TILED(8, 8, 64, 2);
     auto padded = [&](u32 th, u32 tw) { return uint64_t(ceil_div(H, th)) * th * ceil_div(W, tw) * tw; };
     const uint64_t p816 = padded(8, 16), p168 = padded(16, 8), p432 = padded(4, 32);
@@ -405,10 +416,11 @@ static bool tiled_s2_shape(const crb_conv_geom *g) {
            uint64_t(g->IC) * g->IH * g->IW * 4 <= 0xffffffffull && uint64_t(g->IC) * g->OC * 36 <= 0xffffffffull;
 }
 
-// 5x5 / pad 2 / stride 1 (output = input extent) whose images the tiled kernel can address
-static bool tiled_5x5_shape(const crb_conv_geom *g) {
-    return g->FH == 5 && g->FW == 5 && g->sH == 1 && g->sW == 1 && g->pH == 2 && g->pW == 2 && g->IH == g->OH && g->IW == g->OW &&
-           tiled_fits(g->IC > g->OC ? g->IC : g->OC, g->IC > g->OC ? g->OC : g->IC, g->IH, g->IW, 25);
+// F x F (3 or 5), stride 1, the same padding 0 ... F - 1 on both axes, and tensors the tiled kernel can address
+static bool tiled_s1_shape(const crb_conv_geom *g, u32 F) {
+    return g->FH == F && g->FW == F && g->sH == 1 && g->sW == 1 && g->pH == g->pW && g->pH <= F - 1 &&
+           tiled_fits(g->IC > g->OC ? g->IC : g->OC, g->IC > g->OC ? g->OC : g->IC, g->IH > g->OH ? g->IH : g->OH,
+                      g->IW > g->OW ? g->IW : g->OW, F * F);
 }
 
 // 1x1, stride 2, no padding, even input extents, at most 64 channels on either side (conv1x1_s2.h)
@@ -422,17 +434,21 @@ static bool tiny2x2_shape(const crb_conv_geom *g) {
     return direct_shape(g, 1) && g->IH == 2 && g->IW == 2 && uint64_t(g->OC) * g->IC * 16 <= 0x7fffffffull;
 }
 
-// Weight gradient of 3x3 / pad 1 / stride 1 layers on any extent (conv3x3_tiled_wgrad.h), <TH, TW, NOB, NIB, OCC>: 64-pixel tiles of
+// Weight gradient of 3x3 / stride 1 layers with padding 0 ... 2 on any extent (conv3x3_tiled_wgrad.h), <TH, TW, NOB, NIB, OCC>: 64-pixel tiles of
 // the shape that pads the image least, blocks of 64 x 64 channels (32 on a side with at most 32 channels).
 // `run` = false only computes the plan (workspace size).
 static bool wgrad_tiled(const crb_conv_geom *g, bool run, const float *dY, const float *X, float *dW, float *ws, hipStream_t s,
                         TiledWgradPlan &plan, int &status) {
     // (images below 12 x 12 pad their 8 x 8 tiles too much: the engine's flat pixel contraction is as fast or faster there)
-    if (!direct_shape(g, 1) || !tiled_wgrad_fits(g->N, g->IC, g->OC, g->OH, g->OW) || g->OH * g->OW < 144) return false;
+    const bool shape_ok = g->FH == 3 && g->FW == 3 && g->sH == 1 && g->sW == 1 && g->pH == g->pW && g->pH <= 2;
+    if (!shape_ok || !tiled_wgrad_fits(g->N, g->IC, g->OC, std::max(g->IH, g->OH), std::max(g->IW, g->OW)) || g->OH * g->OW < 144)
+        return false;
     const u32 H = g->OH, W = g->OW;
     auto padded = [&](u32 th, u32 tw) { return uint64_t(ceil_div(H, th)) * th * ceil_div(W, tw) * tw; };
     const uint64_t p416 = padded(4, 16), p88 = padded(8, 8), p232 = padded(2, 32);
     const int shape = (p416 <= p88 && p416 <= p232) ? 0 : (p88 <= p232 ? 1 : 2);
+    // tiles at least two thirds full (256 -> 256 @18x18 batch 32, 56 % full: 208 against the engine's 155 us)
+    if (3 * uint64_t(H) * W < 2 * std::min(p416, std::min(p88, p232))) return false;
     // blocks of 32 channels at least three quarters full on both sides, and at least four tiles per workgroup (below that the
     // engine's flat pixel contraction is as fast or faster: 3 -> 64 @224 batch 8 99 against 143 us, 8 -> 8 @100 33 against 43)
     if (g->IC < 24 || g->OC < 24) return false;
@@ -441,7 +457,7 @@ static bool wgrad_tiled(const crb_conv_geom *g, bool run, const float *dY, const
         typedef TiledWgradCfg<TH, TW, NOB, NIB> C;                                                                      \
         plan = tiled_wgrad_plan<C>(g->N, g->IC, g->OC, H, W);                                                           \
         if (uint64_t(plan.tiles_total) * plan.pairs < 1024) return false;                                               \
-        if (run) status = launch_tiled_wgrad<C>(dY, X, dW, ws, plan, g->IC, g->OC, H, W, s, "crb_conv_wgrad");          \
+        if (run) status = launch_tiled_wgrad<C>(dY, X, dW, ws, plan, g->IC, g->OC, H, W, g->IH, g->IW, g->pH, s, "crb_conv_wgrad"); \
         return true;                                                                                                    \
     }
 #define CRB_TW_SHAPES(NOB, NIB)            \
@@ -765,10 +781,13 @@ int crb_conv_fwd(const float *W, const float *X, float *Y, const float *bias_or_
                                                    flags & CRB_FLAG_RELU, s, "crb_conv_fwd", done);
         if (done) return st;
     }
-    if (direct_shape(g, 1) && tiled_fits(g->IC, g->OC, g->IH, g->IW) && tiled_pays(g->N, g->IC, g->OC, g->OH, g->OW, 9))
-        return launch_tiled_any<false>(W, X, Y, bias_or_null, g->N, g->IC, g->OC, g->OH, g->OW, flags & CRB_FLAG_RELU, s, "crb_conv_fwd");
-    if (tiled_5x5_shape(g) && tiled_pays(g->N, g->IC, g->OC, g->OH, g->OW, 25))
-        return launch_tiled_any<false, 1, 5>(W, X, Y, bias_or_null, g->N, g->IC, g->OC, g->OH, g->OW, flags & CRB_FLAG_RELU, s, "crb_conv_fwd");
+    // any other extent, padding 0 ... F - 1 (and operands that are only 4-byte aligned)
+    if (tiled_s1_shape(g, 3) && tiled_pays(g->N, g->IC, g->OC, g->OH, g->OW, 9))
+        return launch_tiled_any<false>(W, X, Y, bias_or_null, g->N, g->IC, g->OC, g->OH, g->OW, flags & CRB_FLAG_RELU, s, "crb_conv_fwd",
+                                       g->IH, g->IW, int(g->pH));
+    if (tiled_s1_shape(g, 5) && tiled_pays(g->N, g->IC, g->OC, g->OH, g->OW, 25))
+        return launch_tiled_any<false, 1, 5>(W, X, Y, bias_or_null, g->N, g->IC, g->OC, g->OH, g->OW, flags & CRB_FLAG_RELU, s, "crb_conv_fwd",
+                                             g->IH, g->IW, int(g->pH));
     if (tiled_s2_shape(g) && tiled_pays(g->N, g->IC, g->OC, g->OH, g->OW, 9))
         return launch_tiled_any<false, 2>(W, X, Y, bias_or_null, g->N, g->IC, g->OC, g->OH, g->OW, flags & CRB_FLAG_RELU, s, "crb_conv_fwd",
                                           g->IH, g->IW);
@@ -804,10 +823,13 @@ int crb_conv_dgrad(const float *W, const float *dY, float *dX, const crb_conv_ge
     }
     if (shortcut_shape(g) && aligned16(dX))
         return launch_sc_dgrad(W, dY, dX, g->N, g->IC, g->OC, g->OH, g->OW, hipStream_t(stream), "crb_conv_dgrad");
-    if (direct_shape(g, 1) && tiled_fits(g->OC, g->IC, g->IH, g->IW) && tiled_pays(g->N, g->OC, g->IC, g->IH, g->IW, 9))
-        return launch_tiled_any<true>(W, dY, dX, nullptr, g->N, g->OC, g->IC, g->OH, g->OW, 0, hipStream_t(stream), "crb_conv_dgrad");
-    if (tiled_5x5_shape(g) && tiled_pays(g->N, g->OC, g->IC, g->IH, g->IW, 25))
-        return launch_tiled_any<true, 1, 5>(W, dY, dX, nullptr, g->N, g->OC, g->IC, g->OH, g->OW, 0, hipStream_t(stream), "crb_conv_dgrad");
+    // any other extent, padding 0 ... F - 1 (and operands that are only 4-byte aligned): the pixel grid is dX, the staged tensor dY
+    if (tiled_s1_shape(g, 3) && tiled_pays(g->N, g->OC, g->IC, g->IH, g->IW, 9))
+        return launch_tiled_any<true>(W, dY, dX, nullptr, g->N, g->OC, g->IC, g->IH, g->IW, 0, hipStream_t(stream), "crb_conv_dgrad", g->OH,
+                                      g->OW, int(2 - g->pH));
+    if (tiled_s1_shape(g, 5) && tiled_pays(g->N, g->OC, g->IC, g->IH, g->IW, 25))
+        return launch_tiled_any<true, 1, 5>(W, dY, dX, nullptr, g->N, g->OC, g->IC, g->IH, g->IW, 0, hipStream_t(stream), "crb_conv_dgrad",
+                                            g->OH, g->OW, int(4 - g->pH));
     const u32 FHW = g->FH * g->FW;
     if ((g->sH > 1 || g->sW > 1) && dgrad_classes_pay(g)) return dgrad_by_classes(W, dY, dX, g, hipStream_t(stream));
     const u32 M = g->IC, N = g->N * g->IH * g->IW, K = g->OC * FHW;
@@ -981,8 +1003,7 @@ size_t crb_conv_fwd_workspace_bytes(const crb_conv_geom *g, int operands_aligned
             try_direct<false, 2>(nullptr, nullptr, nullptr, nullptr, g->N, g->IC, g->OC, g->OH, g->OW, g->IH, 0, nullptr, "", done, true);
         if (done) return 0;
     }
-    if ((direct_shape(g, 1) && tiled_fits(g->IC, g->OC, g->IH, g->IW) && tiled_pays(g->N, g->IC, g->OC, g->OH, g->OW, 9)) ||
-        ((tiled_s2_shape(g) || tiled_5x5_shape(g)) && tiled_pays(g->N, g->IC, g->OC, g->OH, g->OW, g->FH * g->FW)))
+    if (((tiled_s1_shape(g, 3) || tiled_s1_shape(g, 5) || tiled_s2_shape(g)) && tiled_pays(g->N, g->IC, g->OC, g->OH, g->OW, g->FH * g->FW)))
         return 0;  // the tiled kernel
     return nchw_scratch_bytes(g->OC, g->N * g->OH * g->OW, g->IC * g->FH * g->FW);
 }
@@ -1004,8 +1025,7 @@ size_t crb_conv_dgrad_workspace_bytes(const crb_conv_geom *g, int operands_align
         if (done) return 0;
     }
     if (shortcut_shape(g) && operands_aligned16) return 0;
-    if ((direct_shape(g, 1) && tiled_fits(g->OC, g->IC, g->IH, g->IW) && tiled_pays(g->N, g->OC, g->IC, g->IH, g->IW, 9)) ||
-        (tiled_5x5_shape(g) && tiled_pays(g->N, g->OC, g->IC, g->IH, g->IW, 25)))
+    if ((tiled_s1_shape(g, 3) || tiled_s1_shape(g, 5)) && tiled_pays(g->N, g->OC, g->IC, g->IH, g->IW, g->FH * g->FW))
         return 0;  // the tiled kernel
     if ((g->sH > 1 || g->sW > 1) && dgrad_classes_pay(g)) return 0;  // one launch per residue class, none of them cut
     return nchw_scratch_bytes(g->IC, g->N * g->IH * g->IW, g->OC * g->FH * g->FW);

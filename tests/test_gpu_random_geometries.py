@@ -111,6 +111,22 @@ def test_5x5_same_padding_layers(dev, shape):
     run_layer(dev, N, IC, IH, IW, OC, 5, 5, 1, 1, 2, 2, bias=True, seed=sum(shape))
 
 
+# 3x3 and 5x5 at stride 1 with paddings other than "same" (0 ... F - 1): output and input extents differ, the tiled kernels' window
+# origin is an argument (forward and data gradient for both filter sizes, weight gradient for 3x3)
+OTHER_PADDINGS = [
+    # N, IC, IH, IW, OC, F, pad
+    (4, 16, 28, 28, 32, 3, 0), (2, 64, 14, 30, 64, 3, 2), (3, 9, 11, 7, 20, 3, 0), (8, 32, 32, 32, 32, 3, 2), (2, 24, 3, 3, 8, 3, 0),
+    (32, 96, 30, 30, 72, 3, 0), (96, 40, 20, 20, 48, 3, 2),  # the tiled weight gradient: enough tiles and channel blocks to be chosen
+    (4, 6, 14, 14, 16, 5, 0), (2, 16, 28, 28, 32, 5, 1), (2, 32, 12, 20, 24, 5, 3), (1, 8, 6, 5, 40, 5, 4), (8, 20, 24, 24, 50, 5, 0),
+]
+
+
+@pytest.mark.parametrize("shape", OTHER_PADDINGS, ids=lambda s: "x".join(map(str, s)))
+def test_3x3_and_5x5_layers_with_other_paddings(dev, shape):
+    N, IC, IH, IW, OC, F, pad = shape
+    run_layer(dev, N, IC, IH, IW, OC, F, F, 1, 1, pad, pad, bias=True, seed=sum(shape))
+
+
 @pytest.mark.parametrize("seed", [41, 42])
 def test_random_3x3_layers_of_any_extent(dev, seed):
     rng = random.Random(seed)
