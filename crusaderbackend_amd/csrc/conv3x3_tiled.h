@@ -20,6 +20,9 @@
 //
 // Data gradient: the same computation on dY with the filter's channel roles swapped and its taps mirrored
 // (dX(y, x) = sum dY(y + 1 - fh, x + 1 - fw) W[oc][ic][fh][fw]): only the filter staging and the immediates differ.
+//
+// The same kernel also serves 5x5 filters, any padding 0 ... F - 1 at stride 1 (the window origin is an argument), the 3x3
+// forward pass at stride 2, and the data gradient of strided layers one residue class of input pixels at a time (TiledClass).
 #pragma once
 #include <type_traits>
 
@@ -28,8 +31,11 @@
 namespace crb {
 
 // F_: filter size (3, or 5 with pad 2 at stride 1); the header's "3x3", "9" and "halo of one" read F x F, F * F and F / 2.
-template <int TH_, int TW_, int OCT_, int WP_, int CI_, bool DGRAD_, int OCC_, int S_ = 1, int F_ = 3>
+// CLS_: one residue class of a strided data gradient (TiledClass below): F x F (1 ... 4) is the class's tap grid, the output
+// pixels are scattered with the layer's stride.
+template <int TH_, int TW_, int OCT_, int WP_, int CI_, bool DGRAD_, int OCC_, int S_ = 1, int F_ = 3, bool CLS_ = false>
 struct TiledCfg {
+    static constexpr bool CLS = CLS_;
     static constexpr int TH = TH_, TW = TW_, OCT = OCT_, WP = WP_, WO = 4 / WP_, CI = CI_, OCC = OCC_, S = S_;
     static constexpr int F = F_, NT = F_ * F_, PAD = F_ / 2;
     static constexpr bool DGRAD = DGRAD_;
@@ -45,7 +51,7 @@ struct TiledCfg {
     static constexpr int col_pos(int lc) { return S == 1 ? lc : (lc % 2) * HALF + lc / 2; }
     static constexpr int tap_off(int fh, int fw) { return S == 1 ? fh * XS + fw : fh * XS + (fw == 1 ? HALF : fw / 2); }
     static_assert(S == 1 || (S == 2 && !DGRAD_ && F == 3), "stride 2: forward only, 3 x 3 only");
-    static_assert(F == 3 || F == 5, "filter size");
+    static_assert(CLS_ ? (F >= 1 && F <= 4 && DGRAD_ && S == 1) : (F == 3 || F == 5), "filter size");
     static constexpr int XP = XR * XS;                                  // channel plane stride
     static constexpr int X_SIZE = CI * XP;
     static constexpr int KC = CI * NT, KH = KC / 2;                     // contraction per chunk, per lane half
@@ -58,6 +64,21 @@ struct TiledCfg {
     static_assert(CI % 8 == 0 && KH % 4 == 0 && (WSTR % 8) == 4, "16-byte filter fragments, conflict-free rows");
 };
 
+// A residue class of the data gradient at stride (sH, sW): the input pixels (y'' sH + py, x'' sW + px) receive only the taps
+// fh = fh0 + i sH, fw = fw0 + j sW (i < nfh, j < nfw) and read dY (y'' + qh - i, x'' + qw - j): a unit-stride correlation on the
+// class's own pixel grid with an nfh x nfw filter taken out of the layer's, embedded in the kernel's F x F tap grid (the taps
+// beyond nfh x nfw are staged as zeros).
+struct TiledClass {
+    int pad_y, pad_x;                  // window origin of class pixel (y'', x'') in dY: (y'' - pad_y, x'' - pad_x), pad = F - 1 - q
+    u32 fhw, tap0, tap_i, tap_j;       // layer filter: taps per (oc, ic) pair; tap (i, j) of the class is tap0 + i tap_i + j tap_j
+    u32 nfh, nfw;
+    u32 out_hw, out_w;                 // dX: channel stride, row stride
+    u32 osy, osx, oy0, ox0;            // class pixel (y'', x'') is dX pixel (y'' osy + oy0, x'' osx + ox0)
+    u32 H, W, tiles_x, tiles_per_img;  // the class's pixel grid and its tiles (set by the launcher)
+    u32 tile_begin;                    // the class's first tile in the launch's tile list (set by the launcher)
+};
+constexpr int kMaxTiledClasses = 16;  // residue classes of one launch (strides up to 4 x 4)
+
 struct TiledArgs {
     const float *Wt;    // filters, OC x IC x 3 x 3 of the forward convolution
     const float *X;     // input of this pass  (forward: X, data gradient: dY), N x C_IN x H x W
@@ -67,6 +88,8 @@ struct TiledArgs {
     u32 IH, IW;             // extent of the staged tensor
     u32 tiles_x, tiles_per_img, oc_tiles, tiles_total;  // tiles_total = N * tiles_per_img
     u32 relu;
+    TiledClass cls[kMaxTiledClasses];  // CLS configurations only: the launch's classes, tile lists one behind the other
+    u32 ncls;
     u32 pad;  // the window of pixel (y, x) starts at staged (S y - pad, S x - pad): the layer's padding for the forward pass,
               // F - 1 - padding for the data gradient
 };
@@ -85,10 +108,21 @@ __global__ void __launch_bounds__(kThreads, Cfg::OCC) conv3x3_tiled_kernel(Tiled
     // Workgroups are dealt round-robin to the 8 XCDs: the oc_tiles workgroups that read the same input window get ids 8
     // apart, land on the same XCD back to back and share the window through its L2.
     const u32 xcd = bid % kXcds, slot = bid / kXcds;
-    const u32 oct = slot % a.oc_tiles, rest = (slot / a.oc_tiles) * kXcds + xcd;
+    const u32 oct = slot % a.oc_tiles;
+    u32 rest = (slot / a.oc_tiles) * kXcds + xcd;
     if (rest >= a.tiles_total) return;
-    const u32 n = rest / a.tiles_per_img, tile = rest % a.tiles_per_img;
-    const int y0 = int(tile / a.tiles_x) * TH, x0 = int(tile % a.tiles_x) * TW;
+    // residue classes: the tile belongs to the last class whose list starts at or before it (uniform over the workgroup)
+    u32 ci = 0;
+    if constexpr (Cfg::CLS) {
+        for (u32 k = 1; k < a.ncls; ++k)
+            if (rest >= a.cls[k].tile_begin) ci = k;
+        rest -= a.cls[ci].tile_begin;
+    }
+    const TiledClass &cl = a.cls[ci];
+    const u32 gridH = Cfg::CLS ? cl.H : a.H, gridW = Cfg::CLS ? cl.W : a.W;
+    const u32 tiles_x = Cfg::CLS ? cl.tiles_x : a.tiles_x, tiles_per_img = Cfg::CLS ? cl.tiles_per_img : a.tiles_per_img;
+    const u32 n = rest / tiles_per_img, tile = rest % tiles_per_img;
+    const int y0 = int(tile / tiles_x) * TH, x0 = int(tile % tiles_x) * TW;
     const u32 oc0 = oct * OCT;
     const u32 HW = a.H * a.W, IHW = a.IH * a.IW;
 
@@ -108,7 +142,7 @@ __global__ void __launch_bounds__(kThreads, Cfg::OCC) conv3x3_tiled_kernel(Tiled
     for (int i = 0; i < XNP; ++i) {
         const u32 e = t + i * kThreads;
         const u32 c = e / (XR * XC), lr = (e / XC) % XR, lc = e % XC;
-        const int y = Cfg::S * y0 - int(a.pad) + int(lr), x = Cfg::S * x0 - int(a.pad) + int(lc);
+        const int y = Cfg::S * y0 - (Cfg::CLS ? cl.pad_y : int(a.pad)) + int(lr), x = Cfg::S * x0 - (Cfg::CLS ? cl.pad_x : int(a.pad)) + int(lc);
         const bool ok = (XQ % kThreads == 0 || e < XQ) && y >= 0 && y < int(a.IH) && x >= 0 && x < int(a.IW);
         xoff[i] = ok ? (c * IHW + u32(y) * a.IW + u32(x)) * 4u : kNone;
     }
@@ -120,7 +154,11 @@ __global__ void __launch_bounds__(kThreads, Cfg::OCC) conv3x3_tiled_kernel(Tiled
         const u32 e = t + i * kThreads;
         bool ok = WITEMS % kThreads == 0 || e < WITEMS;
         u32 off;
-        if constexpr (Cfg::DGRAD) {
+        if constexpr (Cfg::CLS) {
+            const u32 c = e / (OCT * NT), f = e % (OCT * NT), row = f / NT, ti = (f % NT) / F, tj = (f % NT) % F;
+            ok = ok && oc0 + row < a.C_OUT && ti < cl.nfh && tj < cl.nfw;
+            off = (c * a.C_OUT + row) * cl.fhw + cl.tap0 + ti * cl.tap_i + tj * cl.tap_j;
+        } else if constexpr (Cfg::DGRAD) {
             const u32 c = e / (OCT * NT), f = e % (OCT * NT);
             ok = ok && oc0 * NT + f < a.C_OUT * NT;
             off = c * a.C_OUT * NT + f;
@@ -143,7 +181,8 @@ __global__ void __launch_bounds__(kThreads, Cfg::OCC) conv3x3_tiled_kernel(Tiled
     };
     auto fetch = [&](u32 c0) {
         const char *xc = xin + size_t(c0) * IHW * 4;
-        const char *wc = reinterpret_cast<const char *>(Cfg::DGRAD ? a.Wt + (size_t(c0) * a.C_OUT + oc0) * NT : a.Wt + (size_t(oc0) * a.C_IN + c0) * NT);
+        const u32 wtaps = Cfg::CLS ? cl.fhw : u32(NT);  // floats per (oc, ic) pair in the filter tensor
+        const char *wc = reinterpret_cast<const char *>(Cfg::DGRAD ? a.Wt + (size_t(c0) * a.C_OUT + oc0) * wtaps : a.Wt + (size_t(oc0) * a.C_IN + c0) * NT);
 #pragma unroll
         for (int i = 0; i < XNP; ++i) {
             const bool ok = xoff[i] != kNone && c0 + (t + i * kThreads) / (XR * XC) < a.C_IN;
@@ -265,14 +304,19 @@ __global__ void __launch_bounds__(kThreads, Cfg::OCC) conv3x3_tiled_kernel(Tiled
 #pragma unroll
         for (int p = 0; p < PB; ++p) {
             const int y = y0 + prow + p * Cfg::RB, x = x0 + pcol;
-            const bool pok = y < int(a.H) && x < int(a.W);
-            float *dst = a.Y + size_t(n) * a.C_OUT * HW + size_t(pok ? y : 0) * a.W + (pok ? x : 0);
+            const bool pok = y < int(gridH) && x < int(gridW);
+            const u32 chan = Cfg::CLS ? cl.out_hw : HW;  // channel stride of the output tensor
+            float *dst = a.Y + size_t(n) * a.C_OUT * chan;
+            if constexpr (Cfg::CLS)
+                dst += pok ? size_t(u32(y) * cl.osy + cl.oy0) * cl.out_w + u32(x) * cl.osx + cl.ox0 : size_t(0);
+            else
+                dst += size_t(pok ? y : 0) * a.W + (pok ? x : 0);
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
                 const u32 oc = ocb + 8 * (r / 4) + (r % 4);
                 float v = acc[o][p][r] + bv[r];
                 if (a.relu) v = v > 0.f ? v : 0.f;
-                if (pok && oc < a.C_OUT) dst[size_t(oc) * HW] = v;
+                if (pok && oc < a.C_OUT) dst[size_t(oc) * chan] = v;
             }
         }
     }
@@ -284,27 +328,56 @@ inline bool tiled_fits(u32 C_IN, u32 C_OUT, u32 H, u32 W, u32 taps = 9) {
 }
 
 template <class Cfg>
+inline int launch_tiled_args(TiledArgs &a, u32 N, uint64_t tiles, u32 taps, hipStream_t s, const char *what) {
+    a.oc_tiles = ceil_div(a.C_OUT, u32(Cfg::OCT));
+    const uint64_t wgs = uint64_t(ceil_div(u32(tiles > 0xffffffffull ? 0xffffffffu : tiles), kXcds)) * kXcds * a.oc_tiles;
+    if (tiles > 0x7fffffffull || wgs > 0x7fffffffull) return fail(CRB_EINVAL_SHAPE, "%s: launch grid too large", what);
+    a.tiles_total = u32(tiles);
+    if (!tiled_fits(a.C_IN, a.C_OUT, a.IH, a.IW, taps)) return fail(CRB_EINVAL_SHAPE, "%s: image or filter tensor beyond 4 GB", what);
+    if (!Cfg::DGRAD && a.C_IN % 4 == 0 && reinterpret_cast<uintptr_t>(a.Wt) % 16 == 0)
+        hipLaunchKernelGGL((conv3x3_tiled_kernel<Cfg, !Cfg::DGRAD>), dim3(u32(wgs)), dim3(kThreads), 0, s, a);
+    else
+        hipLaunchKernelGGL((conv3x3_tiled_kernel<Cfg, false>), dim3(u32(wgs)), dim3(kThreads), 0, s, a);
+    return check_launch(what);
+}
+
+template <class Cfg>
 inline int launch_tiled(const float *Wt, const float *X, float *Y, const float *bias, u32 N, u32 C_IN, u32 C_OUT, u32 H, u32 W, u32 relu,
                         hipStream_t s, const char *what, u32 IH = 0, u32 IW = 0, int pad = -1) {
-    TiledArgs a;
+    static_assert(!Cfg::CLS, "residue classes are launched by launch_tiled_classes");
+    TiledArgs a = {};
     a.Wt = Wt, a.X = X, a.Y = Y, a.bias = bias;
     a.C_IN = C_IN, a.C_OUT = C_OUT, a.H = H, a.W = W;
     a.IH = IH ? IH : H, a.IW = IW ? IW : W;
     a.pad = pad < 0 ? u32(Cfg::PAD) : u32(pad);
     a.tiles_x = ceil_div(W, u32(Cfg::TW));
     a.tiles_per_img = a.tiles_x * ceil_div(H, u32(Cfg::TH));
-    a.oc_tiles = ceil_div(C_OUT, u32(Cfg::OCT));
-    const uint64_t tiles = uint64_t(N) * a.tiles_per_img;
-    const uint64_t wgs = uint64_t(ceil_div(u32(tiles > 0xffffffffull ? 0xffffffffu : tiles), kXcds)) * kXcds * a.oc_tiles;
-    if (tiles > 0x7fffffffull || wgs > 0x7fffffffull) return fail(CRB_EINVAL_SHAPE, "%s: launch grid too large", what);
-    a.tiles_total = u32(tiles);
     a.relu = relu;
-    if (!tiled_fits(C_IN, C_OUT, a.IH, a.IW, Cfg::NT)) return fail(CRB_EINVAL_SHAPE, "%s: image or filter tensor beyond 4 GB", what);
-    if (!Cfg::DGRAD && C_IN % 4 == 0 && reinterpret_cast<uintptr_t>(Wt) % 16 == 0)
-        hipLaunchKernelGGL((conv3x3_tiled_kernel<Cfg, !Cfg::DGRAD>), dim3(u32(wgs)), dim3(kThreads), 0, s, a);
-    else
-        hipLaunchKernelGGL((conv3x3_tiled_kernel<Cfg, false>), dim3(u32(wgs)), dim3(kThreads), 0, s, a);
-    return check_launch(what);
+    return launch_tiled_args<Cfg>(a, N, uint64_t(N) * a.tiles_per_img, Cfg::NT, s, what);
+}
+
+// One launch over `ncls` residue classes of a strided data gradient (every class with at most F x F taps): dX's class pixels
+// from dY (N x C_IN x OH x OW) and the layer's filters. cls[k].H / W is the class's pixel grid; the tile fields are set here.
+template <class Cfg>
+inline int launch_tiled_classes(const float *Wt, const float *dY, float *dX, u32 N, u32 C_IN, u32 C_OUT, u32 OH, u32 OW, TiledClass *cls,
+                                u32 ncls, hipStream_t s, const char *what) {
+    static_assert(Cfg::CLS, "kernel form");
+    if (ncls == 0 || ncls > u32(kMaxTiledClasses)) return fail(CRB_EINVAL_SHAPE, "%s: %u residue classes in one launch", what, ncls);
+    TiledArgs a = {};
+    a.Wt = Wt, a.X = dY, a.Y = dX, a.bias = nullptr;
+    a.C_IN = C_IN, a.C_OUT = C_OUT, a.H = 0, a.W = 0, a.IH = OH, a.IW = OW;
+    a.pad = 0, a.tiles_x = 0, a.tiles_per_img = 0, a.relu = 0;
+    uint64_t tiles = 0;
+    for (u32 k = 0; k < ncls; ++k) {
+        cls[k].tiles_x = ceil_div(cls[k].W, u32(Cfg::TW));
+        cls[k].tiles_per_img = cls[k].tiles_x * ceil_div(cls[k].H, u32(Cfg::TH));
+        if (tiles > 0x7fffffffull) return fail(CRB_EINVAL_SHAPE, "%s: launch grid too large", what);
+        cls[k].tile_begin = u32(tiles);
+        tiles += uint64_t(N) * cls[k].tiles_per_img;
+        a.cls[k] = cls[k];
+    }
+    a.ncls = ncls;
+    return launch_tiled_args<Cfg>(a, N, tiles, cls[0].fhw, s, what);
 }
 
 }  // namespace crb

@@ -416,6 +416,95 @@ static bool tiled_s2_shape(const crb_conv_geom *g) {
            uint64_t(g->IC) * g->IH * g->IW * 4 <= 0xffffffffull && uint64_t(g->IC) * g->OC * 36 <= 0xffffffffull;
 }
 
+// Data gradient at stride > 1 through the tiled kernel, one residue class of input pixels per launch (conv3x3_tiled.h,
+// TiledClass): every class is a unit-stride correlation of dY with at most ceil(FH / sH) x ceil(FW / sW) taps, run on the
+// smallest square tap grid F = 1 ... 4 that holds them. Classes no tap reaches (filters smaller than the stride) are zero-filled.
+static bool tiled_class_shape(const crb_conv_geom *g) {
+    return (g->sH > 1 || g->sW > 1) && g->sH * g->sW <= u32(kMaxTiledClasses) && ceil_div(g->FH, g->sH) <= 4 && ceil_div(g->FW, g->sW) <= 4 &&
+           uint64_t(g->OC) * g->OH * g->OW * 4 <= 0xffffffffull && uint64_t(g->IC) * g->OC * g->FH * g->FW * 4 <= 0xffffffffull;
+}
+template <int F>
+static int launch_tiled_class_group(const float *W, const float *dY, float *dX, const crb_conv_geom *g, TiledClass *cls, u32 ncls,
+                                    hipStream_t s, const char *what) {
+    // few taps: more channels per chunk, so that a chunk still holds 32 ... 128 contraction steps between two barriers
+    constexpr int CI = F == 1 ? 32 : (F == 2 ? 16 : 8);
+    if (ceil_div(g->IH, g->sH) <= 8 && ceil_div(g->IW, g->sW) <= 8)
+        return launch_tiled_classes<TiledCfg<8, 8, 64, 2, CI, true, 2, 1, F, true>>(W, dY, dX, g->N, g->OC, g->IC, g->OH, g->OW, cls, ncls, s, what);
+    return launch_tiled_classes<TiledCfg<8, 16, 32, 4, CI, true, 2, 1, F, true>>(W, dY, dX, g->N, g->OC, g->IC, g->OH, g->OW, cls, ncls, s, what);
+}
+// `together`: all classes in one launch on the largest tap grid among them (the smaller classes multiply zero taps, but a
+// small layer fills the chip with one launch); otherwise one launch per tap-grid size.
+static int dgrad_by_tiled_classes(const float *W, const float *dY, float *dX, const crb_conv_geom *g, bool together, hipStream_t s) {
+    const char *what = "crb_conv_dgrad";
+    TiledClass cls[kMaxTiledClasses];
+    int tapgrid[kMaxTiledClasses];
+    u32 ncls = 0;
+    bool empty_class = false;
+    for (u32 py = 0; py < g->sH && py < g->IH; ++py)
+        for (u32 px = 0; px < g->sW && px < g->IW; ++px) {
+            const u32 fh0 = (py + g->pH) % g->sH, fw0 = (px + g->pW) % g->sW;
+            if (fh0 >= g->FH || fw0 >= g->FW) {
+                empty_class = true;
+                continue;
+            }
+            TiledClass &c = cls[ncls];
+            c = TiledClass{};
+            c.nfh = ceil_div(g->FH - fh0, g->sH), c.nfw = ceil_div(g->FW - fw0, g->sW);
+            c.H = ceil_div(g->IH - py, g->sH), c.W = ceil_div(g->IW - px, g->sW);  // the class's pixel grid
+            c.pad_y = -int((py + g->pH) / g->sH), c.pad_x = -int((px + g->pW) / g->sW);  // + F - 1 once the tap grid is known
+            c.fhw = g->FH * g->FW, c.tap0 = fh0 * g->FW + fw0, c.tap_i = g->sH * g->FW, c.tap_j = g->sW;
+            c.out_hw = g->IH * g->IW, c.out_w = g->IW, c.osy = g->sH, c.osx = g->sW, c.oy0 = py, c.ox0 = px;
+            tapgrid[ncls] = int(c.nfh > c.nfw ? c.nfh : c.nfw);
+            ++ncls;
+        }
+    if (empty_class) {
+        const uint64_t count = uint64_t(g->N) * g->IC * g->IH * g->IW;
+        if (int st = crb_tensor_fill(dX, 0.f, uint32_t(count), s)) return st;
+    }
+    int fmax = 1;
+    for (u32 k = 0; k < ncls; ++k) fmax = tapgrid[k] > fmax ? tapgrid[k] : fmax;
+    for (int F = 1; F <= 4; ++F) {
+        TiledClass grp[kMaxTiledClasses];
+        u32 n = 0;
+        for (u32 k = 0; k < ncls; ++k)
+            if (together ? F == fmax : tapgrid[k] == F) {
+                grp[n] = cls[k];
+                grp[n].pad_y += F - 1, grp[n].pad_x += F - 1;
+                ++n;
+            }
+        if (n == 0) continue;
+        int st;
+        switch (F) {
+            case 1: st = launch_tiled_class_group<1>(W, dY, dX, g, grp, n, s, what); break;
+            case 2: st = launch_tiled_class_group<2>(W, dY, dX, g, grp, n, s, what); break;
+            case 3: st = launch_tiled_class_group<3>(W, dY, dX, g, grp, n, s, what); break;
+            default: st = launch_tiled_class_group<4>(W, dY, dX, g, grp, n, s, what); break;
+        }
+        if (st) return st;
+    }
+    return CRB_OK;
+}
+// Every non-empty class is a launch of its own, so a class must bring work: 96 workgroups (24 and 16 contraction channels when it is the only class, as for
+// 1x1 filters), tiles at least a quarter full, five contraction channels. Against the engine's class launches / its one gather
+// over all taps on 240 random layers: 32 -> 16 @56 5x5 stride 3 batch 128 317 -> 108 us, 256 -> 32 @28 7x7 stride 2 batch 32
+// 261 -> 110, 64 -> 256 @14 2x2 stride 2 batch 128 131 -> 59, 3 -> 128 @28 4x4 stride 2 batch 128 208 -> 82; below those counts the
+// engine keeps the call (256 -> 32 @8 7x7 stride 3 batch 32, 3 x 3 pixel classes: 55 us against 115 through nine tiled launches).
+static bool tiled_classes_pay(const crb_conv_geom *g, bool *together = nullptr) {
+    if (!tiled_class_shape(g) || g->OC < 5) return false;
+    u32 nc = 0;
+    for (u32 py = 0; py < g->sH && py < g->IH; ++py)
+        for (u32 px = 0; px < g->sW && px < g->IW; ++px)
+            if ((py + g->pH) % g->sH < g->FH && (px + g->pW) % g->sW < g->FW) ++nc;
+    const u32 CH = ceil_div(g->IH, g->sH), CW = ceil_div(g->IW, g->sW);
+    const bool small = CH <= 8 && CW <= 8;
+    const uint64_t tiles = small ? uint64_t(g->N) : uint64_t(g->N) * ceil_div(CH, 8u) * ceil_div(CW, 16u);
+    const uint64_t wgs = tiles * ceil_div(g->IC, small ? 64u : 32u);  // per class
+    const uint64_t padded = small ? 64 : uint64_t(ceil_div(CH, 8u)) * 8 * ceil_div(CW, 16u) * 16;
+    if (together) *together = wgs < 512;
+    if (nc == 1) return wgs >= 24 && g->OC >= 16;  // (8 -> 3 @64 1x1 stride 2 batch 4: 6.8 against 4.3 us)
+    return wgs * nc >= 128 && 4 * uint64_t(CH) * CW >= padded;
+}
+
 // F x F (3 or 5), stride 1, the same padding 0 ... F - 1 on both axes, and tensors the tiled kernel can address
 static bool tiled_s1_shape(const crb_conv_geom *g, u32 F) {
     return g->FH == F && g->FW == F && g->sH == 1 && g->sW == 1 && g->pH == g->pW && g->pH <= F - 1 &&
@@ -831,6 +920,10 @@ int crb_conv_dgrad(const float *W, const float *dY, float *dX, const crb_conv_ge
         return launch_tiled_any<true, 1, 5>(W, dY, dX, nullptr, g->N, g->OC, g->IC, g->IH, g->IW, 0, hipStream_t(stream), "crb_conv_dgrad",
                                             g->OH, g->OW, int(4 - g->pH));
     const u32 FHW = g->FH * g->FW;
+    {
+        bool together = false;
+        if (tiled_classes_pay(g, &together)) return dgrad_by_tiled_classes(W, dY, dX, g, together, hipStream_t(stream));
+    }
     if ((g->sH > 1 || g->sW > 1) && dgrad_classes_pay(g)) return dgrad_by_classes(W, dY, dX, g, hipStream_t(stream));
     const u32 M = g->IC, N = g->N * g->IH * g->IW, K = g->OC * FHW;
     SepK a{W, g->IC, FHW, g->IC * FHW, 1, FastDiv(FHW)};
@@ -1027,6 +1120,7 @@ size_t crb_conv_dgrad_workspace_bytes(const crb_conv_geom *g, int operands_align
     if (shortcut_shape(g) && operands_aligned16) return 0;
     if ((tiled_s1_shape(g, 3) || tiled_s1_shape(g, 5)) && tiled_pays(g->N, g->OC, g->IC, g->IH, g->IW, g->FH * g->FW))
         return 0;  // the tiled kernel
+    if (tiled_classes_pay(g)) return 0;                              // one tiled launch per residue class
     if ((g->sH > 1 || g->sW > 1) && dgrad_classes_pay(g)) return 0;  // one launch per residue class, none of them cut
     return nchw_scratch_bytes(g->IC, g->N * g->IH * g->IW, g->OC * g->FH * g->FW);
 }

@@ -127,6 +127,23 @@ def test_3x3_and_5x5_layers_with_other_paddings(dev, shape):
     run_layer(dev, N, IC, IH, IW, OC, F, F, 1, 1, pad, pad, bias=True, seed=sum(shape))
 
 
+# Data gradients at stride > 1 that go through the tiled kernel one residue class of input pixels at a time: enough workgroups
+# per class to be chosen (96, or 24 for a single class), tap grids 1 x 1 ... 4 x 4, 8 x 8 and 8 x 16 pixel tiles, ragged class
+# grids, rectangular filters and strides, classes that no tap reaches
+TILED_CLASSES = [
+    # N, IC, IH, IW, OC, FH, FW, sH, sW, pH, pW
+    (24, 40, 28, 28, 24, 4, 4, 2, 2, 1, 1), (24, 64, 30, 30, 16, 3, 3, 2, 2, 1, 1), (24, 33, 27, 31, 12, 5, 5, 2, 2, 2, 2),
+    (24, 64, 32, 32, 8, 7, 7, 2, 2, 3, 3), (48, 24, 48, 48, 20, 3, 3, 3, 3, 1, 1), (96, 64, 16, 16, 32, 2, 2, 2, 2, 0, 0),
+    (8, 96, 20, 20, 32, 1, 1, 2, 2, 0, 0), (16, 70, 17, 23, 40, 1, 1, 3, 3, 0, 0), (32, 32, 20, 20, 16, 3, 3, 2, 1, 1, 1),
+    (24, 48, 24, 24, 16, 3, 5, 2, 2, 1, 2), (100, 36, 15, 15, 24, 2, 2, 2, 2, 1, 1), (24, 40, 29, 29, 17, 4, 4, 2, 2, 0, 0),
+]
+
+
+@pytest.mark.parametrize("shape", TILED_CLASSES, ids=lambda s: "x".join(map(str, s)))
+def test_strided_layers_whose_data_gradient_runs_by_tiled_residue_classes(dev, shape):
+    run_layer(dev, *shape, bias=True, seed=sum(shape))
+
+
 @pytest.mark.parametrize("seed", [41, 42])
 def test_random_3x3_layers_of_any_extent(dev, seed):
     rng = random.Random(seed)
