@@ -33,11 +33,12 @@ namespace crb {
 // F_: filter size (3, or 5 with pad 2 at stride 1); the header's "3x3", "9" and "halo of one" read F x F, F * F and F / 2.
 // CLS_: one residue class of a strided data gradient (TiledClass below): F x F (1 ... 4) is the class's tap grid, the output
 // pixels are scattered with the layer's stride.
-template <int TH_, int TW_, int OCT_, int WP_, int CI_, bool DGRAD_, int OCC_, int S_ = 1, int F_ = 3, bool CLS_ = false>
+// FW_ (class forms): the tap grid is F_ rows x FW_ columns.
+template <int TH_, int TW_, int OCT_, int WP_, int CI_, bool DGRAD_, int OCC_, int S_ = 1, int F_ = 3, bool CLS_ = false, int FW_ = F_>
 struct TiledCfg {
     static constexpr bool CLS = CLS_;
     static constexpr int TH = TH_, TW = TW_, OCT = OCT_, WP = WP_, WO = 4 / WP_, CI = CI_, OCC = OCC_, S = S_;
-    static constexpr int F = F_, NT = F_ * F_, PAD = F_ / 2;
+    static constexpr int F = F_, FW = FW_, NT = F_ * FW_, PAD = F_ / 2;
     static constexpr bool DGRAD = DGRAD_;
     static constexpr int PIX = TH * TW, NPB = PIX / 32, NOB = OCT / 32;  // 32-pixel and 32-channel MFMA blocks
     static constexpr int PB = NPB / WP, OB = NOB / WO;                  // blocks per wave
@@ -45,13 +46,13 @@ struct TiledCfg {
     // staged rows and columns of the input window; LDS row stride. Stride 2 (forward only): a staged row holds the window's
     // even columns (input columns 2 x0 - 1, 2 x0 + 1, ...: taps fw = 0 and 2) and then, HALF floats further, its odd columns
     // (tap fw = 1), so that neighbouring pixels read neighbouring floats for every tap.
-    static constexpr int XR = S * (TH - 1) + F, XC = S * (TW - 1) + F;
+    static constexpr int XR = S * (TH - 1) + F, XC = S * (TW - 1) + FW;
     static constexpr int HALF = TW + 2;
     static constexpr int XS = S == 1 ? TW + 4 : 2 * TW + 4;  // >= XC for both filter sizes
     static constexpr int col_pos(int lc) { return S == 1 ? lc : (lc % 2) * HALF + lc / 2; }
     static constexpr int tap_off(int fh, int fw) { return S == 1 ? fh * XS + fw : fh * XS + (fw == 1 ? HALF : fw / 2); }
     static_assert(S == 1 || (S == 2 && !DGRAD_ && F == 3), "stride 2: forward only, 3 x 3 only");
-    static_assert(CLS_ ? (F >= 1 && F <= 4 && DGRAD_ && S == 1) : (F == 3 || F == 5), "filter size");
+    static_assert(CLS_ ? (F >= 1 && F <= 4 && FW >= 1 && FW <= 4 && DGRAD_ && S == 1) : ((F == 3 || F == 5) && FW == F), "filter size");
     static constexpr int XP = XR * XS;                                  // channel plane stride
     static constexpr int X_SIZE = CI * XP;
     static constexpr int KC = CI * NT, KH = KC / 2;                     // contraction per chunk, per lane half
@@ -67,9 +68,9 @@ struct TiledCfg {
 // A residue class of the data gradient at stride (sH, sW): the input pixels (y'' sH + py, x'' sW + px) receive only the taps
 // fh = fh0 + i sH, fw = fw0 + j sW (i < nfh, j < nfw) and read dY (y'' + qh - i, x'' + qw - j): a unit-stride correlation on the
 // class's own pixel grid with an nfh x nfw filter taken out of the layer's, embedded in the kernel's F x F tap grid (the taps
-// beyond nfh x nfw are staged as zeros).
+// beyond nfh x nfw are staged as zeros; F rows x FW columns in the class forms).
 struct TiledClass {
-    int pad_y, pad_x;                  // window origin of class pixel (y'', x'') in dY: (y'' - pad_y, x'' - pad_x), pad = F - 1 - q
+    int pad_y, pad_x;                  // window origin of class pixel (y'', x'') in dY: (y'' - pad_y, x'' - pad_x), pad = F - 1 - qh, FW - 1 - qw
     u32 fhw, tap0, tap_i, tap_j;       // layer filter: taps per (oc, ic) pair; tap (i, j) of the class is tap0 + i tap_i + j tap_j
     u32 nfh, nfw;
     u32 out_hw, out_w;                 // dX: channel stride, row stride
@@ -99,7 +100,7 @@ template <class Cfg, bool WVEC>
 __global__ void __launch_bounds__(kThreads, Cfg::OCC) conv3x3_tiled_kernel(TiledArgs a) {
     constexpr int TH = Cfg::TH, TW = Cfg::TW, OCT = Cfg::OCT, CI = Cfg::CI, PB = Cfg::PB, OB = Cfg::OB;
     constexpr int XR = Cfg::XR, XC = Cfg::XC, XS = Cfg::XS, XP = Cfg::XP, KC = Cfg::KC, KH = Cfg::KH, WSTR = Cfg::WSTR;
-    constexpr int F = Cfg::F, NT = Cfg::NT;
+    constexpr int F = Cfg::F, FW = Cfg::FW, NT = Cfg::NT;
     __shared__ __attribute__((aligned(16))) float smem[Cfg::SMEM_FLOATS];
     float(*sX)[Cfg::X_SIZE] = reinterpret_cast<float(*)[Cfg::X_SIZE]>(smem);
     float(*sW)[Cfg::W_SIZE] = reinterpret_cast<float(*)[Cfg::W_SIZE]>(smem + 2 * Cfg::X_SIZE);
@@ -155,7 +156,7 @@ __global__ void __launch_bounds__(kThreads, Cfg::OCC) conv3x3_tiled_kernel(Tiled
         bool ok = WITEMS % kThreads == 0 || e < WITEMS;
         u32 off;
         if constexpr (Cfg::CLS) {
-            const u32 c = e / (OCT * NT), f = e % (OCT * NT), row = f / NT, ti = (f % NT) / F, tj = (f % NT) % F;
+            const u32 c = e / (OCT * NT), f = e % (OCT * NT), row = f / NT, ti = (f % NT) / FW, tj = (f % NT) % FW;
             ok = ok && oc0 + row < a.C_OUT && ti < cl.nfh && tj < cl.nfw;
             off = (c * a.C_OUT + row) * cl.fhw + cl.tap0 + ti * cl.tap_i + tj * cl.tap_j;
         } else if constexpr (Cfg::DGRAD) {
@@ -253,7 +254,7 @@ __global__ void __launch_bounds__(kThreads, Cfg::OCC) conv3x3_tiled_kernel(Tiled
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
                 const int s = 4 * sq + e, c = s / NT, tap = s % NT;
-                const int fh = Cfg::DGRAD ? F - 1 - tap / F : tap / F, fw = Cfg::DGRAD ? F - 1 - tap % F : tap % F;
+                const int fh = Cfg::DGRAD ? F - 1 - tap / FW : tap / FW, fw = Cfg::DGRAD ? FW - 1 - tap % FW : tap % FW;
 #pragma unroll
                 for (int p = 0; p < PB; ++p) xv[set][e][p] = xfrag[c * XP + Cfg::S * p * Cfg::RB * XS + Cfg::tap_off(fh, fw)];
             }

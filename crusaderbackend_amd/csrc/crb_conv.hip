@@ -423,22 +423,38 @@ static bool tiled_class_shape(const crb_conv_geom *g) {
     return (g->sH > 1 || g->sW > 1) && g->sH * g->sW <= u32(kMaxTiledClasses) && ceil_div(g->FH, g->sH) <= 4 && ceil_div(g->FW, g->sW) <= 4 &&
            uint64_t(g->OC) * g->OH * g->OW * 4 <= 0xffffffffull && uint64_t(g->IC) * g->OC * g->FH * g->FW * 4 <= 0xffffffffull;
 }
-template <int F>
+template <int FH, int FW>
 static int launch_tiled_class_group(const float *W, const float *dY, float *dX, const crb_conv_geom *g, TiledClass *cls, u32 ncls,
                                     hipStream_t s, const char *what) {
     // few taps: more channels per chunk, so that a chunk still holds 32 ... 128 contraction steps between two barriers
-    constexpr int CI = F == 1 ? 32 : (F == 2 ? 16 : 8);
+    constexpr int CI = FH * FW == 1 ? 32 : (FH * FW <= 4 ? 16 : 8);
+    for (u32 k = 0; k < ncls; ++k) cls[k].pad_y += FH - 1, cls[k].pad_x += FW - 1;
     if (ceil_div(g->IH, g->sH) <= 8 && ceil_div(g->IW, g->sW) <= 8)
-        return launch_tiled_classes<TiledCfg<8, 8, 64, 2, CI, true, 2, 1, F, true>>(W, dY, dX, g->N, g->OC, g->IC, g->OH, g->OW, cls, ncls, s, what);
-    return launch_tiled_classes<TiledCfg<8, 16, 32, 4, CI, true, 2, 1, F, true>>(W, dY, dX, g->N, g->OC, g->IC, g->OH, g->OW, cls, ncls, s, what);
+        return launch_tiled_classes<TiledCfg<8, 8, 64, 2, CI, true, 2, 1, FH, true, FW>>(W, dY, dX, g->N, g->OC, g->IC, g->OH, g->OW, cls, ncls, s,
+                                                                                        what);
+    return launch_tiled_classes<TiledCfg<8, 16, 32, 4, CI, true, 2, 1, FH, true, FW>>(W, dY, dX, g->N, g->OC, g->IC, g->OH, g->OW, cls, ncls, s,
+                                                                                      what);
 }
-// `together`: all classes in one launch on the largest tap grid among them (the smaller classes multiply zero taps, but a
-// small layer fills the chip with one launch); otherwise one launch per tap-grid size.
+// The tap grids that have a kernel; a class runs on the smallest one that holds its nfh x nfw taps.
+struct TapGrid {
+    int fh, fw;
+};
+static constexpr TapGrid kTapGrids[] = {{1, 1}, {1, 2}, {2, 1}, {2, 2}, {2, 3}, {3, 2}, {3, 3}, {3, 4}, {4, 3}, {4, 4}};
+static int tap_grid_for(u32 nfh, u32 nfw) {
+    int best = -1;
+    for (int i = 0; i < int(sizeof(kTapGrids) / sizeof(kTapGrids[0])); ++i)
+        if (kTapGrids[i].fh >= int(nfh) && kTapGrids[i].fw >= int(nfw) &&
+            (best < 0 || kTapGrids[i].fh * kTapGrids[i].fw < kTapGrids[best].fh * kTapGrids[best].fw))
+            best = i;
+    return best;
+}
+// `together`: all classes in one launch on the smallest tap grid that holds them all (the smaller classes multiply zero
+// taps, but a small layer fills the chip with one launch); otherwise one launch per tap grid.
 static int dgrad_by_tiled_classes(const float *W, const float *dY, float *dX, const crb_conv_geom *g, bool together, hipStream_t s) {
     const char *what = "crb_conv_dgrad";
     TiledClass cls[kMaxTiledClasses];
-    int tapgrid[kMaxTiledClasses];
-    u32 ncls = 0;
+    int grid[kMaxTiledClasses];
+    u32 ncls = 0, mh = 1, mw = 1;
     bool empty_class = false;
     for (u32 py = 0; py < g->sH && py < g->IH; ++py)
         for (u32 px = 0; px < g->sW && px < g->IW; ++px) {
@@ -451,44 +467,47 @@ static int dgrad_by_tiled_classes(const float *W, const float *dY, float *dX, co
             c = TiledClass{};
             c.nfh = ceil_div(g->FH - fh0, g->sH), c.nfw = ceil_div(g->FW - fw0, g->sW);
             c.H = ceil_div(g->IH - py, g->sH), c.W = ceil_div(g->IW - px, g->sW);  // the class's pixel grid
-            c.pad_y = -int((py + g->pH) / g->sH), c.pad_x = -int((px + g->pW) / g->sW);  // + F - 1 once the tap grid is known
+            c.pad_y = -int((py + g->pH) / g->sH), c.pad_x = -int((px + g->pW) / g->sW);  // + tap grid - 1 at the launch
             c.fhw = g->FH * g->FW, c.tap0 = fh0 * g->FW + fw0, c.tap_i = g->sH * g->FW, c.tap_j = g->sW;
             c.out_hw = g->IH * g->IW, c.out_w = g->IW, c.osy = g->sH, c.osx = g->sW, c.oy0 = py, c.ox0 = px;
-            tapgrid[ncls] = int(c.nfh > c.nfw ? c.nfh : c.nfw);
+            grid[ncls] = tap_grid_for(c.nfh, c.nfw);
+            mh = c.nfh > mh ? c.nfh : mh, mw = c.nfw > mw ? c.nfw : mw;
             ++ncls;
         }
     if (empty_class) {
         const uint64_t count = uint64_t(g->N) * g->IC * g->IH * g->IW;
         if (int st = crb_tensor_fill(dX, 0.f, uint32_t(count), s)) return st;
     }
-    int fmax = 1;
-    for (u32 k = 0; k < ncls; ++k) fmax = tapgrid[k] > fmax ? tapgrid[k] : fmax;
-    for (int F = 1; F <= 4; ++F) {
+    const int all = tap_grid_for(mh, mw);
+    for (int gi = 0; gi < int(sizeof(kTapGrids) / sizeof(kTapGrids[0])); ++gi) {
         TiledClass grp[kMaxTiledClasses];
         u32 n = 0;
         for (u32 k = 0; k < ncls; ++k)
-            if (together ? F == fmax : tapgrid[k] == F) {
-                grp[n] = cls[k];
-                grp[n].pad_y += F - 1, grp[n].pad_x += F - 1;
-                ++n;
-            }
+            if (together ? gi == all : grid[k] == gi) grp[n++] = cls[k];
         if (n == 0) continue;
         int st;
-        switch (F) {
-            case 1: st = launch_tiled_class_group<1>(W, dY, dX, g, grp, n, s, what); break;
-            case 2: st = launch_tiled_class_group<2>(W, dY, dX, g, grp, n, s, what); break;
-            case 3: st = launch_tiled_class_group<3>(W, dY, dX, g, grp, n, s, what); break;
-            default: st = launch_tiled_class_group<4>(W, dY, dX, g, grp, n, s, what); break;
+        switch (gi) {
+            case 0: st = launch_tiled_class_group<1, 1>(W, dY, dX, g, grp, n, s, what); break;
+            case 1: st = launch_tiled_class_group<1, 2>(W, dY, dX, g, grp, n, s, what); break;
+            case 2: st = launch_tiled_class_group<2, 1>(W, dY, dX, g, grp, n, s, what); break;
+            case 3: st = launch_tiled_class_group<2, 2>(W, dY, dX, g, grp, n, s, what); break;
+            case 4: st = launch_tiled_class_group<2, 3>(W, dY, dX, g, grp, n, s, what); break;
+            case 5: st = launch_tiled_class_group<3, 2>(W, dY, dX, g, grp, n, s, what); break;
+            case 6: st = launch_tiled_class_group<3, 3>(W, dY, dX, g, grp, n, s, what); break;
+            case 7: st = launch_tiled_class_group<3, 4>(W, dY, dX, g, grp, n, s, what); break;
+            case 8: st = launch_tiled_class_group<4, 3>(W, dY, dX, g, grp, n, s, what); break;
+            default: st = launch_tiled_class_group<4, 4>(W, dY, dX, g, grp, n, s, what); break;
         }
         if (st) return st;
     }
     return CRB_OK;
 }
-// Every non-empty class is a launch of its own, so a class must bring work: 96 workgroups (24 and 16 contraction channels when it is the only class, as for
-// 1x1 filters), tiles at least a quarter full, five contraction channels. Against the engine's class launches / its one gather
-// over all taps on 240 random layers: 32 -> 16 @56 5x5 stride 3 batch 128 317 -> 108 us, 256 -> 32 @28 7x7 stride 2 batch 32
-// 261 -> 110, 64 -> 256 @14 2x2 stride 2 batch 128 131 -> 59, 3 -> 128 @28 4x4 stride 2 batch 128 208 -> 82; below those counts the
-// engine keeps the call (256 -> 32 @8 7x7 stride 3 batch 32, 3 x 3 pixel classes: 55 us against 115 through nine tiled launches).
+// The launches must bring work: 128 workgroups over the classes (24 and 16 contraction channels, 64 on class grids up to 8 x 8,
+// when there is a single class, as for 1x1 filters), tiles at least a quarter full, five contraction channels. `together`: a class
+// brings fewer than 512 workgroups, so all classes share one launch. Against the engine's class launches / its one gather over all
+// taps on random layers: 32 -> 16 @56 5x5 stride 3 batch 128 317 -> 85 us, 256 -> 32 @28 7x7 stride 2 batch 32 261 -> 97,
+// 64 -> 256 @14 2x2 stride 2 batch 128 131 -> 23, 3 -> 128 @28 4x4 stride 2 batch 128 208 -> 60; class grids that fill their
+// tiles less stay with the engine (256 -> 32 @8 7x7 stride 3 batch 32, 3 x 3 pixel classes on 8 x 8 tiles: 55 against 115 us).
 static bool tiled_classes_pay(const crb_conv_geom *g, bool *together = nullptr) {
     if (!tiled_class_shape(g) || g->OC < 5) return false;
     u32 nc = 0;
@@ -501,7 +520,8 @@ static bool tiled_classes_pay(const crb_conv_geom *g, bool *together = nullptr) 
     const uint64_t wgs = tiles * ceil_div(g->IC, small ? 64u : 32u);  // per class
     const uint64_t padded = small ? 64 : uint64_t(ceil_div(CH, 8u)) * 8 * ceil_div(CW, 16u) * 16;
     if (together) *together = wgs < 512;
-    if (nc == 1) return wgs >= 24 && g->OC >= 16;  // (8 -> 3 @64 1x1 stride 2 batch 4: 6.8 against 4.3 us)
+    // (8 -> 3 @64 1x1 stride 2 batch 4: 6.8 against 4.3 us; 32 -> 256 @16 1x1 stride 2 batch 32, 8 x 8 class grid: 16.6 against 10.4)
+    if (nc == 1) return wgs >= 24 && g->OC >= (small ? 64u : 16u);
     return wgs * nc >= 128 && 4 * uint64_t(CH) * CW >= padded;
 }
 

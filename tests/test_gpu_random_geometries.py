@@ -128,14 +128,17 @@ def test_3x3_and_5x5_layers_with_other_paddings(dev, shape):
 
 
 # Data gradients at stride > 1 that go through the tiled kernel one residue class of input pixels at a time: enough workgroups
-# per class to be chosen (96, or 24 for a single class), tap grids 1 x 1 ... 4 x 4, 8 x 8 and 8 x 16 pixel tiles, ragged class
-# grids, rectangular filters and strides, classes that no tap reaches
+# in the launch to be chosen (128, or 24 for a single class), tap grids 1 x 1 ... 4 x 4, 8 x 8 and 8 x 16 pixel tiles, ragged
+# class grids, rectangular filters and strides, classes that no tap reaches
 TILED_CLASSES = [
     # N, IC, IH, IW, OC, FH, FW, sH, sW, pH, pW
     (24, 40, 28, 28, 24, 4, 4, 2, 2, 1, 1), (24, 64, 30, 30, 16, 3, 3, 2, 2, 1, 1), (24, 33, 27, 31, 12, 5, 5, 2, 2, 2, 2),
     (24, 64, 32, 32, 8, 7, 7, 2, 2, 3, 3), (48, 24, 48, 48, 20, 3, 3, 3, 3, 1, 1), (96, 64, 16, 16, 32, 2, 2, 2, 2, 0, 0),
     (8, 96, 20, 20, 32, 1, 1, 2, 2, 0, 0), (16, 70, 17, 23, 40, 1, 1, 3, 3, 0, 0), (32, 32, 20, 20, 16, 3, 3, 2, 1, 1, 1),
     (24, 48, 24, 24, 16, 3, 5, 2, 2, 1, 2), (100, 36, 15, 15, 24, 2, 2, 2, 2, 1, 1), (24, 40, 29, 29, 17, 4, 4, 2, 2, 0, 0),
+    # 512 workgroups per class: one launch per tap grid (1x1, 1x2, 2x1, 2x2 / 2x2 ... 3x3 / 3x3 ... 4x4 / a class without a grid of its own)
+    (128, 64, 30, 30, 8, 3, 3, 2, 2, 1, 1), (128, 64, 28, 28, 8, 5, 5, 2, 2, 2, 2), (128, 64, 28, 28, 6, 7, 7, 2, 2, 3, 3),
+    (128, 64, 45, 45, 8, 4, 4, 3, 3, 1, 1), (128, 64, 28, 28, 8, 3, 5, 2, 2, 1, 2),
 ]
 
 
