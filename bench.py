@@ -191,7 +191,7 @@ def measured_hbm_bytes():
         if ln.startswith("Counters taken at commit"):
             commit = ln.split("`")[1] if "`" in ln else None
         if ln.startswith("Kernel source hash"):
-            src_hash = ln.split("`")[1] if "`" in ln else None
+            src_hash = ln.split("`")[-2] if ln.count("`") >= 2 else None  # the line's last quoted token
         if ln.startswith("## HBM bytes per call"):
             on = True
             continue
