@@ -432,7 +432,13 @@ static int launch_tiled_class_group(const float *W, const float *dY, float *dX, 
     if (ceil_div(g->IH, g->sH) <= 8 && ceil_div(g->IW, g->sW) <= 8)
         return launch_tiled_classes<TiledCfg<8, 8, 64, 2, CI, true, 2, 1, FH, true, FW>>(W, dY, dX, g->N, g->OC, g->IC, g->OH, g->OW, cls, ncls, s,
                                                                                         what);
-    return launch_tiled_classes<TiledCfg<8, 16, 32, 4, CI, true, 2, 1, FH, true, FW>>(W, dY, dX, g->N, g->OC, g->IC, g->OH, g->OW, cls, ncls, s,
+    // 8 x 16 tiles, or 4 x 32 where those pad the class grid less (28 x 28: 28 x 32 instead of 32 x 32)
+    const u32 CH = ceil_div(g->IH, g->sH), CW = ceil_div(g->IW, g->sW);
+    constexpr int OCT = 32;  // (64 channels for the grids of up to four taps: 3x3 stride 2 128 -> 128 @56 158 -> 151 us, but 256 -> 256 @28 151 -> 173)
+    if (uint64_t(ceil_div(CH, 4u)) * 4 * ceil_div(CW, 32u) * 32 < uint64_t(ceil_div(CH, 8u)) * 8 * ceil_div(CW, 16u) * 16)
+        return launch_tiled_classes<TiledCfg<4, 32, OCT, 4, CI, true, 2, 1, FH, true, FW>>(W, dY, dX, g->N, g->OC, g->IC, g->OH, g->OW, cls, ncls,
+                                                                                          s, what);
+    return launch_tiled_classes<TiledCfg<8, 16, OCT, 4, CI, true, 2, 1, FH, true, FW>>(W, dY, dX, g->N, g->OC, g->IC, g->OH, g->OW, cls, ncls, s,
                                                                                       what);
 }
 // The tap grids that have a kernel; a class runs on the smallest one that holds its nfh x nfw taps.

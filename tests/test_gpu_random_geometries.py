@@ -139,6 +139,8 @@ TILED_CLASSES = [
     # 512 workgroups per class: one launch per tap grid (1x1, 1x2, 2x1, 2x2 / 2x2 ... 3x3 / 3x3 ... 4x4 / a class without a grid of its own)
     (128, 64, 30, 30, 8, 3, 3, 2, 2, 1, 1), (128, 64, 28, 28, 8, 5, 5, 2, 2, 2, 2), (128, 64, 28, 28, 6, 7, 7, 2, 2, 3, 3),
     (128, 64, 45, 45, 8, 4, 4, 3, 3, 1, 1), (128, 64, 28, 28, 8, 3, 5, 2, 2, 1, 2),
+    # class grids that 4 x 32 tiles pad less than 8 x 16 ones
+    (24, 16, 56, 56, 8, 3, 3, 2, 2, 1, 1), (8, 40, 55, 57, 8, 5, 5, 2, 2, 2, 2),
 ]
 
 
