@@ -233,7 +233,7 @@ def compact(torch, capi, dev, event_time_ms, Layer):
 
 
 def run(torch, capi, dev, event_time_ms, Layer):
-    out = {"gemm": [], "resnet56": [], "vgg16": [], "densenet": [], "dense": []}
+    out = {"gemm": [], "resnet56": [], "vgg16": [], "densenet": [], "dense": [], "offgrid": []}
 
     def rnd(*shape):
         return torch.rand(*shape, device=dev) * 2 - 1
@@ -298,6 +298,15 @@ def run(torch, capi, dev, event_time_ms, Layer):
             dn.append((f"1x1_{base + 12 * i}-48@{H}", base + 12 * i, H, 48, 1, 1, 0))
         dn.append((f"3x3_48-12@{H}", 48, H, 12, 3, 1, 1))
     conv_entries("densenet", dn, 64, True)
+
+    # Layers off the benchmark networks' width grid (no configuration of the baseline; the geometries of ImageNet-style residual
+    # networks, a 5x5 layer, a 3x3 layer without padding, a 4x4 stride-2 layer, a 7x7 stride-2 stem), batch 32
+    conv_entries("offgrid", [("64-64@56", 64, 56, 64, 3, 1, 1), ("128-128@28", 128, 28, 128, 3, 1, 1), ("256-256@14", 256, 14, 256, 3, 1, 1),
+                             ("512-512@7", 512, 7, 512, 3, 1, 1), ("64-128@56s2", 64, 56, 128, 3, 2, 1),
+                             ("128-256@28s2", 128, 28, 256, 3, 2, 1), ("256-512@14s2", 256, 14, 512, 3, 2, 1),
+                             ("sc64-128@56_1x1s2", 64, 56, 128, 1, 2, 0), ("5x5_64-64@28p2", 64, 28, 64, 5, 1, 2),
+                             ("3x3_64-64@30p0", 64, 30, 64, 3, 1, 0), ("4x4s2_64-128@32p1", 64, 32, 128, 4, 2, 1),
+                             ("7x7s2_3-64@224p3", 3, 224, 64, 7, 2, 3)], 32, False)
 
     # config 4 as a whole: the convolution work of one DenseNet-BC-100 training step at batch 64
     pairs = _densenet_pairs(torch, capi, dev, Layer)
@@ -375,7 +384,7 @@ def run(torch, capi, dev, event_time_ms, Layer):
 
 def to_markdown(rep):
     lines = []
-    for key in ("gemm", "resnet56", "vgg16", "densenet", "dense", "elementwise"):
+    for key in ("gemm", "resnet56", "vgg16", "densenet", "offgrid", "dense", "elementwise"):
         if key not in rep:
             continue
         lines += [f"### {key}", "", "| shape.pass | us (smallest of 3 averages) | us (mean of the 3) | GFLOP | MB | AI | TFLOP/s | GB/s | bound | fraction of roofline | cold-cache us | cold GB/s |",
