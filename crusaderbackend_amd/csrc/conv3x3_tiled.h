@@ -242,6 +242,11 @@ __global__ void __launch_bounds__(kThreads, Cfg::OCC) conv3x3_tiled_kernel(Tiled
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[o][p][r] = 0.f;
 
+    u32 tapmask = 0;  // class forms: bit t = tap t of the F x FW grid belongs to this workgroup's class
+    if constexpr (Cfg::CLS) {
+#pragma unroll
+        for (int tp = 0; tp < NT; ++tp) tapmask |= (u32(tp / FW) < cl.nfh && u32(tp % FW) < cl.nfw) ? (1u << tp) : 0u;
+    }
     // Fragments are read one group of four steps ahead of the MFMAs that consume them (two register sets; the scheduler is
     // fenced so that it neither undoes the pipeline nor hoists every read of the chunk to its top).
     auto compute = [&](const float *cx, const float *cw) {
@@ -265,12 +270,16 @@ __global__ void __launch_bounds__(kThreads, Cfg::OCC) conv3x3_tiled_kernel(Tiled
             if (sq + 1 < KH / 4) read_group(sq + 1, (sq + 1) & 1);
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-            for (int e = 0; e < 4; ++e)
+            for (int e = 0; e < 4; ++e) {
+                // class forms: the taps of the shared grid that this class does not have were staged as zeros; their steps
+                // are skipped (uniform over the workgroup)
+                if (Cfg::CLS && !(tapmask >> ((4 * sq + e) % NT) & 1u)) continue;
 #pragma unroll
                 for (int o = 0; o < OB; ++o)
 #pragma unroll
                     for (int p = 0; p < PB; ++p)
                         acc[o][p] = __builtin_amdgcn_mfma_f32_32x32x2f32(wv[sq & 1][o][e], xv[sq & 1][e][p], acc[o][p], 0, 0, 0);
+            }
             __builtin_amdgcn_sched_barrier(0);
         }
     };

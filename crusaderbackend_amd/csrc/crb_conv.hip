@@ -454,8 +454,8 @@ static int tap_grid_for(u32 nfh, u32 nfw) {
             best = i;
     return best;
 }
-// `together`: all classes in one launch on the smallest tap grid that holds them all (the smaller classes multiply zero
-// taps, but a small layer fills the chip with one launch); otherwise one launch per tap grid.
+// `together`: all classes in one launch on the smallest tap grid that holds them all (a workgroup skips the steps of the taps
+// its class does not have; one launch fills the chip where four would not); otherwise one launch per tap grid.
 static int dgrad_by_tiled_classes(const float *W, const float *dY, float *dX, const crb_conv_geom *g, bool together, hipStream_t s) {
     const char *what = "crb_conv_dgrad";
     TiledClass cls[kMaxTiledClasses];
@@ -510,7 +510,7 @@ static int dgrad_by_tiled_classes(const float *W, const float *dY, float *dX, co
 }
 // The launches must bring work: 128 workgroups over the classes (24 and 16 contraction channels, 64 on class grids up to 8 x 8,
 // when there is a single class, as for 1x1 filters), tiles at least a quarter full, five contraction channels. `together`: a class
-// brings fewer than 512 workgroups, so all classes share one launch. Against the engine's class launches / its one gather over all
+// brings fewer than 1024 workgroups, so all classes share one launch (the steps of the taps a class does not have are skipped). Against the engine's class launches / its one gather over all
 // taps on random layers: 32 -> 16 @56 5x5 stride 3 batch 128 317 -> 85 us, 256 -> 32 @28 7x7 stride 2 batch 32 261 -> 97,
 // 64 -> 256 @14 2x2 stride 2 batch 128 131 -> 23, 3 -> 128 @28 4x4 stride 2 batch 128 208 -> 60; class grids that fill their
 // tiles less stay with the engine (256 -> 32 @8 7x7 stride 3 batch 32, 3 x 3 pixel classes on 8 x 8 tiles: 55 against 115 us).
@@ -525,7 +525,7 @@ static bool tiled_classes_pay(const crb_conv_geom *g, bool *together = nullptr) 
     const uint64_t tiles = small ? uint64_t(g->N) : uint64_t(g->N) * ceil_div(CH, 8u) * ceil_div(CW, 16u);
     const uint64_t wgs = tiles * ceil_div(g->IC, small ? 64u : 32u);  // per class
     const uint64_t padded = small ? 64 : uint64_t(ceil_div(CH, 8u)) * 8 * ceil_div(CW, 16u) * 16;
-    if (together) *together = wgs < 512;
+    if (together) *together = wgs < 1024;
     // (8 -> 3 @64 1x1 stride 2 batch 4: 6.8 against 4.3 us; 32 -> 256 @16 1x1 stride 2 batch 32, 8 x 8 class grid: 16.6 against 10.4)
     if (nc == 1) return wgs >= 24 && g->OC >= (small ? 64u : 16u);
     return wgs * nc >= 128 && 4 * uint64_t(CH) * CW >= padded;

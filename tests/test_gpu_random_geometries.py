@@ -136,9 +136,11 @@ TILED_CLASSES = [
     (24, 64, 32, 32, 8, 7, 7, 2, 2, 3, 3), (48, 24, 48, 48, 20, 3, 3, 3, 3, 1, 1), (96, 64, 16, 16, 32, 2, 2, 2, 2, 0, 0),
     (8, 96, 20, 20, 32, 1, 1, 2, 2, 0, 0), (16, 70, 17, 23, 40, 1, 1, 3, 3, 0, 0), (32, 32, 20, 20, 16, 3, 3, 2, 1, 1, 1),
     (24, 48, 24, 24, 16, 3, 5, 2, 2, 1, 2), (100, 36, 15, 15, 24, 2, 2, 2, 2, 1, 1), (24, 40, 29, 29, 17, 4, 4, 2, 2, 0, 0),
-    # 512 workgroups per class: one launch per tap grid (1x1, 1x2, 2x1, 2x2 / 2x2 ... 3x3 / 3x3 ... 4x4 / a class without a grid of its own)
-    (128, 64, 30, 30, 8, 3, 3, 2, 2, 1, 1), (128, 64, 28, 28, 8, 5, 5, 2, 2, 2, 2), (128, 64, 28, 28, 6, 7, 7, 2, 2, 3, 3),
-    (128, 64, 45, 45, 8, 4, 4, 3, 3, 1, 1), (128, 64, 28, 28, 8, 3, 5, 2, 2, 1, 2),
+    # 1024 workgroups per class: one launch per tap grid (1x1, 1x2, 2x1, 2x2 / 2x2 ... 3x3 / 3x3 ... 4x4 / a class without a grid of its own)
+    (256, 64, 30, 30, 8, 3, 3, 2, 2, 1, 1), (256, 64, 28, 28, 8, 5, 5, 2, 2, 2, 2), (256, 64, 28, 28, 6, 7, 7, 2, 2, 3, 3),
+    (256, 64, 45, 45, 8, 4, 4, 3, 3, 1, 1), (256, 64, 28, 28, 8, 3, 5, 2, 2, 1, 2),
+    # the same layers at half the batch: all classes in one launch on the shared tap grid, absent taps skipped
+    (128, 64, 30, 30, 8, 3, 3, 2, 2, 1, 1), (128, 64, 28, 28, 8, 5, 5, 2, 2, 2, 2), (128, 64, 28, 28, 8, 3, 5, 2, 2, 1, 2),
     # class grids that 4 x 32 tiles pad less than 8 x 16 ones
     (24, 16, 56, 56, 8, 3, 3, 2, 2, 1, 1), (8, 40, 55, 57, 8, 5, 5, 2, 2, 2, 2),
 ]
